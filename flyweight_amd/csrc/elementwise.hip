@@ -1,0 +1,239 @@
+// Row-wise kernels: embedding gather, RMS norm, SwiGLU, rotation tables, argmax/top-k.
+// All reductions run in float32 in an order fixed by the row alone.
+#include "fw_common.h"
+#include "fw_kernels.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+// ---- error channel ---------------------------------------------------------------------
+static thread_local char fw_error_text[1024] = "";
+
+void fw_set_error(const char* format, ...) {
+    va_list args;
+    va_start(args, format);
+    vsnprintf(fw_error_text, sizeof(fw_error_text), format, args);
+    va_end(args);
+}
+extern "C" const char* fw_last_error(void) { return fw_error_text; }
+extern "C" int fw_abi_version(void) { return 1; }
+
+// ---- embedding -------------------------------------------------------------------------
+// The reference gathers one row per token and widens it to float32
+// (native/include/flyweight_v2_native_kernels.hpp:98-151).
+template <typename W>
+__global__ void embed_rows_kernel(const W* __restrict__ table, const int32_t* __restrict__ ids,
+                                  float* __restrict__ out, int hidden) {
+    const int row = blockIdx.y;
+    const size_t base = (size_t)ids[row] * hidden;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < hidden; i += gridDim.x * blockDim.x)
+        out[(size_t)row * hidden + i] = load_as_float(table, base + i);
+}
+
+extern "C" int fw_embed_rows(const void* table, int table_dtype, const int32_t* ids, float* out,
+                             int rows, int hidden, int vocab, void* stream) {
+    FW_REQUIRE(rows >= 0 && hidden > 0 && vocab > 0, "embed_rows: bad sizes rows=%d hidden=%d vocab=%d", rows, hidden, vocab);
+    FW_REQUIRE(rows <= 65535, "embed_rows: at most 65535 rows per call, got %d", rows);
+    if (rows == 0) return 0;
+    dim3 grid(fw_ceil_div(hidden, 256) > 64 ? 64 : fw_ceil_div(hidden, 256), rows);
+    if (table_dtype == FW_F32)
+        embed_rows_kernel<float><<<grid, 256, 0, (hipStream_t)stream>>>((const float*)table, ids, out, hidden);
+    else if (table_dtype == FW_BF16)
+        embed_rows_kernel<bf16_t><<<grid, 256, 0, (hipStream_t)stream>>>((const bf16_t*)table, ids, out, hidden);
+    else
+        FW_REQUIRE(false, "embed_rows: unknown table dtype %d", table_dtype);
+    FW_LAUNCH_CHECK("embed_rows");
+    return 0;
+}
+
+// ---- RMS norm --------------------------------------------------------------------------
+// y = x * rsqrt(mean(x^2) + eps) * w; the weight multiplies directly unless one_centered
+// (native/include/flyweight_v2_qwen_kernels.hpp:425-447, rows variant :1180-1207).
+template <typename T>
+__global__ void rmsnorm_rows_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                                    T* __restrict__ out, const int32_t* __restrict__ row_index,
+                                    int hidden, float eps, int one_centered) {
+    __shared__ float scratch[16];
+    const int row = blockIdx.x;
+    const size_t src = (size_t)(row_index ? row_index[row] : row) * hidden;
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float v = x[src + i];
+        sum += v * v;
+    }
+    sum = block_sum(sum, scratch);
+    const float inv = rsqrtf(sum / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float w = one_centered ? 1.0f + weight[i] : weight[i];
+        store_from_float(out, (size_t)row * hidden + i, x[src + i] * inv * w);
+    }
+}
+
+extern "C" int fw_rmsnorm_rows(const float* x, const float* weight, void* out, int out_dtype,
+                               const int32_t* row_index, int rows, int hidden, float eps,
+                               int one_centered, void* stream) {
+    FW_REQUIRE(rows >= 0 && hidden > 0, "rmsnorm_rows: bad sizes rows=%d hidden=%d", rows, hidden);
+    FW_REQUIRE(eps > 0.0f, "rmsnorm_rows: eps must be positive");
+    if (rows == 0) return 0;
+    if (out_dtype == FW_F32)
+        rmsnorm_rows_kernel<float><<<rows, 256, 0, (hipStream_t)stream>>>(x, weight, (float*)out, row_index, hidden, eps, one_centered);
+    else if (out_dtype == FW_BF16)
+        rmsnorm_rows_kernel<bf16_t><<<rows, 256, 0, (hipStream_t)stream>>>(x, weight, (bf16_t*)out, row_index, hidden, eps, one_centered);
+    else
+        FW_REQUIRE(false, "rmsnorm_rows: unknown out dtype %d", out_dtype);
+    FW_LAUNCH_CHECK("rmsnorm_rows");
+    return 0;
+}
+
+// ---- SwiGLU ----------------------------------------------------------------------------
+// silu(g) * u with a sigmoid that cannot overflow
+// (native/include/flyweight_v2_qwen_kernels.hpp:1209-1223).
+__device__ __forceinline__ float stable_sigmoid(float g) {
+    if (g >= 0.0f) return 1.0f / (1.0f + expf(-g));
+    const float e = expf(g);
+    return e / (1.0f + e);
+}
+
+template <typename T>
+__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int intermediate) {
+    const int row = blockIdx.y;
+    const T* source = gate_up + (size_t)row * 2 * intermediate;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < intermediate; i += gridDim.x * blockDim.x) {
+        const float g = load_as_float(source, i);
+        const float u = load_as_float(source, (size_t)intermediate + i);
+        store_from_float(out, (size_t)row * intermediate + i, g * stable_sigmoid(g) * u);
+    }
+}
+
+extern "C" int fw_swiglu(const void* gate_up, void* out, int dtype, int rows, int intermediate, void* stream) {
+    FW_REQUIRE(rows >= 0 && intermediate > 0, "swiglu: bad sizes rows=%d width=%d", rows, intermediate);
+    FW_REQUIRE(rows <= 65535, "swiglu: at most 65535 rows per call, got %d", rows);
+    if (rows == 0) return 0;
+    int bx = fw_ceil_div(intermediate, 256);
+    if (bx > 32) bx = 32;
+    dim3 grid(bx, rows);
+    if (dtype == FW_F32)
+        swiglu_kernel<float><<<grid, 256, 0, (hipStream_t)stream>>>((const float*)gate_up, (float*)out, intermediate);
+    else if (dtype == FW_BF16)
+        swiglu_kernel<bf16_t><<<grid, 256, 0, (hipStream_t)stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate);
+    else
+        FW_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
+    FW_LAUNCH_CHECK("swiglu");
+    return 0;
+}
+
+// ---- rotation tables -------------------------------------------------------------------
+// angle = position * theta^(-2i/d) (native/include/flyweight_v2_native_kernels.hpp:993-1008
+// computes the same angle per element in float32). The product is formed in float64 so that
+// a large position does not lose the low bits of the angle; cos and sin are float32.
+__global__ void rope_table_kernel(const int32_t* __restrict__ positions, const double* __restrict__ inv_freq,
+                                  float* __restrict__ cos_out, float* __restrict__ sin_out, int rows, int half) {
+    const int index = blockIdx.x * blockDim.x + threadIdx.x;
+    if (index >= rows * half) return;
+    const int row = index / half;
+    const int pair = index - row * half;
+    const double angle = (double)positions[row] * inv_freq[pair];
+    cos_out[index] = (float)cos(angle);
+    sin_out[index] = (float)sin(angle);
+}
+
+extern "C" int fw_rope_table(const int32_t* positions, const double* inv_freq, float* cos_out, float* sin_out,
+                             int rows, int half, void* stream) {
+    FW_REQUIRE(rows >= 0 && half > 0, "rope_table: bad sizes rows=%d half=%d", rows, half);
+    if (rows == 0) return 0;
+    const long long total = (long long)rows * half;
+    rope_table_kernel<<<fw_ceil_div(total, 256), 256, 0, (hipStream_t)stream>>>(positions, inv_freq, cos_out, sin_out, rows, half);
+    FW_LAUNCH_CHECK("rope_table");
+    return 0;
+}
+
+// ---- argmax / top-k --------------------------------------------------------------------
+// A candidate is ordered by (value descending, id ascending); NaN sorts last. The key packs
+// both so that one 64-bit max finds the winner, as the reference's fused LM-head argmax
+// does (native/include/flyweight_v2_qwen_kernels.hpp:2391-2405): ties go to the lowest id.
+__device__ __forceinline__ unsigned long long candidate_key(float value, int id) {
+    uint32_t bits = __float_as_uint(value);
+    uint32_t ordered;
+    if (value != value) ordered = 0u;                                   // NaN: below everything
+    else ordered = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u); // monotone in value
+    return ((unsigned long long)ordered << 32) | (unsigned long long)(0xffffffffu - (uint32_t)id);
+}
+
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) {
+        const unsigned long long other = __shfl_xor(v, offset, 64);
+        v = other > v ? other : v;
+    }
+    return v;
+}
+
+__device__ __forceinline__ unsigned long long block_max_u64(unsigned long long v, unsigned long long* scratch) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = (blockDim.x + 63) >> 6;
+    v = wave_max_u64(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    unsigned long long best = 0;
+    for (int i = 0; i < waves; ++i) best = scratch[i] > best ? scratch[i] : best;
+    return best;
+}
+
+// One block per row; `k` rounds, each picks the best key strictly below the last winner.
+__global__ void topk_rows_kernel(const float* __restrict__ logits, float* __restrict__ values,
+                                 int32_t* __restrict__ ids, int vocab, int k) {
+    __shared__ unsigned long long scratch[16];
+    const int row = blockIdx.x;
+    const float* source = logits + (size_t)row * vocab;
+    unsigned long long ceiling = ~0ull;
+    for (int round = 0; round < k; ++round) {
+        unsigned long long best = 0;
+        for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+            const unsigned long long key = candidate_key(source[i], i);
+            if (key < ceiling && key > best) best = key;
+        }
+        best = block_max_u64(best, scratch);
+        if (threadIdx.x == 0) {
+            const int id = (int)(0xffffffffu - (uint32_t)(best & 0xffffffffull));
+            ids[(size_t)row * k + round] = id;
+            if (values) values[(size_t)row * k + round] = source[id];
+        }
+        ceiling = best;
+    }
+}
+
+extern "C" int fw_topk_rows(const float* logits, float* values, int32_t* ids, int rows, int vocab, int k,
+                            void* stream) {
+    FW_REQUIRE(rows >= 0 && vocab > 0, "topk_rows: bad sizes rows=%d vocab=%d", rows, vocab);
+    FW_REQUIRE(k >= 1 && k <= vocab && k <= 256, "topk_rows: k must be in 1..min(256, vocab), got %d", k);
+    if (rows == 0) return 0;
+    topk_rows_kernel<<<rows, 1024, 0, (hipStream_t)stream>>>(logits, values, ids, vocab, k);
+    FW_LAUNCH_CHECK("topk_rows");
+    return 0;
+}
+
+extern "C" int fw_argmax_rows(const float* logits, int32_t* ids, int rows, int vocab, void* stream) {
+    FW_REQUIRE(rows >= 0 && vocab > 0, "argmax_rows: bad sizes rows=%d vocab=%d", rows, vocab);
+    if (rows == 0) return 0;
+    topk_rows_kernel<<<rows, 1024, 0, (hipStream_t)stream>>>(logits, nullptr, ids, vocab, 1);
+    FW_LAUNCH_CHECK("argmax_rows");
+    return 0;
+}
+
+// ---- fill ------------------------------------------------------------------------------
+__global__ void fill_zero_kernel(uint32_t* __restrict__ ptr, long long words) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < words;
+         i += (long long)gridDim.x * blockDim.x)
+        ptr[i] = 0u;
+}
+
+extern "C" int fw_fill_zero(void* ptr, long long bytes, void* stream) {
+    FW_REQUIRE(bytes >= 0 && bytes % 4 == 0, "fill_zero: byte count %lld must be a multiple of 4", bytes);
+    if (bytes == 0) return 0;
+    const long long words = bytes / 4;
+    int blocks = fw_ceil_div(words, 256);
+    if (blocks > 2048) blocks = 2048;
+    fill_zero_kernel<<<blocks, 256, 0, (hipStream_t)stream>>>((uint32_t*)ptr, words);
+    FW_LAUNCH_CHECK("fill_zero");
+    return 0;
+}

@@ -1,0 +1,99 @@
+// Shared device helpers for the gfx950 kernels: storage types, conversions, wave64
+// reductions, and the error channel behind the flat C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// dtype codes used across the C ABI
+#define FW_F32 0
+#define FW_BF16 1
+
+// ---- error channel: every entry point returns 0 or -1 and leaves a message ---------
+void fw_set_error(const char* format, ...);
+#define FW_REQUIRE(cond, ...)                    \
+    do {                                         \
+        if (!(cond)) {                           \
+            fw_set_error(__VA_ARGS__);           \
+            return -1;                           \
+        }                                        \
+    } while (0)
+#define FW_LAUNCH_CHECK(name)                                                     \
+    do {                                                                          \
+        hipError_t fw_status__ = hipGetLastError();                               \
+        if (fw_status__ != hipSuccess) {                                          \
+            fw_set_error("%s: launch failed: %s", name, hipGetErrorString(fw_status__)); \
+            return -1;                                                            \
+        }                                                                         \
+    } while (0)
+
+// ---- bfloat16 as raw bits ----------------------------------------------------------
+struct bf16_t {
+    uint16_t bits;
+};
+
+__device__ __forceinline__ float bf16_to_float(bf16_t v) {
+    return __uint_as_float(((uint32_t)v.bits) << 16);
+}
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t bits) {
+    return __uint_as_float(bits << 16);
+}
+// round to nearest, ties to even; NaN stays NaN
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ bf16_t float_to_bf16(float f) {
+    bf16_t r;
+    r.bits = float_to_bf16_bits(f);
+    return r;
+}
+
+template <typename T> __device__ __forceinline__ float load_as_float(const T* p, size_t i);
+template <> __device__ __forceinline__ float load_as_float<float>(const float* p, size_t i) { return p[i]; }
+template <> __device__ __forceinline__ float load_as_float<bf16_t>(const bf16_t* p, size_t i) {
+    return bf16_to_float(p[i]);
+}
+template <typename T> __device__ __forceinline__ void store_from_float(T* p, size_t i, float v);
+template <> __device__ __forceinline__ void store_from_float<float>(float* p, size_t i, float v) { p[i] = v; }
+template <> __device__ __forceinline__ void store_from_float<bf16_t>(bf16_t* p, size_t i, float v) {
+    p[i] = float_to_bf16(v);
+}
+// the value a store of this type would leave behind (used where a value is both kept
+// in registers and written, so later reads from memory see the same number)
+template <typename T> __device__ __forceinline__ float round_through(float v);
+template <> __device__ __forceinline__ float round_through<float>(float v) { return v; }
+template <> __device__ __forceinline__ float round_through<bf16_t>(float v) {
+    return bf16_bits_to_float(float_to_bf16_bits(v));
+}
+
+// ---- wave64 reductions (fixed butterfly order: the result does not depend on
+//      anything but the 64 inputs) -----------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, 64));
+    return v;
+}
+
+// block-wide sum for blocks of up to 1024 threads; every thread gets the result
+__device__ __forceinline__ float block_sum(float v, float* scratch /* >= 16 floats */) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int waves = (blockDim.x + 63) >> 6;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    float total = 0.0f;
+    for (int i = 0; i < waves; ++i) total += scratch[i];
+    return total;
+}
+
+static inline int fw_ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }

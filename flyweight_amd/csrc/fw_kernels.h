@@ -1,0 +1,77 @@
+// Flat C ABI of the gfx950 kernel library. Every pointer is a device pointer unless a
+// comment says otherwise; `stream` is a hipStream_t. Every function returns 0 on success
+// and -1 on failure, after which fw_last_error() describes what was refused. Shapes are
+// checked on the host before anything is launched; a kernel never runs on operands it
+// was not written for.
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* fw_last_error(void);
+int fw_abi_version(void);
+
+// out[r][:] = table[ids[r]][:]  (float32 out: the residual stream)
+int fw_embed_rows(const void* table, int table_dtype, const int32_t* ids, float* out,
+                  int rows, int hidden, int vocab, void* stream);
+
+// RMS norm of float32 rows: out[r] = x[src] * rsqrt(mean(x[src]^2) + eps) * w, where
+// src = row_index ? row_index[r] : r.  one_centered: multiply by (1 + w) instead of w.
+int fw_rmsnorm_rows(const float* x, const float* weight, void* out, int out_dtype,
+                    const int32_t* row_index, int rows, int hidden, float eps,
+                    int one_centered, void* stream);
+
+// out = a[M][K] . w[N][K]^T (+ bias[N]); out_mode 0: store in out_dtype,
+// 1: out (float32) += result (the residual sum).
+int fw_gemm_generic(const void* a, int a_dtype, const void* w, int w_dtype, const float* bias,
+                    void* out, int out_dtype, int out_mode, int M, int N, int K, void* stream);
+
+// out[r][i] = silu(gu[r][i]) * gu[r][I + i]
+int fw_swiglu(const void* gate_up, void* out, int dtype, int rows, int intermediate, void* stream);
+
+// cos/sin of position * inv_freq for every row: tables [rows][half]
+int fw_rope_table(const int32_t* positions, const double* inv_freq, float* cos_out, float* sin_out,
+                  int rows, int half, void* stream);
+
+// Gated short convolution over a mixed batch. bcx [rows][3H] = (B | C | x); taps [H][L]
+// oldest first; conv_bias [H] or null; state [slots][H][L-1] float32, oldest first.
+// Row r belongs to segment row_seg[r]; segment s covers rows seg_row0[s]..seg_row0[s+1]
+// and continues the sequence whose state lives in slot seg_slot[s].
+int fw_shortconv(const void* bcx, void* out, int dtype, const float* taps, const float* conv_bias,
+                 float* state, const int32_t* row_seg, const int32_t* seg_row0,
+                 const int32_t* seg_slot, int rows, int segments, int hidden, int kernel_size,
+                 int slots, void* stream);
+
+// Per-head RMS norm of q and k (weights may be null: no norm), half-split rotation of the
+// first rotary_dim channels by the row's angle, q out, k and v appended to the pages of
+// the row's segment. qkv [rows][(nh + 2 nkv) hd]. k_pages [pages][nkv][P][hd];
+// v_pages [pages][nkv][hd][P]. block_table [segments][table_stride].
+int fw_qk_norm_rope_kv_write(const void* qkv, void* q_out, int dtype, const float* q_norm_weight,
+                             const float* k_norm_weight, float eps, const float* cos_table,
+                             const float* sin_table, int rotary_dim, void* k_pages, void* v_pages,
+                             const int32_t* block_table, int table_stride, const int32_t* row_seg,
+                             const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
+                             int head_dim, int page_size, int num_pages, int write_kv, void* stream);
+
+// Causal attention of every row over the cached keys 0..row_pos[r] (or the last `window`
+// of them) of its segment. out [rows][nh*hd].
+int fw_attention_generic(const void* q, void* out, int dtype, const void* k_pages,
+                         const void* v_pages, const int32_t* block_table, int table_stride,
+                         const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
+                         int num_kv_heads, int head_dim, float scale, int window, int page_size,
+                         int num_pages, void* stream);
+
+// ids[r] = argmax(logits[r]) with ties to the lowest id
+int fw_argmax_rows(const float* logits, int32_t* ids, int rows, int vocab, void* stream);
+
+// the k largest logits of every row, sorted by (value descending, id ascending)
+int fw_topk_rows(const float* logits, float* values, int32_t* ids, int rows, int vocab, int k,
+                 void* stream);
+
+int fw_fill_zero(void* ptr, long long bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif

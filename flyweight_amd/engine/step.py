@@ -1,0 +1,188 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+A step holds *segments*: a request's next ``n >= 1`` tokens, whether a portion of its
+prompt or one decoded token. Any mix, cut anywhere. The step runs only the tokens it is
+given, against the cache earlier steps left, appends to that cache, and returns float32
+logits at the wanted places. The reference has three disjoint entry points instead (one
+token -> argmax, native/src/v2_runtime.cpp:27525; R rows of one sequence without logits,
+native/src/v2_mtp_verifier.inc:4086-4121) and never a mixed batch.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import CacheManager, OutOfPages
+from .model import CacheView, CausalLM
+
+
+class StepError(ValueError):
+    pass
+
+
+@dataclass
+class StepEntry:
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()       # places among ``tokens`` whose logits are asked for
+
+
+class StepContext:
+    """The batch as the kernels see it: per-row and per-segment index arrays on the
+    device (one upload), block tables per page group, and per-step tables of the position
+    encodings."""
+
+    def __init__(self, entries: Sequence[StepEntry], cache: CacheManager, device: torch.device, vocab_size: int,
+                 max_positions: int):
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        seen = set()
+        tokens: List[int] = []
+        row_pos: List[int] = []
+        row_seg: List[int] = []
+        seg_row0: List[int] = [0]
+        seg_slot: List[int] = []
+        want_rows: List[int] = []
+        self.requests: List[Hashable] = []
+        self.new_lengths: List[int] = []
+        for seg, entry in enumerate(entries):
+            if entry.request in seen:
+                raise StepError(f"request {entry.request!r} appears twice in one step")
+            seen.add(entry.request)
+            n = len(entry.tokens)
+            if n < 1:
+                raise StepError(f"request {entry.request!r} brings no tokens")
+            start = cache.length_of(entry.request)
+            if start + n > max_positions:
+                raise StepError(f"request {entry.request!r} would reach {start + n} tokens; the model's limit is {max_positions}")
+            for t in entry.tokens:
+                if not 0 <= int(t) < vocab_size:
+                    raise StepError(f"token id {t} of request {entry.request!r} is outside the vocabulary (0..{vocab_size - 1})")
+            for place in entry.want:
+                if not 0 <= int(place) < n:
+                    raise StepError(f"request {entry.request!r} wants logits at place {place} of {n} tokens")
+                want_rows.append(len(tokens) + int(place))
+            tokens.extend(int(t) for t in entry.tokens)
+            row_pos.extend(range(start, start + n))
+            row_seg.extend([seg] * n)
+            seg_row0.append(len(tokens))
+            seg_slot.append(cache.slot_of(entry.request))
+            self.requests.append(entry.request)
+            self.new_lengths.append(start + n)
+        self.num_rows = len(tokens)
+        self.num_segments = len(entries)
+        self.num_wanted = len(want_rows)
+        self.all_decode = self.num_rows == self.num_segments
+        self.max_context = max(self.new_lengths)
+        self.device = device
+        self.host_row_pos = row_pos
+        self.host_seg_row0 = seg_row0
+
+        tables = [cache.block_table_rows(g, self.requests) for g in range(len(cache.groups))]
+        pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows)]
+        pieces += [t.reshape(-1) for t in tables]
+        packed = torch.from_numpy(np.concatenate(pieces)).to(device)
+        views = []
+        offset = 0
+        for piece in pieces:
+            views.append(packed[offset:offset + piece.size])
+            offset += piece.size
+        (self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows) = views[:6]
+        self.block_tables = [v.view(t.shape) for v, t in zip(views[6:], tables)]
+        self._position_tables: Dict = {}
+
+    def position_tables(self, part):
+        key = part.key()
+        if key not in self._position_tables:
+            self._position_tables[key] = part.tables(self)
+        return self._position_tables[key]
+
+    def cache_view(self, cache: CacheManager, entry) -> CacheView:
+        if entry.cache is None:
+            return CacheView(writes=False)
+        if entry.cache in cache.entry_group:
+            return CacheView(k_pages=cache.k_pages[entry.cache], v_pages=cache.v_pages[entry.cache],
+                             block_table=self.block_tables[cache.entry_group[entry.cache]], writes=entry.writes_cache)
+        if entry.cache in cache.state:
+            return CacheView(state=cache.state[entry.cache], writes=entry.writes_cache)
+        return CacheView(writes=entry.writes_cache)
+
+
+class Stepper:
+    """Owns the model's cache and runs steps. ``admit`` a request before its first step,
+    ``release`` it when it ends."""
+
+    def __init__(self, model: CausalLM, num_pages: int, max_requests: int, page_size: int = 64):
+        if not model.bound:
+            raise StepError("the model has no weights yet")
+        self.model = model
+        self.device = model.device
+        max_pages = (model.spec.max_positions + page_size - 1) // page_size
+        self.cache = CacheManager(model.cache_needs(), num_pages=num_pages, max_requests=max_requests,
+                                  page_size=page_size, max_pages_per_request=max_pages, dtype=model.dtype,
+                                  device=model.device)
+        self.steps = 0
+        self.tokens_run = 0
+
+    def admit(self, request: Hashable) -> None:
+        self.cache.admit(request)
+
+    def release(self, request: Hashable) -> None:
+        self.cache.release(request)
+
+    def is_live(self, request: Hashable) -> bool:
+        return request in self.cache.requests
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Returns float32 logits [wanted, vocab] on the device, rows in the order of the
+        entries and of each entry's ``want`` (None if nothing is wanted). Raises
+        OutOfPages, having changed nothing, when the cache cannot hold the new tokens."""
+        cache = self.cache
+        spec = self.model.spec
+        if not entries:
+            raise StepError("a step needs at least one entry")
+        seen = set()
+        for entry in entries:
+            if entry.request not in cache.requests:
+                raise StepError(f"request {entry.request!r} was not admitted")
+            if entry.request in seen:
+                raise StepError(f"request {entry.request!r} appears twice in one step")
+            seen.add(entry.request)
+            if len(entry.tokens) < 1:
+                raise StepError(f"request {entry.request!r} brings no tokens")
+            if cache.length_of(entry.request) + len(entry.tokens) > spec.max_positions:
+                raise StepError(f"request {entry.request!r} would reach "
+                                f"{cache.length_of(entry.request) + len(entry.tokens)} tokens; the model's limit is "
+                                f"{spec.max_positions}")
+            for t in entry.tokens:
+                if not 0 <= int(t) < spec.vocab_size:
+                    raise StepError(f"token id {t} of request {entry.request!r} is outside the vocabulary "
+                                    f"(0..{spec.vocab_size - 1})")
+            for place in entry.want:
+                if not 0 <= int(place) < len(entry.tokens):
+                    raise StepError(f"request {entry.request!r} wants logits at place {place} of {len(entry.tokens)} tokens")
+        # reserve everything first so that a failure leaves no request half-served
+        needed = {g: 0 for g in range(len(cache.groups))}
+        for entry in entries:
+            new_length = cache.length_of(entry.request) + len(entry.tokens)
+            if cache.pages_for(new_length) > cache.max_pages_per_request:
+                raise OutOfPages(f"request {entry.request!r} would need {cache.pages_for(new_length)} pages; "
+                                 f"a block table holds {cache.max_pages_per_request}")
+            for g, count in cache.pages_missing(entry.request, new_length).items():
+                needed[g] += count
+        for g, count in needed.items():
+            if cache.groups[g].pool.free_count < count:
+                raise OutOfPages(f"out of cache pages: the step needs {count} more, {cache.groups[g].pool.free_count} free")
+        for entry in entries:
+            cache.reserve(entry.request, cache.length_of(entry.request) + len(entry.tokens))
+        ctx = StepContext(entries, cache, self.device, self.model.spec.vocab_size, self.model.spec.max_positions)
+        logits = self.model.forward(ctx, cache)
+        for request, length in zip(ctx.requests, ctx.new_lengths):
+            cache.commit(request, length)
+        self.steps += 1
+        self.tokens_run += ctx.num_rows
+        return logits

@@ -1,0 +1,147 @@
+"""Builds the gfx950 kernel library from ``csrc/*.hip`` with hipcc.
+
+The library is built in-tree (``csrc/_build/libflyweight_hip.so``) so that it travels
+with the source tree; when the tree is not writable it is built under the temporary
+folder instead. ``ensure_built()`` builds only when no current library is found, and
+prints a line per file meanwhile, since a first build takes a minute or two.
+"""
+
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+from concurrent.futures import ThreadPoolExecutor
+from typing import List, Optional
+
+CSRC = os.path.normpath(os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "csrc"))
+LIB_NAME = "libflyweight_hip.so"
+ARCH = "gfx950"
+# packed float32 instructions are switched off: the compiler otherwise forms them from
+# ordinary float code
+FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature",
+         "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+
+
+def _say(text: str) -> None:
+    print(f"[flyweight_amd] {text}", file=sys.stderr, flush=True)
+
+
+def sources() -> List[str]:
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def _fingerprint() -> str:
+    digest = hashlib.sha256()
+    for path in sources() + sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")):
+        digest.update(os.path.basename(path).encode())
+        with open(path, "rb") as handle:
+            digest.update(handle.read())
+    digest.update(" ".join(FLAGS).encode())
+    return digest.hexdigest()
+
+
+def _hipcc() -> str:
+    found = shutil.which("hipcc")
+    if found:
+        return found
+    for candidate in ("/opt/rocm/bin/hipcc",):
+        if os.path.isfile(candidate):
+            return candidate
+    raise RuntimeError("hipcc not found: the gfx950 kernels cannot be built")
+
+
+def build_dirs() -> List[str]:
+    uid = os.getuid() if hasattr(os, "getuid") else 0
+    return [os.path.join(CSRC, "_build"),
+            os.path.join(tempfile.gettempdir(), f"flyweight_amd_build_{uid}")]
+
+
+def find_library(require_current: bool = True) -> Optional[str]:
+    wanted = _fingerprint() if require_current else None
+    for folder in build_dirs():
+        lib = os.path.join(folder, LIB_NAME)
+        stamp = os.path.join(folder, "build.stamp")
+        if not os.path.isfile(lib):
+            continue
+        if wanted is None:
+            return lib
+        if os.path.isfile(stamp):
+            with open(stamp, "r", encoding="utf-8") as handle:
+                if handle.read().strip() == wanted:
+                    return lib
+    return None
+
+
+def _writable_dir() -> str:
+    for folder in build_dirs():
+        try:
+            os.makedirs(folder, exist_ok=True)
+            probe = os.path.join(folder, f".probe_{os.getpid()}")
+            with open(probe, "w") as handle:
+                handle.write("x")
+            os.remove(probe)
+            return folder
+        except OSError:
+            continue
+    raise RuntimeError("no writable folder to build the kernel library in")
+
+
+def build(verbose: bool = True) -> str:
+    """Compile every source and link the library; returns its path."""
+    hipcc = _hipcc()
+    folder = _writable_dir()
+    files = sources()
+    started = time.time()
+    if verbose:
+        _say(f"building {LIB_NAME} for {ARCH} from {len(files)} sources in {folder}")
+    env = dict(os.environ)
+    env.setdefault("HOME", tempfile.gettempdir())
+
+    def compile_one(path: str) -> str:
+        obj = os.path.join(folder, os.path.basename(path)[:-4] + ".o")
+        begun = time.time()
+        result = subprocess.run([hipcc, *FLAGS, "-c", path, "-o", obj], capture_output=True, text=True, env=env)
+        if result.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {path}:\n{result.stderr}")
+        if verbose:
+            _say(f"  compiled {os.path.basename(path)} in {time.time() - begun:.0f} s")
+        return obj
+
+    workers = max(1, min(8, len(files), (os.cpu_count() or 2)))
+    with ThreadPoolExecutor(max_workers=workers) as pool:
+        objects = list(pool.map(compile_one, files))
+    lib = os.path.join(folder, LIB_NAME)
+    partial = lib + f".{os.getpid()}.tmp"
+    result = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", partial, *objects],
+                            capture_output=True, text=True, env=env)
+    if result.returncode != 0:
+        raise RuntimeError(f"linking {LIB_NAME} failed:\n{result.stderr}")
+    os.replace(partial, lib)
+    with open(os.path.join(folder, "build.stamp"), "w", encoding="utf-8") as handle:
+        handle.write(_fingerprint())
+    if verbose:
+        _say(f"built {lib} in {time.time() - started:.0f} s")
+    return lib
+
+
+def ensure_built() -> str:
+    lib = find_library(require_current=True)
+    if lib is not None:
+        return lib
+    try:
+        return build()
+    except RuntimeError:
+        stale = find_library(require_current=False)
+        if stale is not None:
+            _say(f"warning: could not rebuild; loading {stale}, which is older than the sources")
+            return stale
+        raise
+
+
+if __name__ == "__main__":
+    build()

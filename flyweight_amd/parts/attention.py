@@ -1,0 +1,95 @@
+"""Grouped-query attention over the paged cache.
+
+q = W_q h, k = W_k h, v = W_v h; optional per-head RMS norm of q and k (one weight of
+head_dim shared by all heads); position encoding on q and k; k and v appended to the
+cache; scores q.k / sqrt(head_dim) over the cached keys the row may see (causal, optionally
+only the last ``window``), softmax in float32, weighted sum of values; out = W_o o.
+Query head i reads kv head i // (num_heads / num_kv_heads). Formulas as the reference's
+LFM2 attention branch computes them (native/src/v2_runtime.cpp:28429-28478).
+"""
+
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..cache.needs import PagedKV
+from ..config.spec import ConfigError
+from ..kernels import ops
+from ..weights.loader import TensorDecl
+from .base import Mixer, build_part, register_mixer
+from .linear import Linear
+
+_DEFAULT_NAMES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj", "q_norm": "q_norm", "k_norm": "k_norm"}
+
+
+@register_mixer("gqa_attention")
+class GQAttention(Mixer):
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.hidden = int(spec["hidden_size"])
+        self.num_heads = int(spec["num_heads"])
+        self.num_kv_heads = int(spec["num_kv_heads"])
+        self.head_dim = int(spec["head_dim"])
+        self.qk_norm = bool(spec.get("qk_norm", False))
+        self.qk_norm_eps = float(spec.get("qk_norm_eps", 1e-6)) if self.qk_norm else 1.0
+        self.window = spec.get("window")
+        self.scale = float(spec.get("softmax_scale", self.head_dim ** -0.5))
+        self.bias = bool(spec.get("bias", False))
+        self.names = {**_DEFAULT_NAMES, **dict(spec.get("names", {}))}
+        self.position = build_part("position", spec["position"])
+        if self.num_heads % self.num_kv_heads:
+            raise ConfigError(f"{self.num_heads} heads are not a multiple of {self.num_kv_heads} kv heads")
+        if self.head_dim > ops.MAX_HEAD_DIM:
+            raise ConfigError(f"head_dim {self.head_dim} exceeds the kernels' limit of {ops.MAX_HEAD_DIM}")
+        if self.window is not None and int(self.window) <= 0:
+            raise ConfigError("an attention window must be positive (or None for all keys)")
+
+    def cache_need(self):
+        return PagedKV(self.num_kv_heads, self.head_dim, None if self.window is None else int(self.window))
+
+    def _name(self, which: str, leaf: str = "weight") -> str:
+        return f"{self.prefix}{self.names[which]}.{leaf}"
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        q_width, kv_width = self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
+        declared = {
+            self._name("q"): TensorDecl((q_width, self.hidden)),
+            self._name("k"): TensorDecl((kv_width, self.hidden)),
+            self._name("v"): TensorDecl((kv_width, self.hidden)),
+            self._name("o"): TensorDecl((self.hidden, q_width)),
+        }
+        if self.bias:
+            declared[self._name("q", "bias")] = TensorDecl((q_width,), "vector", "bias")
+            declared[self._name("k", "bias")] = TensorDecl((kv_width,), "vector", "bias")
+            declared[self._name("v", "bias")] = TensorDecl((kv_width,), "vector", "bias")
+            declared[self._name("o", "bias")] = TensorDecl((self.hidden,), "vector", "bias")
+        if self.qk_norm:
+            declared[self._name("q_norm")] = TensorDecl((self.head_dim,), "vector", "norm")
+            declared[self._name("k_norm")] = TensorDecl((self.head_dim,), "vector", "norm")
+        return declared
+
+    def bind(self, tensors, dtype, device) -> None:
+        super().bind(tensors, dtype, device)
+        self.position.bind(tensors, dtype, device)
+        q, k, v = (tensors[self._name(n)] for n in ("q", "k", "v"))
+        if not (q.dtype == k.dtype == v.dtype):
+            raise ConfigError(f"{self.prefix}: q, k and v projections are stored in different precisions")
+        # one operand for the three projections: rows are q heads, then k heads, then v heads
+        bias = torch.cat([tensors[self._name(n, "bias")] for n in ("q", "k", "v")]) if self.bias else None
+        self.qkv = Linear(torch.cat([q, k, v], dim=0), bias)
+        self.out = Linear(tensors[self._name("o")], tensors[self._name("o", "bias")] if self.bias else None)
+        self.q_norm_weight = tensors[self._name("q_norm")] if self.qk_norm else None
+        self.k_norm_weight = tensors[self._name("k_norm")] if self.qk_norm else None
+
+    def forward(self, h, residual, ctx, cache) -> None:
+        qkv = self.qkv.forward(h)
+        cos, sin = ctx.position_tables(self.position)
+        q = ops.qk_norm_rope_kv_write(
+            qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight,
+            self.qk_norm_eps, cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table,
+            ctx.row_seg, ctx.row_pos, write_kv=cache.writes)
+        attended = ops.attention(q, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
+                                 cache.block_table, ctx, self.scale, int(self.window or 0))
+        self.out.accumulate(attended, residual)

@@ -1,0 +1,111 @@
+"""Interfaces of the parts a layer is made of, and the registries that map a part's
+``kind`` to its class.
+
+A part is built from a :class:`PartSpec` (its sizes and constants) and knows nothing of
+the model it sits in. It declares the tensors it needs by full checkpoint name, is bound
+to them once, and is then called by the step function with a :class:`StepContext` that
+describes the batch. To add a part, subclass one of the four bases and register it:
+
+* **Norm** - ``forward(x, ctx, row_index=None) -> h``: float32 rows in, activation dtype out.
+* **PositionEncoding** - ``tables(ctx)``: whatever the mixer's kernels need for the rows of
+  this step (computed once per step and shared by all layers with the same parameters).
+* **Mixer** - ``cache_need()`` says what per-request memory it needs (paged keys/values, a
+  fixed-size state, or nothing); ``forward(h, residual, ctx, cache)`` must ADD its output to
+  ``residual`` (float32, in place).
+* **FeedForward** - ``forward(h, residual, ctx)`` must ADD its output to ``residual``.
+
+The reference keeps the same seams as per-layer flags and tensor slots of one plan
+struct (native/src/v2_runtime.cpp:395-560,4177-4184).
+"""
+
+from __future__ import annotations
+
+from typing import Callable, Dict, Mapping, Optional, Type
+
+import torch
+
+from ..config.spec import ConfigError, PartSpec
+from ..weights.loader import TensorDecl
+
+
+class Part:
+    def __init__(self, spec: PartSpec):
+        self.spec = spec
+        self.prefix = spec.prefix
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        """Full checkpoint name -> declaration, for every tensor this part needs."""
+        return {}
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], dtype: torch.dtype, device: torch.device) -> None:
+        """Take the loaded tensors (already on ``device``); ``dtype`` is the activation dtype."""
+        self.dtype = dtype
+        self.device = device
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, ctx, row_index: Optional[torch.Tensor] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def key(self):
+        """Parts with equal keys share one set of per-step tables."""
+        return (type(self).__name__, tuple(sorted((k, v) for k, v in self.spec.params.items())))
+
+    def tables(self, ctx):
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_need(self):
+        return None
+
+    def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx, cache) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx) -> None:
+        raise NotImplementedError
+
+
+_REGISTRIES: Dict[str, Dict[str, Type[Part]]] = {"norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}}
+
+
+def _register(family: str, kind: str) -> Callable[[Type], Type]:
+    def decorate(cls: Type) -> Type:
+        _REGISTRIES[family][kind] = cls
+        return cls
+    return decorate
+
+
+def register_norm(kind: str):
+    return _register("norm", kind)
+
+
+def register_position_encoding(kind: str):
+    return _register("position", kind)
+
+
+def register_mixer(kind: str):
+    return _register("mixer", kind)
+
+
+def register_feed_forward(kind: str):
+    return _register("ffn", kind)
+
+
+def register_block(kind: str):
+    return _register("block", kind)
+
+
+def build_part(family: str, spec: PartSpec):
+    registry = _REGISTRIES[family]
+    if spec.kind not in registry:
+        raise ConfigError(f"unknown {family} kind '{spec.kind}'; registered: {', '.join(sorted(registry)) or 'none'}")
+    return registry[spec.kind](spec)
+
+
+def registered(family: str):
+    return tuple(sorted(_REGISTRIES[family]))

@@ -1,0 +1,44 @@
+"""The arrangement of parts in a layer.
+
+``pre_norm_residual``: x <- x + mixer(norm1(x)); x <- x + ffn(norm2(x)), the residual
+stream x in float32 (native/src/v2_runtime.cpp:28077,28282,28774,29133-29136). Another
+arrangement (post-norm, parallel mixer and feed-forward) is another class registered here.
+"""
+
+from __future__ import annotations
+
+from typing import Dict
+
+from ..weights.loader import TensorDecl
+from .base import build_part, register_block
+
+
+@register_block("pre_norm_residual")
+class PreNormResidualBlock:
+    def __init__(self, spec):
+        self.spec = spec
+        self.mixer_norm = build_part("norm", spec.mixer_norm)
+        self.mixer = build_part("mixer", spec.mixer)
+        self.ffn_norm = build_part("norm", spec.ffn_norm)
+        self.ffn = build_part("ffn", spec.ffn)
+
+    def parts(self):
+        return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        declared: Dict[str, TensorDecl] = {}
+        for part in self.parts():
+            declared.update(part.tensors())
+        return declared
+
+    def bind(self, tensors, dtype, device) -> None:
+        for part in self.parts():
+            part.bind(tensors, dtype, device)
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def forward(self, x, ctx, cache) -> None:
+        """``x`` [rows, hidden] float32 is updated in place."""
+        self.mixer.forward(self.mixer_norm.forward(x, ctx), x, ctx, cache)
+        self.ffn.forward(self.ffn_norm.forward(x, ctx), x, ctx)
