@@ -16,9 +16,9 @@
 // the rest values. Per-head RMS norm then half-split rotation: channel i pairs with
 // i + rotary_dim/2; out[i] = a cos - b sin, out[i + half] = b cos + a sin
 // (native/include/flyweight_v2_native_kernels.hpp:1015-1050). Values are stored untouched.
-template <typename T>
+template <typename TI, typename T>
 __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
-    const T* __restrict__ qkv, T* __restrict__ q_out, const float* __restrict__ q_norm_weight,
+    const TI* __restrict__ qkv, T* __restrict__ q_out, const float* __restrict__ q_norm_weight,
     const float* __restrict__ k_norm_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rotary_dim, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
@@ -28,7 +28,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
     const int vec = blockIdx.y;
     const int lane = threadIdx.x;
     const int width = (num_heads + 2 * num_kv_heads) * head_dim;
-    const T* source = qkv + (size_t)row * width + (size_t)vec * head_dim;
+    const TI* source = qkv + (size_t)row * width + (size_t)vec * head_dim;
     const int pos = row_pos[row];
     const int page = block_table[(size_t)row_seg[row] * table_stride + pos / ATTN_PAGE];
     const int slot = pos % ATTN_PAGE;
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
     if (vec >= num_heads + num_kv_heads) {      // value head: transposed store
         const int kvh = vec - num_heads - num_kv_heads;
         T* dest = v_pages + ((size_t)page * num_kv_heads + kvh) * head_dim * ATTN_PAGE;
-        for (int d = lane; d < head_dim; d += 64) dest[(size_t)d * ATTN_PAGE + slot] = source[d];
+        for (int d = lane; d < head_dim; d += 64) store_from_float(dest, (size_t)d * ATTN_PAGE + slot, load_as_float(source, d));
         return;
     }
     const bool is_query = vec < num_heads;
@@ -72,7 +72,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
     }
 }
 
-extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, void* q_out, int dtype, const float* q_norm_weight,
+extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int dtype, const float* q_norm_weight,
                                         const float* k_norm_weight, float eps, const float* cos_table,
                                         const float* sin_table, int rotary_dim, void* k_pages, void* v_pages,
                                         const int32_t* block_table, int table_stride, const int32_t* row_seg,
@@ -90,16 +90,16 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, void* q_out, int dtype,
     const int vectors = write_kv ? num_heads + 2 * num_kv_heads : num_heads;
     FW_REQUIRE(vectors <= 65535, "qk_norm_rope: too many heads (%d)", vectors);
     dim3 grid(rows, vectors);
-    if (dtype == FW_F32)
-        qk_norm_rope_kv_write_kernel<float><<<grid, 64, 0, (hipStream_t)stream>>>(
-            (const float*)qkv, (float*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim,
-            (float*)k_pages, (float*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim);
-    else if (dtype == FW_BF16)
-        qk_norm_rope_kv_write_kernel<bf16_t><<<grid, 64, 0, (hipStream_t)stream>>>(
-            (const bf16_t*)qkv, (bf16_t*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim,
-            (bf16_t*)k_pages, (bf16_t*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim);
-    else
-        FW_REQUIRE(false, "qk_norm_rope: unknown dtype %d", dtype);
+    hipStream_t s = (hipStream_t)stream;
+#define FW_QK_LAUNCH(TI, T)                                                                                          \
+    qk_norm_rope_kv_write_kernel<TI, T><<<grid, 64, 0, s>>>(                                                         \
+        (const TI*)qkv, (T*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim, (T*)k_pages, \
+        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim)
+    if (in_dtype == FW_F32 && dtype == FW_F32) FW_QK_LAUNCH(float, float);
+    else if (in_dtype == FW_F32 && dtype == FW_BF16) FW_QK_LAUNCH(float, bf16_t);
+    else if (in_dtype == FW_BF16 && dtype == FW_BF16) FW_QK_LAUNCH(bf16_t, bf16_t);
+    else FW_REQUIRE(false, "qk_norm_rope: unsupported dtypes in=%d out=%d", in_dtype, dtype);
+#undef FW_QK_LAUNCH
     FW_LAUNCH_CHECK("qk_norm_rope_kv_write");
     return 0;
 }

@@ -94,10 +94,10 @@ __device__ __forceinline__ float stable_sigmoid(float g) {
     return e / (1.0f + e);
 }
 
-template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int intermediate) {
+template <typename TI, typename TO>
+__global__ void swiglu_kernel(const TI* __restrict__ gate_up, TO* __restrict__ out, int intermediate) {
     const int row = blockIdx.y;
-    const T* source = gate_up + (size_t)row * 2 * intermediate;
+    const TI* source = gate_up + (size_t)row * 2 * intermediate;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < intermediate; i += gridDim.x * blockDim.x) {
         const float g = load_as_float(source, i);
         const float u = load_as_float(source, (size_t)intermediate + i);
@@ -105,19 +105,23 @@ __global__ void swiglu_kernel(const T* __restrict__ gate_up, T* __restrict__ out
     }
 }
 
-extern "C" int fw_swiglu(const void* gate_up, void* out, int dtype, int rows, int intermediate, void* stream) {
+extern "C" int fw_swiglu(const void* gate_up, int in_dtype, void* out, int out_dtype, int rows, int intermediate,
+                         void* stream) {
     FW_REQUIRE(rows >= 0 && intermediate > 0, "swiglu: bad sizes rows=%d width=%d", rows, intermediate);
     FW_REQUIRE(rows <= 65535, "swiglu: at most 65535 rows per call, got %d", rows);
     if (rows == 0) return 0;
     int bx = fw_ceil_div(intermediate, 256);
     if (bx > 32) bx = 32;
     dim3 grid(bx, rows);
-    if (dtype == FW_F32)
-        swiglu_kernel<float><<<grid, 256, 0, (hipStream_t)stream>>>((const float*)gate_up, (float*)out, intermediate);
-    else if (dtype == FW_BF16)
-        swiglu_kernel<bf16_t><<<grid, 256, 0, (hipStream_t)stream>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate);
+    hipStream_t s = (hipStream_t)stream;
+    if (in_dtype == FW_F32 && out_dtype == FW_F32)
+        swiglu_kernel<float, float><<<grid, 256, 0, s>>>((const float*)gate_up, (float*)out, intermediate);
+    else if (in_dtype == FW_F32 && out_dtype == FW_BF16)
+        swiglu_kernel<float, bf16_t><<<grid, 256, 0, s>>>((const float*)gate_up, (bf16_t*)out, intermediate);
+    else if (in_dtype == FW_BF16 && out_dtype == FW_BF16)
+        swiglu_kernel<bf16_t, bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)gate_up, (bf16_t*)out, intermediate);
     else
-        FW_REQUIRE(false, "swiglu: unknown dtype %d", dtype);
+        FW_REQUIRE(false, "swiglu: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
     FW_LAUNCH_CHECK("swiglu");
     return 0;
 }

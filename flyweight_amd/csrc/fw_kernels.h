@@ -28,8 +28,9 @@ int fw_rmsnorm_rows(const float* x, const float* weight, void* out, int out_dtyp
 int fw_gemm_generic(const void* a, int a_dtype, const void* w, int w_dtype, const float* bias,
                     void* out, int out_dtype, int out_mode, int M, int N, int K, void* stream);
 
-// out[r][i] = silu(gu[r][i]) * gu[r][I + i]
-int fw_swiglu(const void* gate_up, void* out, int dtype, int rows, int intermediate, void* stream);
+// out[r][i] = silu(gu[r][i]) * gu[r][I + i]; the input may be float32 beside a bfloat16 output
+int fw_swiglu(const void* gate_up, int in_dtype, void* out, int out_dtype, int rows, int intermediate,
+              void* stream);
 
 // cos/sin of position * inv_freq for every row: tables [rows][half]
 int fw_rope_table(const int32_t* positions, const double* inv_freq, float* cos_out, float* sin_out,
@@ -39,8 +40,8 @@ int fw_rope_table(const int32_t* positions, const double* inv_freq, float* cos_o
 // oldest first; conv_bias [H] or null; state [slots][H][L-1] float32, oldest first.
 // Row r belongs to segment row_seg[r]; segment s covers rows seg_row0[s]..seg_row0[s+1]
 // and continues the sequence whose state lives in slot seg_slot[s].
-int fw_shortconv(const void* bcx, void* out, int dtype, const float* taps, const float* conv_bias,
-                 float* state, const int32_t* row_seg, const int32_t* seg_row0,
+int fw_shortconv(const void* bcx, int in_dtype, void* out, int out_dtype, const float* taps,
+                 const float* conv_bias, float* state, const int32_t* row_seg, const int32_t* seg_row0,
                  const int32_t* seg_slot, int rows, int segments, int hidden, int kernel_size,
                  int slots, void* stream);
 
@@ -48,7 +49,7 @@ int fw_shortconv(const void* bcx, void* out, int dtype, const float* taps, const
 // first rotary_dim channels by the row's angle, q out, k and v appended to the pages of
 // the row's segment. qkv [rows][(nh + 2 nkv) hd]. k_pages [pages][nkv][P][hd];
 // v_pages [pages][nkv][hd][P]. block_table [segments][table_stride].
-int fw_qk_norm_rope_kv_write(const void* qkv, void* q_out, int dtype, const float* q_norm_weight,
+int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int dtype, const float* q_norm_weight,
                              const float* k_norm_weight, float eps, const float* cos_table,
                              const float* sin_table, int rotary_dim, void* k_pages, void* v_pages,
                              const int32_t* block_table, int table_stride, const int32_t* row_seg,

@@ -20,8 +20,8 @@ __device__ __forceinline__ float bx_at(const T* __restrict__ bcx, int row, int c
     return load_as_float(source, channel) * load_as_float(source, 2 * (size_t)hidden + channel);
 }
 
-template <typename T>
-__global__ void shortconv_rows_kernel(const T* __restrict__ bcx, T* __restrict__ out,
+template <typename T, typename TO>
+__global__ void shortconv_rows_kernel(const T* __restrict__ bcx, TO* __restrict__ out,
                                       const float* __restrict__ taps, const float* __restrict__ conv_bias,
                                       const float* __restrict__ state, const int32_t* __restrict__ row_seg,
                                       const int32_t* __restrict__ seg_row0, const int32_t* __restrict__ seg_slot,
@@ -67,8 +67,8 @@ __global__ void shortconv_state_kernel(const T* __restrict__ bcx, float* __restr
 }
 
 // every segment is one row: output and state shift in one pass
-template <typename T>
-__global__ void shortconv_decode_kernel(const T* __restrict__ bcx, T* __restrict__ out,
+template <typename T, typename TO>
+__global__ void shortconv_decode_kernel(const T* __restrict__ bcx, TO* __restrict__ out,
                                         const float* __restrict__ taps, const float* __restrict__ conv_bias,
                                         float* __restrict__ state, const int32_t* __restrict__ seg_slot,
                                         int hidden, int kernel_size) {
@@ -89,24 +89,24 @@ __global__ void shortconv_decode_kernel(const T* __restrict__ bcx, T* __restrict
     store_from_float(out, (size_t)row * hidden + channel, gate * y);
 }
 
-template <typename T>
+template <typename T, typename TO>
 static void launch(const void* bcx, void* out, const float* taps, const float* conv_bias, float* state,
                    const int32_t* row_seg, const int32_t* seg_row0, const int32_t* seg_slot, int rows,
                    int segments, int hidden, int kernel_size, hipStream_t stream) {
     const int bx = fw_ceil_div(hidden, 256);
     if (rows == segments) {
-        shortconv_decode_kernel<T><<<dim3(bx, rows), 256, 0, stream>>>(
-            (const T*)bcx, (T*)out, taps, conv_bias, state, seg_slot, hidden, kernel_size);
+        shortconv_decode_kernel<T, TO><<<dim3(bx, rows), 256, 0, stream>>>(
+            (const T*)bcx, (TO*)out, taps, conv_bias, state, seg_slot, hidden, kernel_size);
         return;
     }
-    shortconv_rows_kernel<T><<<dim3(bx, rows), 256, 0, stream>>>(
-        (const T*)bcx, (T*)out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, hidden, kernel_size);
+    shortconv_rows_kernel<T, TO><<<dim3(bx, rows), 256, 0, stream>>>(
+        (const T*)bcx, (TO*)out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, hidden, kernel_size);
     shortconv_state_kernel<T><<<dim3(bx, segments), 256, 0, stream>>>(
         (const T*)bcx, state, seg_row0, seg_slot, hidden, kernel_size);
 }
 
-extern "C" int fw_shortconv(const void* bcx, void* out, int dtype, const float* taps, const float* conv_bias,
-                            float* state, const int32_t* row_seg, const int32_t* seg_row0,
+extern "C" int fw_shortconv(const void* bcx, int in_dtype, void* out, int out_dtype, const float* taps,
+                            const float* conv_bias, float* state, const int32_t* row_seg, const int32_t* seg_row0,
                             const int32_t* seg_slot, int rows, int segments, int hidden, int kernel_size,
                             int slots, void* stream) {
     FW_REQUIRE(rows >= 0 && segments >= 0 && hidden > 0, "shortconv: bad sizes rows=%d segments=%d hidden=%d", rows, segments, hidden);
@@ -115,9 +115,11 @@ extern "C" int fw_shortconv(const void* bcx, void* out, int dtype, const float* 
     FW_REQUIRE(rows <= 65535 && segments <= slots, "shortconv: rows=%d (max 65535), segments=%d, slots=%d", rows, segments, slots);
     if (rows == 0) return 0;
     FW_REQUIRE(segments >= 1, "shortconv: rows without a segment");
-    if (dtype == FW_F32) launch<float>(bcx, out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, rows, segments, hidden, kernel_size, (hipStream_t)stream);
-    else if (dtype == FW_BF16) launch<bf16_t>(bcx, out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, rows, segments, hidden, kernel_size, (hipStream_t)stream);
-    else FW_REQUIRE(false, "shortconv: unknown dtype %d", dtype);
+    hipStream_t s = (hipStream_t)stream;
+    if (in_dtype == FW_F32 && out_dtype == FW_F32) launch<float, float>(bcx, out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, rows, segments, hidden, kernel_size, s);
+    else if (in_dtype == FW_F32 && out_dtype == FW_BF16) launch<float, bf16_t>(bcx, out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, rows, segments, hidden, kernel_size, s);
+    else if (in_dtype == FW_BF16 && out_dtype == FW_BF16) launch<bf16_t, bf16_t>(bcx, out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, rows, segments, hidden, kernel_size, s);
+    else FW_REQUIRE(false, "shortconv: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
     FW_LAUNCH_CHECK("shortconv");
     return 0;
 }

@@ -1,0 +1,223 @@
+"""The Python entry point, in the manner of the reference's binding: a ``Model`` opened
+from a folder and a ``Runtime`` over it (``V2Model`` / ``V2QwenRuntime``,
+src/flyweight/v2.py:2188-2440,3297-4029). Method names and meanings follow the reference
+where it has them: ``prepare``, ``decode``, ``generate(prompt, max_tokens, callback)``,
+``task_submit``, ``engine_step`` -> [(task id, token, kind)], ``task_cancel``,
+``task_error``, ``reset``, ``info``, ``close``. ``step`` (logits of a mixed batch) has no
+counterpart there: the reference returns tokens, never logits.
+"""
+
+from __future__ import annotations
+
+import time
+from typing import Callable, Dict, Hashable, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache import OutOfPages
+from ..sampling import GREEDY, SamplingConfig, sample_rows
+from .model import CausalLM, load_model, parse_dtype
+from .scheduler import (EVENT_ERROR, EVENT_FINISHED, EVENT_PREFILL, EVENT_TOKEN, Request, Scheduler,
+                        SchedulerError)
+from .step import StepEntry, Stepper
+
+PAGE_SIZE = 64
+
+
+class EngineError(RuntimeError):
+    pass
+
+
+class Model:
+    """A model folder (config.json + safetensors) loaded onto the GPU."""
+
+    def __init__(self, path: str, dtype="bfloat16", device: str = "cuda:0"):
+        self.path = path
+        self.dtype = parse_dtype(dtype)
+        self.config, self.model = load_model(path, dtype=self.dtype, device=device)
+
+    @property
+    def spec(self):
+        return self.model.spec
+
+    def tensors(self) -> Dict[str, Tuple[Tuple[int, ...], str]]:
+        return {name: (decl.shape, decl.role) for name, decl in self.model.tensors().items()}
+
+    def native_runtime(self, **options) -> "Runtime":
+        return Runtime(self, **options)
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+class Runtime:
+    def __init__(self, model: Model, context_limit: Optional[int] = None, parallel_sequences: int = 16,
+                 num_pages: Optional[int] = None, max_batch_tokens: int = 2048, prefill_rows: int = 512):
+        """``context_limit``: most tokens (prompt + output) of one request, at most the
+        model's ``max_position_embeddings``. ``parallel_sequences``: most requests live at
+        once. ``num_pages``: cache pages (of 64 tokens) per page group; by default enough
+        for every live request at the full context. ``prefill_rows``: most tokens of one
+        prompt portion; ``max_batch_tokens``: most tokens of one step."""
+        self.model = model
+        spec = model.spec
+        self.context_limit = min(context_limit or spec.max_positions, spec.max_positions)
+        self.parallel_sequences = max(1, int(parallel_sequences))
+        per_request = (self.context_limit + PAGE_SIZE - 1) // PAGE_SIZE
+        self.num_pages = int(num_pages) if num_pages else per_request * self.parallel_sequences
+        self.max_batch_tokens = int(max_batch_tokens)
+        self.prefill_rows = int(prefill_rows)
+        self.stepper: Optional[Stepper] = None
+        self.scheduler: Optional[Scheduler] = None
+        self._errors: Dict[int, str] = {}
+        self._decode_request: Optional[Hashable] = None
+        self._counters = {"decode_calls": 0, "decode_ns": 0, "prefill_calls": 0, "prefill_tokens": 0, "prefill_ns": 0,
+                          "steps": 0}
+
+    # ----- lifetime ---------------------------------------------------------------------
+    def prepare(self) -> "Runtime":
+        if self.stepper is None:
+            self.stepper = Stepper(self.model.model, num_pages=self.num_pages, max_requests=self.parallel_sequences,
+                                   page_size=PAGE_SIZE)
+            self.scheduler = Scheduler(self.stepper.cache, max_positions=self.context_limit,
+                                       max_batch_tokens=self.max_batch_tokens, chunk_size=self.prefill_rows,
+                                       max_live=self.parallel_sequences)
+        return self
+
+    def reset(self) -> None:
+        """Forget every request and give all cache memory back (state slots are zeroed
+        again when next handed out)."""
+        self.prepare()
+        for request in list(self.stepper.cache.requests):
+            self.stepper.cache.release(request)
+        self.scheduler = Scheduler(self.stepper.cache, max_positions=self.context_limit,
+                                   max_batch_tokens=self.max_batch_tokens, chunk_size=self.prefill_rows,
+                                   max_live=self.parallel_sequences)
+        self._decode_request = None
+        self._errors.clear()
+
+    def close(self) -> None:
+        self.stepper = None
+        self.scheduler = None
+
+    def __enter__(self):
+        return self.prepare()
+
+    def __exit__(self, *exc):
+        self.close()
+        return False
+
+    # ----- logits -----------------------------------------------------------------------
+    def admit(self, request: Hashable) -> None:
+        self.prepare().stepper.admit(request)
+
+    def release(self, request: Hashable) -> None:
+        self.stepper.release(request)
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """One mixed batch -> float32 logits [wanted, vocab] on the device."""
+        return self.prepare().stepper.step(entries)
+
+    # ----- single sequence, as the reference's decode(token) -> token ---------------------
+    def decode(self, token: int) -> int:
+        """Feeds one token to the runtime's own sequence and returns the greedy next token."""
+        self.prepare()
+        if self._decode_request is None:
+            self._decode_request = ("decode", id(self))
+            self.stepper.admit(self._decode_request)
+        began = time.perf_counter_ns()
+        logits = self.stepper.step([StepEntry(self._decode_request, [int(token)], [0])])
+        token = sample_rows(logits, [GREEDY], [None])[0]
+        self._counters["decode_calls"] += 1
+        self._counters["decode_ns"] += time.perf_counter_ns() - began
+        return token
+
+    # ----- tasks ------------------------------------------------------------------------
+    def task_submit(self, prompt: Sequence[int], max_tokens: int, stop_tokens: Sequence[int] = (),
+                    temperature: float = 0.0, top_k: int = 20, top_p: float = 0.95, min_p: float = 0.0,
+                    seed: Optional[int] = None) -> int:
+        self.prepare()
+        sampling = SamplingConfig(temperature=temperature, top_k=top_k, top_p=top_p, min_p=min_p, seed=seed)
+        try:
+            return self.scheduler.submit(prompt, max_tokens, sampling, stop_tokens).id
+        except SchedulerError as error:
+            raise EngineError(str(error)) from None
+
+    def task_cancel(self, task_id: int) -> bool:
+        return self.scheduler.cancel(task_id)
+
+    def task_error(self, task_id: int) -> Optional[str]:
+        return self._errors.get(task_id)
+
+    def engine_step(self) -> List[Tuple[int, int, int]]:
+        """One step of everything that can move: returns (task id, token or progress, kind)
+        with kind 0 token, 1 finished, 2 error, 3 prefill progress."""
+        self.prepare()
+        scheduler = self.scheduler
+        if not scheduler.has_work():
+            return []
+        plan = scheduler.schedule()
+        for request in plan.failed:
+            self._errors[request.id] = request.error or "failed"
+        sampled: Dict[int, int] = {}
+        if plan.segments:
+            entries = [StepEntry(s.request.id, s.tokens, [len(s.tokens) - 1] if s.wants_logits else [])
+                       for s in plan.segments]
+            began = time.perf_counter_ns()
+            logits = self.stepper.step(entries)
+            wanting = [s.request for s in plan.segments if s.wants_logits]
+            if wanting:
+                tokens = sample_rows(logits, [r.sampling for r in wanting], [r.rng for r in wanting])
+                sampled = {r.id: t for r, t in zip(wanting, tokens)}
+            elapsed = time.perf_counter_ns() - began
+            self._counters["steps"] += 1
+            prompt_tokens = sum(len(s.tokens) for s in plan.segments if len(s.tokens) > 1)
+            if prompt_tokens:
+                self._counters["prefill_calls"] += 1
+                self._counters["prefill_tokens"] += prompt_tokens
+                self._counters["prefill_ns"] += elapsed
+            else:
+                self._counters["decode_calls"] += len(plan.segments)
+                self._counters["decode_ns"] += elapsed
+        return scheduler.complete(plan, sampled)
+
+    # ----- blocking generation ------------------------------------------------------------
+    def generate(self, prompt: Sequence[int], max_tokens: int,
+                 callback: Optional[Callable[[int], Optional[bool]]] = None, **sampling) -> List[int]:
+        """Generates up to ``max_tokens`` tokens after ``prompt``; ``callback(token)`` is
+        called for each and stops the generation by returning False (as the reference's
+        generate, src/flyweight/v2.py:3837-3876). Greedy unless sampling settings are given."""
+        task = self.task_submit(prompt, max_tokens, **sampling)
+        produced: List[int] = []
+        while True:
+            events = self.engine_step()
+            for task_id, value, kind in events:
+                if task_id != task:
+                    continue
+                if kind == EVENT_TOKEN:
+                    produced.append(value)
+                    if callback is not None and callback(value) is False:
+                        self.task_cancel(task)
+                elif kind == EVENT_ERROR:
+                    raise EngineError(self.task_error(task) or "generation failed")
+                elif kind == EVENT_FINISHED:
+                    return produced
+            if not self.scheduler.has_work():
+                return produced
+
+    def run(self) -> Dict[int, List[int]]:
+        """Steps until every submitted task has ended; returns task id -> generated tokens."""
+        while self.scheduler.has_work():
+            self.engine_step()
+        return {task: list(request.generated) for task, request in self.scheduler.requests.items()}
+
+    # ----- counters ---------------------------------------------------------------------
+    @property
+    def info(self) -> Dict[str, int]:
+        data = dict(self._counters)
+        if self.stepper is not None:
+            data.update(self.stepper.cache.stats())
+            data["preemptions"] = self.scheduler.preemptions
+        return data

@@ -81,6 +81,7 @@ class StepContext:
         self.device = device
         self.host_row_pos = row_pos
         self.host_seg_row0 = seg_row0
+        self.host_seg_slot = seg_slot
 
         tables = [cache.block_table_rows(g, self.requests) for g in range(len(cache.groups))]
         pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows)]

@@ -147,17 +147,20 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] 
     return target
 
 
-def swiglu(gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+def swiglu(gate_up: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """silu(gate) * up of [rows, gate | up]; the input may be float32 beside a bfloat16 output."""
     _dev(gate_up, out)
+    out_dtype = out_dtype or gate_up.dtype
     rows, width = gate_up.shape
     if width % 2:
         raise KernelError("swiglu: the input holds gate and up halves; its width must be even")
     inter = width // 2
     if out is None:
-        out = torch.empty((rows, inter), dtype=gate_up.dtype, device=gate_up.device)
-    if out.shape != (rows, inter) or out.dtype != gate_up.dtype:
+        out = torch.empty((rows, inter), dtype=out_dtype, device=gate_up.device)
+    if out.shape != (rows, inter) or out.dtype != out_dtype:
         raise KernelError("swiglu: out has the wrong shape or dtype")
-    _check(library().fw_swiglu(_p(gate_up), _p(out), _code(gate_up.dtype), rows, inter, _stream()))
+    _check(library().fw_swiglu(_p(gate_up), _code(gate_up.dtype), _p(out), _code(out_dtype), rows, inter, _stream()))
     return out
 
 
@@ -175,9 +178,11 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor):
 
 def shortconv(bcx: torch.Tensor, taps: torch.Tensor, conv_bias: Optional[torch.Tensor], state: torch.Tensor,
               row_seg: torch.Tensor, seg_row0: torch.Tensor, seg_slot: torch.Tensor, segments: int,
-              out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """state [slots, H, L-1] is read and updated in place."""
+              out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """state [slots, H, L-1] is read and updated in place. ``bcx`` may be float32 beside a
+    bfloat16 output."""
     _dev(bcx, taps, conv_bias, state, row_seg, seg_row0, seg_slot, out)
+    out_dtype = out_dtype or bcx.dtype
     rows, width = bcx.shape
     hidden, kernel = taps.shape
     if width != 3 * hidden:
@@ -195,10 +200,10 @@ def shortconv(bcx: torch.Tensor, taps: torch.Tensor, conv_bias: Optional[torch.T
         if t.numel() < n:
             raise KernelError(f"shortconv: {name} holds {t.numel()} entries, needs {n}")
     if out is None:
-        out = torch.empty((rows, hidden), dtype=bcx.dtype, device=bcx.device)
-    if out.shape != (rows, hidden) or out.dtype != bcx.dtype:
+        out = torch.empty((rows, hidden), dtype=out_dtype, device=bcx.device)
+    if out.shape != (rows, hidden) or out.dtype != out_dtype:
         raise KernelError("shortconv: out has the wrong shape or dtype")
-    _check(library().fw_shortconv(_p(bcx), _p(out), _code(bcx.dtype), _p(taps), _p(conv_bias), _p(state), _p(row_seg),
+    _check(library().fw_shortconv(_p(bcx), _code(bcx.dtype), _p(out), _code(out_dtype), _p(taps), _p(conv_bias), _p(state), _p(row_seg),
                                   _p(seg_row0), _p(seg_slot), rows, segments, hidden, kernel, state.shape[0], _stream()))
     return out
 
@@ -219,11 +224,12 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, 
                           cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rotary_dim: int,
                           k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                           row_seg: torch.Tensor, row_pos: torch.Tensor, write_kv: bool = True) -> torch.Tensor:
+    """The output and the cache take the pages' dtype; ``qkv`` may be float32 beside bfloat16 pages."""
     _dev(qkv, q_norm_weight, k_norm_weight, cos, sin, k_pages, v_pages, block_table, row_seg, row_pos)
     rows, width = qkv.shape
     if width != (num_heads + 2 * num_kv_heads) * head_dim:
         raise KernelError(f"qk_norm_rope: qkv width {width} != ({num_heads} + 2 x {num_kv_heads}) x {head_dim}")
-    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, qkv.dtype)
+    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, k_pages.dtype)
     for w in (q_norm_weight, k_norm_weight):
         if w is not None:
             _want(w, torch.float32, "norm weight")
@@ -239,9 +245,9 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, 
     _want(row_pos, torch.int32, "row_pos")
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("qk_norm_rope: batch index arrays are too short")
-    q_out = torch.empty((rows, num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    q_out = torch.empty((rows, num_heads * head_dim), dtype=k_pages.dtype, device=qkv.device)
     _check(library().fw_qk_norm_rope_kv_write(
-        _p(qkv), _p(q_out), _code(qkv.dtype), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin),
+        _p(qkv), _code(qkv.dtype), _p(q_out), _code(k_pages.dtype), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin),
         rotary_dim, _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(row_seg), _p(row_pos), rows,
         num_heads, num_kv_heads, head_dim, PAGE_SIZE, pages, int(write_kv), _stream()))
     return q_out

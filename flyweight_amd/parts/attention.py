@@ -84,7 +84,7 @@ class GQAttention(Mixer):
         self.k_norm_weight = tensors[self._name("k_norm")] if self.qk_norm else None
 
     def forward(self, h, residual, ctx, cache) -> None:
-        qkv = self.qkv.forward(h)
+        qkv = self.qkv.forward(h, out_dtype=torch.float32)      # normed, rotated and rounded once, below
         cos, sin = ctx.position_tables(self.position)
         q = ops.qk_norm_rope_kv_write(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight,

@@ -57,7 +57,7 @@ class ShortConv(Mixer):
         self.conv_bias = tensors[p + "conv.bias"] if self.bias else None
 
     def forward(self, h, residual, ctx, cache) -> None:
-        bcx = self.in_proj.forward(h)
+        bcx = self.in_proj.forward(h, out_dtype=torch.float32)  # B * x and the taps' sum stay in float32
         gated = ops.shortconv(bcx, self.taps, self.conv_bias, cache.state, ctx.row_seg, ctx.seg_row0, ctx.seg_slot,
-                              ctx.num_segments)
+                              ctx.num_segments, out_dtype=self.dtype)
         self.out_proj.accumulate(gated, residual)

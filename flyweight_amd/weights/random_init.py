@@ -11,6 +11,7 @@ see identical values.
 
 from __future__ import annotations
 
+import math
 import os
 from typing import Dict, Mapping
 
@@ -22,8 +23,21 @@ from .safetensors_io import write_file
 _STD = {"matrix": 0.02, "conv": 0.1, "bias": 0.01}
 
 
+def _std(decl: TensorDecl, scale: str) -> float:
+    """``scale`` "small": the fixed widths above. "fan_in": every linear map keeps the size
+    of what passes through it (matrices 1/sqrt(columns), taps 0.5, biases 0.1), so that each
+    part of a layer contributes visibly to the output; meant for tests."""
+    if scale == "small":
+        return _STD[decl.init]
+    if scale != "fan_in":
+        raise ValueError(f"unknown scale '{scale}'")
+    if decl.init == "matrix":
+        return 1.0 / math.sqrt(decl.shape[-1])
+    return {"conv": 0.5, "bias": 0.1}[decl.init]
+
+
 def random_tensors(declared: Mapping[str, TensorDecl], seed: int,
-                   matrix_dtype: torch.dtype = torch.bfloat16) -> Dict[str, torch.Tensor]:
+                   matrix_dtype: torch.dtype = torch.bfloat16, scale: str = "small") -> Dict[str, torch.Tensor]:
     generator = torch.Generator(device="cpu")
     generator.manual_seed(int(seed))
     tensors: Dict[str, torch.Tensor] = {}
@@ -37,19 +51,19 @@ def random_tensors(declared: Mapping[str, TensorDecl], seed: int,
         elif decl.init == "zeros":
             value = torch.zeros(decl.shape, dtype=torch.float32)
         else:
-            value = torch.randn(decl.shape, generator=generator, dtype=torch.float32) * _STD[decl.init]
+            value = torch.randn(decl.shape, generator=generator, dtype=torch.float32) * _std(decl, scale)
         tensors[name] = value.to(matrix_dtype) if decl.role == "matrix" else value
     return tensors
 
 
 def write_random_model(folder: str, config, seed: int,
-                       matrix_dtype: torch.dtype = torch.bfloat16) -> str:
+                       matrix_dtype: torch.dtype = torch.bfloat16, scale: str = "small") -> str:
     """``config`` is a registered architecture's configuration object."""
     from ..engine.model import declared_tensors      # parts decide which tensors exist
     os.makedirs(folder, exist_ok=True)
     config.save(folder)
     declared = declared_tensors(config.model_spec())
-    tensors = random_tensors(declared, seed, matrix_dtype)
+    tensors = random_tensors(declared, seed, matrix_dtype, scale)
     write_file(os.path.join(folder, "model.safetensors"), tensors,
                metadata={"format": "pt", "seed": str(int(seed))})
     return folder

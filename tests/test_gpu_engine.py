@@ -1,0 +1,241 @@
+"""The engine in-process on the GPU: the step function under many cuts, generation through
+the entry point, the scheduler under page pressure."""
+
+import numpy as np
+import pytest
+import torch
+
+import plain_lfm2 as plain
+from gpu_common import Loaded, feed
+from helpers import assert_close, make_model, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("models")
+    return {name: make_model(str(root / name), name, seed=21) for name in ("A", "B")}
+
+
+@pytest.fixture(scope="module")
+def loaded(folders):
+    cache = {}
+
+    def get(name, dtype):
+        if (name, dtype) not in cache:
+            cache[(name, dtype)] = Loaded(folders[name], dtype)
+        return cache[(name, dtype)]
+    return get
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens_and_lengths_across_every_boundary(loaded, name, dtype):
+    # prompt lengths of the reference's path-parity test (tests/test_v2_path_parity.py:129), whole and cut
+    m = loaded(name, dtype)
+    stepper = m.stepper(num_pages=6, max_requests=2)
+    for length in (1, 2, 3, 9, 40, 300):
+        tokens = random_tokens(m.config.vocab_size, length, seed=length)
+        want = m.expected(tokens)
+        for cuts in ([length], [1] * min(length, 5), [2, 1, 3, 64, 63, 1, 65]):
+            stepper.admit("r")
+            assert_close(feed(stepper, "r", tokens, cuts), want, dtype, f"length {length} cuts {cuts[:4]}")
+            stepper.release("r")
+    stepper.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(loaded, dtype):
+    m = loaded("B", dtype)
+    tokens = random_tokens(m.config.vocab_size, 330, seed=8)
+    stepper = m.stepper(num_pages=6, max_requests=1)
+    stepper.admit("r")
+    assert_close(feed(stepper, "r", tokens, [30] + [1] * 300), m.expected(tokens), dtype, "300 decoded tokens")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_cuts_agree_with_each_other_more_closely_than_with_the_plain_model(loaded, dtype):
+    """Whole, token by token and in portions differ by rounding only; in float32 that is
+    far below the distance to the float64 model."""
+    m = loaded("A", dtype)
+    tokens = random_tokens(m.config.vocab_size, 150, seed=4)
+    stepper = m.stepper(num_pages=3, max_requests=1)
+    runs = []
+    for cuts in ([150], [1] * 150, [7, 2, 16, 3, 2, 64, 5]):
+        stepper.admit("r")
+        runs.append(feed(stepper, "r", tokens, cuts))
+        stepper.release("r")
+    scale = np.abs(runs[0]).max()
+    limit = {"float32": 2e-6, "bfloat16": 1e-2}[dtype] * scale
+    assert np.abs(runs[1] - runs[0]).max() <= limit and np.abs(runs[2] - runs[0]).max() <= limit
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_pages_and_slots_that_are_used_again_carry_nothing_over(loaded, dtype):
+    """After a request ends its pages and state slot are filled with NaN; the next request
+    gets exactly those (the pools are LIFO) and must not be touched by what they hold."""
+    m = loaded("B", dtype)
+    stepper = m.stepper(num_pages=4, max_requests=1)
+    first = random_tokens(m.config.vocab_size, 200, seed=1)
+    stepper.admit("a")
+    feed(stepper, "a", first, [200])
+    held = list(stepper.cache.groups[0].tables["a"])
+    stepper.release("a")
+    for pages in list(stepper.cache.k_pages.values()) + list(stepper.cache.v_pages.values()):
+        pages.fill_(float("nan"))
+    for state in stepper.cache.state.values():
+        state.fill_(float("nan"))
+    second = random_tokens(m.config.vocab_size, 130, seed=2)
+    stepper.admit("b")
+    got = feed(stepper, "b", second, [70, 3, 1, 1, 55])
+    assert set(stepper.cache.groups[0].tables["b"]) <= set(held)
+    assert_close(got, m.expected(second), dtype, "second request on poisoned pages")
+
+
+@pytest.mark.parametrize("dtype", ["float32"])
+def test_a_far_key_among_hundreds_decides_the_output(loaded, dtype, tmp_path):
+    """The query of the last token is made to match the key of token 3 (of 400) far better
+    than any other, by scaling the q- and k-norm weights of the attention layers: if a step
+    dropped or misplaced one key, the logits would move by far more than the tolerance. The
+    plain model sees the same weights, so this is an ordinary comparison with a sharp
+    attention pattern. In 32-bit only: so sharp a softmax magnifies bfloat16's rounding of
+    the scores just as it magnifies a fault (the bfloat16 kernels are given single dominant
+    keys in their own tests instead)."""
+    import os
+    from flyweight_amd.weights import SafetensorsFile, write_file
+    m = loaded("A", dtype)
+    with SafetensorsFile(os.path.join(m.folder, "model.safetensors")) as handle:
+        tensors = {n: handle.tensor(n) for n in handle.names()}
+    for n in tensors:
+        if n.endswith("k_layernorm.weight") or n.endswith("q_layernorm.weight"):
+            tensors[n] = tensors[n] * 3.0       # scores nine times larger: softmax picks single keys
+    folder = str(tmp_path / "sharp")
+    os.makedirs(folder)
+    write_file(os.path.join(folder, "model.safetensors"), tensors)
+    m.config.save(folder)
+    sharp = Loaded(folder, dtype)
+    tokens = random_tokens(sharp.config.vocab_size, 380, seed=9)
+    want = sharp.expected(tokens)
+    stepper = sharp.stepper(num_pages=6, max_requests=1)
+    stepper.admit("r")
+    assert_close(feed(stepper, "r", tokens, [100, 1, 1, 150, 2, 126]), want, dtype, "sharp attention")
+
+
+def _runtime(m, **kw):
+    from flyweight_amd.engine import Model, Runtime
+    model = Model.__new__(Model)
+    model.path, model.dtype, model.config, model.model = m.folder, m.model.dtype, m.config, m.model
+    return Runtime(model, **kw).prepare()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_greedy_generation_through_the_entry_point(folders, name, dtype):
+    import flyweight_amd
+    model = flyweight_amd.Model(folders[name], dtype=dtype)
+    config, weights = plain.read_folder(folders[name])
+    with flyweight_amd.Runtime(model, parallel_sequences=2, prefill_rows=16, max_batch_tokens=24) as runtime:
+        for length in (5, 17, 31):
+            prompt = random_tokens(config["vocab_size"], length, seed=length)
+            seen = []
+            produced = runtime.generate(prompt, 8, callback=seen.append)
+            assert produced == seen
+            if dtype == "float32":
+                assert produced == plain.greedy(config, weights, prompt, 8)
+            else:   # bfloat16 may legitimately pick another of two near-equal logits; check each choice instead
+                context = list(prompt)
+                for token in produced:
+                    logits = plain.forward(config, weights, context)[-1]
+                    assert logits[token] >= logits.max() - 2e-2 * np.abs(logits).max()
+                    context.append(token)
+        # decode(token) -> token, the reference's single-sequence call
+        runtime.reset()
+        prompt = random_tokens(config["vocab_size"], 6, seed=1)
+        token = None
+        for t in prompt:
+            token = runtime.decode(t)
+        if dtype == "float32":
+            assert token == plain.greedy(config, weights, prompt, 1)[0]
+        assert runtime.info["decode_calls"] >= 6
+
+
+def test_engine_tasks_equal_blocking_generation_and_survive_preemption(loaded):
+    m = loaded("B", "float32")
+    config, weights = m.plain_config, m.plain_weights
+    prompts = [random_tokens(m.config.vocab_size, n, seed=n) for n in (1, 9, 64, 100)]
+    expected = [plain.greedy(config, weights, p, 16) for p in prompts]
+    # a roomy engine, portions of 16 beside decode rows
+    runtime = _runtime(m, parallel_sequences=4, prefill_rows=16, max_batch_tokens=32)
+    ids = [runtime.task_submit(p, 16) for p in prompts]
+    events = []
+    while runtime.scheduler.has_work():
+        events += runtime.engine_step()
+    for task, want in zip(ids, expected):
+        assert [e[1] for e in events if e[0] == task and e[2] == 0] == want
+        assert [e[2] for e in events if e[0] == task][-1] == 1
+    # so few pages that the newest request must give way while decoding and be recomputed: same tokens
+    tight = _runtime(m, parallel_sequences=4, prefill_rows=32, max_batch_tokens=64, num_pages=3)
+    pressed = [(prompts[2], 40), (random_tokens(m.config.vocab_size, 60, seed=77), 80)]    # 104 and 140 tokens: 2 + 3 pages
+    ids = [tight.task_submit(p, n) for p, n in pressed]
+    result = tight.run()
+    assert tight.info["preemptions"] >= 1
+    for task, (prompt, n) in zip(ids, pressed):
+        assert result[task] == plain.greedy(config, weights, prompt, n)
+    assert tight.info["pages_free"] == 3 and tight.info["live_requests"] == 0
+    tight.stepper.cache.check_invariants()
+
+
+def test_seeded_sampling_does_not_depend_on_the_batch(loaded):
+    """Temperature 0.8, seed 7, portions of 16 mixed with decode rows: a request draws the
+    same tokens alone and among others, and they are the plain sampler's tokens given the
+    plain model's logits."""
+    m = loaded("B", "float32")
+    prompts = [random_tokens(m.config.vocab_size, n, seed=n + 3) for n in (1, 9, 64, 200)]
+    settings = dict(temperature=0.8, top_k=40, top_p=0.95, min_p=0.05, seed=7)
+    together = _runtime(m, parallel_sequences=4, prefill_rows=16, max_batch_tokens=40)
+    ids = [together.task_submit(p, 16, **settings) for p in prompts]
+    batch = together.run()
+    for task, prompt in zip(ids, prompts):
+        alone = _runtime(m, parallel_sequences=1, prefill_rows=512)
+        assert alone.generate(prompt, 16, **settings) == batch[task]
+    rng = plain.XorShift64Star(7)
+    context, want = list(prompts[1]), []
+    for _ in range(16):
+        logits = plain.forward(m.plain_config, m.plain_weights, context)[-1]
+        want.append(plain.sample(logits.astype(np.float32), 0.8, 40, 0.95, 0.05, rng))
+        context.append(want[-1])
+    assert batch[ids[1]] == want
+    # top_k = 0 takes the host path over the whole vocabulary
+    full = _runtime(m, parallel_sequences=1)
+    a = full.generate(prompts[1], 6, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, seed=3)
+    b = full.generate(prompts[1], 6, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, seed=3)
+    assert a == b and len(a) == 6
+
+
+def test_errors_are_reported_not_hidden(loaded):
+    from flyweight_amd.engine import EngineError, StepEntry, StepError
+    from flyweight_amd.cache import OutOfPages
+    m = loaded("A", "float32")
+    runtime = _runtime(m, parallel_sequences=2, num_pages=2)
+    with pytest.raises(EngineError, match="exceeds the context"):
+        runtime.task_submit([1] * 300, 200)
+    with pytest.raises(EngineError, match="empty"):
+        runtime.task_submit([], 2)
+    task = runtime.task_submit([1] * 100, 100)       # needs 4 pages, the pool has 2
+    events = runtime.engine_step()
+    assert (task, 0, 2) in events and "pages" in runtime.task_error(task)
+    stepper = m.stepper(num_pages=1, max_requests=2)
+    stepper.admit("a")
+    with pytest.raises(StepError, match="outside the vocabulary"):
+        stepper.step([StepEntry("a", [m.config.vocab_size], [0])])
+    with pytest.raises(StepError, match="not admitted"):
+        stepper.step([StepEntry("zz", [1], [0])])
+    with pytest.raises(StepError, match="twice"):
+        stepper.step([StepEntry("a", [1], [0]), StepEntry("a", [2], [0])])
+    with pytest.raises(OutOfPages):
+        stepper.step([StepEntry("a", [1] * 65, [])])
+    assert stepper.cache.length_of("a") == 0 and stepper.cache.groups[0].pool.in_use == 0   # nothing half-done
+    assert stepper.step([StepEntry("a", [1] * 64, [63])]).shape == (1, m.config.vocab_size)

@@ -1,0 +1,336 @@
+"""Each kernel alone against a plain float64 computation, at other sizes than the engine's
+tiny models use: widths and vocabularies that are no power of two, head sizes in steps of
+16, odd numbers of heads and groups."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+TOL = {torch.float32: 3e-6, torch.bfloat16: 1.2e-2}     # relative to the largest expected value
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from flyweight_amd.kernels import ops
+    ops.library()
+    return ops
+
+
+def gen(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed + sum(shape))
+    return torch.randn(*shape, generator=g, dtype=torch.float64) * scale
+
+
+def close(found, expected, dtype, factor=1.0):
+    found = found.detach().cpu().to(torch.float64)
+    assert found.shape == expected.shape
+    assert torch.isfinite(found).all()
+    limit = TOL[dtype] * factor * max(1.0, float(expected.abs().max()))
+    worst = float((found - expected).abs().max())
+    assert worst <= limit, f"largest difference {worst:.3e} exceeds {limit:.3e}"
+
+
+def as_dev(t, dtype):
+    return t.to(dtype).to(DEV).contiguous()
+
+
+def back(t):
+    """What the kernel really saw after rounding to its dtype."""
+    return t.detach().cpu().to(torch.float64)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_rows(ops, dtype):
+    table = as_dev(gen(301, 100), dtype)
+    ids = torch.tensor([0, 300, 7, 7, 150], dtype=torch.int32, device=DEV)
+    out = ops.embed_rows(table, ids)
+    assert out.dtype == torch.float32 and torch.equal(out.cpu(), table.float().cpu()[ids.cpu().long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [100, 4100])
+def test_rmsnorm_rows(ops, dtype, hidden):
+    x = gen(7, hidden, scale=3).float()
+    w = (1 + 0.1 * gen(hidden)).float()
+    want = x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-4) * w.double()
+    close(ops.rmsnorm_rows(x.to(DEV), w.to(DEV), 1e-4, dtype), want, dtype)
+    index = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    close(ops.rmsnorm_rows(x.to(DEV), w.to(DEV), 1e-4, dtype, row_index=index), want[[6, 0, 3]], dtype)
+    centered = x.double() / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-4) * (1 + w.double())
+    close(ops.rmsnorm_rows(x.to(DEV), w.to(DEV), 1e-4, dtype, one_centered=True), centered, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 70, 130), (5, 200, 96), (67, 129, 257), (130, 64, 40)])
+def test_gemm(ops, dtype, M, N, K):
+    a, w = as_dev(gen(M, K), dtype), as_dev(gen(N, K, seed=1, scale=K ** -0.5), dtype)
+    bias = gen(N, seed=2).float().to(DEV)
+    want = back(a) @ back(w).T
+    close(ops.gemm(a, w), want, dtype)
+    close(ops.gemm(a, w, bias, out_dtype=torch.float32), want + bias.cpu().double(), torch.float32)
+    residual = gen(M, N, seed=3).float().to(DEV)
+    before = residual.cpu().double()
+    ops.gemm(a, w, accumulate_into=residual)
+    close(residual, before + want, torch.float32)      # float32 sums of the rounded operands either way
+    if dtype == torch.bfloat16:     # a 32-bit weight beside bfloat16 activations stays 32-bit
+        w32 = gen(N, K, seed=1, scale=K ** -0.5).float().to(DEV)
+        close(ops.gemm(a, w32, out_dtype=torch.float32), back(a) @ w32.cpu().double().T, torch.float32)
+
+
+def test_gemm_rows_do_not_depend_on_the_batch(ops):
+    a, w = as_dev(gen(70, 200), torch.float32), as_dev(gen(90, 200, seed=1), torch.float32)
+    whole = ops.gemm(a, w)
+    assert torch.equal(ops.gemm(a[13:14].contiguous(), w)[0], whole[13])
+    assert torch.equal(ops.gemm(a[60:70].contiguous(), w), whole[60:70])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu(ops, dtype):
+    gu = as_dev(gen(5, 2 * 77, scale=4), dtype)
+    gu[0, 0], gu[0, 1] = 80.0, -80.0        # the sigmoid must not overflow
+    g, u = back(gu)[:, :77], back(gu)[:, 77:]
+    out = ops.swiglu(gu)
+    close(out, F.silu(g) * u, dtype)
+    wide = as_dev(gen(5, 2 * 77, scale=4), torch.float32)       # float32 in, rounded once on the way out
+    close(ops.swiglu(wide, out_dtype=dtype), F.silu(back(wide)[:, :77]) * back(wide)[:, 77:], dtype)
+
+
+def test_rope_table(ops):
+    positions = torch.tensor([0, 1, 63, 64, 4095, 131071], dtype=torch.int32, device=DEV)
+    inv = (1e6 ** (-torch.arange(24, dtype=torch.float64) * 2 / 48)).to(DEV)
+    cos, sin = ops.rope_table(positions, inv)
+    angle = positions.cpu().double()[:, None] * inv.cpu()[None]
+    assert float((cos.cpu().double() - torch.cos(angle)).abs().max()) < 1e-6
+    assert float((sin.cpu().double() - torch.sin(angle)).abs().max()) < 1e-6
+
+
+def conv_reference(bcx, taps, bias, state, segments):
+    """Per segment: the plain left-padded convolution over [state | segment]."""
+    rows, width = bcx.shape
+    H, L = taps.shape
+    out = torch.zeros(rows, H, dtype=torch.float64)
+    new_state = state.clone()
+    for first, count, slot in segments:
+        part = bcx[first:first + count]
+        bx = part[:, :H] * part[:, 2 * H:]
+        seq = torch.cat([state[slot].T, bx], dim=0)                 # [L-1 + count, H]
+        for t in range(count):
+            y = (taps.T * seq[t:t + L]).sum(0)
+            if bias is not None:
+                y = y + bias
+            out[first + t] = part[t, H:2 * H] * y
+        new_state[slot] = seq[-(L - 1):].T
+    return out, new_state
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,L,with_bias", [(70, 3, False), (130, 4, True), (257, 2, True), (64, 7, False)])
+def test_shortconv_mixed_segments(ops, dtype, H, L, with_bias):
+    # segments of 1, 2 (< L-1 for L = 4), L-1 and many rows; slots out of order
+    counts = [5, 1, 2, L - 1, 40, 1]
+    slots = [3, 0, 6, 2, 5, 1]
+    segments, first = [], 0
+    for count, slot in zip(counts, slots):
+        segments.append((first, count, slot))
+        first += count
+    rows = first
+    bcx = as_dev(gen(rows, 3 * H), dtype)
+    taps = gen(H, L, seed=1).float()
+    bias = gen(H, seed=2).float() if with_bias else None
+    state = gen(7, H, L - 1, seed=3).float()
+    want_out, want_state = conv_reference(back(bcx), taps.double(), None if bias is None else bias.double(), state.double(), segments)
+    row_seg = torch.tensor([s for s, (_, c, _) in enumerate(segments) for _ in range(c)], dtype=torch.int32, device=DEV)
+    seg_row0 = torch.tensor([f for f, _, _ in segments] + [rows], dtype=torch.int32, device=DEV)
+    seg_slot = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    dev_state = state.to(DEV)
+    out = ops.shortconv(bcx, taps.to(DEV), None if bias is None else bias.to(DEV), dev_state, row_seg, seg_row0, seg_slot, len(segments))
+    close(out, want_out, dtype)
+    close(dev_state, want_state, torch.float32, 10.0 if dtype == torch.bfloat16 else 1.0)
+    # all single rows: the fused decode variant, from the state the first call left
+    n = 4
+    bcx1 = as_dev(gen(n, 3 * H, seed=5), dtype)
+    segs1 = [(i, 1, s) for i, s in enumerate([2, 6, 0, 4])]
+    want_out1, want_state1 = conv_reference(back(bcx1), taps.double(), None if bias is None else bias.double(),
+                                            dev_state.cpu().double(), segs1)
+    ids = torch.arange(n, dtype=torch.int32, device=DEV)
+    out1 = ops.shortconv(bcx1, taps.to(DEV), None if bias is None else bias.to(DEV), dev_state, ids,
+                         torch.arange(n + 1, dtype=torch.int32, device=DEV), torch.tensor([2, 6, 0, 4], dtype=torch.int32, device=DEV), n)
+    close(out1, want_out1, dtype)
+    close(dev_state, want_state1, torch.float32, 10.0 if dtype == torch.bfloat16 else 1.0)
+
+
+def rope_reference(x, cos, sin, rotary):
+    half = rotary // 2
+    a, b, rest = x[..., :half], x[..., half:rotary], x[..., rotary:]
+    return torch.cat([a * cos - b * sin, b * cos + a * sin, rest], dim=-1)
+
+
+def scatter_setup(rows_per_seg, starts, num_pages, seed=0):
+    """Block tables with scattered pages, and the per-row index arrays."""
+    rng = np.random.default_rng(seed)
+    pages = rng.permutation(num_pages).tolist()
+    stride = max((s + n + 63) // 64 for s, n in zip(starts, rows_per_seg))
+    table = np.zeros((len(starts), stride), dtype=np.int32)
+    for i, (s, n) in enumerate(zip(starts, rows_per_seg)):
+        for b in range((s + n + 63) // 64):
+            table[i, b] = pages.pop()
+    row_seg = np.concatenate([np.full(n, i) for i, n in enumerate(rows_per_seg)]).astype(np.int32)
+    row_pos = np.concatenate([np.arange(s, s + n) for s, n in zip(starts, rows_per_seg)]).astype(np.int32)
+    return table, row_seg, row_pos
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,rotary,normed", [(4, 2, 16, 16, True), (3, 1, 48, 48, True), (6, 3, 80, 32, False),
+                                                     (2, 2, 128, 128, True), (5, 5, 256, 0, True)])
+def test_qk_norm_rope_kv_write(ops, dtype, nh, nkv, hd, rotary, normed):
+    rows_per_seg, starts = [3, 1, 70], [0, 63, 60]
+    table, row_seg, row_pos = scatter_setup(rows_per_seg, starts, num_pages=9)
+    rows = sum(rows_per_seg)
+    qkv = as_dev(gen(rows, (nh + 2 * nkv) * hd), dtype)
+    qw, kw = (1 + 0.1 * gen(hd, seed=1)).float(), (1 + 0.1 * gen(hd, seed=2)).float()
+    eps = 1e-5
+    inv = (1e4 ** (-torch.arange(max(rotary // 2, 1), dtype=torch.float64) * 2 / max(rotary, 1)))
+    angle = torch.tensor(row_pos, dtype=torch.float64)[:, None] * inv[None]
+    cos, sin = torch.cos(angle), torch.sin(angle)
+    k_pages = torch.full((9, nkv, 64, hd), 77.0, dtype=dtype, device=DEV)
+    v_pages = torch.full((9, nkv, hd, 64), 77.0, dtype=dtype, device=DEV)
+    d = lambda a: torch.tensor(a, device=DEV)       # noqa: E731
+    q_out = ops.qk_norm_rope_kv_write(qkv, nh, nkv, hd, qw.to(DEV) if normed else None, kw.to(DEV) if normed else None, eps,
+                                      cos.float().to(DEV) if rotary else None, sin.float().to(DEV) if rotary else None, rotary,
+                                      k_pages, v_pages, d(table), d(row_seg), d(row_pos))
+    x = back(qkv)
+    q = x[:, :nh * hd].reshape(rows, nh, hd)
+    k = x[:, nh * hd:(nh + nkv) * hd].reshape(rows, nkv, hd)
+    v = x[:, (nh + nkv) * hd:].reshape(rows, nkv, hd)
+    if normed:
+        q = q / torch.sqrt((q ** 2).mean(-1, keepdim=True) + eps) * qw.double()
+        k = k / torch.sqrt((k ** 2).mean(-1, keepdim=True) + eps) * kw.double()
+    if rotary:
+        q, k = rope_reference(q, cos[:, None], sin[:, None], rotary), rope_reference(k, cos[:, None], sin[:, None], rotary)
+    close(q_out, q.reshape(rows, nh * hd), dtype)
+    kp, vp = k_pages.cpu().double(), v_pages.cpu().double()
+    for r in range(rows):
+        page, slot = table[row_seg[r], row_pos[r] // 64], row_pos[r] % 64
+        close(kp[page, :, slot, :], k[r], dtype)
+        assert torch.equal(vp[page, :, :, slot], v[r])          # values are stored untouched
+    written = torch.zeros(9, 64, dtype=torch.bool)
+    for r in range(rows):
+        written[table[row_seg[r], row_pos[r] // 64], row_pos[r] % 64] = True
+    assert bool((kp.permute(0, 2, 1, 3)[~written] == 77.0).all()) and bool((vp.permute(0, 3, 1, 2)[~written] == 77.0).all())
+
+
+def attention_reference(q, keys, values, pos, scale, window, group):
+    out = torch.zeros_like(q)
+    for head in range(q.shape[0]):
+        lo = 0 if not window else max(0, pos - window + 1)
+        s = (keys[lo:pos + 1, head // group] @ q[head]) * scale
+        p = torch.softmax(s, dim=0)
+        out[head] = p @ values[lo:pos + 1, head // group]
+    return out
+
+
+def paged(keys, values, table_row, num_pages, dtype, poison=float("nan")):
+    """Scatter [T, nkv, hd] keys/values into pages; everything else is poison."""
+    T, nkv, hd = keys.shape
+    k_pages = torch.full((num_pages, nkv, 64, hd), poison, dtype=torch.float64)
+    v_pages = torch.full((num_pages, nkv, hd, 64), poison, dtype=torch.float64)
+    for t in range(T):
+        k_pages[table_row[t // 64], :, t % 64, :] = keys[t]
+        v_pages[table_row[t // 64], :, :, t % 64] = values[t]
+    return k_pages.to(dtype).to(DEV), v_pages.to(dtype).to(DEV)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (3, 1, 48, 0), (6, 3, 80, 0), (2, 2, 128, 0), (5, 1, 256, 0),
+                                              (4, 2, 32, 70), (4, 4, 64, 64), (2, 1, 64, 1)])
+def test_attention_over_scattered_pages(ops, dtype, nh, nkv, hd, window):
+    # the block table of the reference's contract test: pages {9, 2, 14, 5} of a pool of 16
+    # (native/tests/paged_kv_contract.cpp:89-242)
+    T = 250
+    table_row = [9, 2, 14, 5]
+    keys, values = gen(T, nkv, hd).to(dtype).double(), gen(T, nkv, hd, seed=1).to(dtype).double()
+    k_pages, v_pages = paged(keys, values, table_row, 16, dtype)
+    positions = [0, 1, 62, 63, 64, 65, 127, 128, 129, 200, 249]
+    q = as_dev(gen(len(positions), nh * hd, seed=2), dtype)
+    scale = 1 / math.sqrt(hd)
+    table = torch.tensor([table_row], dtype=torch.int32, device=DEV)
+    row_seg = torch.zeros(len(positions), dtype=torch.int32, device=DEV)
+    row_pos = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    out = ops.attention_generic(q, nh, nkv, hd, k_pages, v_pages, table, row_seg, row_pos, scale, window)
+    want = torch.stack([attention_reference(back(q)[i].reshape(nh, hd), keys, values, p, scale, window, nh // nkv).reshape(-1)
+                        for i, p in enumerate(positions)])
+    close(out, want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_one_far_key_and_the_edges_of_a_window(ops, dtype):
+    """One key is made to match the query far better than all others, so the output is
+    that key's value: at a far position, at both sides of every page edge, and just inside
+    and just outside a window."""
+    nh, nkv, hd, T = 2, 1, 64, 700
+    table_row = list(range(11))
+    scale = 1 / math.sqrt(hd)
+    keys = gen(T, nkv, hd, scale=0.1)
+    values = gen(T, nkv, hd, seed=1)
+    direction = torch.zeros(hd, dtype=torch.float64); direction[5] = 1.0
+    q = torch.zeros(1, nh * hd, dtype=torch.float64)
+    q[0, 5] = q[0, hd + 5] = 60.0
+    table = torch.tensor([table_row], dtype=torch.int32, device=DEV)
+    zero = torch.zeros(1, dtype=torch.int32, device=DEV)
+    pos = torch.tensor([T - 1], dtype=torch.int32, device=DEV)
+    for target in (3, 63, 64, 127, 128, 640, 698, 699):
+        k = keys.clone(); k[target, 0] = direction * 8
+        k_pages, v_pages = paged(k.to(dtype).double(), values.to(dtype).double(), table_row, 11, dtype)
+        out = ops.attention_generic(as_dev(q, dtype), nh, nkv, hd, k_pages, v_pages, table, zero, pos, scale, 0)
+        close(out[0, :hd], values[target, 0].to(dtype).double(), dtype)
+    window = 100            # the row at 699 sees 600..699
+    for target, seen in ((600, True), (599, False), (640, True)):
+        k = keys.clone(); k[target, 0] = direction * 8
+        k_pages, v_pages = paged(k.to(dtype).double(), values.to(dtype).double(), table_row, 11, dtype)
+        out = ops.attention_generic(as_dev(q, dtype), nh, nkv, hd, k_pages, v_pages, table, zero, pos, scale, window)
+        hit = float((out[0, :hd].cpu().double() - values[target, 0].to(dtype).double()).abs().max()) < 0.05
+        assert hit == seen, f"key {target} with a window of {window} at position {T - 1}"
+
+
+def test_argmax_and_topk(ops):
+    logits = gen(5, 1000).float()
+    logits[0, 17] = logits[0, 900] = 50.0               # ties go to the lowest id
+    logits[1, 999] = 60.0                               # the last entry of a vocabulary that is no power of two
+    logits[2, :] = -3.0                                 # all equal
+    logits[3, 5] = float("nan"); logits[3, 6] = 40.0    # NaN sorts last
+    ids = ops.argmax_rows(logits.to(DEV)).cpu().tolist()
+    assert ids[:4] == [17, 999, 0, 6] and ids[4] == int(logits[4].argmax())
+    values, top = ops.topk_rows(logits.to(DEV), 7)
+    assert top[0, :2].cpu().tolist() == [17, 900] and top[2].cpu().tolist() == list(range(7))
+    order = sorted(range(1000), key=lambda i: (-float(logits[4, i]), i))[:7]
+    assert top[4].cpu().tolist() == order and torch.equal(values[4].cpu(), logits[4][order])
+
+
+def test_kernels_refuse_what_they_were_not_written_for(ops):
+    from flyweight_amd.kernels.ops import KernelError
+    x = torch.zeros(2, 8, device=DEV)
+    with pytest.raises(KernelError, match="GPU only"):
+        ops.rmsnorm_rows(torch.zeros(2, 8), torch.ones(8), 1e-5, torch.float32)
+    with pytest.raises(KernelError, match="weight"):
+        ops.rmsnorm_rows(x, torch.ones(9, device=DEV), 1e-5, torch.float32)
+    with pytest.raises(KernelError):
+        ops.gemm(x, torch.zeros(4, 9, device=DEV))
+    with pytest.raises(KernelError, match="float32 or bfloat16"):
+        ops.gemm(x.half(), torch.zeros(4, 8, device=DEV).half())
+    with pytest.raises(KernelError, match="head_dim"):
+        ops.attention_generic(torch.zeros(1, 512, device=DEV), 1, 1, 512, torch.zeros(1, 1, 64, 512, device=DEV),
+                              torch.zeros(1, 1, 512, 64, device=DEV), torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+                              torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV), 1.0)
+    with pytest.raises(KernelError, match="k must be"):
+        ops.topk_rows(torch.zeros(1, 300, device=DEV), 257)
+    with pytest.raises(KernelError, match="kernel size"):
+        ops.shortconv(torch.zeros(1, 24, device=DEV), torch.zeros(8, 17, device=DEV), None, torch.zeros(1, 8, 16, device=DEV),
+                      torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(2, dtype=torch.int32, device=DEV),
+                      torch.zeros(1, dtype=torch.int32, device=DEV), 1)

@@ -1,0 +1,309 @@
+"""Each part of a layer alone, built from its PartSpec with its own sizes, against the
+plain implementation's function for that part; and a toy mixer with state of its own,
+defined here, that is registered, built and stepped without touching the framework."""
+
+import dataclasses
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_lfm2 as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = torch.device("cuda:0")
+DTYPES = [torch.float32, torch.bfloat16]
+TOL = {torch.float32: 5e-6, torch.bfloat16: 2e-2}
+
+
+def close(found, expected, dtype):
+    found = found.detach().cpu().double().numpy()
+    limit = TOL[dtype] * max(1.0, float(np.abs(expected).max()))
+    assert found.shape == expected.shape and np.isfinite(found).all()
+    assert float(np.abs(found - expected).max()) <= limit, f"{float(np.abs(found - expected).max()):.3e} > {limit:.3e}"
+
+
+def bound(part, dtype, seed=0):
+    """Random tensors for a part, bound on the GPU; returns them as float64 numpy too."""
+    from flyweight_amd.weights import random_tensors
+    from flyweight_amd.weights.loader import storage_dtype
+    tensors = random_tensors(part.tensors(), seed, torch.bfloat16, scale="fan_in")
+    device = {n: t.to(storage_dtype(part.tensors()[n].role, t.dtype, dtype)).to(DEV) for n, t in tensors.items()}
+    part.bind(device, dtype, DEV)
+    return {n: t.double().numpy() for n, t in tensors.items()}
+
+
+def context(part_needs, segments, num_pages=8):
+    """segments: (request, start, count). Sequences are first advanced to ``start``."""
+    from flyweight_amd.cache import CacheManager
+    from flyweight_amd.engine.step import StepContext, StepEntry
+    return CacheManager, StepContext, StepEntry
+
+
+class Harness:
+    """A cache for one mixer and step contexts over it."""
+
+    def __init__(self, mixer, dtype, num_pages=8, max_requests=4):
+        from flyweight_amd.cache import CacheManager
+        need = mixer.cache_need()
+        self.cache = CacheManager({0: need} if need is not None else {}, num_pages=num_pages, max_requests=max_requests,
+                                  dtype=dtype, device=DEV)
+        self.mixer = mixer
+
+    def run(self, entries, h):
+        """entries: [(request, count)]; h: [rows, hidden] on the device. Returns the mixer's
+        contribution to the residual."""
+        from flyweight_amd.config import ScheduleEntry
+        from flyweight_amd.engine.step import StepContext, StepEntry
+        step = []
+        for request, count in entries:
+            if request not in self.cache.requests:
+                self.cache.admit(request)
+            self.cache.reserve(request, self.cache.length_of(request) + count)
+            step.append(StepEntry(request, [0] * count, []))
+        ctx = StepContext(step, self.cache, DEV, vocab_size=1, max_positions=1 << 20)
+        residual = torch.zeros(h.shape[0], self.mixer.hidden, dtype=torch.float32, device=DEV)
+        self.mixer.forward(h, residual, ctx, ctx.cache_view(self.cache, ScheduleEntry(0, cache=0)))
+        for request, length in zip(ctx.requests, ctx.new_lengths):
+            self.cache.commit(request, length)
+        return residual
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_part(dtype):
+    from flyweight_amd.config import PartSpec
+    from flyweight_amd.parts import build_part
+    part = build_part("norm", PartSpec("rmsnorm", {"size": 100, "eps": 3e-4}, prefix="n."))
+    w = bound(part, dtype)
+    x = torch.randn(6, 100, generator=torch.Generator().manual_seed(1)) * 2
+    close(part.forward(x.to(DEV), None), plain.rms_norm(x.double().numpy(), w["n.weight"], 3e-4), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_swiglu_part(dtype):
+    from flyweight_amd.config import PartSpec
+    from flyweight_amd.parts import build_part
+    part = build_part("ffn", PartSpec("swiglu", {"hidden_size": 72, "intermediate_size": 200,
+                                                 "names": {"gate": "w1", "up": "w3", "down": "w2"}}, prefix="f."))
+    w = bound(part, dtype)
+    h = (torch.randn(9, 72, generator=torch.Generator().manual_seed(2))).to(dtype)
+    residual = torch.ones(9, 72, dtype=torch.float32, device=DEV)
+    part.forward(h.to(DEV), residual, None)
+    close(residual, 1.0 + plain.swiglu(h.double().numpy(), w, "f."), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,kernel,bias", [(72, 3, False), (40, 5, True)])
+def test_short_conv_part_whole_and_cut(dtype, hidden, kernel, bias):
+    from flyweight_amd.config import PartSpec
+    from flyweight_amd.parts import build_part
+    part = build_part("mixer", PartSpec("short_conv", {"hidden_size": hidden, "kernel_size": kernel, "bias": bias}, prefix="c."))
+    w = bound(part, dtype, seed=3)
+    T = 50
+    h = torch.randn(T, hidden, generator=torch.Generator().manual_seed(4)).to(dtype)
+    want = plain.short_conv_mixer(h.double().numpy(), w, "c.", {"hidden_size": hidden, "conv_bias": bias})
+    harness = Harness(part, dtype)
+    close(harness.run([("whole", T)], h.to(DEV)), want, dtype)
+    pieces, at = [], 0
+    for n in (3, 1, 2, 20, 1, 1, 22):       # portions shorter than the kernel's reach too
+        pieces.append(harness.run([("cut", n)], h[at:at + n].contiguous().to(DEV)))
+        at += n
+    close(torch.cat(pieces), want, dtype)
+    # two sequences in one batch, one decoding while the other is in a portion
+    other = torch.randn(8, hidden, generator=torch.Generator().manual_seed(5)).to(dtype)
+    want_other = plain.short_conv_mixer(other.double().numpy(), w, "c.", {"hidden_size": hidden, "conv_bias": bias})
+    first = harness.run([("x", 7), ("y", 5)], torch.cat([other[:7], h[:5]]).to(DEV))
+    second = harness.run([("y", 3), ("x", 1)], torch.cat([h[5:8], other[7:8]]).to(DEV))
+    close(torch.cat([first[:7], second[3:4]]), want_other, dtype)
+    close(torch.cat([first[7:], second[:3]]), want[:8], dtype)
+
+
+def attention_spec(hidden, nh, nkv, hd, theta, rotary, eps, window=None, qk_norm=True):
+    from flyweight_amd.config import PartSpec
+    return PartSpec("gqa_attention", {
+        "hidden_size": hidden, "num_heads": nh, "num_kv_heads": nkv, "head_dim": hd, "qk_norm": qk_norm, "qk_norm_eps": eps,
+        "window": window, "softmax_scale": 1 / math.sqrt(hd),
+        "position": PartSpec("rotary_neox", {"theta": theta, "rotary_dim": rotary, "head_dim": hd}),
+        "names": {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "out_proj", "q_norm": "q_layernorm", "k_norm": "k_layernorm"},
+    }, prefix="a.")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,nh,nkv,hd,theta,eps", [(96, 6, 2, 16, 100.0, 1e-5), (144, 3, 3, 48, 1e6, 1e-6)])
+def test_attention_part_whole_cut_and_batched(dtype, hidden, nh, nkv, hd, theta, eps):
+    from flyweight_amd.parts import build_part
+    part = build_part("mixer", attention_spec(hidden, nh, nkv, hd, theta, hd, eps))
+    w = bound(part, dtype, seed=6)
+    T = 150
+    h = torch.randn(T, hidden, generator=torch.Generator().manual_seed(7)).to(dtype)
+    config = {"num_attention_heads": nh, "num_key_value_heads": nkv, "hidden_size": nh * hd, "norm_eps": eps, "rope_theta": theta}
+    want = plain.attention_mixer(h.double().numpy(), w, "a.", config)
+    harness = Harness(part, dtype)
+    close(harness.run([("whole", T)], h.to(DEV)), want, dtype)
+    pieces, at = [], 0
+    for n in (60, 4, 1, 1, 63, 2, 19):
+        pieces.append(harness.run([("cut", n)], h[at:at + n].contiguous().to(DEV)))
+        at += n
+    close(torch.cat(pieces), want, dtype)
+    # shifting every position changes nothing: only distances count (first 64 positions skipped)
+    shifted = Harness(part, dtype)
+    shifted.run([("s", 64)], torch.zeros(64, hidden, dtype=dtype, device=DEV))
+    # ... but the zero rows are keys too, so compare with the plain model given the same prefix
+    prefix = np.concatenate([np.zeros((64, hidden)), h[:40].double().numpy()])
+    close(shifted.run([("s", 40)], h[:40].contiguous().to(DEV)), plain.attention_mixer(prefix, w, "a.", config)[64:], dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_part_with_a_window_and_partial_rotation(dtype):
+    """Options LFM2 does not use but the part takes as parameters."""
+    from flyweight_amd.parts import build_part
+    hidden, nh, nkv, hd, window, rotary = 64, 4, 2, 32, 70, 16
+    part = build_part("mixer", attention_spec(hidden, nh, nkv, hd, 1e4, rotary, 1e-5, window=window, qk_norm=False))
+    w = bound(part, dtype, seed=8)
+    T = 200
+    h = torch.randn(T, hidden, generator=torch.Generator().manual_seed(9)).to(dtype)
+    x = h.double().numpy()
+    q = (x @ w["a.q_proj.weight"].T).reshape(T, nh, hd)
+    k = (x @ w["a.k_proj.weight"].T).reshape(T, nkv, hd)
+    v = (x @ w["a.v_proj.weight"].T).reshape(T, nkv, hd)
+    cos, sin = plain.rope_angles(np.arange(T), rotary, 1e4)
+    q, k = plain.rope_half_split(q, cos, sin), plain.rope_half_split(k, cos, sin)
+    want = plain.causal_attention(q, k, v, 1 / math.sqrt(hd), window=window).reshape(T, nh * hd) @ w["a.out_proj.weight"].T
+    harness = Harness(part, dtype, num_pages=4)
+    pieces, at = [], 0
+    for n in (100, 1, 1, 30, 68):
+        pieces.append(harness.run([("r", n)], h[at:at + n].contiguous().to(DEV)))
+        at += n
+    close(torch.cat(pieces), want, dtype)
+    # the next query (position 200) sees keys 131..200: blocks 0 and 1 are passed, their pages back in the pool
+    assert harness.cache.groups[0].tables["r"][:2] == [-1, -1] and harness.cache.groups[0].pool.in_use == 2
+
+
+# ----- a toy mixer with state of its own ----------------------------------------------------
+def register_toy():
+    from flyweight_amd.cache import FixedState
+    from flyweight_amd.parts import Linear, Mixer, register_mixer
+    from flyweight_amd.weights import TensorDecl
+
+    @register_mixer("toy_running_mean")
+    class RunningMean(Mixer):
+        """out_t = W . mean(h_0..h_t). State per request: the running sum and the count."""
+
+        def __init__(self, spec):
+            super().__init__(spec)
+            self.hidden = int(spec["hidden_size"])
+
+        def cache_need(self):
+            return FixedState((self.hidden + 1,), torch.float32)
+
+        def tensors(self):
+            return {self.prefix + "mix.weight": TensorDecl((self.hidden, self.hidden))}
+
+        def bind(self, tensors, dtype, device):
+            super().bind(tensors, dtype, device)
+            self.mix = Linear(tensors[self.prefix + "mix.weight"])
+
+        def forward(self, h, residual, ctx, cache):
+            means = torch.empty_like(h)
+            for seg in range(ctx.num_segments):
+                lo, hi, slot = ctx.host_seg_row0[seg], ctx.host_seg_row0[seg + 1], ctx.host_seg_slot[seg]
+                state = cache.state[slot]
+                sums = state[:self.hidden] + torch.cumsum(h[lo:hi].float(), dim=0)
+                counts = state[self.hidden] + torch.arange(1, hi - lo + 1, device=h.device, dtype=torch.float32)
+                means[lo:hi] = (sums / counts[:, None]).to(h.dtype)
+                state[:self.hidden] = sums[-1]
+                state[self.hidden] = counts[-1]
+            self.mix.accumulate(means, residual)
+    return RunningMean
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_mixer_with_its_own_state_is_registered_built_and_stepped(tmp_path, dtype):
+    from flyweight_amd.config import LayerSpec, PartSpec, ScheduleEntry, config_from_dict
+    from flyweight_amd.engine import CausalLM, StepEntry, Stepper
+    from flyweight_amd.engine.model import parse_dtype
+    from flyweight_amd.weights import load_tensors, random_tensors, write_file
+    from helpers import TINY_A
+    register_toy()
+    base = config_from_dict(TINY_A).model_spec()
+    toy_layer = dataclasses.replace(base.layers[0], mixer=PartSpec("toy_running_mean", {"hidden_size": 64}, prefix="model.layers.0.toy."))
+    # layers: toy, attention, conv, attention; the schedule runs the toy layer twice (two states)
+    # and lets a second execution of layer 1 read the keys its first execution wrote
+    spec = dataclasses.replace(base, layers=(toy_layer,) + base.layers[1:], schedule=(
+        ScheduleEntry(0, cache=0), ScheduleEntry(1, cache=1), ScheduleEntry(2, cache=2), ScheduleEntry(0, cache=5),
+        ScheduleEntry(1, cache=1, writes_cache=False), ScheduleEntry(3, cache=3)))
+    model = CausalLM(spec)
+    folder = str(tmp_path / "toy")
+    os.makedirs(folder)
+    write_file(os.path.join(folder, "model.safetensors"), random_tensors(model.tensors(), 4, scale="fan_in"))
+    torch_dtype = parse_dtype(dtype)
+    tensors = load_tensors(folder, model.tensors(), torch_dtype, DEV)
+    model.bind(tensors, torch_dtype, DEV)
+    assert set(model.cache_needs()) == {0, 1, 2, 3, 5}
+    w = {n: t.double().cpu().numpy() for n, t in tensors.items()}
+
+    def expected(tokens):
+        config = dict(TINY_A)
+        eps = config["norm_eps"]
+        x = w["model.embed_tokens.weight"][tokens]
+        def toy(x):
+            h = plain.rms_norm(x, w["model.layers.0.operator_norm.weight"], eps)
+            means = np.cumsum(h, axis=0) / np.arange(1, len(h) + 1)[:, None]
+            x = x + means @ w["model.layers.0.toy.mix.weight"].T
+            return x + plain.swiglu(plain.rms_norm(x, w["model.layers.0.ffn_norm.weight"], eps), w, "model.layers.0.feed_forward.")
+        def attention(x, i, reuse=None):
+            p = f"model.layers.{i}."
+            h = plain.rms_norm(x, w[p + "operator_norm.weight"], eps)
+            T, nh, nkv, hd = len(x), 4, 2, 16
+            q = plain.rms_norm((h @ w[p + "self_attn.q_proj.weight"].T).reshape(T, nh, hd), w[p + "self_attn.q_layernorm.weight"], eps)
+            cos, sin = plain.rope_angles(np.arange(T), hd, config["rope_theta"])
+            q = plain.rope_half_split(q, cos, sin)
+            if reuse is None:
+                k = plain.rms_norm((h @ w[p + "self_attn.k_proj.weight"].T).reshape(T, nkv, hd), w[p + "self_attn.k_layernorm.weight"], eps)
+                reuse = (plain.rope_half_split(k, cos, sin), (h @ w[p + "self_attn.v_proj.weight"].T).reshape(T, nkv, hd))
+            out = plain.causal_attention(q, reuse[0], reuse[1], 0.25).reshape(T, nh * hd) @ w[p + "self_attn.out_proj.weight"].T
+            x = x + out
+            return x + plain.swiglu(plain.rms_norm(x, w[p + "ffn_norm.weight"], eps), w, p + "feed_forward."), reuse
+        def conv(x, i):
+            p = f"model.layers.{i}."
+            x = x + plain.short_conv_mixer(plain.rms_norm(x, w[p + "operator_norm.weight"], eps), w, p + "conv.", config)
+            return x + plain.swiglu(plain.rms_norm(x, w[p + "ffn_norm.weight"], eps), w, p + "feed_forward.")
+        x = toy(x)
+        x, kv = attention(x, 1)
+        x = conv(x, 2)
+        x = toy(x)
+        x, _ = attention(x, 1, reuse=kv)
+        x, _ = attention(x, 3)
+        return plain.rms_norm(x, w["model.embedding_norm.weight"], eps) @ w["model.embed_tokens.weight"].T
+
+    rng = np.random.default_rng(0)
+    a, b = rng.integers(0, 256, 90).tolist(), rng.integers(0, 256, 70).tolist()
+    stepper = Stepper(model, num_pages=4, max_requests=2)
+    stepper.admit("a"); stepper.admit("b")
+    got = {"a": [], "b": []}
+    plan = [[("a", 40)], [("a", 1), ("b", 30)], [("b", 2), ("a", 9)], [("a", 40), ("b", 38)]]
+    at = {"a": 0, "b": 0}
+    for step in plan:
+        entries = []
+        for request, n in step:
+            tokens = (a if request == "a" else b)[at[request]:at[request] + n]
+            entries.append(StepEntry(request, tokens, list(range(n))))
+            at[request] += n
+        logits = stepper.step(entries).cpu().numpy()
+        row = 0
+        for request, n in step:
+            got[request].append(logits[row:row + n])
+            row += n
+    tolerance = {"float32": 2e-5, "bfloat16": 2e-2}[dtype]
+    for request, tokens in (("a", a), ("b", b)):
+        want = expected(tokens)
+        found = np.concatenate(got[request])
+        assert np.abs(found - want).max() <= tolerance * np.abs(want).max()
+    # the toy state slot is zeroed for the next request
+    stepper.release("a")
+    stepper.admit("c")
+    again = stepper.step([StepEntry("c", a[:20], list(range(20)))]).cpu().numpy()
+    assert np.abs(again - expected(a[:20])).max() <= tolerance * np.abs(expected(a[:20])).max()

@@ -1,0 +1,199 @@
+"""Pins the plain implementation (tests/plain_lfm2.py) by what fixes it beside the
+reference's text: special cases that reduce to a library routine, invariants, and the
+reference's own recurrences, each chosen so that a plausible mistake fails it."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_lfm2 as plain
+from helpers import CONFIGS, make_model, random_tokens
+
+RNG = np.random.default_rng(0)
+
+
+def test_rms_norm():
+    x = RNG.normal(size=(5, 24)) * 3
+    w = RNG.normal(size=24)
+    eps = 1e-3
+    y = plain.rms_norm(x, np.ones(24), eps)
+    n = x.shape[-1]
+    sq = (x * x).sum(-1)
+    np.testing.assert_allclose((y * y).sum(-1), n * sq / (sq + n * eps), rtol=1e-12)
+    np.testing.assert_allclose(plain.rms_norm(x, w, eps), x / np.sqrt((x * x).mean(-1, keepdims=True) + eps) * w, rtol=1e-12)
+    # the weight multiplies directly (not 1 + w): a zero weight gives zero
+    assert np.abs(plain.rms_norm(x, np.zeros(24), eps)).max() == 0.0
+    # scale invariance up to eps; eps inside the root (a large eps shrinks the output)
+    np.testing.assert_allclose(plain.rms_norm(1e4 * x, w, 1e-12), plain.rms_norm(x, w, 1e-12), rtol=1e-6)
+    assert np.abs(plain.rms_norm(x, w, 100.0)).max() < np.abs(plain.rms_norm(x, w, eps)).max() / 3
+
+
+def test_short_conv_is_a_left_padded_depthwise_convolution():
+    T, H, L = 11, 6, 4
+    bx, taps = RNG.normal(size=(T, H)), RNG.normal(size=(H, L))
+    y = plain.causal_depthwise_conv(bx, taps)
+    lib = F.conv1d(torch.tensor(bx.T[None]), torch.tensor(taps[:, None, :]), groups=H, padding=L - 1)[0, :, :T].T.numpy()
+    np.testing.assert_allclose(y, lib, rtol=1e-12, atol=1e-12)
+    for c in range(H):      # np.convolve flips its kernel
+        np.testing.assert_allclose(y[:, c], np.convolve(bx[:, c], taps[c, ::-1])[:T], rtol=1e-12, atol=1e-12)
+    # the last tap multiplies the current token
+    identity = np.zeros((H, L)); identity[:, -1] = 1.0
+    np.testing.assert_allclose(plain.causal_depthwise_conv(bx, identity), bx)
+    oldest = np.zeros((H, L)); oldest[:, 0] = 1.0
+    np.testing.assert_allclose(plain.causal_depthwise_conv(bx, oldest)[L - 1:], bx[:T - L + 1])
+    assert np.abs(plain.causal_depthwise_conv(bx, oldest)[:L - 1]).max() == 0.0     # zero before the start
+
+
+def test_short_conv_equals_the_reference_ring_recurrence():
+    # native/include/flyweight_v2_native_kernels.hpp:1302-1319: state = last L-1 values of bx, oldest first
+    T, H, L = 9, 5, 3
+    bx, taps = RNG.normal(size=(T, H)), RNG.normal(size=(H, L))
+    state = np.zeros((H, L - 1))
+    rows = []
+    for t in range(T):
+        value = taps[:, L - 1] * bx[t]
+        for i in range(L - 1):
+            value = value + taps[:, i] * state[:, i]
+        state = np.concatenate([state[:, 1:], bx[t][:, None]], axis=1)
+        rows.append(value)
+    np.testing.assert_allclose(plain.causal_depthwise_conv(bx, taps), np.stack(rows), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(state, bx[-(L - 1):].T)      # the state is the last L-1 columns of bx
+
+
+def _conv_weights(H, L, bias):
+    w = {"p.in_proj.weight": RNG.normal(size=(3 * H, H)), "p.conv.weight": RNG.normal(size=(H, 1, L)),
+         "p.out_proj.weight": RNG.normal(size=(H, H))}
+    if bias:
+        w.update({"p.in_proj.bias": RNG.normal(size=3 * H), "p.conv.bias": RNG.normal(size=H), "p.out_proj.bias": RNG.normal(size=H)})
+    return w
+
+
+def test_in_proj_thirds_are_b_c_x():
+    H, L, T = 8, 3, 6
+    config = {"hidden_size": H, "conv_bias": False}
+    w = _conv_weights(H, L, False)
+    h = RNG.normal(size=(T, H))
+    out = plain.short_conv_mixer(h, w, "p.", config)
+    swapped = dict(w)
+    m = w["p.in_proj.weight"]
+    swapped["p.in_proj.weight"] = np.concatenate([m[2 * H:], m[H:2 * H], m[:H]])       # B <-> x: B*x is unchanged
+    np.testing.assert_allclose(plain.short_conv_mixer(h, swapped, "p.", config), out, rtol=1e-12)
+    gate_off = dict(w)
+    gate_off["p.in_proj.weight"] = np.concatenate([m[:H], np.zeros((H, H)), m[2 * H:]])  # C = 0 silences the mixer
+    assert np.abs(plain.short_conv_mixer(h, gate_off, "p.", config)).max() == 0.0
+    other = dict(w)
+    other["p.in_proj.weight"] = np.concatenate([np.zeros((H, H)), m[H:]])               # so does B = 0
+    assert np.abs(plain.short_conv_mixer(h, other, "p.", config)).max() == 0.0
+    # C gates after the convolution: with identity taps the mixer is out_proj(C * B * x)
+    ident = dict(w); taps = np.zeros((H, 1, L)); taps[:, 0, -1] = 1.0; ident["p.conv.weight"] = taps
+    bcx = h @ m.T
+    np.testing.assert_allclose(plain.short_conv_mixer(h, ident, "p.", config),
+                               (bcx[:, H:2 * H] * bcx[:, :H] * bcx[:, 2 * H:]) @ w["p.out_proj.weight"].T, rtol=1e-12)
+
+
+def test_conv_biases_sit_after_each_linear_map():
+    H, L, T = 4, 4, 5
+    w = _conv_weights(H, L, True)
+    h = RNG.normal(size=(T, H))
+    out = plain.short_conv_mixer(h, w, "p.", {"hidden_size": H, "conv_bias": True})
+    bcx = h @ w["p.in_proj.weight"].T + w["p.in_proj.bias"]
+    y = plain.causal_depthwise_conv(bcx[:, :H] * bcx[:, 2 * H:], w["p.conv.weight"].reshape(H, L)) + w["p.conv.bias"]
+    np.testing.assert_allclose(out, (bcx[:, H:2 * H] * y) @ w["p.out_proj.weight"].T + w["p.out_proj.bias"], rtol=1e-12)
+    lib = F.conv1d(torch.tensor((bcx[:, :H] * bcx[:, 2 * H:]).T[None]), torch.tensor(w["p.conv.weight"]),
+                   bias=torch.tensor(w["p.conv.bias"]), groups=H, padding=L - 1)[0, :, :T].T.numpy()
+    np.testing.assert_allclose(y, lib, rtol=1e-12)
+
+
+def test_rope():
+    hd, theta = 16, 100.0
+    x = RNG.normal(size=(7, 3, hd))
+    cos, sin = plain.rope_angles(np.arange(7), hd, theta)
+    np.testing.assert_allclose(np.arctan2(sin[3], cos[3]) % (2 * np.pi), (3 * theta ** (-np.arange(8) * 2 / hd)) % (2 * np.pi), rtol=1e-9)
+    rotated = plain.rope_half_split(x, cos, sin)
+    np.testing.assert_allclose(rotated[0], x[0])                                        # position 0: identity
+    np.testing.assert_allclose((rotated ** 2).sum(-1), (x ** 2).sum(-1), rtol=1e-12)    # a rotation
+    # half-split pairing: a one-hot channel 0 leaks into channel hd/2, not channel 1
+    onehot = np.zeros((1, 1, hd)); onehot[0, 0, 0] = 1.0
+    c1, s1 = plain.rope_angles(np.array([1]), hd, theta)
+    r = plain.rope_half_split(onehot, c1, s1)[0, 0]
+    assert abs(r[0] - math.cos(1.0)) < 1e-12 and abs(r[hd // 2] - math.sin(1.0)) < 1e-12 and r[1] == 0.0
+    # scores depend on distances only
+    q, k = RNG.normal(size=(1, 1, hd)), RNG.normal(size=(1, 1, hd))
+    def score(p, t):
+        cp, sp = plain.rope_angles(np.array([p]), hd, theta)
+        ct, st = plain.rope_angles(np.array([t]), hd, theta)
+        return float((plain.rope_half_split(q, cp, sp) * plain.rope_half_split(k, ct, st)).sum())
+    assert abs(score(9, 4) - score(105, 100)) < 1e-9 and abs(score(9, 4) - score(4, 9)) > 1e-3
+    # a partial rotation leaves the tail alone
+    cp, sp = plain.rope_angles(np.arange(7), 8, theta)
+    np.testing.assert_allclose(plain.rope_half_split(x, cp, sp)[..., 8:], x[..., 8:])
+
+
+def test_attention_special_cases_and_library_agreement():
+    T, nh, nkv, hd = 9, 6, 2, 8
+    q, k, v = RNG.normal(size=(T, nh, hd)), RNG.normal(size=(T, nkv, hd)), RNG.normal(size=(T, nkv, hd))
+    scale = 1 / math.sqrt(hd)
+    out = plain.causal_attention(q, k, v, scale)
+    group = nh // nkv
+    np.testing.assert_allclose(out[0], np.repeat(v[0], group, axis=0))                  # one key: the value itself
+    same = plain.causal_attention(q, np.repeat(k[:1], T, axis=0), v, scale)
+    np.testing.assert_allclose(same[4, 0], v[:5, 0].mean(0), rtol=1e-12)                # equal keys: the mean
+    tq, tk, tv = (torch.tensor(a).transpose(0, 1)[None] for a in (q, k, v))
+    lib = F.scaled_dot_product_attention(tq, tk.repeat_interleave(group, 1), tv.repeat_interleave(group, 1), is_causal=True)
+    np.testing.assert_allclose(out, lib[0].transpose(0, 1).numpy(), rtol=1e-10, atol=1e-12)
+    # causality: a later token changes nothing earlier
+    k2, v2 = k.copy(), v.copy(); k2[6] += 1.0; v2[6] -= 2.0
+    np.testing.assert_allclose(plain.causal_attention(q, k2, v2, scale)[:6], out[:6])
+    # a window of w keys: the row sees exactly its last w
+    windowed = plain.causal_attention(q, k, v, scale, window=3)
+    np.testing.assert_allclose(windowed[:3], out[:3])
+    np.testing.assert_allclose(windowed[7], plain.causal_attention(q[5:8], k[5:8], v[5:8], scale)[2], rtol=1e-12)
+
+
+def test_swiglu_and_its_tails():
+    h = RNG.normal(size=(4, 6))
+    w = {"f.w1.weight": RNG.normal(size=(10, 6)), "f.w3.weight": RNG.normal(size=(10, 6)), "f.w2.weight": RNG.normal(size=(6, 10))}
+    th = torch.tensor(h)
+    lib = (F.silu(th @ torch.tensor(w["f.w1.weight"]).T) * (th @ torch.tensor(w["f.w3.weight"]).T)) @ torch.tensor(w["f.w2.weight"]).T
+    np.testing.assert_allclose(plain.swiglu(h, w, "f."), lib.numpy(), rtol=1e-12)
+    assert np.isfinite(plain.silu(np.array([-700.0, 700.0]))).all()
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_block_order_head_and_whole_model_invariants(tmp_path, name):
+    folder = make_model(str(tmp_path / name), name, seed=3)
+    config, w = plain.read_folder(folder)
+    assert plain.feed_forward_width(config) == w["model.layers.0.feed_forward.w1.weight"].shape[0]
+    tokens = random_tokens(config["vocab_size"], 40, 1)
+    logits = plain.forward(config, w, tokens)
+    assert logits.shape == (40, config["vocab_size"])
+    # causality of the whole model
+    changed = list(tokens); changed[30] = (changed[30] + 1) % config["vocab_size"]
+    again = plain.forward(config, w, changed)
+    np.testing.assert_allclose(again[:30], logits[:30], rtol=1e-12)
+    assert np.abs(again[30:] - logits[30:]).max() > 1e-3
+    # silencing every mixer's and feed-forward's last map makes the blocks the identity
+    silent = dict(w)
+    for key in w:
+        if key.endswith(("out_proj.weight", "out_proj.bias", "feed_forward.w2.weight")):
+            silent[key] = np.zeros_like(w[key])
+    tied = config.get("tie_word_embeddings", True)
+    head = w["model.embed_tokens.weight"] if tied else w["lm_head.weight"]
+    bare = plain.rms_norm(w["model.embed_tokens.weight"][tokens], w["model.embedding_norm.weight"], config["norm_eps"]) @ head.T
+    np.testing.assert_allclose(plain.forward(config, silent, tokens), bare, rtol=1e-12)
+    if not tied:        # an untied model ignores the embedding table at the head
+        other = dict(w); other["lm_head.weight"] = w["lm_head.weight"] * 2
+        np.testing.assert_allclose(plain.forward(config, other, tokens), 2 * logits, rtol=1e-12)
+    # each part matters at this weight scale: removing it changes the logits visibly
+    for suffix in ("conv.conv.weight", "self_attn.v_proj.weight", "feed_forward.w3.weight"):
+        cut = {k: (np.zeros_like(v) if k.endswith(suffix) else v) for k, v in w.items()}
+        assert np.abs(plain.forward(config, cut, tokens) - logits).max() > 0.05 * np.abs(logits).max()
+    # greedy: lowest id among equals
+    assert plain.greedy(config, w, tokens[:5], 3) == plain.greedy(config, w, tokens[:5], 3)
+
+
+def test_greedy_ties_go_to_the_lowest_id():
+    assert int(np.argmax(np.array([1.0, 3.0, 3.0, 2.0]))) == 1

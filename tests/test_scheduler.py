@@ -1,0 +1,181 @@
+"""The scheduler's decisions (no GPU): a fake "model" answers with a token that depends on
+the request's tokens so far, so preemption and recomputation must reproduce it."""
+
+import pytest
+
+from flyweight_amd.cache import CacheManager, FixedState, PagedKV
+from flyweight_amd.engine.scheduler import (EVENT_ERROR, EVENT_FINISHED, EVENT_PREFILL, EVENT_TOKEN, Scheduler,
+                                            SchedulerError)
+from flyweight_amd.sampling import GREEDY
+
+NEEDS = {0: PagedKV(2, 16), 1: FixedState((4, 2))}
+
+
+def oracle(tokens):
+    return (sum(tokens) * 31 + len(tokens)) % 97
+
+
+def make(num_pages=8, max_requests=4, **kw):
+    cache = CacheManager(NEEDS, num_pages=num_pages, max_requests=max_requests)
+    return cache, Scheduler(cache, max_positions=kw.pop("max_positions", 4096), **kw)
+
+
+def drive(scheduler, cache, max_steps=10000, log=None):
+    """Runs to completion; returns request id -> (tokens, finished-event count)."""
+    seen = {}
+    steps = 0
+    while scheduler.has_work():
+        plan = scheduler.schedule()
+        # what the step function would check
+        ids = [s.request.id for s in plan.segments]
+        assert len(ids) == len(set(ids)), "a request appears twice in a step"
+        assert plan.num_tokens <= scheduler.max_batch_tokens
+        for segment in plan.segments:
+            r = segment.request
+            assert r.live and segment.tokens == r.tokens[r.computed:r.computed + len(segment.tokens)]
+            assert cache.pages_missing(r.id, r.computed + len(segment.tokens)) == {0: 0}, "pages were not reserved"
+            assert segment.wants_logits == (r.computed + len(segment.tokens) == len(r.tokens))
+        sampled = {s.request.id: oracle(s.request.tokens) for s in plan.segments if s.wants_logits}
+        if log is not None:
+            log.append(plan)
+        for event in scheduler.complete(plan, sampled):
+            seen.setdefault(event[0], []).append(event)
+        cache.check_invariants()
+        steps += 1
+        assert steps < max_steps, "the scheduler does not make progress"
+    return seen
+
+
+def expected_tokens(prompt, count, stop=()):
+    tokens, out = list(prompt), []
+    for _ in range(count):
+        t = oracle(tokens)
+        out.append(t)
+        tokens.append(t)
+        if t in stop:
+            break
+    return out
+
+
+def test_submit_validation():
+    cache, scheduler = make(max_positions=100)
+    with pytest.raises(SchedulerError, match="empty"):
+        scheduler.submit([], 4)
+    with pytest.raises(SchedulerError, match="exceeds the context"):
+        scheduler.submit([1] * 90, 11)
+    with pytest.raises(SchedulerError, match="at least 1"):
+        scheduler.submit([1], 0)
+    scheduler.submit([1] * 90, 10)
+    for _ in range(255):
+        scheduler.submit([1], 1)
+    with pytest.raises(SchedulerError, match="queue"):
+        scheduler.submit([1], 1)
+
+
+def test_prompt_is_cut_into_portions_under_the_budget_and_decodes_come_first():
+    cache, scheduler = make(num_pages=16, max_batch_tokens=24, chunk_size=16)
+    a = scheduler.submit(list(range(40)), 5)
+    log = []
+    plan = scheduler.schedule()
+    assert [(s.request.id, len(s.tokens), s.wants_logits) for s in plan.segments] == [(a.id, 16, False)]
+    scheduler.complete(plan, {})
+    b = scheduler.submit(list(range(10)), 3)
+    plan = scheduler.schedule()          # a's next portion, and b's prompt in what is left of the budget
+    assert [(s.request.id, len(s.tokens), s.wants_logits) for s in plan.segments] == [(a.id, 16, False), (b.id, 8, False)]
+    scheduler.complete(plan, {})
+    plan = scheduler.schedule()
+    assert [(s.request.id, len(s.tokens), s.wants_logits) for s in plan.segments] == [(a.id, 8, True), (b.id, 2, True)]
+    scheduler.complete(plan, {a.id: oracle(a.tokens), b.id: oracle(b.tokens)})
+    c = scheduler.submit(list(range(30)), 2)
+    plan = scheduler.schedule()          # both decode rows first, then the newcomer's portion
+    assert [(s.request.id, len(s.tokens)) for s in plan.segments] == [(a.id, 1), (b.id, 1), (c.id, 16)]
+    assert all(s.wants_logits for s in plan.segments[:2]) and not plan.segments[2].wants_logits
+
+
+def test_runs_to_the_same_tokens_as_one_request_alone():
+    cache, scheduler = make(num_pages=32, max_batch_tokens=32, chunk_size=16)
+    prompts = [list(range(5)), list(range(3, 20)), list(range(7, 38)), [9]]
+    requests = [scheduler.submit(p, 8) for p in prompts]
+    seen = drive(scheduler, cache)
+    for request, prompt in zip(requests, prompts):
+        assert request.generated == expected_tokens(prompt, 8)
+        kinds = [e[2] for e in seen[request.id]]
+        assert kinds.count(EVENT_FINISHED) == 1 and kinds[-1] == EVENT_FINISHED and kinds.count(EVENT_TOKEN) == 8
+    assert cache.stats()["pages_free"] == 32 and cache.slots.free_count == 4 and not cache.requests
+
+
+def test_stop_token_and_position_limit_end_a_request():
+    cache, scheduler = make(max_positions=12)
+    prompt = [1, 2, 3]
+    stop = expected_tokens(prompt, 4)[2]
+    a = scheduler.submit(prompt, 9, stop_tokens=[stop])
+    b = scheduler.submit([5] * 8, 4)
+    drive(scheduler, cache)
+    assert a.generated == expected_tokens(prompt, 9, stop=(stop,)) and a.generated[-1] == stop
+    assert len(b.generated) == 4 and len(b.prompt) + len(b.generated) == 12
+
+
+def test_out_of_pages_preempts_the_newest_and_never_the_oldest():
+    # 4 pages of 64: two requests of 100 + 120 tokens cannot both finish
+    cache, scheduler = make(num_pages=4, max_batch_tokens=256, chunk_size=128)
+    old = scheduler.submit([3] * 100, 120)
+    new = scheduler.submit([4] * 100, 120)
+    log = []
+    seen = drive(scheduler, cache, log=log)
+    assert scheduler.preemptions >= 1 and old.preemptions == 0 and new.preemptions >= 1
+    assert old.generated == expected_tokens([3] * 100, 120)
+    assert new.generated == expected_tokens([4] * 100, 120)     # recomputed, nothing lost or doubled
+    preempting = [p for p in log if p.preempted]
+    assert all(p.preempted[0] is new for p in preempting)
+    assert all(not p.admitted for p in preempting), "nobody is admitted in a step in which somebody gave way"
+    assert [e[2] for e in seen[new.id]].count(EVENT_FINISHED) == 1
+    # a preempted request recomputes prompt + generated as portions and asks for logits only at the end
+    after = log[log.index(preempting[0]) + 1:]
+    recompute = [s for p in after for s in p.segments if s.request is new and len(s.tokens) > 1]
+    assert recompute and recompute[0].tokens[:100] == [4] * 100
+    assert cache.stats()["pages_free"] == 4
+
+
+def test_a_request_that_cannot_fit_alone_fails_and_the_rest_goes_on():
+    cache, scheduler = make(num_pages=2, max_batch_tokens=256, chunk_size=256)
+    big = scheduler.submit([1] * 100, 100)       # 200 tokens need 4 pages, the pool has 2
+    small = scheduler.submit([2] * 10, 5)
+    seen = drive(scheduler, cache)
+    assert big.finished and big.error and "pages" in big.error and [e[2] for e in seen[big.id]] == [EVENT_ERROR]
+    assert small.generated == expected_tokens([2] * 10, 5)
+    assert cache.stats()["pages_free"] == 2
+
+
+def test_prefills_that_block_each_other_are_untangled():
+    # two prompts of 150 tokens need 3 pages each, the pool has 4: the second must give way
+    cache, scheduler = make(num_pages=4, max_batch_tokens=128, chunk_size=64)
+    a = scheduler.submit([1] * 150, 4)
+    b = scheduler.submit([2] * 150, 4)
+    drive(scheduler, cache)
+    assert a.generated == expected_tokens([1] * 150, 4) and b.generated == expected_tokens([2] * 150, 4)
+    assert a.preemptions == 0
+
+
+def test_live_limit_and_slots_bound_admission():
+    cache, scheduler = make(num_pages=64, max_requests=2, max_batch_tokens=64, chunk_size=8)
+    requests = [scheduler.submit([i + 1] * 4, 3) for i in range(5)]
+    log = []
+    drive(scheduler, cache, log=log)
+    assert max(len({s.request.id for s in p.segments}) for p in log) <= 2
+    assert all(r.generated == expected_tokens(r.prompt, 3) for r in requests)
+    order = [r.id for p in log for r in p.admitted]
+    assert order == sorted(order)                # first come, first admitted
+
+
+def test_cancel_frees_everything():
+    cache, scheduler = make()
+    a = scheduler.submit([1] * 70, 50)
+    b = scheduler.submit([2] * 5, 50)
+    for _ in range(3):
+        plan = scheduler.schedule()
+        scheduler.complete(plan, {s.request.id: oracle(s.request.tokens) for s in plan.segments if s.wants_logits})
+    assert scheduler.cancel(a.id) and scheduler.cancel(b.id) and not scheduler.cancel(12345)
+    plan = scheduler.schedule()
+    events = scheduler.complete(plan, {})
+    assert sorted(e[0] for e in events if e[2] == EVENT_FINISHED) == [a.id, b.id]
+    assert not scheduler.has_work() and cache.stats()["pages_free"] == 8 and cache.slots.free_count == 4
