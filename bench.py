@@ -1,0 +1,189 @@
+"""Measures the engine on the LFM2-1.2B shape with random weights on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the whole batch. Prints ONE JSON line: decoded tokens a second
+at batch 8 (``value``), the same at batch 1 and 64 (``points``), the 2,048-token prefill
+(``prefill``) and the decode step's achieved fraction of the HBM roofline (``roofline``).
+Peaks are the MI355X's published ones: HBM 8 TB/s, dense bfloat16 MFMA 2.5 PFLOP/s.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK = 2.5e15
+
+# BASELINE.json configs[2]: the LFM2-1.2B shape
+SHAPE = dict(
+    architectures=["Lfm2ForCausalLM"], model_type="lfm2", vocab_size=65536, hidden_size=2048, num_hidden_layers=16,
+    num_attention_heads=32, num_key_value_heads=8, intermediate_size=12288, block_auto_adjust_ff_dim=True,
+    block_ffn_dim_multiplier=1.0, block_multiple_of=256, norm_eps=1e-5, rope_theta=1000000.0, conv_L_cache=3,
+    conv_bias=False, tie_word_embeddings=True, max_position_embeddings=4096, full_attn_idxs=[2, 5, 8, 10, 12, 14])
+PROMPT = 2048
+CONTEXT = 4096
+
+
+def log(text: str) -> None:
+    print(f"[bench] {text}", file=sys.stderr, flush=True)
+
+
+def model_bytes(model) -> int:
+    """Bytes of every weight a decode step reads once (the tied table is read as the head)."""
+    seen, total = set(), 0
+    def add(t):
+        nonlocal total
+        if t is not None and t.data_ptr() not in seen:
+            seen.add(t.data_ptr())
+            total += t.numel() * t.element_size()
+    lm = model.model
+    add(lm.head.weight)
+    add(lm.final_norm.weight)
+    for block in lm.layers:
+        add(block.mixer_norm.weight), add(block.ffn_norm.weight)
+        add(block.ffn.gate_up.weight), add(block.ffn.down.weight)
+        mixer = block.mixer
+        for name in ("qkv", "out", "in_proj", "out_proj"):
+            if hasattr(mixer, name):
+                add(getattr(mixer, name).weight), add(getattr(mixer, name).bias)
+        for name in ("q_norm_weight", "k_norm_weight", "taps", "conv_bias"):
+            add(getattr(mixer, name, None))
+    return total
+
+
+def matmul_params(config) -> int:
+    h, ff = config.hidden_size, config.ff_dim
+    per_ffn = 3 * h * ff
+    conv = 3 * h * h + h * h
+    attn = (config.num_attention_heads + 2 * config.num_key_value_heads) * config.head_dim * h + h * config.num_attention_heads * config.head_dim
+    n_attn = len(config.full_attn_idxs)
+    return config.num_hidden_layers * per_ffn + (config.num_hidden_layers - n_attn) * conv + n_attn * attn
+
+
+def decode_run(torch, model, config, batch: int, steps: int, warmup: int, seed: int = 0):
+    """``batch`` requests with 2,048-token prompts; returns (seconds for ``steps`` decode steps, mean context)."""
+    import numpy as np
+    from flyweight_amd import Runtime
+    # requests admitted earlier decode while later prompts are still running (continuous
+    # batching), so they are up to ``batch`` tokens ahead when the timed steps begin
+    new_tokens = warmup + steps + batch + 2
+    pages_each = (PROMPT + new_tokens + 63) // 64
+    runtime = Runtime(model, context_limit=CONTEXT, parallel_sequences=batch, num_pages=pages_each * batch,
+                      max_batch_tokens=PROMPT + batch, prefill_rows=PROMPT).prepare()
+    rng = np.random.default_rng(seed)
+    for _ in range(batch):
+        runtime.task_submit(rng.integers(0, config.vocab_size, PROMPT).tolist(), new_tokens)
+    # prompts: until every request has produced its first token
+    while any(r.computed < len(r.prompt) for r in runtime.scheduler.requests.values()):
+        runtime.engine_step()
+    for _ in range(warmup):
+        runtime.engine_step()
+    requests = list(runtime.scheduler.requests.values())
+    before = sum(r.computed for r in requests) / batch
+    torch.cuda.synchronize()
+    began = time.perf_counter()
+    for _ in range(steps):
+        events = runtime.engine_step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - began
+    assert sum(1 for e in events if e[2] == 0) == batch, "a timed step did not decode the whole batch"
+    mean_context = before + 1 + (steps - 1) / 2.0      # keys a row sees, averaged over requests and steps
+    runtime.close()
+    return elapsed, mean_context
+
+
+def prefill_run(torch, model, config, repeats: int = 3):
+    import numpy as np
+    from flyweight_amd import Runtime, StepEntry
+    runtime = Runtime(model, context_limit=CONTEXT, parallel_sequences=1, num_pages=PROMPT // 64 + 1).prepare()
+    tokens = np.random.default_rng(1).integers(0, config.vocab_size, PROMPT).tolist()
+    best = None
+    for i in range(repeats + 1):
+        runtime.admit(i)
+        torch.cuda.synchronize()
+        began = time.perf_counter()
+        runtime.step([StepEntry(i, tokens, [PROMPT - 1])])
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - began
+        runtime.release(i)
+        if i > 0:
+            best = elapsed if best is None else min(best, elapsed)
+    return best
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=256)
+    parser.add_argument("--warmup", type=int, default=16)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
+    args = parser.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for {args.gpus})", flush=True)
+        return 2
+    if PROMPT + args.warmup + args.steps + 64 + 2 > CONTEXT:
+        print("bench.py: warmup + steps must leave the 4,096-token context room", flush=True)
+        return 2
+
+    import torch
+    from flyweight_amd import Model
+    from flyweight_amd.config import config_from_dict
+
+    config = config_from_dict(SHAPE)
+    log("building the LFM2-1.2B shape with random bfloat16 weights")
+    model = Model.random(config, seed=0, dtype="bfloat16")
+    weights = model_bytes(model)
+    kv_per_token = len(config.full_attn_idxs) * 2 * config.num_key_value_heads * config.head_dim * 2
+    state_per_request = (config.num_hidden_layers - len(config.full_attn_idxs)) * config.hidden_size * (config.conv_L_cache - 1) * 4
+
+    log("prefill of 2,048 tokens")
+    prefill_s = prefill_run(torch, model, config)
+    head_flops = 2 * config.vocab_size * config.hidden_size
+    attention_flops = len(config.full_attn_idxs) * 2 * config.num_attention_heads * config.head_dim * PROMPT * PROMPT
+    prefill_flops = 2 * matmul_params(config) * PROMPT + head_flops + attention_flops
+
+    log(f"decode at batch {args.batch}: {args.warmup} warm-up and {args.steps} timed steps")
+    elapsed, mean_context = decode_run(torch, model, config, args.batch, args.steps, args.warmup)
+    value = args.batch * args.steps / elapsed
+    step_bytes = weights + args.batch * (mean_context * kv_per_token + state_per_request)
+    achieved = step_bytes / (elapsed / args.steps) / 1e9
+
+    points = {}
+    if not args.skip_points:
+        for batch, steps in ((1, min(args.steps, 128)), (64, min(args.steps, 64))):
+            log(f"decode at batch {batch}")
+            seconds, _ = decode_run(torch, model, config, batch, steps, min(args.warmup, 8))
+            points[f"decode_b{batch}"] = round(batch * steps / seconds, 1)
+
+    print(json.dumps({
+        "metric": "decode tok/s @ batch 8 (LFM2-1.2B shape, 2,048-token prompts, context 4,096)",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic: seeded uniform token ids, random-init weights",
+        "config": {"model": "LFM2-1.2B shape", "layers": config.num_hidden_layers, "layers_of_named_config": 16,
+                   "hidden": config.hidden_size, "heads": config.num_attention_heads,
+                   "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim, "ff_dim": config.ff_dim,
+                   "vocab": config.vocab_size, "attention_layers": len(config.full_attn_idxs),
+                   "conv_L_cache": config.conv_L_cache, "global_batch": args.batch, "prompt_len": PROMPT,
+                   "seq_len": CONTEXT, "parallelism": "single GPU"},
+        "prefill": {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
+                    "frac": round(prefill_flops / prefill_s / MFMA_BF16_PEAK, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": points,
+    }), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,358 @@
+// Attention over the paged cache on the matrix cores (bfloat16 cache, float32 softmax).
+//
+// One wave works on 16 "columns" against the keys of one kv head. For a prompt portion a
+// column is a query row (16 consecutive rows of one segment, one head per wave, the heads of
+// a kv group side by side in a workgroup so that they find the same pages in L1). For decode
+// a column is one of the query heads that share the kv head, and the keys are split between
+// workgroups in runs of SPLIT_PAGES pages whose partial results (running maximum, sum and
+// unnormalised output) a second kernel merges in order.
+//
+// The products are formed transposed so that nothing has to change lanes between them:
+//   S^T[key][col] = K[key][d] . Q^T[d][col]        (v_mfma_f32_16x16x32_bf16, k = d)
+//   O^T[d][col]  += V^T[d][key] . P^T[key][col]    (k = key)
+// Lane (col, g) receives the scores of keys 4g..4g+3 of each 16-key tile, which is exactly
+// what it must supply as P^T for keys {4g..4g+3} of two tiles if the 32 keys of the second
+// product are taken in that order; V^T is fetched in the same order, which its layout
+// ([page][kv_head][head_dim][64 keys]: a channel's keys together) makes two 8-byte loads.
+// K ([page][kv_head][64 keys][head_dim]) is fetched straight into operand registers too.
+// Maximum, exponentials, sums and the rescaling of O are float32; P is rounded to bfloat16
+// for the second product. The reference's fast decode tier has the same split-and-merge shape
+// (native/src/split_kv.h:77-124, native/src/v2_runtime.cpp:24241-24267).
+#include "fw_common.h"
+#include "fw_kernels.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define PAGE 64
+#define SPLIT_PAGES 4           // keys per decode split = 256, whatever the batch
+#define NEG_BIG (-1.0e30f)
+#define PART_STRIDE(head_dim) ((head_dim) + 4)   // unnormalised output, maximum, sum, two unused: rows stay 16-byte aligned
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    return (uint32_t)float_to_bf16_bits(lo) | ((uint32_t)float_to_bf16_bits(hi) << 16);
+}
+
+// State of one wave: 16 columns, HD channels (HD a multiple of 32; channels >= head_dim are zero).
+template <int HD>
+struct Columns {
+    bf16x8 q[HD / 32];          // this lane's part of Q^T: column lane % 16, d = 32 c + 8 (lane / 16) ..
+    f32x4 o[HD / 16];           // O^T: column lane % 16, d = 16 t + 4 (lane / 16) + r
+    float m, l;                 // running maximum (in units of log2) and this lane's share of the sum
+};
+
+// One page of 64 keys. `lo`/`hi`: the keys of this page that this lane's column may see are
+// those with lo <= key <= hi (page-relative; hi < 0: none). `last_written`: keys beyond it
+// hold whatever an earlier owner of the page left, and are zeroed before they meet P = 0.
+template <int HD>
+__device__ __forceinline__ void attend_page(Columns<HD>& c, const uint16_t* __restrict__ k_page,
+                                            const uint16_t* __restrict__ v_page, int head_dim, float scale_log2,
+                                            int lo, int hi, int last_written) {
+    const int lane = threadIdx.x & 63;
+    const int i16 = lane & 15, g = lane >> 4;
+    f32x4 s[4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+        s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const uint16_t* key = k_page + (size_t)(kt * 16 + i16) * head_dim + g * 8;
+#pragma unroll
+        for (int dc = 0; dc < HD / 32; ++dc) {
+            bf16x8 kf = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (dc * 32 + g * 8 < head_dim) kf = *reinterpret_cast<const bf16x8*>(key + dc * 32);
+            s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, c.q[dc], s[kt], 0, 0, 0);
+        }
+    }
+    // mask, then the running maximum of this column: over this lane's 16 scores, then over
+    // the four lanes that share the column
+    float page_max = NEG_BIG;
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int key = kt * 16 + g * 4 + r;
+            const float v = (key >= lo && key <= hi) ? s[kt][r] * scale_log2 : NEG_BIG;
+            s[kt][r] = v;
+            page_max = fmaxf(page_max, v);
+        }
+    page_max = fmaxf(page_max, __shfl_xor(page_max, 16, 64));
+    page_max = fmaxf(page_max, __shfl_xor(page_max, 32, 64));
+    const float new_max = fmaxf(c.m, page_max);
+    const float alpha = exp2f(c.m - new_max);
+    c.m = new_max;
+    float sum = 0.0f;
+    uint32_t p[4][2];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+        float e[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            e[r] = s[kt][r] > 0.5f * NEG_BIG ? exp2f(s[kt][r] - new_max) : 0.0f;
+            sum += e[r];
+        }
+        p[kt][0] = pack_bf16(e[0], e[1]);
+        p[kt][1] = pack_bf16(e[2], e[3]);
+    }
+    c.l = c.l * alpha + sum;
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t) c.o[t] *= alpha;
+    const bool partial_page = last_written < PAGE - 1;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+        u32x4 pw = {p[2 * kb][0], p[2 * kb][1], p[2 * kb + 1][0], p[2 * kb + 1][1]};
+        const bf16x8 pf = __builtin_bit_cast(bf16x8, pw);
+        const int key_a = kb * 32 + g * 4, key_b = key_a + 16;
+#pragma unroll
+        for (int t = 0; t < HD / 16; ++t) {
+            if (t * 16 >= head_dim) break;
+            const uint16_t* value = v_page + (size_t)(t * 16 + i16) * PAGE;
+            u32x2 va = *reinterpret_cast<const u32x2*>(value + key_a);
+            u32x2 vb = *reinterpret_cast<const u32x2*>(value + key_b);
+            if (partial_page) {
+                // keep keys <= last_written only: two keys per 32-bit word, low half first
+                auto keep = [&](uint32_t word, int first_key) -> uint32_t {
+                    if (first_key + 1 <= last_written) return word;
+                    if (first_key <= last_written) return word & 0xffffu;
+                    return 0u;
+                };
+                va = u32x2{keep(va[0], key_a), keep(va[1], key_a + 2)};
+                vb = u32x2{keep(vb[0], key_b), keep(vb[1], key_b + 2)};
+            }
+            u32x4 vw = {va[0], va[1], vb[0], vb[1]};
+            c.o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vw), pf, c.o[t], 0, 0, 0);
+        }
+    }
+}
+
+template <int HD>
+__device__ __forceinline__ void load_query(Columns<HD>& c, const uint16_t* __restrict__ q_row, int head_dim, bool valid) {
+    const int g = (threadIdx.x & 63) >> 4;
+#pragma unroll
+    for (int dc = 0; dc < HD / 32; ++dc) {
+        c.q[dc] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (valid && dc * 32 + g * 8 < head_dim) c.q[dc] = *reinterpret_cast<const bf16x8*>(q_row + dc * 32 + g * 8);
+    }
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t) c.o[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    c.m = NEG_BIG;
+    c.l = 0.0f;
+}
+
+// ---- prompt portions ---------------------------------------------------------------------------
+// grid (query tiles, kv heads); one wave per query head of the group. tile_seg / tile_row0:
+// the segment of each tile of 16 rows and its first row (a tile never spans two segments).
+template <int HD>
+__global__ void attention_prefill_kernel(
+    const uint16_t* __restrict__ q, uint16_t* __restrict__ out, const uint16_t* __restrict__ k_pages,
+    const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
+    const int32_t* __restrict__ tile_seg, const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ seg_row0,
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, float scale_log2, int window) {
+    const int tile = blockIdx.x, kvh = blockIdx.y;
+    const int group = num_heads / num_kv_heads;
+    const int head = kvh * group + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63, col = lane & 15, g = lane >> 4;
+    const int seg = tile_seg[tile];
+    const int row0 = tile_row0[tile];
+    const int seg_end = seg_row0[seg + 1];
+    const int rows = seg_end - row0 < 16 ? seg_end - row0 : 16;
+    const bool valid = col < rows;
+    const int my_row = row0 + (valid ? col : 0);
+    const int my_pos = row_pos[my_row];
+    const int pos_lo = row_pos[row0], pos_hi = row_pos[row0 + rows - 1];
+    const int my_first = window > 0 && my_pos - window + 1 > 0 ? my_pos - window + 1 : 0;
+    const int tile_first = window > 0 && pos_lo - window + 1 > 0 ? pos_lo - window + 1 : 0;
+
+    Columns<HD> c;
+    load_query<HD>(c, q + ((size_t)my_row * num_heads + head) * head_dim, head_dim, valid);
+    const int32_t* table = block_table + (size_t)seg * table_stride;
+    const size_t page_elems = (size_t)PAGE * head_dim;
+    for (int block = tile_first / PAGE; block <= pos_hi / PAGE; ++block) {
+        const int page = table[block];
+        const size_t at = ((size_t)page * num_kv_heads + kvh) * page_elems;
+        const int base = block * PAGE;
+        const int lo = valid ? my_first - base : PAGE;
+        const int hi = valid ? my_pos - base : -1;
+        attend_page<HD>(c, k_pages + at, v_pages + at, head_dim, scale_log2, lo, hi, pos_hi - base);
+    }
+    float l = c.l;
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!valid) return;
+    const float inv = 1.0f / l;
+    uint16_t* dest = out + ((size_t)my_row * num_heads + head) * head_dim;
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t) {
+        if (t * 16 >= head_dim) break;
+        u32x2 packed = {pack_bf16(c.o[t][0] * inv, c.o[t][1] * inv), pack_bf16(c.o[t][2] * inv, c.o[t][3] * inv)};
+        *reinterpret_cast<u32x2*>(dest + t * 16 + g * 4) = packed;
+    }
+}
+
+// ---- decode ------------------------------------------------------------------------------------
+// grid (rows, kv heads * head tiles, splits); one wave. Columns are the query heads of the kv
+// group (16 per head tile). partial [rows][heads][max_splits][head_dim + 4]: unnormalised
+// output, then maximum and sum; a split with nothing to do writes nothing.
+template <int HD>
+__global__ __launch_bounds__(64) void attention_decode_split_kernel(
+    const uint16_t* __restrict__ q, float* __restrict__ partial, const uint16_t* __restrict__ k_pages,
+    const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
+    const int32_t* __restrict__ row_seg, const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads,
+    int head_dim, float scale_log2, int window, int max_splits) {
+    const int row = blockIdx.x, split = blockIdx.z;
+    const int group = num_heads / num_kv_heads;
+    const int head_tiles = (group + 15) / 16;
+    const int kvh = blockIdx.y / head_tiles, head_tile = blockIdx.y % head_tiles;
+    const int lane = threadIdx.x & 63, col = lane & 15, g = lane >> 4;
+    const int pos = row_pos[row];
+    const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+    // splits are counted from the first page that holds a visible key
+    const int first_block = first / PAGE + split * SPLIT_PAGES;
+    const int last_block = pos / PAGE;
+    if (first_block > last_block) return;
+    const int end_block = first_block + SPLIT_PAGES - 1 < last_block ? first_block + SPLIT_PAGES - 1 : last_block;
+    const int in_group = head_tile * 16 + col;
+    const bool valid = in_group < group;
+    const int head = kvh * group + (valid ? in_group : 0);
+
+    Columns<HD> c;
+    load_query<HD>(c, q + ((size_t)row * num_heads + head) * head_dim, head_dim, valid);
+    const int32_t* table = block_table + (size_t)row_seg[row] * table_stride;
+    const size_t page_elems = (size_t)PAGE * head_dim;
+    for (int block = first_block; block <= end_block; ++block) {
+        const int page = table[block];
+        const size_t at = ((size_t)page * num_kv_heads + kvh) * page_elems;
+        const int base = block * PAGE;
+        attend_page<HD>(c, k_pages + at, v_pages + at, head_dim, scale_log2, valid ? first - base : PAGE,
+                        valid ? pos - base : -1, pos - base);
+    }
+    float l = c.l;
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!valid) return;
+    float* dest = partial + (((size_t)row * num_heads + head) * max_splits + split) * PART_STRIDE(head_dim);
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t) {
+        if (t * 16 >= head_dim) break;
+        *reinterpret_cast<f32x4*>(dest + t * 16 + g * 4) = c.o[t];
+    }
+    if (g == 0) {
+        dest[head_dim] = c.m;
+        dest[head_dim + 1] = l;
+    }
+}
+
+// grid (rows, heads): merges the splits of one (row, head) in order of the keys.
+__global__ __launch_bounds__(64) void attention_decode_merge_kernel(
+    const float* __restrict__ partial, uint16_t* __restrict__ out, const int32_t* __restrict__ row_pos, int num_heads,
+    int head_dim, int window, int max_splits) {
+    const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const int pos = row_pos[row];
+    const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+    const int blocks = pos / PAGE - first / PAGE + 1;
+    const int splits = (blocks + SPLIT_PAGES - 1) / SPLIT_PAGES;
+    const float* source = partial + ((size_t)row * num_heads + head) * max_splits * PART_STRIDE(head_dim);
+    float m = NEG_BIG;
+    for (int s = 0; s < splits; ++s) m = fmaxf(m, source[(size_t)s * PART_STRIDE(head_dim) + head_dim]);
+    float total = 0.0f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < splits; ++s) {
+        const float* part = source + (size_t)s * PART_STRIDE(head_dim);
+        const float weight = exp2f(part[head_dim] - m);
+        total += weight * part[head_dim + 1];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int d = lane + 64 * j;
+            if (d < head_dim) acc[j] += weight * part[d];
+        }
+    }
+    const float inv = 1.0f / total;
+    uint16_t* dest = out + ((size_t)row * num_heads + head) * head_dim;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int d = lane + 64 * j;
+        if (d < head_dim) dest[d] = float_to_bf16_bits(acc[j] * inv);
+    }
+}
+
+static const float LOG2E = 1.4426950408889634f;
+
+static int check_common(const char* name, int rows, int num_heads, int num_kv_heads, int head_dim, int page_size,
+                        int window, int num_pages, int table_stride) {
+    FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
+               "%s: heads %d must be a positive multiple of kv heads %d", name, num_heads, num_kv_heads);
+    FW_REQUIRE(head_dim >= 16 && head_dim <= 256 && head_dim % 16 == 0, "%s: head_dim %d must be a multiple of 16 in 16..256", name, head_dim);
+    FW_REQUIRE(page_size == PAGE, "%s: page size must be %d, got %d", name, PAGE, page_size);
+    FW_REQUIRE(window >= 0, "%s: window must be 0 (all keys) or positive, got %d", name, window);
+    FW_REQUIRE(num_pages > 0 && table_stride > 0, "%s: empty cache (pages=%d, table stride=%d)", name, num_pages, table_stride);
+    return 0;
+}
+
+#define FW_BY_HEAD_DIM(head_dim, CALL)      \
+    do {                                    \
+        if (head_dim <= 32) { CALL(32); }   \
+        else if (head_dim <= 64) { CALL(64); } \
+        else if (head_dim <= 128) { CALL(128); } \
+        else { CALL(256); }                 \
+    } while (0)
+
+// bfloat16 q [rows][heads * head_dim] -> out (same shape). tile_seg / tile_row0 [tiles].
+extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                    const int32_t* block_table, int table_stride, const int32_t* tile_seg,
+                                    const int32_t* tile_row0, int tiles, const int32_t* seg_row0,
+                                    const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim,
+                                    float scale, int window, int page_size, int num_pages, void* stream) {
+    if (check_common("attention_prefill", rows, num_heads, num_kv_heads, head_dim, page_size, window, num_pages, table_stride)) return -1;
+    FW_REQUIRE(num_heads / num_kv_heads <= 16, "attention_prefill: at most 16 query heads per kv head, got %d", num_heads / num_kv_heads);
+    FW_REQUIRE(tiles >= 0 && tiles <= rows && num_kv_heads <= 65535, "attention_prefill: %d tiles for %d rows", tiles, rows);
+    if (rows == 0 || tiles == 0) return 0;
+    dim3 grid(tiles, num_kv_heads);
+    const int threads = 64 * (num_heads / num_kv_heads);
+#define CALL(HD)                                                                                                   \
+    attention_prefill_kernel<HD><<<grid, threads, 0, (hipStream_t)stream>>>(                                        \
+        (const uint16_t*)q, (uint16_t*)out, (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table,        \
+        table_stride, tile_seg, tile_row0, seg_row0, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window)
+    FW_BY_HEAD_DIM(head_dim, CALL);
+#undef CALL
+    FW_LAUNCH_CHECK("attention_prefill");
+    return 0;
+}
+
+// One row per request. partial: float32 workspace of rows * heads * max_splits * (head_dim + 4).
+// max_context: no row's position reaches it (the caller knows; the kernel cannot check);
+// max_splits must cover the keys such a row sees, in runs of 4 pages.
+extern "C" int fw_attention_decode(const void* q, void* out, float* partial, int max_splits, int max_context,
+                                   const void* k_pages,
+                                   const void* v_pages, const int32_t* block_table, int table_stride,
+                                   const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
+                                   int num_kv_heads, int head_dim, float scale, int window, int page_size,
+                                   int num_pages, void* stream) {
+    if (check_common("attention_decode", rows, num_heads, num_kv_heads, head_dim, page_size, window, num_pages, table_stride)) return -1;
+    FW_REQUIRE(max_splits >= 1 && max_splits <= 65535, "attention_decode: max_splits %d outside 1..65535", max_splits);
+    FW_REQUIRE(max_context >= 1, "attention_decode: max_context must be positive");
+    {
+        int blocks = (max_context + PAGE - 1) / PAGE;
+        if (window > 0 && (window + PAGE - 2) / PAGE + 1 < blocks) blocks = (window + PAGE - 2) / PAGE + 1;
+        FW_REQUIRE(max_splits * SPLIT_PAGES >= blocks, "attention_decode: %d splits of %d pages do not cover %d pages of context",
+                   max_splits, SPLIT_PAGES, blocks);
+        FW_REQUIRE((max_context + PAGE - 1) / PAGE <= table_stride, "attention_decode: a context of %d tokens exceeds the block table (%d pages)",
+                   max_context, table_stride);
+    }
+    if (rows == 0) return 0;
+    const int group = num_heads / num_kv_heads;
+    const int head_tiles = (group + 15) / 16;
+    FW_REQUIRE(rows <= 1 << 20 && num_kv_heads * head_tiles <= 65535 && num_heads <= 65535, "attention_decode: grid too large");
+    dim3 grid(rows, num_kv_heads * head_tiles, max_splits);
+#define CALL(HD)                                                                                                   \
+    attention_decode_split_kernel<HD><<<grid, 64, 0, (hipStream_t)stream>>>(                                        \
+        (const uint16_t*)q, partial, (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table, table_stride, \
+        row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits)
+    FW_BY_HEAD_DIM(head_dim, CALL);
+#undef CALL
+    FW_LAUNCH_CHECK("attention_decode_split");
+    attention_decode_merge_kernel<<<dim3(rows, num_heads), 64, 0, (hipStream_t)stream>>>(
+        partial, (uint16_t*)out, row_pos, num_heads, head_dim, window, max_splits);
+    FW_LAUNCH_CHECK("attention_decode_merge");
+    return 0;
+}

@@ -28,6 +28,16 @@ int fw_rmsnorm_rows(const float* x, const float* weight, void* out, int out_dtyp
 int fw_gemm_generic(const void* a, int a_dtype, const void* w, int w_dtype, const float* bias,
                     void* out, int out_dtype, int out_mode, int M, int N, int K, void* stream);
 
+// bfloat16 matrix products on the matrix cores, float32 accumulation. a [M][K], w [N][K], K a
+// multiple of 8. mode 0: out = a . w^T (+ bias) stored as out_dtype; mode 1: out (float32) +=
+// a . w^T (+ bias); mode 2 (SwiGLU): w is [2N][K], gate rows then up rows, out [M][N] bfloat16 =
+// silu(a . gate^T) * (a . up^T). fw_gemm_skinny streams w once for M <= 64 (decode);
+// fw_gemm_mfma tiles both operands through LDS (prompts).
+int fw_gemm_skinny(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
+                   int M, int N, int K, void* stream);
+int fw_gemm_mfma(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
+                 int M, int N, int K, void* stream);
+
 // out[r][i] = silu(gu[r][i]) * gu[r][I + i]; the input may be float32 beside a bfloat16 output
 int fw_swiglu(const void* gate_up, int in_dtype, void* out, int out_dtype, int rows, int intermediate,
               void* stream);
@@ -63,6 +73,22 @@ int fw_attention_generic(const void* q, void* out, int dtype, const void* k_page
                          const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                          int num_kv_heads, int head_dim, float scale, int window, int page_size,
                          int num_pages, void* stream);
+
+// The same attention on the matrix cores, bfloat16 only, head_dim a multiple of 16 up to 256.
+// Prompt portions: rows are cut into tiles of 16 that never span two segments (tile_seg,
+// tile_row0); at most 16 query heads per kv head.
+int fw_attention_prefill(const void* q, void* out, const void* k_pages, const void* v_pages,
+                         const int32_t* block_table, int table_stride, const int32_t* tile_seg,
+                         const int32_t* tile_row0, int tiles, const int32_t* seg_row0, const int32_t* row_pos,
+                         int rows, int num_heads, int num_kv_heads, int head_dim, float scale, int window,
+                         int page_size, int num_pages, void* stream);
+// Decode (one row per request): the keys are split between workgroups in runs of 4 pages and
+// merged in order. partial: float32 workspace [rows][heads][max_splits][head_dim + 4];
+// max_context: an upper bound on position + 1 of every row, known to the caller.
+int fw_attention_decode(const void* q, void* out, float* partial, int max_splits, int max_context,
+                        const void* k_pages, const void* v_pages, const int32_t* block_table, int table_stride,
+                        const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
+                        int head_dim, float scale, int window, int page_size, int num_pages, void* stream);
 
 // ids[r] = argmax(logits[r]) with ties to the lowest id
 int fw_argmax_rows(const float* logits, int32_t* ids, int rows, int vocab, void* stream);

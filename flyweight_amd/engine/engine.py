@@ -36,6 +36,23 @@ class Model:
         self.dtype = parse_dtype(dtype)
         self.config, self.model = load_model(path, dtype=self.dtype, device=device)
 
+    @classmethod
+    def random(cls, config, seed: int = 0, dtype="bfloat16", device: str = "cuda:0", scale: str = "small") -> "Model":
+        """A model of ``config`` (a registered architecture's configuration) with random
+        weights drawn on the device; nothing is written to disk."""
+        from ..kernels import ops
+        from ..weights import random_tensors_on_device
+        from .model import CausalLM
+        self = cls.__new__(cls)
+        self.path, self.dtype, self.config = None, parse_dtype(dtype), config
+        target = torch.device(device)
+        if target.type != "cuda" or not torch.cuda.is_available():
+            raise RuntimeError("flyweight_amd runs on a GPU only (no CPU path); no HIP device is available")
+        ops.library()
+        self.model = CausalLM(config.model_spec())
+        self.model.bind(random_tensors_on_device(self.model.tensors(), seed, target, self.dtype, scale), self.dtype, target)
+        return self
+
     @property
     def spec(self):
         return self.model.spec

@@ -17,6 +17,7 @@ import numpy as np
 import torch
 
 from ..cache import CacheManager, OutOfPages
+from ..kernels import ops
 from .model import CacheView, CausalLM
 
 
@@ -83,8 +84,10 @@ class StepContext:
         self.host_seg_row0 = seg_row0
         self.host_seg_slot = seg_slot
 
+        tile_seg, tile_row0 = ops.query_tiles(seg_row0)        # tiles of 16 rows for the prompt attention kernel
         tables = [cache.block_table_rows(g, self.requests) for g in range(len(cache.groups))]
-        pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows)]
+        pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows,
+                                                          tile_seg, tile_row0)]
         pieces += [t.reshape(-1) for t in tables]
         packed = torch.from_numpy(np.concatenate(pieces)).to(device)
         views = []
@@ -92,8 +95,9 @@ class StepContext:
         for piece in pieces:
             views.append(packed[offset:offset + piece.size])
             offset += piece.size
-        (self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows) = views[:6]
-        self.block_tables = [v.view(t.shape) for v, t in zip(views[6:], tables)]
+        (self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows, self.tile_seg,
+         self.tile_row0) = views[:8]
+        self.block_tables = [v.view(t.shape) for v, t in zip(views[8:], tables)]
         self._position_tables: Dict = {}
 
     def position_tables(self, part):

@@ -298,13 +298,142 @@ def fill_zero(t: torch.Tensor) -> None:
     _check(library().fw_fill_zero(_p(t), ctypes.c_longlong(t.numel() * t.element_size()), _stream()))
 
 
+def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int) -> None:
+    """bfloat16 operands on the matrix cores: the skinny kernel for up to 64 rows, the tiled one beyond."""
+    M, K = a.shape
+    entry = library().fw_gemm_skinny if M <= SKINNY_MAX_ROWS else library().fw_gemm_mfma
+    _check(entry(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K, _stream()))
+
+
+SKINNY_MAX_ROWS = 64
+
+
+def _fast_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[0] >= 1 and a.shape[1] % 8 == 0
+            and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
 # ---- dispatch: which kernel serves a call ------------------------------------------------
 def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
          out_dtype: Optional[torch.dtype] = None, accumulate_into: Optional[torch.Tensor] = None) -> torch.Tensor:
-    return gemm_generic(a, w, bias, out_dtype=out_dtype, accumulate_into=accumulate_into)
+    """a [M, K] . w [N, K]^T (+ bias): bfloat16 operands go to the matrix-core kernels,
+    everything else (float32, mixed) to the generic float32 one."""
+    if not _fast_ok(a, w):
+        return gemm_generic(a, w, bias, out_dtype=out_dtype, accumulate_into=accumulate_into)
+    _dev(a, w, bias, accumulate_into)
+    M, K = a.shape
+    N, K2 = w.shape
+    if K != K2:
+        raise KernelError(f"gemm: a is {tuple(a.shape)} but w is {tuple(w.shape)}")
+    if bias is not None and (bias.dtype != torch.float32 or bias.shape != (N,)):
+        raise KernelError("gemm: bias must be float32 [N]")
+    if accumulate_into is not None:
+        _want(accumulate_into, torch.float32, "accumulate_into")
+        if accumulate_into.shape != (M, N):
+            raise KernelError(f"gemm: destination is {tuple(accumulate_into.shape)}, expected {(M, N)}")
+        _fast_gemm(a, w, bias, accumulate_into, F32, 1, N)
+        return accumulate_into
+    out_dtype = out_dtype or a.dtype
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    _fast_gemm(a, w, bias, out, _code(out_dtype), 0, N)
+    return out
+
+
+def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(a . gate^T) * (a . up^T) with w_gate_up = [gate rows; up rows]: [M, I] in a's dtype.
+    On the bfloat16 path the activation is formed from the float32 sums inside the product's
+    kernel; otherwise the [M, 2I] intermediate is float32 and a second kernel forms it."""
+    rows2, K = w_gate_up.shape
+    if rows2 % 2:
+        raise KernelError("gemm_swiglu: the operand holds gate and up rows; their number must be even")
+    if _fast_ok(a, w_gate_up):
+        _dev(a, w_gate_up)
+        if a.shape[1] != K:
+            raise KernelError(f"gemm_swiglu: a is {tuple(a.shape)} but w is {tuple(w_gate_up.shape)}")
+        out = torch.empty((a.shape[0], rows2 // 2), dtype=torch.bfloat16, device=a.device)
+        _fast_gemm(a, w_gate_up, None, out, BF16, 2, rows2 // 2)
+        return out
+    return swiglu(gemm_generic(a, w_gate_up, out_dtype=torch.float32), out_dtype=a.dtype)
+
+
+DECODE_SPLIT_PAGES = 4
+
+
+def query_tiles(seg_row0):
+    """Cuts the rows of each segment into tiles of 16 that never span two segments:
+    (segment of each tile, first row of each tile), as lists."""
+    tile_seg, tile_row0 = [], []
+    for seg in range(len(seg_row0) - 1):
+        for row in range(seg_row0[seg], seg_row0[seg + 1], 16):
+            tile_seg.append(seg)
+            tile_row0.append(row)
+    return tile_seg, tile_row0
+
+
+def decode_splits(max_context: int, window: int = 0) -> int:
+    blocks = (max_context + PAGE_SIZE - 1) // PAGE_SIZE
+    if window > 0:
+        blocks = min(blocks, (window + PAGE_SIZE - 2) // PAGE_SIZE + 1)
+    return max(1, (blocks + DECODE_SPLIT_PAGES - 1) // DECODE_SPLIT_PAGES)
+
+
+def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
+                      v_pages: torch.Tensor, block_table: torch.Tensor, tile_seg: torch.Tensor, tile_row0: torch.Tensor,
+                      seg_row0: torch.Tensor, row_pos: torch.Tensor, scale: float, window: int = 0) -> torch.Tensor:
+    _dev(q, k_pages, v_pages, block_table, tile_seg, tile_row0, seg_row0, row_pos)
+    _want(q, torch.bfloat16, "q")
+    rows = q.shape[0]
+    if q.shape != (rows, num_heads * head_dim):
+        raise KernelError(f"attention: q is {tuple(q.shape)}, expected {(rows, num_heads * head_dim)}")
+    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, torch.bfloat16)
+    for name, t in (("block_table", block_table), ("tile_seg", tile_seg), ("tile_row0", tile_row0),
+                    ("seg_row0", seg_row0), ("row_pos", row_pos)):
+        _want(t, torch.int32, name)
+    if block_table.dim() != 2 or row_pos.numel() < rows or tile_seg.numel() != tile_row0.numel():
+        raise KernelError("attention: batch index arrays are inconsistent")
+    out = torch.empty_like(q)
+    _check(library().fw_attention_prefill(
+        _p(q), _p(out), _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(tile_seg), _p(tile_row0),
+        tile_seg.numel(), _p(seg_row0), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale),
+        int(window), PAGE_SIZE, pages, _stream()))
+    return out
+
+
+def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
+                     v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
+                     scale: float, max_context: int, window: int = 0) -> torch.Tensor:
+    """One row per request; ``max_context`` bounds position + 1 of every row (the host knows it)."""
+    _dev(q, k_pages, v_pages, block_table, row_seg, row_pos)
+    _want(q, torch.bfloat16, "q")
+    rows = q.shape[0]
+    if q.shape != (rows, num_heads * head_dim):
+        raise KernelError(f"attention: q is {tuple(q.shape)}, expected {(rows, num_heads * head_dim)}")
+    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, torch.bfloat16)
+    for name, t in (("block_table", block_table), ("row_seg", row_seg), ("row_pos", row_pos)):
+        _want(t, torch.int32, name)
+    if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
+        raise KernelError("attention: batch index arrays are too short")
+    splits = decode_splits(max_context, window)
+    partial = torch.empty((rows, num_heads, splits, head_dim + 4), dtype=torch.float32, device=q.device)
+    out = torch.empty_like(q)
+    _check(library().fw_attention_decode(
+        _p(q), _p(out), _p(partial), splits, int(max_context), _p(k_pages), _p(v_pages), _p(block_table),
+        block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale),
+        int(window), PAGE_SIZE, pages, _stream()))
+    return out
 
 
 def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
               v_pages: torch.Tensor, block_table: torch.Tensor, ctx, scale: float, window: int = 0) -> torch.Tensor:
+    """bfloat16 with a head size in steps of 16 runs on the matrix cores (the split-key
+    decode kernel when every segment is one row, the tiled one otherwise); float32 and
+    everything else on the generic kernel."""
+    fast = q.dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= MAX_HEAD_DIM
+    if fast and ctx.all_decode:
+        return attention_decode(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
+                                ctx.row_pos, scale, ctx.max_context, window)
+    if fast and num_heads // num_kv_heads <= 16:
+        return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.tile_seg,
+                                 ctx.tile_row0, ctx.seg_row0, ctx.row_pos, scale, window)
     return attention_generic(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                              ctx.row_pos, scale, window)

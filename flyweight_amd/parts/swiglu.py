@@ -44,5 +44,5 @@ class SwiGLU(FeedForward):
         self.down = Linear(tensors[self._name("down")])
 
     def forward(self, h, residual, ctx) -> None:
-        gate_up = self.gate_up.forward(h, out_dtype=torch.float32)      # the activation is formed in float32
-        self.down.accumulate(ops.swiglu(gate_up, out_dtype=self.dtype), residual)
+        # the activation is formed from float32 sums and rounded once
+        self.down.accumulate(ops.gemm_swiglu(h, self.gate_up.weight), residual)

@@ -67,3 +67,24 @@ def write_random_model(folder: str, config, seed: int,
     write_file(os.path.join(folder, "model.safetensors"), tensors,
                metadata={"format": "pt", "seed": str(int(seed))})
     return folder
+
+
+def random_tensors_on_device(declared: Mapping[str, TensorDecl], seed: int, device: torch.device,
+                             run_dtype: torch.dtype = torch.bfloat16, scale: str = "small") -> Dict[str, torch.Tensor]:
+    """The same distributions drawn on the device, in the dtypes a loaded model would hold
+    (for measurements on shapes too large to write to disk first; the values differ from
+    ``random_tensors`` of the same seed)."""
+    generator = torch.Generator(device=device)
+    generator.manual_seed(int(seed))
+    tensors: Dict[str, torch.Tensor] = {}
+    for name, decl in declared.items():
+        if decl.role == "table":
+            tensors[name] = torch.zeros(decl.shape, dtype=torch.int32, device=device)
+        elif decl.init == "norm":
+            tensors[name] = 0.9 + 0.2 * torch.rand(decl.shape, generator=generator, dtype=torch.float32, device=device)
+        elif decl.init == "zeros":
+            tensors[name] = torch.zeros(decl.shape, dtype=torch.float32, device=device)
+        else:
+            value = torch.randn(decl.shape, generator=generator, dtype=torch.float32, device=device) * _std(decl, scale)
+            tensors[name] = value.to(run_dtype) if decl.role == "matrix" else value
+    return tensors

@@ -334,3 +334,155 @@ def test_kernels_refuse_what_they_were_not_written_for(ops):
         ops.shortconv(torch.zeros(1, 24, device=DEV), torch.zeros(8, 17, device=DEV), None, torch.zeros(1, 8, 16, device=DEV),
                       torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(2, dtype=torch.int32, device=DEV),
                       torch.zeros(1, dtype=torch.int32, device=DEV), 1)
+
+
+# ----- the matrix-core products ----------------------------------------------------------------
+@pytest.mark.parametrize("M", [1, 8, 17, 64, 65, 128, 300])
+@pytest.mark.parametrize("N,K", [(70, 64), (129, 96), (272, 136), (4100, 2056)])
+def test_fast_gemm_every_epilogue(ops, M, N, K):
+    a = as_dev(gen(M, K), torch.bfloat16)
+    w = as_dev(gen(N, K, seed=1, scale=K ** -0.5), torch.bfloat16)
+    bias = gen(N, seed=2).float().to(DEV)
+    want = back(a) @ back(w).T
+    close(ops.gemm(a, w, out_dtype=torch.float32), want, torch.float32, 2.0)
+    close(ops.gemm(a, w, bias, out_dtype=torch.float32), want + bias.cpu().double(), torch.float32, 2.0)
+    close(ops.gemm(a, w), want, torch.bfloat16, 0.4)        # one rounding of the result
+    residual = gen(M, N, seed=3).float().to(DEV)
+    before = residual.cpu().double()
+    ops.gemm(a, w, accumulate_into=residual)
+    close(residual, before + want, torch.float32, 2.0)
+    if N % 2 == 0:
+        half = N // 2
+        act = F.silu(want[:, :half]) * want[:, half:]
+        close(ops.gemm_swiglu(a, w), act, torch.bfloat16, 0.4)
+
+
+def test_fast_gemm_rows_do_not_depend_on_the_batch(ops):
+    a = as_dev(gen(300, 256), torch.bfloat16)
+    w = as_dev(gen(200, 256, seed=1), torch.bfloat16)
+    whole = ops.gemm(a, w, out_dtype=torch.float32)
+    assert torch.equal(ops.gemm(a[100:230].contiguous(), w, out_dtype=torch.float32), whole[100:230])
+    few = ops.gemm(a[:40].contiguous(), w, out_dtype=torch.float32)
+    assert torch.equal(ops.gemm(a[7:8].contiguous(), w, out_dtype=torch.float32)[0], few[7])
+    # the decode and the prompt kernel sum in different orders: equal up to float32 rounding
+    close(few, whole[:40].cpu().double(), torch.float32, 2.0)
+
+
+# ----- attention on the matrix cores -------------------------------------------------------------
+def _mfma_setup(nh, nkv, hd, lengths, num_pages, seed=0):
+    """Several sequences with scattered pages; everything not written is NaN."""
+    rng = np.random.default_rng(seed)
+    order = rng.permutation(num_pages).tolist()
+    stride = max((n + 63) // 64 for n in lengths)
+    table = np.zeros((len(lengths), stride), dtype=np.int32)
+    keys, values = [], []
+    k_pages = torch.full((num_pages, nkv, 64, hd), float("nan"), dtype=torch.float64)
+    v_pages = torch.full((num_pages, nkv, hd, 64), float("nan"), dtype=torch.float64)
+    for i, n in enumerate(lengths):
+        k = gen(n, nkv, hd, seed=seed + 10 * i).to(torch.bfloat16).double()
+        v = gen(n, nkv, hd, seed=seed + 10 * i + 1).to(torch.bfloat16).double()
+        keys.append(k); values.append(v)
+        for b in range((n + 63) // 64):
+            table[i, b] = order.pop()
+        for t in range(n):
+            k_pages[table[i, t // 64], :, t % 64, :] = k[t]
+            v_pages[table[i, t // 64], :, :, t % 64] = v[t]
+    return keys, values, table, k_pages.to(torch.bfloat16).to(DEV), v_pages.to(torch.bfloat16).to(DEV)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (3, 1, 48, 0), (6, 3, 80, 0), (32, 8, 64, 0), (2, 2, 128, 0),
+                                              (16, 1, 256, 0), (4, 2, 32, 70), (4, 4, 64, 64), (2, 1, 64, 1)])
+def test_attention_prefill_on_the_matrix_cores(ops, nh, nkv, hd, window):
+    # segments: a whole prompt, a continuation across a page edge, single rows, a tile and one row
+    lengths = [150, 200, 64, 65, 33]
+    starts = [0, 120, 63, 64, 16]
+    keys, values, table, k_pages, v_pages = _mfma_setup(nh, nkv, hd, lengths, num_pages=14, seed=3)
+    counts = [n - s for n, s in zip(lengths, starts)]
+    seg_row0 = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    row_pos = np.concatenate([np.arange(s, n) for s, n in zip(starts, lengths)]).astype(np.int32)
+    row_seg = np.concatenate([np.full(c, i) for i, c in enumerate(counts)]).astype(np.int32)
+    tile_seg, tile_row0 = ops.query_tiles(seg_row0.tolist())
+    rows = int(seg_row0[-1])
+    q = as_dev(gen(rows, nh * hd, seed=2), torch.bfloat16)
+    scale = 1 / math.sqrt(hd)
+    d = lambda a: torch.tensor(np.asarray(a, dtype=np.int32), device=DEV)       # noqa: E731
+    out = ops.attention_prefill(q, nh, nkv, hd, k_pages, v_pages, d(table), d(tile_seg), d(tile_row0), d(seg_row0),
+                                d(row_pos), scale, window)
+    want = torch.stack([attention_reference(back(q)[r].reshape(nh, hd), keys[row_seg[r]], values[row_seg[r]], int(row_pos[r]),
+                                            scale, window, nh // nkv).reshape(-1) for r in range(rows)])
+    close(out, want, torch.bfloat16)
+    # the generic kernel on the same cache agrees (it runs the same rows when the batch is float32)
+    generic = ops.attention_generic(q, nh, nkv, hd, torch.nan_to_num(k_pages), torch.nan_to_num(v_pages), d(table),
+                                    d(row_seg), d(row_pos), scale, window)
+    close(generic, want, torch.bfloat16)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (3, 1, 48, 0), (6, 3, 80, 0), (32, 8, 64, 0), (2, 2, 128, 0),
+                                              (20, 1, 256, 0), (4, 2, 32, 300), (4, 4, 64, 64), (2, 1, 64, 1)])
+def test_attention_decode_on_the_matrix_cores(ops, nh, nkv, hd, window):
+    lengths = [1, 64, 65, 256, 257, 700, 1000]
+    keys, values, table, k_pages, v_pages = _mfma_setup(nh, nkv, hd, lengths, num_pages=40, seed=5)
+    rows = len(lengths)
+    q = as_dev(gen(rows, nh * hd, seed=2), torch.bfloat16)
+    scale = 1 / math.sqrt(hd)
+    d = lambda a: torch.tensor(np.asarray(a, dtype=np.int32), device=DEV)       # noqa: E731
+    positions = [n - 1 for n in lengths]
+    out = ops.attention_decode(q, nh, nkv, hd, k_pages, v_pages, d(table), d(np.arange(rows)), d(positions), scale,
+                               max_context=max(lengths), window=window)
+    want = torch.stack([attention_reference(back(q)[r].reshape(nh, hd), keys[r], values[r], positions[r], scale, window,
+                                            nh // nkv).reshape(-1) for r in range(rows)])
+    close(out, want, torch.bfloat16)
+    # a larger bound on the context changes the grid, not the result
+    again = ops.attention_decode(q, nh, nkv, hd, k_pages, v_pages, d(table), d(np.arange(rows)), d(positions), scale,
+                                 max_context=1024, window=window)
+    assert torch.equal(again, out)
+    # a row's result does not depend on the rest of the batch
+    alone = ops.attention_decode(q[5:6].contiguous(), nh, nkv, hd, k_pages, v_pages, d(table[5:6]), d([0]), d([positions[5]]),
+                                 scale, max_context=lengths[5], window=window)
+    assert torch.equal(alone[0], out[5])
+    from flyweight_amd.kernels.ops import KernelError
+    with pytest.raises(KernelError, match="do not cover|exceeds the block table"):
+        ops.library()
+        import ctypes
+        partial = torch.empty(rows * nh * (hd + 4), device=DEV)
+        status = ops.library().fw_attention_decode(
+            ctypes.c_void_p(q.data_ptr()), ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(partial.data_ptr()), 1, 100000,
+            ctypes.c_void_p(k_pages.data_ptr()), ctypes.c_void_p(v_pages.data_ptr()), ctypes.c_void_p(d(table).data_ptr()),
+            table.shape[1], ctypes.c_void_p(d(np.arange(rows)).data_ptr()), ctypes.c_void_p(d(positions).data_ptr()), rows, nh,
+            nkv, hd, ctypes.c_float(scale), 0, 64, 40, None)
+        ops._check(status)
+
+
+def test_matrix_core_attention_finds_one_far_key_and_the_edges_of_a_window(ops):
+    """The same single-dominant-key cases as for the generic kernel, for both fast kernels."""
+    nh, nkv, hd, T = 8, 2, 64, 700
+    scale = 1 / math.sqrt(hd)
+    table = np.arange(11, dtype=np.int32)[None]
+    base_keys = gen(T, nkv, hd, scale=0.1)
+    values = gen(T, nkv, hd, seed=1).to(torch.bfloat16).double()
+    direction = torch.zeros(hd, dtype=torch.float64); direction[5] = 1.0
+    q = torch.zeros(1, nh * hd, dtype=torch.float64)
+    q[0, 5::hd] = 60.0
+    d = lambda a: torch.tensor(np.asarray(a, dtype=np.int32), device=DEV)       # noqa: E731
+
+    def run(target, window):
+        k = base_keys.clone(); k[target, :] = direction * 8
+        k_pages = torch.full((11, nkv, 64, hd), float("nan"), dtype=torch.float64)
+        v_pages = torch.full((11, nkv, hd, 64), float("nan"), dtype=torch.float64)
+        for t in range(T):
+            k_pages[t // 64, :, t % 64, :] = k[t]
+            v_pages[t // 64, :, :, t % 64] = values[t]
+        k_pages, v_pages = k_pages.to(torch.bfloat16).to(DEV), v_pages.to(torch.bfloat16).to(DEV)
+        qd = as_dev(q, torch.bfloat16)
+        dec = ops.attention_decode(qd, nh, nkv, hd, k_pages, v_pages, d(table), d([0]), d([T - 1]), scale, T, window)
+        pre = ops.attention_prefill(qd, nh, nkv, hd, k_pages, v_pages, d(table), d([0]), d([0]), d([0, 1]), d([T - 1]), scale, window)
+        return dec[0].cpu().double().reshape(nh, hd), pre[0].cpu().double().reshape(nh, hd)
+
+    for target in (3, 63, 64, 127, 128, 255, 256, 640, 698, 699):
+        for found in run(target, 0):
+            for head in range(nh):
+                assert float((found[head] - values[target, head // 4]).abs().max()) < 0.05, f"key {target}"
+    for target, seen in ((600, True), (599, False), (640, True)):
+        for found in run(target, 100):
+            hit = float((found[0] - values[target, 0]).abs().max()) < 0.05
+            assert hit == seen, f"key {target} with a window of 100 at position {T - 1}"
