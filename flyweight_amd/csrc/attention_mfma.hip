@@ -53,17 +53,38 @@ __device__ __forceinline__ void attend_page(Columns<HD>& c, const uint16_t* __re
                                             int lo, int hi, int last_written) {
     const int lane = threadIdx.x & 63;
     const int i16 = lane & 15, g = lane >> 4;
+    // all loads of the page are issued before the first product (for heads up to 64 channels
+    // the values too: they do not depend on the scores)
+    bf16x8 kf[4][HD / 32];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+        const uint16_t* key = k_page + (size_t)(kt * 16 + i16) * head_dim + g * 8;
+#pragma unroll
+        for (int dc = 0; dc < HD / 32; ++dc) {
+            kf[kt][dc] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (dc * 32 + g * 8 < head_dim) kf[kt][dc] = *reinterpret_cast<const bf16x8*>(key + dc * 32);
+        }
+    }
+    constexpr bool EARLY_V = HD <= 64;
+    u32x2 vearly[EARLY_V ? 2 : 1][EARLY_V ? HD / 16 : 1][2];
+    if (EARLY_V) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int t = 0; t < HD / 16; ++t) {
+                if (t * 16 >= head_dim) break;
+                const uint16_t* value = v_page + (size_t)(t * 16 + i16) * PAGE + kb * 32 + g * 4;
+                vearly[kb][t][0] = *reinterpret_cast<const u32x2*>(value);
+                vearly[kb][t][1] = *reinterpret_cast<const u32x2*>(value + 16);
+            }
+    }
     f32x4 s[4];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
         s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const uint16_t* key = k_page + (size_t)(kt * 16 + i16) * head_dim + g * 8;
 #pragma unroll
-        for (int dc = 0; dc < HD / 32; ++dc) {
-            bf16x8 kf = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (dc * 32 + g * 8 < head_dim) kf = *reinterpret_cast<const bf16x8*>(key + dc * 32);
-            s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, c.q[dc], s[kt], 0, 0, 0);
-        }
+        for (int dc = 0; dc < HD / 32; ++dc)
+            s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kt][dc], c.q[dc], s[kt], 0, 0, 0);
     }
     // mask, then the running maximum of this column: over this lane's 16 scores, then over
     // the four lanes that share the column
@@ -107,9 +128,15 @@ __device__ __forceinline__ void attend_page(Columns<HD>& c, const uint16_t* __re
 #pragma unroll
         for (int t = 0; t < HD / 16; ++t) {
             if (t * 16 >= head_dim) break;
-            const uint16_t* value = v_page + (size_t)(t * 16 + i16) * PAGE;
-            u32x2 va = *reinterpret_cast<const u32x2*>(value + key_a);
-            u32x2 vb = *reinterpret_cast<const u32x2*>(value + key_b);
+            u32x2 va, vb;
+            if (EARLY_V) {
+                va = vearly[kb][t][0];
+                vb = vearly[kb][t][1];
+            } else {
+                const uint16_t* value = v_page + (size_t)(t * 16 + i16) * PAGE;
+                va = *reinterpret_cast<const u32x2*>(value + key_a);
+                vb = *reinterpret_cast<const u32x2*>(value + key_b);
+            }
             if (partial_page) {
                 // keep keys <= last_written only: two keys per 32-bit word, low half first
                 auto keep = [&](uint32_t word, int first_key) -> uint32_t {
@@ -191,38 +218,39 @@ __global__ void attention_prefill_kernel(
 }
 
 // ---- decode ------------------------------------------------------------------------------------
-// grid (rows, kv heads * head tiles, splits); one wave. Columns are the query heads of the kv
-// group (16 per head tile). partial [rows][heads][max_splits][head_dim + 4]: unnormalised
-// output, then maximum and sum; a split with nothing to do writes nothing.
+// grid (rows, kv heads * head tiles, splits); four waves, each takes one page of the split's
+// SPLIT_PAGES, and their results are merged in LDS in the order of the keys. Columns are the
+// query heads of the kv group (16 per head tile). partial [rows][heads][max_splits][head_dim + 4]:
+// unnormalised output, then maximum and sum; a split with nothing to do writes nothing.
 template <int HD>
-__global__ __launch_bounds__(64) void attention_decode_split_kernel(
+__global__ __launch_bounds__(64 * SPLIT_PAGES) void attention_decode_split_kernel(
     const uint16_t* __restrict__ q, float* __restrict__ partial, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ row_seg, const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads,
     int head_dim, float scale_log2, int window, int max_splits) {
+    __shared__ f32x4 shared_o[SPLIT_PAGES][HD / 16][64];
+    __shared__ float shared_m[SPLIT_PAGES][16], shared_l[SPLIT_PAGES][16];
     const int row = blockIdx.x, split = blockIdx.z;
     const int group = num_heads / num_kv_heads;
     const int head_tiles = (group + 15) / 16;
     const int kvh = blockIdx.y / head_tiles, head_tile = blockIdx.y % head_tiles;
-    const int lane = threadIdx.x & 63, col = lane & 15, g = lane >> 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, g = lane >> 4;
     const int pos = row_pos[row];
     const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
     // splits are counted from the first page that holds a visible key
     const int first_block = first / PAGE + split * SPLIT_PAGES;
     const int last_block = pos / PAGE;
-    if (first_block > last_block) return;
-    const int end_block = first_block + SPLIT_PAGES - 1 < last_block ? first_block + SPLIT_PAGES - 1 : last_block;
+    if (first_block > last_block) return;       // the whole workgroup
     const int in_group = head_tile * 16 + col;
     const bool valid = in_group < group;
     const int head = kvh * group + (valid ? in_group : 0);
 
     Columns<HD> c;
     load_query<HD>(c, q + ((size_t)row * num_heads + head) * head_dim, head_dim, valid);
-    const int32_t* table = block_table + (size_t)row_seg[row] * table_stride;
-    const size_t page_elems = (size_t)PAGE * head_dim;
-    for (int block = first_block; block <= end_block; ++block) {
-        const int page = table[block];
-        const size_t at = ((size_t)page * num_kv_heads + kvh) * page_elems;
+    const int block = first_block + wave;
+    if (block <= last_block) {
+        const int page = block_table[(size_t)row_seg[row] * table_stride + block];
+        const size_t at = ((size_t)page * num_kv_heads + kvh) * PAGE * head_dim;
         const int base = block * PAGE;
         attend_page<HD>(c, k_pages + at, v_pages + at, head_dim, scale_log2, valid ? first - base : PAGE,
                         valid ? pos - base : -1, pos - base);
@@ -230,16 +258,35 @@ __global__ __launch_bounds__(64) void attention_decode_split_kernel(
     float l = c.l;
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
-    if (!valid) return;
+#pragma unroll
+    for (int t = 0; t < HD / 16; ++t) shared_o[wave][t][lane] = c.o[t];
+    if (g == 0) {
+        shared_m[wave][col] = c.m;
+        shared_l[wave][col] = l;
+    }
+    __syncthreads();
+    if (wave != 0 || !valid) return;
+    float m = NEG_BIG;
+#pragma unroll
+    for (int w = 0; w < SPLIT_PAGES; ++w) m = fmaxf(m, shared_m[w][col]);
+    float total = 0.0f, weight[SPLIT_PAGES];
+#pragma unroll
+    for (int w = 0; w < SPLIT_PAGES; ++w) {
+        weight[w] = exp2f(shared_m[w][col] - m);        // a wave without a page has l = 0 and o = 0
+        total += weight[w] * shared_l[w][col];
+    }
     float* dest = partial + (((size_t)row * num_heads + head) * max_splits + split) * PART_STRIDE(head_dim);
 #pragma unroll
     for (int t = 0; t < HD / 16; ++t) {
         if (t * 16 >= head_dim) break;
-        *reinterpret_cast<f32x4*>(dest + t * 16 + g * 4) = c.o[t];
+        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < SPLIT_PAGES; ++w) sum += weight[w] * shared_o[w][t][lane];
+        *reinterpret_cast<f32x4*>(dest + t * 16 + g * 4) = sum;
     }
     if (g == 0) {
-        dest[head_dim] = c.m;
-        dest[head_dim + 1] = l;
+        dest[head_dim] = m;
+        dest[head_dim + 1] = total;
     }
 }
 
@@ -345,7 +392,7 @@ extern "C" int fw_attention_decode(const void* q, void* out, float* partial, int
     FW_REQUIRE(rows <= 1 << 20 && num_kv_heads * head_tiles <= 65535 && num_heads <= 65535, "attention_decode: grid too large");
     dim3 grid(rows, num_kv_heads * head_tiles, max_splits);
 #define CALL(HD)                                                                                                   \
-    attention_decode_split_kernel<HD><<<grid, 64, 0, (hipStream_t)stream>>>(                                        \
+    attention_decode_split_kernel<HD><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                                        \
         (const uint16_t*)q, partial, (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table, table_stride, \
         row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits)
     FW_BY_HEAD_DIM(head_dim, CALL);

@@ -100,6 +100,53 @@ class StepContext:
         self.block_tables = [v.view(t.shape) for v, t in zip(views[8:], tables)]
         self._position_tables: Dict = {}
 
+    @classmethod
+    def for_decode_graph(cls, batch: int, cache: CacheManager, device: torch.device, max_context: int,
+                         table_stride: int) -> "StepContext":
+        """A context of ``batch`` single-token segments whose index arrays live in ONE
+        persistent device buffer, refreshed before every replay of the captured step."""
+        self = cls.__new__(cls)
+        self.num_rows = self.num_segments = self.num_wanted = batch
+        self.all_decode = True
+        self.max_context = max_context          # bounds the split-key grid, not the result
+        self.device = device
+        self.host_row_pos = self.host_seg_row0 = self.host_seg_slot = None     # not for captured steps
+        sizes = [batch, batch, batch, batch + 1, batch, batch, batch, batch] + [batch * table_stride] * len(cache.groups)
+        self.host_buffer = torch.empty(sum(sizes), dtype=torch.int32, pin_memory=True)
+        self.device_buffer = torch.zeros(sum(sizes), dtype=torch.int32, device=device)
+        views, host_views, offset = [], [], 0
+        for size in sizes:
+            views.append(self.device_buffer[offset:offset + size])
+            host_views.append(self.host_buffer[offset:offset + size].numpy())
+            offset += size
+        (self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows, self.tile_seg,
+         self.tile_row0) = views[:8]
+        self.block_tables = [v.view(batch, table_stride) for v in views[8:]]
+        self._host = host_views
+        self._table_stride = table_stride
+        # what never changes between replays
+        rows = np.arange(batch, dtype=np.int32)
+        host_views[2][:] = rows
+        host_views[3][:] = np.arange(batch + 1, dtype=np.int32)
+        host_views[5][:] = rows
+        host_views[6][:] = rows
+        host_views[7][:] = rows
+        self._position_tables = {}
+        return self
+
+    def refresh(self, entries: Sequence[StepEntry], cache: CacheManager) -> None:
+        """Writes this step's tokens, positions, slots and block tables and uploads them."""
+        host = self._host
+        self.requests = [e.request for e in entries]
+        starts = [cache.length_of(r) for r in self.requests]
+        self.new_lengths = [s + 1 for s in starts]
+        host[0][:] = [int(e.tokens[0]) for e in entries]
+        host[1][:] = starts
+        host[4][:] = [cache.slot_of(r) for r in self.requests]
+        for g in range(len(cache.groups)):
+            host[8 + g][:] = cache.block_table_rows(g, self.requests, stride=self._table_stride).reshape(-1)
+        self.device_buffer.copy_(self.host_buffer, non_blocking=True)
+
     def position_tables(self, part):
         key = part.key()
         if key not in self._position_tables:
@@ -132,6 +179,12 @@ class Stepper:
                                   device=model.device)
         self.steps = 0
         self.tokens_run = 0
+        # decode steps (every segment one token) are captured in a HIP graph per batch size and
+        # replayed, if every part of the model allows it
+        self.use_graphs = all(block.graph_safe for block in model.layers) and model.final_norm.graph_safe
+        self._graphs: Dict[int, "_CapturedDecode"] = {}
+        self._eager_decodes: Dict[int, int] = {}
+        self.graph_replays = 0
 
     def admit(self, request: Hashable) -> None:
         self.cache.admit(request)
@@ -184,6 +237,10 @@ class Stepper:
                 raise OutOfPages(f"out of cache pages: the step needs {count} more, {cache.groups[g].pool.free_count} free")
         for entry in entries:
             cache.reserve(entry.request, cache.length_of(entry.request) + len(entry.tokens))
+        if self.use_graphs and all(len(entry.tokens) == 1 for entry in entries):
+            captured = self._captured_decode(len(entries))
+            if captured is not None:
+                return self._replay(captured, entries)
         ctx = StepContext(entries, cache, self.device, self.model.spec.vocab_size, self.model.spec.max_positions)
         logits = self.model.forward(ctx, cache)
         for request, length in zip(ctx.requests, ctx.new_lengths):
@@ -191,3 +248,55 @@ class Stepper:
         self.steps += 1
         self.tokens_run += ctx.num_rows
         return logits
+
+    # ----- captured decode steps ----------------------------------------------------------
+    def _captured_decode(self, batch: int) -> Optional["_CapturedDecode"]:
+        """The graph for this batch size; the first decode step of a size runs eagerly (it
+        also sets the kernels' attributes), the second is captured."""
+        captured = self._graphs.get(batch)
+        if captured is not None:
+            return captured
+        seen = self._eager_decodes.get(batch, 0)
+        self._eager_decodes[batch] = seen + 1
+        if seen < 1:
+            return None
+        cache = self.cache
+        ctx = StepContext.for_decode_graph(batch, cache, self.device, max_context=self.model.spec.max_positions,
+                                           table_stride=cache.max_pages_per_request)
+        captured = _CapturedDecode(ctx)
+        self._graphs[batch] = captured
+        return captured
+
+    def _replay(self, captured: "_CapturedDecode", entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        cache = self.cache
+        ctx = captured.ctx
+        ctx.refresh(entries, cache)
+        if captured.graph is None:
+            # record the step once; recording runs nothing, the replay below does
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                with torch.cuda.graph(graph, stream=side):
+                    captured.logits = self.model.forward(ctx, cache)
+            torch.cuda.current_stream().wait_stream(side)
+            captured.graph = graph
+        captured.graph.replay()
+        self.graph_replays += 1
+        for request, length in zip(ctx.requests, ctx.new_lengths):
+            cache.commit(request, length)
+        self.steps += 1
+        self.tokens_run += ctx.num_rows
+        wanted = [i for i, entry in enumerate(entries) if len(entry.want)]
+        if not wanted:
+            return None
+        if len(wanted) == len(entries):
+            return captured.logits          # overwritten by the next replay of this batch size
+        return captured.logits[wanted]
+
+
+class _CapturedDecode:
+    def __init__(self, ctx: StepContext):
+        self.ctx = ctx
+        self.graph = None
+        self.logits = None

@@ -29,6 +29,11 @@ from ..weights.loader import TensorDecl
 
 
 class Part:
+    # True when ``forward`` only launches work on the current stream from device-side batch
+    # data (no host reads of the batch, no synchronisation): a decode step made of such parts
+    # may be captured in a HIP graph and replayed. Parts that look at ``ctx.host_*`` leave it False.
+    graph_safe = False
+
     def __init__(self, spec: PartSpec):
         self.spec = spec
         self.prefix = spec.prefix

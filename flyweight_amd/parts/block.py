@@ -38,6 +38,11 @@ class PreNormResidualBlock:
     def cache_need(self):
         return self.mixer.cache_need()
 
+    @property
+    def graph_safe(self) -> bool:
+        position = getattr(self.mixer, "position", None)
+        return all(part.graph_safe for part in self.parts()) and (position is None or position.graph_safe)
+
     def forward(self, x, ctx, cache) -> None:
         """``x`` [rows, hidden] float32 is updated in place."""
         self.mixer.forward(self.mixer_norm.forward(x, ctx), x, ctx, cache)

@@ -14,6 +14,8 @@ from .base import Norm, register_norm
 
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.size = int(spec["size"])

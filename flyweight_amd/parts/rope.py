@@ -15,6 +15,8 @@ from .base import PositionEncoding, register_position_encoding
 
 @register_position_encoding("rotary_neox")
 class RotaryNeox(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.theta = float(spec["theta"])
@@ -38,6 +40,8 @@ class RotaryNeox(PositionEncoding):
 
 @register_position_encoding("none")
 class NoPosition(PositionEncoding):
+    graph_safe = True
+
     rotary_dim = 0
 
     def tables(self, ctx):

@@ -24,6 +24,8 @@ from .linear import Linear
 
 @register_mixer("short_conv")
 class ShortConv(Mixer):
+    graph_safe = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.hidden = int(spec["hidden_size"])

@@ -19,6 +19,8 @@ _DEFAULT_NAMES = {"gate": "gate_proj", "up": "up_proj", "down": "down_proj"}
 
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, spec):
         super().__init__(spec)
         self.hidden = int(spec["hidden_size"])

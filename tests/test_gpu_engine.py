@@ -239,3 +239,36 @@ def test_errors_are_reported_not_hidden(loaded):
         stepper.step([StepEntry("a", [1] * 65, [])])
     assert stepper.cache.length_of("a") == 0 and stepper.cache.groups[0].pool.in_use == 0   # nothing half-done
     assert stepper.step([StepEntry("a", [1] * 64, [63])]).shape == (1, m.config.vocab_size)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_captured_decode_steps_replay_to_the_eager_result(loaded, dtype):
+    """Decode steps are recorded in a HIP graph per batch size and replayed. Every replay,
+    with eager prompt portions and synchronisations between them and with the batch changing
+    size, must give what the eager step gives."""
+    from flyweight_amd.engine import StepEntry
+    m = loaded("B", dtype)
+    vocab = m.config.vocab_size
+    runs = []
+    for use_graphs in (False, True):
+        stepper = m.stepper(num_pages=12, max_requests=4)
+        assert stepper.use_graphs
+        stepper.use_graphs = use_graphs
+        rng = np.random.default_rng(5)
+        out = []
+        for request in ("a", "b", "c"):
+            stepper.admit(request)
+        stepper.step([StepEntry("a", rng.integers(0, vocab, 70).tolist(), []), StepEntry("b", rng.integers(0, vocab, 3).tolist(), [])])
+        for step in range(40):
+            entries = [StepEntry("a", [int(rng.integers(0, vocab))], [0]), StepEntry("b", [int(rng.integers(0, vocab))], [0])]
+            if step % 7 == 3:       # an eager step between replays: a prompt portion of a third request
+                out.append(stepper.step([StepEntry("c", rng.integers(0, vocab, 5).tolist(), [4])]).cpu().numpy())
+            if step >= 20:          # the batch grows: another graph
+                entries.append(StepEntry("c", [int(rng.integers(0, vocab))], [] if step % 2 else [0]))
+            logits = stepper.step(entries)
+            out.append(logits.cpu().numpy())
+        runs.append(out)
+        if use_graphs:
+            assert stepper.graph_replays >= 30 and set(stepper._graphs) == {2, 3}
+    for eager, replayed in zip(*runs):
+        assert eager.shape == replayed.shape and np.array_equal(eager, replayed)
