@@ -38,6 +38,18 @@ int fw_gemm_skinny(const void* a, const void* w, const float* bias, void* out, i
 int fw_gemm_mfma(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                  int M, int N, int K, void* stream);
 
+// Fused product for decode steps of up to 16 rows. prologue 0: a is bfloat16 [M][K]; 1: a is
+// float32 rows, RMS-normed with norm_weight/eps (rows gathered through row_index if given) inside
+// the kernel. epilogue 0: store out_dtype [M][N]; 1: float32 out += ; 2: SwiGLU, w = [gate rows;
+// up rows], out bfloat16 [M][N]; 3: gated short convolution of single-token segments, w = [B rows;
+// C rows; x rows] of N channels each, state [slots][N][kernel_size - 1] read and shifted.
+// fw_gemm_decode_fits says whether a shape is taken (1) or must go to separate kernels (0).
+int fw_gemm_decode(int prologue, const void* a, const float* norm_weight, const int32_t* row_index, float eps,
+                   int one_centered, const void* w, const float* bias, void* out, int out_dtype, int epilogue,
+                   int M, int N, int K, const float* taps, const float* conv_bias, float* state,
+                   const int32_t* seg_slot, int kernel_size, void* stream);
+int fw_gemm_decode_fits(int M, int N, int K, int epilogue);
+
 // out[r][i] = silu(gu[r][i]) * gu[r][I + i]; the input may be float32 beside a bfloat16 output
 int fw_swiglu(const void* gate_up, int in_dtype, void* out, int out_dtype, int rows, int intermediate,
               void* stream);

@@ -13,6 +13,7 @@ from ..config import ModelSpec, load_config
 from ..config.spec import ConfigError
 from ..kernels import ops
 from ..parts import Linear, build_part
+from ..parts.norm import LazyNorm
 from ..parts.base import _REGISTRIES
 from ..weights.loader import TensorDecl, load_tensors
 
@@ -100,8 +101,7 @@ class CausalLM:
             self.layers[entry.layer].forward(x, ctx, ctx.cache_view(cache, entry))
         if ctx.num_wanted == 0:
             return None
-        h = self.final_norm.forward(x, ctx, row_index=ctx.want_rows)
-        return self.head.forward(h, out_dtype=torch.float32)
+        return self.head.forward(LazyNorm(self.final_norm, x, ctx, row_index=ctx.want_rows), out_dtype=torch.float32)
 
 
 def declared_tensors(spec: ModelSpec) -> Dict[str, TensorDecl]:

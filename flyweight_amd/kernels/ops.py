@@ -356,6 +356,69 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     return swiglu(gemm_generic(a, w_gate_up, out_dtype=torch.float32), out_dtype=a.dtype)
 
 
+# ---- fused products for decode steps of up to 16 rows --------------------------------------------
+EPILOGUE_STORE, EPILOGUE_ACCUMULATE, EPILOGUE_SWIGLU, EPILOGUE_CONV = 0, 1, 2, 3
+DECODE_MAX_ROWS = 16
+
+
+def gemm_decode_fits(rows: int, features: int, k: int, epilogue: int) -> bool:
+    return bool(library().fw_gemm_decode_fits(int(rows), int(features), int(k), int(epilogue)))
+
+
+def gemm_decode(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Optional[torch.Tensor] = None,
+                norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0, one_centered: bool = False,
+                row_index: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
+                accumulate_into: Optional[torch.Tensor] = None, taps: Optional[torch.Tensor] = None,
+                conv_bias: Optional[torch.Tensor] = None, state: Optional[torch.Tensor] = None,
+                seg_slot: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One kernel for (optional RMS norm of float32 rows) -> product with bfloat16 ``w`` -> epilogue.
+    With ``norm_weight`` ``a`` holds float32 rows (gathered through ``row_index`` if given), else
+    bfloat16 activations. See fw_gemm_decode in fw_kernels.h for the epilogues."""
+    _dev(a, w, bias, norm_weight, row_index, accumulate_into, taps, conv_bias, state, seg_slot)
+    _want(w, torch.bfloat16, "w")
+    normed = norm_weight is not None
+    rows = row_index.numel() if (normed and row_index is not None) else a.shape[0]
+    K = a.shape[1]
+    tiles = {EPILOGUE_SWIGLU: 2, EPILOGUE_CONV: 3}.get(epilogue, 1)
+    if w.shape[1] != K or w.shape[0] % tiles:
+        raise KernelError(f"gemm_decode: a is {tuple(a.shape)} but w is {tuple(w.shape)}")
+    N = w.shape[0] // tiles
+    if normed:
+        _want(a, torch.float32, "a")
+        _want(norm_weight, torch.float32, "norm_weight")
+        if norm_weight.shape != (K,):
+            raise KernelError("gemm_decode: the norm weight must be [K]")
+        if row_index is not None:
+            _want(row_index, torch.int32, "row_index")
+    else:
+        _want(a, torch.bfloat16, "a")
+    if bias is not None and (bias.dtype != torch.float32 or bias.shape != (w.shape[0],)):
+        raise KernelError("gemm_decode: bias must be float32, one entry per row of w")
+    kernel_size = 0
+    if epilogue == EPILOGUE_CONV:
+        _want(taps, torch.float32, "taps")
+        _want(state, torch.float32, "state")
+        _want(seg_slot, torch.int32, "seg_slot")
+        kernel_size = taps.shape[1]
+        if taps.shape != (N, kernel_size) or state.dim() != 3 or state.shape[1:] != (N, kernel_size - 1):
+            raise KernelError("gemm_decode: taps must be [N, L] and state [slots, N, L - 1]")
+        if seg_slot.numel() < rows or (conv_bias is not None and conv_bias.shape != (N,)):
+            raise KernelError("gemm_decode: seg_slot or the convolution bias has the wrong size")
+    if epilogue == EPILOGUE_ACCUMULATE:
+        _want(accumulate_into, torch.float32, "accumulate_into")
+        if accumulate_into.shape != (rows, N):
+            raise KernelError(f"gemm_decode: destination is {tuple(accumulate_into.shape)}, expected {(rows, N)}")
+        target, out_dtype = accumulate_into, torch.float32
+    else:
+        out_dtype = out_dtype or torch.bfloat16
+        target = torch.empty((rows, N), dtype=out_dtype, device=a.device)
+    _check(library().fw_gemm_decode(
+        int(normed), _p(a), _p(norm_weight), _p(row_index), ctypes.c_float(eps), int(one_centered), _p(w), _p(bias),
+        _p(target), _code(out_dtype), int(epilogue), rows, N, K, _p(taps), _p(conv_bias), _p(state), _p(seg_slot),
+        int(kernel_size), _stream()))
+    return target
+
+
 DECODE_SPLIT_PAGES = 4
 
 

@@ -27,6 +27,7 @@ _DEFAULT_NAMES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj", "q
 @register_mixer("gqa_attention")
 class GQAttention(Mixer):
     graph_safe = True
+    accepts_lazy_norm = True
 
     def __init__(self, spec):
         super().__init__(spec)

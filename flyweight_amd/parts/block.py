@@ -11,6 +11,7 @@ from typing import Dict
 
 from ..weights.loader import TensorDecl
 from .base import build_part, register_block
+from .norm import LazyNorm
 
 
 @register_block("pre_norm_residual")
@@ -45,5 +46,8 @@ class PreNormResidualBlock:
 
     def forward(self, x, ctx, cache) -> None:
         """``x`` [rows, hidden] float32 is updated in place."""
-        self.mixer.forward(self.mixer_norm.forward(x, ctx), x, ctx, cache)
-        self.ffn.forward(self.ffn_norm.forward(x, ctx), x, ctx)
+        # a part that can take the norm into its own first kernel gets it unevaluated
+        h = LazyNorm(self.mixer_norm, x, ctx)
+        self.mixer.forward(h if getattr(self.mixer, "accepts_lazy_norm", False) else h.tensor(), x, ctx, cache)
+        h = LazyNorm(self.ffn_norm, x, ctx)
+        self.ffn.forward(h if getattr(self.ffn, "accepts_lazy_norm", False) else h.tensor(), x, ctx)

@@ -1,17 +1,24 @@
 """A matrix product with a stored weight: out = a . W^T (+ bias).
 
 ``forward`` returns activations; ``accumulate`` adds the product to the float32 residual
-stream in the kernel's epilogue, so the residual sum never leaves float32. Which kernel
-runs is chosen here from the operand types and the number of rows.
+stream in the kernel's epilogue, so the residual sum never leaves float32; ``swiglu`` and
+``short_conv`` finish the product with that part's arithmetic. Which kernel runs is chosen
+here from the operand types and the number of rows: for up to 16 rows of a bfloat16 model one
+fused kernel takes the RMS norm before the product (handed over as a :class:`LazyNorm`) and
+the epilogue after it; otherwise the norm runs on its own and the skinny, tiled or generic
+product follows.
 """
 
 from __future__ import annotations
 
-from typing import Optional
+from typing import Optional, Union
 
 import torch
 
 from ..kernels import ops
+from .norm import LazyNorm
+
+Input = Union[torch.Tensor, LazyNorm]
 
 
 class Linear:
@@ -22,8 +29,58 @@ class Linear:
         self.bias = bias
         self.out_features, self.in_features = weight.shape
 
-    def forward(self, a: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-        return ops.gemm(a, self.weight, self.bias, out_dtype=out_dtype or a.dtype)
+    # ----- which path ---------------------------------------------------------------------
+    def _fused(self, a: Input, features: int, epilogue: int) -> bool:
+        if self.weight.dtype != torch.bfloat16 or a.dtype != torch.bfloat16:
+            return False
+        rows = a.rows if isinstance(a, LazyNorm) else a.shape[0]
+        if not 1 <= rows <= ops.DECODE_MAX_ROWS:
+            return False
+        if isinstance(a, LazyNorm) and a.rms_parameters() is None:
+            return False
+        return ops.gemm_decode_fits(rows, features, self.in_features, epilogue)
+
+    @staticmethod
+    def _norm_arguments(a: Input) -> dict:
+        if not isinstance(a, LazyNorm):
+            return {}
+        weight, eps, one_centered = a.rms_parameters()
+        return {"norm_weight": weight, "eps": eps, "one_centered": one_centered, "row_index": a.row_index}
+
+    @staticmethod
+    def _rows_of(a: Input) -> torch.Tensor:
+        return a.x if isinstance(a, LazyNorm) else a
+
+    @staticmethod
+    def _tensor_of(a: Input) -> torch.Tensor:
+        return a.tensor() if isinstance(a, LazyNorm) else a
+
+    # ----- products -----------------------------------------------------------------------
+    def forward(self, a: Input, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        out_dtype = out_dtype or a.dtype
+        if self._fused(a, self.out_features, ops.EPILOGUE_STORE):
+            return ops.gemm_decode(self._rows_of(a), self.weight, ops.EPILOGUE_STORE, bias=self.bias, out_dtype=out_dtype,
+                                   **self._norm_arguments(a))
+        return ops.gemm(self._tensor_of(a), self.weight, self.bias, out_dtype=out_dtype)
 
     def accumulate(self, a: torch.Tensor, residual: torch.Tensor) -> None:
+        if self._fused(a, self.out_features, ops.EPILOGUE_ACCUMULATE):
+            ops.gemm_decode(a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias, accumulate_into=residual)
+            return
         ops.gemm(a, self.weight, self.bias, accumulate_into=residual)
+
+    def swiglu(self, a: Input) -> torch.Tensor:
+        """The weight holds gate rows then up rows: silu(a . gate^T) * (a . up^T)."""
+        if self.bias is None and self._fused(a, self.out_features // 2, ops.EPILOGUE_SWIGLU):
+            return ops.gemm_decode(self._rows_of(a), self.weight, ops.EPILOGUE_SWIGLU, out_dtype=torch.bfloat16,
+                                   **self._norm_arguments(a))
+        return ops.gemm_swiglu(self._tensor_of(a), self.weight)
+
+    def short_conv_decode(self, a: Input, taps: torch.Tensor, conv_bias: Optional[torch.Tensor], state: torch.Tensor,
+                          seg_slot: torch.Tensor, out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+        """For single-token segments: the weight holds B, C and x rows; returns C * conv(B * x)
+        with the state shifted, or None when the fused kernel does not take the shape."""
+        if not self._fused(a, self.out_features // 3, ops.EPILOGUE_CONV):
+            return None
+        return ops.gemm_decode(self._rows_of(a), self.weight, ops.EPILOGUE_CONV, bias=self.bias, out_dtype=out_dtype,
+                               taps=taps, conv_bias=conv_bias, state=state, seg_slot=seg_slot, **self._norm_arguments(a))

@@ -12,6 +12,33 @@ from ..weights.loader import TensorDecl
 from .base import Norm, register_norm
 
 
+class LazyNorm:
+    """A norm that has not run yet: the rows ``x`` (optionally gathered through ``row_index``)
+    and the norm to apply. A product that can apply an RMS norm in its own kernel takes it as
+    it is (``rms_parameters``); anything else calls ``tensor()``, which runs the norm once."""
+
+    def __init__(self, norm: Norm, x: torch.Tensor, ctx, row_index: Optional[torch.Tensor] = None):
+        self.norm, self.x, self.ctx, self.row_index = norm, x, ctx, row_index
+        self._tensor = None
+
+    @property
+    def rows(self) -> int:
+        return self.row_index.numel() if self.row_index is not None else self.x.shape[0]
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.norm.dtype
+
+    def rms_parameters(self):
+        """(weight, eps, one_centered) if the norm is a plain RMS norm, else None."""
+        return self.norm.rms_parameters() if hasattr(self.norm, "rms_parameters") else None
+
+    def tensor(self) -> torch.Tensor:
+        if self._tensor is None:
+            self._tensor = self.norm.forward(self.x, self.ctx, row_index=self.row_index)
+        return self._tensor
+
+
 @register_norm("rmsnorm")
 class RMSNorm(Norm):
     graph_safe = True
@@ -28,6 +55,9 @@ class RMSNorm(Norm):
     def bind(self, tensors, dtype, device) -> None:
         super().bind(tensors, dtype, device)
         self.weight = tensors[self.prefix + "weight"]
+
+    def rms_parameters(self):
+        return self.weight, self.eps, self.one_centered
 
     def forward(self, x: torch.Tensor, ctx, row_index: Optional[torch.Tensor] = None) -> torch.Tensor:
         return ops.rmsnorm_rows(x, self.weight, self.eps, self.dtype, row_index=row_index,

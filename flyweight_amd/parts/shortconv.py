@@ -25,6 +25,7 @@ from .linear import Linear
 @register_mixer("short_conv")
 class ShortConv(Mixer):
     graph_safe = True
+    accepts_lazy_norm = True
 
     def __init__(self, spec):
         super().__init__(spec)
@@ -59,6 +60,11 @@ class ShortConv(Mixer):
         self.conv_bias = tensors[p + "conv.bias"] if self.bias else None
 
     def forward(self, h, residual, ctx, cache) -> None:
+        if ctx.all_decode:      # single-token segments: norm, in_proj, convolution and state shift in one kernel
+            gated = self.in_proj.short_conv_decode(h, self.taps, self.conv_bias, cache.state, ctx.seg_slot, self.dtype)
+            if gated is not None:
+                self.out_proj.accumulate(gated, residual)
+                return
         bcx = self.in_proj.forward(h, out_dtype=torch.float32)  # B * x and the taps' sum stay in float32
         gated = ops.shortconv(bcx, self.taps, self.conv_bias, cache.state, ctx.row_seg, ctx.seg_row0, ctx.seg_slot,
                               ctx.num_segments, out_dtype=self.dtype)

@@ -20,6 +20,7 @@ _DEFAULT_NAMES = {"gate": "gate_proj", "up": "up_proj", "down": "down_proj"}
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
     graph_safe = True
+    accepts_lazy_norm = True
 
     def __init__(self, spec):
         super().__init__(spec)
@@ -47,4 +48,4 @@ class SwiGLU(FeedForward):
 
     def forward(self, h, residual, ctx) -> None:
         # the activation is formed from float32 sums and rounded once
-        self.down.accumulate(ops.gemm_swiglu(h, self.gate_up.weight), residual)
+        self.down.accumulate(self.gate_up.swiglu(h), residual)

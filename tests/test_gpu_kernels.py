@@ -486,3 +486,114 @@ def test_matrix_core_attention_finds_one_far_key_and_the_edges_of_a_window(ops):
         for found in run(target, 100):
             hit = float((found[0] - values[target, 0]).abs().max()) < 0.05
             assert hit == seen, f"key {target} with a window of 100 at position {T - 1}"
+
+
+# ----- the fused decode product -----------------------------------------------------------------
+def _normed(x, weight, eps, one_centered=False):
+    w = 1 + weight if one_centered else weight
+    return x / torch.sqrt((x ** 2).mean(-1, keepdim=True) + eps) * w
+
+
+def _kernel_norm(ops, x, norm_w, eps, index=None, one_centered=False):
+    """The normed rows exactly as the fused kernel rounds them to bfloat16: its product with an
+    identity matrix (exact). They are checked against the float64 norm to one rounding; the
+    products are then checked against THESE rows, so that a value the kernel's float32 norm
+    rounds the other way than float64 would does not pass for an error of the product."""
+    K = x.shape[1]
+    identity = torch.eye(K, dtype=torch.bfloat16, device=DEV)
+    h = ops.gemm_decode(x.to(DEV), identity, ops.EPILOGUE_STORE, norm_weight=norm_w.to(DEV), eps=eps, one_centered=one_centered,
+                        row_index=None if index is None else index.to(DEV), out_dtype=torch.float32).cpu().double()
+    exact = _normed(x.double(), norm_w.double(), eps, one_centered)
+    exact = exact if index is None else exact[index.long()]
+    assert float(((h - exact).abs() / exact.abs().clamp_min(1e-3)).max()) <= 2.0 ** -8        # bfloat16: 8 bits of mantissa
+    return h
+
+
+@pytest.mark.parametrize("M", [1, 5, 8, 9, 16])
+@pytest.mark.parametrize("N,K", [(72, 64), (200, 96), (4096, 512), (4104, 136), (16400, 256), (2048, 4096)])
+def test_fused_decode_product(ops, M, N, K):
+    """Norm prologue or plain activations, every epilogue, outputs narrower and wider than one
+    tile per compute unit, K that is no multiple of the chunk."""
+    x = gen(M + 3, K, scale=2).float()
+    norm_w = (1 + 0.1 * gen(K, seed=1)).float()
+    w = as_dev(gen(N, K, seed=2, scale=K ** -0.5), torch.bfloat16)
+    bias = gen(N, seed=3).float()
+    eps = 1e-5
+    index = torch.tensor(list(range(M + 2, 2, -1)), dtype=torch.int32)      # rows gathered in reverse
+    h = _kernel_norm(ops, x, norm_w, eps, index)         # what the kernel keeps in LDS
+    want = h @ back(w).T
+    assert ops.gemm_decode_fits(M, N, K, ops.EPILOGUE_STORE)
+    got = ops.gemm_decode(x.to(DEV), w, ops.EPILOGUE_STORE, norm_weight=norm_w.to(DEV), eps=eps, row_index=index.to(DEV),
+                          out_dtype=torch.float32)
+    close(got, want, torch.float32, 2.0)
+    got = ops.gemm_decode(x.to(DEV), w, ops.EPILOGUE_STORE, norm_weight=norm_w.to(DEV), eps=eps, row_index=index.to(DEV),
+                          bias=bias.to(DEV), out_dtype=torch.bfloat16)
+    close(got, want + bias.double(), torch.bfloat16, 0.4)
+    centered = _kernel_norm(ops, x[:M].contiguous(), norm_w, eps, one_centered=True) @ back(w).T
+    got = ops.gemm_decode(x[:M].contiguous().to(DEV), w, ops.EPILOGUE_STORE, norm_weight=norm_w.to(DEV), eps=eps, one_centered=True,
+                          out_dtype=torch.float32)
+    close(got, centered, torch.float32, 2.0)
+    # plain bfloat16 activations; adding into the residual stream
+    a = as_dev(gen(M, K, seed=4), torch.bfloat16)
+    plain = back(a) @ back(w).T
+    close(ops.gemm_decode(a, w, ops.EPILOGUE_STORE, out_dtype=torch.float32), plain, torch.float32, 2.0)
+    residual = gen(M, N, seed=5).float().to(DEV)
+    before = residual.cpu().double()
+    ops.gemm_decode(a, w, ops.EPILOGUE_ACCUMULATE, accumulate_into=residual, bias=bias.to(DEV))
+    close(residual, before + plain + bias.double(), torch.float32, 2.0)
+    # the same product from the skinny kernel agrees to float32 rounding
+    close(ops.gemm(a, w, out_dtype=torch.float32), plain, torch.float32, 2.0)
+    if N % 2 == 0:
+        half = N // 2
+        close(ops.gemm_decode(a, w, ops.EPILOGUE_SWIGLU), F.silu(plain[:, :half]) * plain[:, half:], torch.bfloat16, 0.4)
+        got = ops.gemm_decode(x.to(DEV), w, ops.EPILOGUE_SWIGLU, norm_weight=norm_w.to(DEV), eps=eps, row_index=index.to(DEV))
+        close(got, F.silu(want[:, :half]) * want[:, half:], torch.bfloat16, 0.4)
+
+
+@pytest.mark.parametrize("M", [1, 7, 16])
+@pytest.mark.parametrize("H,L,with_bias", [(72, 3, False), (136, 4, True), (4096, 2, True)])
+def test_fused_decode_product_with_the_convolution_epilogue(ops, M, H, L, with_bias):
+    K = 256 if H > 1000 else H
+    x = gen(M, K, scale=2).float()
+    norm_w = (1 + 0.1 * gen(K, seed=1)).float()
+    w = as_dev(gen(3 * H, K, seed=2, scale=K ** -0.5), torch.bfloat16)
+    in_bias = gen(3 * H, seed=3).float() if with_bias else None
+    taps = gen(H, L, seed=4).float()
+    conv_bias = gen(H, seed=5).float() if with_bias else None
+    state = gen(M + 2, H, L - 1, seed=6).float()
+    slots = torch.tensor(list(range(M + 1, 1, -1)), dtype=torch.int32)
+    eps = 1e-6
+    h = _kernel_norm(ops, x, norm_w, eps)
+    bcx = h @ back(w).T + (in_bias.double() if with_bias else 0)
+    segments = [(i, 1, int(slots[i])) for i in range(M)]
+    want_out, want_state = conv_reference(bcx, taps.double(), None if conv_bias is None else conv_bias.double(), state.double(), segments)
+    dev_state = state.to(DEV)
+    d = lambda t: None if t is None else t.to(DEV)      # noqa: E731
+    got = ops.gemm_decode(x.to(DEV), w, ops.EPILOGUE_CONV, norm_weight=norm_w.to(DEV), eps=eps, bias=d(in_bias), taps=taps.to(DEV),
+                          conv_bias=d(conv_bias), state=dev_state, seg_slot=slots.to(DEV), out_dtype=torch.bfloat16)
+    close(got, want_out, torch.bfloat16, 0.6)
+    close(dev_state, want_state, torch.float32, 4.0)
+    # and from bfloat16 activations, float32 out
+    a = as_dev(gen(M, K, seed=7), torch.bfloat16)
+    bcx = back(a) @ back(w).T + (in_bias.double() if with_bias else 0)
+    want_out, want_state2 = conv_reference(bcx, taps.double(), None if conv_bias is None else conv_bias.double(), want_state, segments)
+    got = ops.gemm_decode(a, w, ops.EPILOGUE_CONV, bias=d(in_bias), taps=taps.to(DEV), conv_bias=d(conv_bias), state=dev_state,
+                          seg_slot=slots.to(DEV), out_dtype=torch.float32)
+    close(got, want_out, torch.float32, 4.0)
+    close(dev_state, want_state2, torch.float32, 4.0)
+
+
+def test_fused_decode_product_limits(ops):
+    from flyweight_amd.kernels.ops import KernelError
+    assert not ops.gemm_decode_fits(17, 64, 64, ops.EPILOGUE_STORE)
+    assert not ops.gemm_decode_fits(16, 64, 8192, ops.EPILOGUE_STORE)        # 16 rows of 8192 do not fit in LDS
+    assert ops.gemm_decode_fits(8, 64, 8192, ops.EPILOGUE_STORE) and ops.gemm_decode_fits(16, 64, 8192, ops.EPILOGUE_ACCUMULATE)
+    a = torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(KernelError, match="1..16 rows"):
+        ops.gemm_decode(a, torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV), ops.EPILOGUE_STORE)
+    # 16 rows and a long K: the accumulating product reads its activations from global memory instead
+    a = as_dev(gen(16, 8192), torch.bfloat16)
+    w = as_dev(gen(136, 8192, seed=1, scale=0.01), torch.bfloat16)
+    residual = torch.zeros(16, 136, device=DEV)
+    ops.gemm_decode(a, w, ops.EPILOGUE_ACCUMULATE, accumulate_into=residual)
+    close(residual, back(a) @ back(w).T, torch.float32, 2.0)
