@@ -1,22 +1,26 @@
 // Fused matrix products for decode steps of up to 16 rows.
 //
-// A decode step of a small batch is a chain of ~130 short kernels, each of which costs a few
-// microseconds to start and to drain whatever it computes; the weights themselves stream in
-// well under a millisecond. This kernel folds the neighbours of each matrix product into it:
+// A decode step of a small batch is a chain of short kernels, each of which costs a few
+// microseconds to start and to drain whatever it computes, while the weights themselves
+// stream in well under a millisecond. This kernel folds the neighbours of each matrix product
+// into it, without putting anything in front of the stream of W:
 //
-//  prologue   none: a is bfloat16 [M][K];  or RMS norm: a = bf16(x * rsqrt(mean(x^2) + eps) * w)
-//             of float32 rows x (optionally gathered through row_index), computed by the
-//             workgroup itself and kept in LDS (a wave per row, two passes over the row);
-//  product    as the skinny kernel: W streams once from global memory straight into
-//             v_mfma_f32_16x16x32_bf16 operands, K split over the waves of the workgroup, the
-//             first chunk of W requested before the prologue starts; a comes from LDS;
+//  prologue   none: a is bfloat16 [M][K];  or RMS norm of float32 rows x (optionally gathered
+//             through row_index). The norm is not applied before the product: with
+//             h = x * r * w (r the row's 1/rms, w the norm weight) the product is
+//             r * sum_k bf16(x_k w_k) W_nk, so every wave turns its own slices of x into operands
+//             as it goes (rounded to bfloat16 before the scale instead of after it: the same
+//             relative rounding), adds up x^2 of what it reads, and the row's r multiplies the
+//             sums in the epilogue;
+//  product    W streams once from global memory straight into v_mfma_f32_16x16x32_bf16
+//             operands, K split over the waves of the workgroup in chunks of 128;
 //  epilogue   store | add into the float32 residual stream | SwiGLU (tiles: gate, up) |
 //             gated short convolution for single-token segments (tiles: B, C, x of the same
 //             channels; reads and shifts the request's state; see shortconv.hip).
 //
-// A workgroup owns 16 (or 8, so that narrow outputs still fill the chip) features per tile.
-// Partial sums meet in LDS and are added in wave order: results do not depend on timing or on
-// what else is in the batch.
+// A workgroup owns 16 (or 8, so that narrow outputs still fill the chip) features per tile and
+// may take several tiles in turn. Partial sums (and sums of squares) meet in LDS and are added
+// in wave order: results do not depend on timing or on what else is in the batch.
 #include "fw_common.h"
 #include "fw_kernels.h"
 
@@ -25,7 +29,6 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 #define DG_CHUNK 128
-#define DG_PAD 8            // bf16 elements of padding per LDS row of a: consecutive rows shift by four banks
 #define DG_MAX_TAPS 16
 
 enum { DG_STORE = 0, DG_ACCUMULATE = 1, DG_SWIGLU = 2, DG_CONV = 3 };
@@ -55,211 +58,168 @@ __device__ __forceinline__ float dg_silu(float g) {
     return g * e / (1.0f + e);
 }
 
-template <int RT, int WAVES, int ROWS, int PRO, int EPI, bool STAGE, typename TO>
-__global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGemmArgs p) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    float (*partial)[RT][64][4] = reinterpret_cast<float (*)[RT][64][4]>(lds);
-    uint16_t* a_lds = reinterpret_cast<uint16_t*>(lds + sizeof(float) * WAVES * RT * 64 * 4);
+template <int RT, int WAVES, int ROWS, int PRO, int EPI, typename TO>
+__global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGemmArgs p, const int num_tiles) {
+    __shared__ float partial[WAVES][RT][64][4];
+    __shared__ float squares[WAVES][16];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
     const int M = p.M, N = p.N, K = p.K;
-    const int n0 = blockIdx.x * ROWS;
-    const int a_stride = K + DG_PAD;
+    constexpr bool TILED = EPI == DG_SWIGLU || EPI == DG_CONV;    // the tiles of a workgroup are kinds of one feature
 
-    const uint16_t* w_row[RT];
-    bool w_ok[RT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-        const int feature = n0 + (ROWS == 16 ? r16 : (r16 & 7));
-        int n;
-        if (EPI == DG_SWIGLU || EPI == DG_CONV) n = feature + rt * p.tile_stride;
-        else n = feature + rt * ROWS * gridDim.x;      // plain outputs: tile rt covers features [rt * N / RT ...)
-        w_ok[rt] = (EPI == DG_SWIGLU || EPI == DG_CONV) ? feature < N : n < N;
-        w_row[rt] = p.w + (size_t)(w_ok[rt] ? n : 0) * K + g * 8;
-    }
+    const bool a_ok = r16 < M;
+    const int a_index = a_ok ? (PRO == 1 && p.row_index ? p.row_index[r16] : r16) : 0;
+    const uint16_t* a_bf16 = static_cast<const uint16_t*>(p.a) + (size_t)a_index * K + g * 8;
+    const float* a_f32 = static_cast<const float*>(p.a) + (size_t)a_index * K + g * 8;
+    const float* norm_w = p.norm_weight + g * 8;
+    const float one = p.one_centered ? 1.0f : 0.0f;
 
-    auto fetch_w = [&](bf16x8 (&wf)[RT][4], int k0) {
+    for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
+        const uint16_t* w_row[RT];
+        bool w_ok[RT];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int k = k0 + j * 32;
-            const bool ok = k + g * 8 < K;
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-                wf[rt][j] = (ok && w_ok[rt]) ? *reinterpret_cast<const bf16x8*>(w_row[rt] + k) : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        for (int rt = 0; rt < RT; ++rt) {
+            const int feature = tile * ROWS + (ROWS == 16 ? r16 : (r16 & 7));
+            const int n = TILED ? feature + rt * p.tile_stride : feature + rt * ROWS * num_tiles;
+            w_ok[rt] = TILED ? feature < N : n < N;
+            w_row[rt] = p.w + (size_t)(w_ok[rt] ? n : 0) * K + g * 8;
         }
-    };
-
-    // the first chunk of W is on its way while a is prepared
-    bf16x8 w_next[RT][4];
-    int k0 = wave * DG_CHUNK;
-    if (k0 < K) fetch_w(w_next, k0);
-
-    if (STAGE) {
-        if (PRO == 1) {
-            const float* x = static_cast<const float*>(p.a);
-            for (int row = wave; row < M; row += WAVES) {
-                const float* source = x + (size_t)(p.row_index ? p.row_index[row] : row) * K;
-                float sum = 0.0f;
-                for (int k = lane * 8; k < K; k += 512) {
-                    const f32x4 lo = *reinterpret_cast<const f32x4*>(source + k);
-                    const f32x4 hi = *reinterpret_cast<const f32x4*>(source + k + 4);
+        f32x4 acc[RT];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) sum += lo[e] * lo[e] + hi[e] * hi[e];
-                }
-                const float inv = rsqrtf(wave_sum(sum) / (float)K + p.eps);
-                for (int k = lane * 8; k < K; k += 512) {
-                    const f32x4 lo = *reinterpret_cast<const f32x4*>(source + k);
-                    const f32x4 hi = *reinterpret_cast<const f32x4*>(source + k + 4);
-                    const f32x4 wl = *reinterpret_cast<const f32x4*>(p.norm_weight + k);
-                    const f32x4 wh = *reinterpret_cast<const f32x4*>(p.norm_weight + k + 4);
-                    u32x4 packed;
+        for (int rt = 0; rt < RT; ++rt) acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        float square = 0.0f;
+#pragma unroll 2
+        for (int k0 = wave * DG_CHUNK; k0 < K; k0 += WAVES * DG_CHUNK) {
+            bf16x8 wf[RT][4], af[4];
 #pragma unroll
-                    for (int e = 0; e < 2; ++e) {
-                        const float w0 = p.one_centered ? 1.0f + wl[2 * e] : wl[2 * e];
-                        const float w1 = p.one_centered ? 1.0f + wl[2 * e + 1] : wl[2 * e + 1];
-                        const float w2 = p.one_centered ? 1.0f + wh[2 * e] : wh[2 * e];
-                        const float w3 = p.one_centered ? 1.0f + wh[2 * e + 1] : wh[2 * e + 1];
-                        packed[e] = (uint32_t)float_to_bf16_bits(lo[2 * e] * inv * w0) |
-                                    ((uint32_t)float_to_bf16_bits(lo[2 * e + 1] * inv * w1) << 16);
-                        packed[2 + e] = (uint32_t)float_to_bf16_bits(hi[2 * e] * inv * w2) |
-                                        ((uint32_t)float_to_bf16_bits(hi[2 * e + 1] * inv * w3) << 16);
+            for (int j = 0; j < 4; ++j) {
+                const int k = k0 + j * 32;
+                const bool ok = k + g * 8 < K;          // K is a multiple of 8: a run of 8 is in or out as a whole
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    wf[rt][j] = (ok && w_ok[rt]) ? *reinterpret_cast<const bf16x8*>(w_row[rt] + k) : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (PRO == 0) {
+                    af[j] = (ok && a_ok) ? *reinterpret_cast<const bf16x8*>(a_bf16 + k) : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                } else {
+                    u32x4 packed = {0u, 0u, 0u, 0u};
+                    if (ok && a_ok) {
+                        const f32x4 lo = *reinterpret_cast<const f32x4*>(a_f32 + k);
+                        const f32x4 hi = *reinterpret_cast<const f32x4*>(a_f32 + k + 4);
+                        const f32x4 wl = *reinterpret_cast<const f32x4*>(norm_w + k);
+                        const f32x4 wh = *reinterpret_cast<const f32x4*>(norm_w + k + 4);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) square += lo[e] * lo[e] + hi[e] * hi[e];
+#pragma unroll
+                        for (int e = 0; e < 2; ++e) {
+                            packed[e] = (uint32_t)float_to_bf16_bits(lo[2 * e] * (one + wl[2 * e])) |
+                                        ((uint32_t)float_to_bf16_bits(lo[2 * e + 1] * (one + wl[2 * e + 1])) << 16);
+                            packed[2 + e] = (uint32_t)float_to_bf16_bits(hi[2 * e] * (one + wh[2 * e])) |
+                                            ((uint32_t)float_to_bf16_bits(hi[2 * e + 1] * (one + wh[2 * e + 1])) << 16);
+                        }
                     }
-                    *reinterpret_cast<u32x4*>(a_lds + (size_t)row * a_stride + k) = packed;
+                    af[j] = __builtin_bit_cast(bf16x8, packed);
                 }
             }
-        } else {
-            const uint16_t* a = static_cast<const uint16_t*>(p.a);
-            const int chunks = K / 8;
-            for (int index = threadIdx.x; index < M * chunks; index += WAVES * 64) {
-                const int row = index / chunks, kc = index - row * chunks;
-                *reinterpret_cast<u32x4*>(a_lds + (size_t)row * a_stride + kc * 8) =
-                    *reinterpret_cast<const u32x4*>(a + (size_t)row * K + kc * 8);
-            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][j], af[j], acc[rt], 0, 0, 0);
+        }
+
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) partial[wave][rt][lane][r] = acc[rt][r];
+        if (PRO == 1) {
+            // this wave's share of sum x^2 of row r16: over the four k groups
+            square += __shfl_xor(square, 16, 64);
+            square += __shfl_xor(square, 32, 64);
+            if (g == 0) squares[wave][r16] = square;
         }
         __syncthreads();
-    }
 
-    f32x4 acc[RT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const bool a_ok = r16 < M;
-    const uint16_t* a_direct = STAGE ? nullptr : static_cast<const uint16_t*>(p.a) + (size_t)(a_ok ? r16 : 0) * K + g * 8;
-    const uint16_t* a_staged = a_lds + (size_t)(a_ok ? r16 : 0) * a_stride + g * 8;
-    for (; k0 < K; k0 += WAVES * DG_CHUNK) {
-        bf16x8 wf[RT][4];
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) wf[rt][j] = w_next[rt][j];
-        if (k0 + WAVES * DG_CHUNK < K) fetch_w(w_next, k0 + WAVES * DG_CHUNK);
-        bf16x8 af[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int k = k0 + j * 32;
-            const bool ok = a_ok && k + g * 8 < K;
-            if (STAGE) af[j] = ok ? *reinterpret_cast<const bf16x8*>(a_staged + k) : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-            else af[j] = ok ? *reinterpret_cast<const bf16x8*>(a_direct + k) : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        // D layout: lane holds W row 4 * (lane / 16) + r of the tile for row lane % 16 of a.
+        // With 8 features per tile the rows 8..15 repeat rows 0..7 and are dropped.
+        const int m = r16;
+        const bool mine = m < M && !(ROWS == 8 && g >= 2);
+        const int n0 = tile * ROWS;
+        float inv = 1.0f;
+        if (PRO == 1 && mine) {
+            float total = 0.0f;
+            for (int v = 0; v < WAVES; ++v) total += squares[v][m];
+            inv = rsqrtf(total / (float)K + p.eps);
         }
+        if (!TILED) {
+            if (mine) {
+                for (int rt = wave; rt < RT; rt += WAVES) {
+                    float total[4] = {0.f, 0.f, 0.f, 0.f};
+                    for (int v = 0; v < WAVES; ++v)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+                        for (int r = 0; r < 4; ++r) total[r] += partial[v][rt][lane][r];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int n = n0 + g * 4 + r + rt * ROWS * num_tiles;
+                        if (n >= N) continue;
+                        float value = total[r] * inv;
+                        if (p.bias) value += p.bias[n];
+                        TO* out = static_cast<TO*>(p.out);
+                        const size_t at = (size_t)m * N + n;
+                        if (EPI == DG_ACCUMULATE) value += load_as_float(out, at);
+                        store_from_float(out, at, value);
+                    }
+                }
+            }
+        } else if (wave == 0 && mine) {
+            float total[RT][4];
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
-                acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][j], af[j], acc[rt], 0, 0, 0);
-    }
-
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) partial[wave][rt][lane][r] = acc[rt][r];
-    __syncthreads();
-
-    // D layout: lane holds W row 4 * (lane / 16) + r of the tile for row lane % 16 of a.
-    // With 8 features per tile the rows 8..15 repeat rows 0..7 and are dropped.
-    const int m = r16;
-    if (m >= M || (ROWS == 8 && g >= 2)) return;
-    if (EPI == DG_STORE || EPI == DG_ACCUMULATE) {
-        for (int rt = wave; rt < RT; rt += WAVES) {
-            float total[4] = {0.f, 0.f, 0.f, 0.f};
+                for (int r = 0; r < 4; ++r) total[rt][r] = 0.0f;
             for (int v = 0; v < WAVES; ++v)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) total[r] += partial[v][rt][lane][r];
+                for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) total[rt][r] += partial[v][rt][lane][r];
+            TO* out = static_cast<TO*>(p.out);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int n = n0 + g * 4 + r + rt * ROWS * gridDim.x;
+                const int n = n0 + g * 4 + r;
                 if (n >= N) continue;
-                float value = total[r];
-                if (p.bias) value += p.bias[n];
-                TO* out = static_cast<TO*>(p.out);
-                const size_t at = (size_t)m * N + n;
-                if (EPI == DG_ACCUMULATE) value += load_as_float(out, at);
-                store_from_float(out, at, value);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    total[rt][r] *= inv;
+                    if (p.bias) total[rt][r] += p.bias[n + rt * p.tile_stride];
+                }
+                if (EPI == DG_SWIGLU) {
+                    store_from_float(out, (size_t)m * N + n, dg_silu(total[0][r]) * total[RT > 1 ? 1 : 0][r]);
+                } else {        // DG_CONV: tiles are B, C, x of channel n; the row is a segment of one token
+                    const int history = p.kernel_size - 1;
+                    float* channel_state = p.state + ((size_t)p.seg_slot[m] * N + n) * history;
+                    const float* channel_taps = p.taps + (size_t)n * p.kernel_size;
+                    float window[DG_MAX_TAPS];
+                    for (int k = 0; k < history; ++k) window[k] = channel_state[k];
+                    window[history] = total[0][r] * total[RT > 2 ? 2 : 0][r];
+                    float y = 0.0f;
+                    for (int j = 0; j < p.kernel_size; ++j) y = fmaf(channel_taps[j], window[j], y);
+                    if (p.conv_bias) y += p.conv_bias[n];
+                    for (int k = 0; k < history; ++k) channel_state[k] = window[k + 1];
+                    store_from_float(out, (size_t)m * N + n, total[RT > 1 ? 1 : 0][r] * y);
+                }
             }
         }
-        return;
-    }
-    if (wave != 0) return;
-    float total[RT][4];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) total[rt][r] = 0.0f;
-    for (int v = 0; v < WAVES; ++v)
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) total[rt][r] += partial[v][rt][lane][r];
-    TO* out = static_cast<TO*>(p.out);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int n = n0 + g * 4 + r;
-        if (n >= N) continue;
-        if (p.bias) {
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt) total[rt][r] += p.bias[n + rt * p.tile_stride];
-        }
-        if (EPI == DG_SWIGLU) {
-            store_from_float(out, (size_t)m * N + n, dg_silu(total[0][r]) * total[RT > 1 ? 1 : 0][r]);
-        } else {        // DG_CONV: tiles are B, C, x of channel n; the row is a segment of one token
-            const int history = p.kernel_size - 1;
-            float* channel_state = p.state + ((size_t)p.seg_slot[m] * N + n) * history;
-            const float* channel_taps = p.taps + (size_t)n * p.kernel_size;
-            float window[DG_MAX_TAPS];
-            for (int k = 0; k < history; ++k) window[k] = channel_state[k];
-            window[history] = total[0][r] * total[RT > 2 ? 2 : 0][r];
-            float y = 0.0f;
-            for (int j = 0; j < p.kernel_size; ++j) y = fmaf(channel_taps[j], window[j], y);
-            if (p.conv_bias) y += p.conv_bias[n];
-            for (int k = 0; k < history; ++k) channel_state[k] = window[k + 1];
-            store_from_float(out, (size_t)m * N + n, total[RT > 1 ? 1 : 0][r] * y);
-        }
+        if (tile + (int)gridDim.x < num_tiles) __syncthreads();       // the partial sums are free again
     }
 }
 
-template <int RT, int WAVES, int ROWS, int PRO, int EPI, bool STAGE, typename TO>
-static int launch(const DecodeGemmArgs& args, int stage_rows, hipStream_t stream) {
-    const int tiles_features = (EPI == DG_STORE || EPI == DG_ACCUMULATE) ? ROWS * RT : ROWS;
-    const int blocks = fw_ceil_div(args.N, tiles_features);
-    const size_t lds_bytes = sizeof(float) * WAVES * RT * 64 * 4 + (STAGE ? (size_t)stage_rows * (args.K + DG_PAD) * 2 : 0);
-    static size_t configured = 0;       // per instantiation: the largest LDS size asked for so far
-    if (lds_bytes > configured) {
-        hipError_t status = hipFuncSetAttribute((const void*)decode_gemm_kernel<RT, WAVES, ROWS, PRO, EPI, STAGE, TO>,
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (status != hipSuccess) {
-            fw_set_error("gemm_decode: cannot reserve %zu bytes of LDS: %s", lds_bytes, hipGetErrorString(status));
-            return -1;
-        }
-        configured = lds_bytes;
-    }
-    decode_gemm_kernel<RT, WAVES, ROWS, PRO, EPI, STAGE, TO><<<blocks, WAVES * 64, lds_bytes, stream>>>(args);
+#define DG_MAX_BLOCKS 1024
+
+template <int RT, int WAVES, int ROWS, int PRO, int EPI, typename TO>
+static int launch(const DecodeGemmArgs& args, hipStream_t stream) {
+    const int tile_features = (EPI == DG_STORE || EPI == DG_ACCUMULATE) ? ROWS * RT : ROWS;
+    const int num_tiles = fw_ceil_div(args.N, tile_features);
+    const int blocks = num_tiles > DG_MAX_BLOCKS ? DG_MAX_BLOCKS : num_tiles;
+    decode_gemm_kernel<RT, WAVES, ROWS, PRO, EPI, TO><<<blocks, WAVES * 64, 0, stream>>>(args, num_tiles);
     return 0;
-}
-
-#define DG_LDS_LIMIT (150 * 1024)
-
-// How much LDS the staged variant needs; 0 if a cannot be staged (the caller then uses
-// other kernels).
-static size_t staged_bytes(int M, int K, int rt, int waves) {
-    const int rows = M <= 8 ? 8 : 16;
-    return sizeof(float) * waves * rt * 64 * 4 + (size_t)rows * (K + DG_PAD) * 2;
 }
 
 // prologue 0: a bfloat16 [M][K]; 1: RMS norm of float32 rows (norm_weight, eps, one_centered,
@@ -277,52 +237,40 @@ extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_wei
     FW_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemm_decode: unknown epilogue %d", epilogue);
     FW_REQUIRE(prologue == 0 || (norm_weight != nullptr && eps > 0.0f), "gemm_decode: the norm prologue needs its weight and eps");
     FW_REQUIRE(epilogue != DG_ACCUMULATE || out_dtype == FW_F32, "gemm_decode: accumulation needs a float32 destination");
+    FW_REQUIRE(epilogue != DG_ACCUMULATE || prologue == 0, "gemm_decode: the accumulating product takes bfloat16 activations");
     FW_REQUIRE(epilogue != DG_SWIGLU || out_dtype == FW_BF16, "gemm_decode: SwiGLU stores bfloat16");
     FW_REQUIRE(out_dtype == FW_F32 || out_dtype == FW_BF16, "gemm_decode: unknown out dtype %d", out_dtype);
     FW_REQUIRE(epilogue != DG_CONV || (taps && state && seg_slot && kernel_size >= 2 && kernel_size <= DG_MAX_TAPS),
                "gemm_decode: the convolution epilogue needs taps, state, slots and a kernel size in 2..%d", DG_MAX_TAPS);
-    FW_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_decode: operands must be 16-byte aligned");
+    FW_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)norm_weight % 16 == 0),
+               "gemm_decode: operands must be 16-byte aligned");
     DecodeGemmArgs args;
     args.a = a; args.norm_weight = norm_weight; args.row_index = row_index; args.eps = eps; args.one_centered = one_centered;
     args.w = (const uint16_t*)w; args.bias = bias; args.out = out; args.M = M; args.N = N; args.K = K;
     args.tile_stride = (epilogue == DG_SWIGLU || epilogue == DG_CONV) ? N : 0;
     args.taps = taps; args.conv_bias = conv_bias; args.state = state; args.seg_slot = seg_slot; args.kernel_size = kernel_size;
     hipStream_t s = (hipStream_t)stream;
-    const int stage_rows = M <= 8 ? 8 : 16;
     const bool narrow = N < 256 * 16;       // fewer than one 16-feature tile per compute unit: use 8-feature tiles
     int status = -2;
-#define DG_TRY(RT, WAVES, ROWS, PRO, EPI, STAGE, TO) \
-    status = launch<RT, WAVES, ROWS, PRO, EPI, STAGE, TO>(args, stage_rows, s)
+#define DG_TRY(RT, WAVES, ROWS, PRO, EPI, TO) status = launch<RT, WAVES, ROWS, PRO, EPI, TO>(args, s)
     if (epilogue == DG_ACCUMULATE) {
-        FW_REQUIRE(prologue == 0, "gemm_decode: the accumulating product takes bfloat16 activations");
-        const int waves = K >= 4096 ? 16 : 8;
-        const bool stage = staged_bytes(M, K, 1, waves) <= DG_LDS_LIMIT;
-        if (waves == 16) {
-            if (narrow) { if (stage) DG_TRY(1, 16, 8, 0, DG_ACCUMULATE, true, float); else DG_TRY(1, 16, 8, 0, DG_ACCUMULATE, false, float); }
-            else { if (stage) DG_TRY(1, 16, 16, 0, DG_ACCUMULATE, true, float); else DG_TRY(1, 16, 16, 0, DG_ACCUMULATE, false, float); }
-        } else {
-            if (narrow) { if (stage) DG_TRY(1, 8, 8, 0, DG_ACCUMULATE, true, float); else DG_TRY(1, 8, 8, 0, DG_ACCUMULATE, false, float); }
-            else { if (stage) DG_TRY(1, 8, 16, 0, DG_ACCUMULATE, true, float); else DG_TRY(1, 8, 16, 0, DG_ACCUMULATE, false, float); }
-        }
-    } else {
-        const int rt = epilogue == DG_SWIGLU ? 2 : epilogue == DG_CONV ? 3 : (N >= 16384 ? 2 : 1);
-        FW_REQUIRE(staged_bytes(M, K, rt, 8) <= DG_LDS_LIMIT, "gemm_decode: %d rows of K = %d do not fit in LDS", M, K);
-        if (epilogue == DG_STORE) {
+        if (K >= 4096) { if (narrow) DG_TRY(1, 16, 8, 0, DG_ACCUMULATE, float); else DG_TRY(1, 16, 16, 0, DG_ACCUMULATE, float); }
+        else { if (narrow) DG_TRY(1, 8, 8, 0, DG_ACCUMULATE, float); else DG_TRY(1, 8, 16, 0, DG_ACCUMULATE, float); }
+    } else if (epilogue == DG_STORE) {
 #define DG_STORE_CASE(RT, ROWS)                                                                     \
-    if (prologue == 1) { if (out_dtype == FW_F32) DG_TRY(RT, 8, ROWS, 1, DG_STORE, true, float); else DG_TRY(RT, 8, ROWS, 1, DG_STORE, true, bf16_t); } \
-    else { if (out_dtype == FW_F32) DG_TRY(RT, 8, ROWS, 0, DG_STORE, true, float); else DG_TRY(RT, 8, ROWS, 0, DG_STORE, true, bf16_t); }
-            if (rt == 2) { DG_STORE_CASE(2, 16) } else if (narrow) { DG_STORE_CASE(1, 8) } else { DG_STORE_CASE(1, 16) }
+    if (prologue == 1) { if (out_dtype == FW_F32) DG_TRY(RT, 8, ROWS, 1, DG_STORE, float); else DG_TRY(RT, 8, ROWS, 1, DG_STORE, bf16_t); } \
+    else { if (out_dtype == FW_F32) DG_TRY(RT, 8, ROWS, 0, DG_STORE, float); else DG_TRY(RT, 8, ROWS, 0, DG_STORE, bf16_t); }
+        if (N >= 16384) { DG_STORE_CASE(2, 16) } else if (narrow) { DG_STORE_CASE(1, 8) } else { DG_STORE_CASE(1, 16) }
 #undef DG_STORE_CASE
-        } else if (epilogue == DG_SWIGLU) {
-            if (prologue == 1) { if (narrow) DG_TRY(2, 8, 8, 1, DG_SWIGLU, true, bf16_t); else DG_TRY(2, 8, 16, 1, DG_SWIGLU, true, bf16_t); }
-            else { if (narrow) DG_TRY(2, 8, 8, 0, DG_SWIGLU, true, bf16_t); else DG_TRY(2, 8, 16, 0, DG_SWIGLU, true, bf16_t); }
-        } else {
+    } else if (epilogue == DG_SWIGLU) {
+        if (prologue == 1) { if (narrow) DG_TRY(2, 8, 8, 1, DG_SWIGLU, bf16_t); else DG_TRY(2, 8, 16, 1, DG_SWIGLU, bf16_t); }
+        else { if (narrow) DG_TRY(2, 8, 8, 0, DG_SWIGLU, bf16_t); else DG_TRY(2, 8, 16, 0, DG_SWIGLU, bf16_t); }
+    } else {
 #define DG_CONV_CASE(ROWS)                                                                          \
-    if (prologue == 1) { if (out_dtype == FW_F32) DG_TRY(3, 8, ROWS, 1, DG_CONV, true, float); else DG_TRY(3, 8, ROWS, 1, DG_CONV, true, bf16_t); } \
-    else { if (out_dtype == FW_F32) DG_TRY(3, 8, ROWS, 0, DG_CONV, true, float); else DG_TRY(3, 8, ROWS, 0, DG_CONV, true, bf16_t); }
-            if (narrow) { DG_CONV_CASE(8) } else { DG_CONV_CASE(16) }
+    if (prologue == 1) { if (out_dtype == FW_F32) DG_TRY(3, 8, ROWS, 1, DG_CONV, float); else DG_TRY(3, 8, ROWS, 1, DG_CONV, bf16_t); } \
+    else { if (out_dtype == FW_F32) DG_TRY(3, 8, ROWS, 0, DG_CONV, float); else DG_TRY(3, 8, ROWS, 0, DG_CONV, bf16_t); }
+        if (narrow) { DG_CONV_CASE(8) } else { DG_CONV_CASE(16) }
 #undef DG_CONV_CASE
-        }
     }
 #undef DG_TRY
     if (status != 0) return -1;
@@ -332,8 +280,6 @@ extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_wei
 
 // Whether fw_gemm_decode takes this shape (the caller falls back to separate kernels if not).
 extern "C" int fw_gemm_decode_fits(int M, int N, int K, int epilogue) {
-    if (M < 1 || M > 16 || K <= 0 || K % 8 != 0 || N <= 0) return 0;
-    if (epilogue == DG_ACCUMULATE) return 1;
-    const int rt = epilogue == DG_SWIGLU ? 2 : epilogue == DG_CONV ? 3 : (N >= 16384 ? 2 : 1);
-    return staged_bytes(M, K, rt, 8) <= DG_LDS_LIMIT ? 1 : 0;
+    (void)epilogue;
+    return (M >= 1 && M <= 16 && K > 0 && K % 8 == 0 && N > 0) ? 1 : 0;
 }

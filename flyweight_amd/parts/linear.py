@@ -22,6 +22,8 @@ Input = Union[torch.Tensor, LazyNorm]
 
 
 class Linear:
+    WIDE = 32768
+
     def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor] = None):
         if weight.dim() != 2:
             raise ValueError("a linear weight is [out, in]")
@@ -36,8 +38,8 @@ class Linear:
         rows = a.rows if isinstance(a, LazyNorm) else a.shape[0]
         if not 1 <= rows <= ops.DECODE_MAX_ROWS:
             return False
-        if isinstance(a, LazyNorm) and a.rms_parameters() is None:
-            return False
+        if isinstance(a, LazyNorm) and (a.rms_parameters() is None or features >= self.WIDE):
+            return False        # very wide outputs (a vocabulary): norming once beats norming in every workgroup
         return ops.gemm_decode_fits(rows, features, self.in_features, epilogue)
 
     @staticmethod

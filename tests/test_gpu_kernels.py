@@ -495,10 +495,11 @@ def _normed(x, weight, eps, one_centered=False):
 
 
 def _kernel_norm(ops, x, norm_w, eps, index=None, one_centered=False):
-    """The normed rows exactly as the fused kernel rounds them to bfloat16: its product with an
-    identity matrix (exact). They are checked against the float64 norm to one rounding; the
-    products are then checked against THESE rows, so that a value the kernel's float32 norm
-    rounds the other way than float64 would does not pass for an error of the product."""
+    """The normed rows exactly as the fused kernel forms them (x * w rounded to bfloat16, times
+    the row's 1/rms): its product with an identity matrix. They are checked against the float64
+    norm to one bfloat16 rounding; the products are then checked against THESE rows, so that a
+    value the kernel rounds the other way than float64 would does not pass for an error of the
+    product."""
     K = x.shape[1]
     identity = torch.eye(K, dtype=torch.bfloat16, device=DEV)
     h = ops.gemm_decode(x.to(DEV), identity, ops.EPILOGUE_STORE, norm_weight=norm_w.to(DEV), eps=eps, one_centered=one_centered,
@@ -585,13 +586,12 @@ def test_fused_decode_product_with_the_convolution_epilogue(ops, M, H, L, with_b
 
 def test_fused_decode_product_limits(ops):
     from flyweight_amd.kernels.ops import KernelError
-    assert not ops.gemm_decode_fits(17, 64, 64, ops.EPILOGUE_STORE)
-    assert not ops.gemm_decode_fits(16, 64, 8192, ops.EPILOGUE_STORE)        # 16 rows of 8192 do not fit in LDS
-    assert ops.gemm_decode_fits(8, 64, 8192, ops.EPILOGUE_STORE) and ops.gemm_decode_fits(16, 64, 8192, ops.EPILOGUE_ACCUMULATE)
+    assert not ops.gemm_decode_fits(17, 64, 64, ops.EPILOGUE_STORE) and not ops.gemm_decode_fits(4, 64, 68, ops.EPILOGUE_STORE)
+    assert ops.gemm_decode_fits(16, 64, 8192, ops.EPILOGUE_STORE) and ops.gemm_decode_fits(1, 64, 8, ops.EPILOGUE_ACCUMULATE)
     a = torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(KernelError, match="1..16 rows"):
         ops.gemm_decode(a, torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV), ops.EPILOGUE_STORE)
-    # 16 rows and a long K: the accumulating product reads its activations from global memory instead
+    # 16 rows and a long K
     a = as_dev(gen(16, 8192), torch.bfloat16)
     w = as_dev(gen(136, 8192, seed=1, scale=0.01), torch.bfloat16)
     residual = torch.zeros(16, 136, device=DEV)
