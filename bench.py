@@ -127,6 +127,7 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=16)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
+    parser.add_argument("--only", choices=("decode", "prefill"), help="run one phase and print no JSON (for profiling)")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for {args.gpus})", flush=True)
@@ -146,8 +147,15 @@ def main() -> int:
     kv_per_token = len(config.full_attn_idxs) * 2 * config.num_key_value_heads * config.head_dim * 2
     state_per_request = (config.num_hidden_layers - len(config.full_attn_idxs)) * config.hidden_size * (config.conv_L_cache - 1) * 4
 
+    if args.only == "decode":
+        elapsed, _ = decode_run(torch, model, config, args.batch, args.steps, args.warmup)
+        log(f"{args.batch * args.steps / elapsed:.1f} tokens/s")
+        return 0
     log("prefill of 2,048 tokens")
     prefill_s = prefill_run(torch, model, config)
+    if args.only == "prefill":
+        log(f"{PROMPT / prefill_s:.1f} tokens/s")
+        return 0
     head_flops = 2 * config.vocab_size * config.hidden_size
     attention_flops = len(config.full_attn_idxs) * 2 * config.num_attention_heads * config.head_dim * PROMPT * PROMPT
     prefill_flops = 2 * matmul_params(config) * PROMPT + head_flops + attention_flops
