@@ -1,8 +1,8 @@
 // Attention over the paged cache on the matrix cores (bfloat16 cache, float32 softmax).
 //
 // One wave works on 16 "columns" against the keys of one kv head. For a prompt portion a
-// column is a query row (16 consecutive rows of one segment, one head per wave, the heads of
-// a kv group side by side in a workgroup so that they find the same pages in L1). For decode
+// column is a query row (16 consecutive rows of one segment and one head per wave, four such
+// waves per workgroup sharing the pages through LDS). For decode
 // a column is one of the query heads that share the kv head, and the keys are split between
 // workgroups in runs of SPLIT_PAGES pages whose partial results (running maximum, sum and
 // unnormalised output) a second kernel merges in order.
@@ -50,22 +50,22 @@ struct Columns {
 template <int HD>
 __device__ __forceinline__ void attend_page(Columns<HD>& c, const uint16_t* __restrict__ k_page,
                                             const uint16_t* __restrict__ v_page, int head_dim, float scale_log2,
-                                            int lo, int hi, int last_written) {
+                                            int lo, int hi, int last_written, int k_stride, int v_stride) {
     const int lane = threadIdx.x & 63;
     const int i16 = lane & 15, g = lane >> 4;
-    // all loads of the page are issued before the first product (for heads up to 64 channels
-    // the values too: they do not depend on the scores)
+    // all key loads of the page are issued before the first product; with the 64-channel
+    // instantiation (the measured case) the values too: they do not depend on the scores
     bf16x8 kf[4][HD / 32];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
-        const uint16_t* key = k_page + (size_t)(kt * 16 + i16) * head_dim + g * 8;
+        const uint16_t* key = k_page + (size_t)(kt * 16 + i16) * k_stride + g * 8;
 #pragma unroll
         for (int dc = 0; dc < HD / 32; ++dc) {
             kf[kt][dc] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
             if (dc * 32 + g * 8 < head_dim) kf[kt][dc] = *reinterpret_cast<const bf16x8*>(key + dc * 32);
         }
     }
-    constexpr bool EARLY_V = HD <= 64;
+    constexpr bool EARLY_V = HD == 64;
     u32x2 vearly[EARLY_V ? 2 : 1][EARLY_V ? HD / 16 : 1][2];
     if (EARLY_V) {
 #pragma unroll
@@ -73,7 +73,7 @@ __device__ __forceinline__ void attend_page(Columns<HD>& c, const uint16_t* __re
 #pragma unroll
             for (int t = 0; t < HD / 16; ++t) {
                 if (t * 16 >= head_dim) break;
-                const uint16_t* value = v_page + (size_t)(t * 16 + i16) * PAGE + kb * 32 + g * 4;
+                const uint16_t* value = v_page + (size_t)(t * 16 + i16) * v_stride + kb * 32 + g * 4;
                 vearly[kb][t][0] = *reinterpret_cast<const u32x2*>(value);
                 vearly[kb][t][1] = *reinterpret_cast<const u32x2*>(value + 16);
             }
@@ -133,7 +133,7 @@ __device__ __forceinline__ void attend_page(Columns<HD>& c, const uint16_t* __re
                 va = vearly[kb][t][0];
                 vb = vearly[kb][t][1];
             } else {
-                const uint16_t* value = v_page + (size_t)(t * 16 + i16) * PAGE;
+                const uint16_t* value = v_page + (size_t)(t * 16 + i16) * v_stride;
                 va = *reinterpret_cast<const u32x2*>(value + key_a);
                 vb = *reinterpret_cast<const u32x2*>(value + key_b);
             }
@@ -168,26 +168,37 @@ __device__ __forceinline__ void load_query(Columns<HD>& c, const uint16_t* __res
 }
 
 // ---- prompt portions ---------------------------------------------------------------------------
-// grid (query tiles, kv heads); one wave per query head of the group. tile_seg / tile_row0:
-// the segment of each tile of 16 rows and its first row (a tile never spans two segments).
+// grid (tiles of 64 query rows, heads); four waves, 16 rows each, all of one head. The pages of
+// the kv head are copied global -> registers -> LDS one page ahead of the one being worked on
+// (two LDS buffers, one barrier per page), so that the copy hides behind the softmax
+// arithmetic. tile_seg / tile_row0: the segment of each tile and its first row (a tile never
+// spans two segments). LDS rows are padded by 16 bytes against bank conflicts.
+#define KV_PAD 8
 template <int HD>
-__global__ void attention_prefill_kernel(
+__global__ __launch_bounds__(256) void attention_prefill_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ tile_seg, const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ seg_row0,
     const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, float scale_log2, int window) {
-    const int tile = blockIdx.x, kvh = blockIdx.y;
-    const int group = num_heads / num_kv_heads;
-    const int head = kvh * group + (threadIdx.x >> 6);
-    const int lane = threadIdx.x & 63, col = lane & 15, g = lane >> 4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    const int k_stride = head_dim + KV_PAD, v_stride = PAGE + KV_PAD;
+    const int k_elems = PAGE * k_stride, v_elems = head_dim * v_stride;
+    uint16_t* lds = reinterpret_cast<uint16_t*>(lds_raw);      // [buffer][K tile | V tile]
+
+    const int tile = blockIdx.x, head = blockIdx.y;
+    const int kvh = head / (num_heads / num_kv_heads);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, g = lane >> 4;
     const int seg = tile_seg[tile];
-    const int row0 = tile_row0[tile];
+    const int tile_first_row = tile_row0[tile];
     const int seg_end = seg_row0[seg + 1];
-    const int rows = seg_end - row0 < 16 ? seg_end - row0 : 16;
+    const int tile_rows = seg_end - tile_first_row < 64 ? seg_end - tile_first_row : 64;
+    const int row0 = tile_first_row + wave * 16;                        // this wave's rows
+    const int rows = tile_rows - wave * 16 < 16 ? tile_rows - wave * 16 : 16;     // may be <= 0
     const bool valid = col < rows;
-    const int my_row = row0 + (valid ? col : 0);
+    const int my_row = valid ? row0 + col : tile_first_row;
     const int my_pos = row_pos[my_row];
-    const int pos_lo = row_pos[row0], pos_hi = row_pos[row0 + rows - 1];
+    const int wave_hi = rows > 0 ? row_pos[row0 + rows - 1] : -1;       // last position of this wave
+    const int pos_lo = row_pos[tile_first_row], pos_hi = row_pos[tile_first_row + tile_rows - 1];
     const int my_first = window > 0 && my_pos - window + 1 > 0 ? my_pos - window + 1 : 0;
     const int tile_first = window > 0 && pos_lo - window + 1 > 0 ? pos_lo - window + 1 : 0;
 
@@ -195,13 +206,51 @@ __global__ void attention_prefill_kernel(
     load_query<HD>(c, q + ((size_t)my_row * num_heads + head) * head_dim, head_dim, valid);
     const int32_t* table = block_table + (size_t)seg * table_stride;
     const size_t page_elems = (size_t)PAGE * head_dim;
-    for (int block = tile_first / PAGE; block <= pos_hi / PAGE; ++block) {
-        const int page = table[block];
-        const size_t at = ((size_t)page * num_kv_heads + kvh) * page_elems;
+
+    // the copy: a page's K is 64 rows of head_dim, its V head_dim rows of 64; runs of 16 bytes
+    const int k_runs = PAGE * head_dim / 8, v_runs = head_dim * PAGE / 8;        // equal
+    constexpr int MAX_RUNS = HD * PAGE / 8 / 256;                                // per thread, per operand
+    u32x4 hold_k[MAX_RUNS], hold_v[MAX_RUNS];
+    auto fetch = [&](int block) {
+        const size_t at = ((size_t)table[block] * num_kv_heads + kvh) * page_elems;
+#pragma unroll
+        for (int u = 0; u < MAX_RUNS; ++u) {
+            const int run = tid + u * 256;
+            if (run < k_runs) {
+                hold_k[u] = *reinterpret_cast<const u32x4*>(k_pages + at + (size_t)run * 8);
+                hold_v[u] = *reinterpret_cast<const u32x4*>(v_pages + at + (size_t)run * 8);
+            }
+        }
+    };
+    auto stash = [&](int buffer) {
+        uint16_t* kt = lds + (size_t)buffer * (k_elems + v_elems);
+        uint16_t* vt = kt + k_elems;
+        const int k_per_row = head_dim / 8;
+#pragma unroll
+        for (int u = 0; u < MAX_RUNS; ++u) {
+            const int run = tid + u * 256;
+            if (run < k_runs) {
+                *reinterpret_cast<u32x4*>(kt + (run / k_per_row) * k_stride + (run % k_per_row) * 8) = hold_k[u];
+                *reinterpret_cast<u32x4*>(vt + (run / 8) * v_stride + (run % 8) * 8) = hold_v[u];
+            }
+        }
+    };
+
+    const int first_block = tile_first / PAGE, last_block = pos_hi / PAGE;
+    fetch(first_block);
+    stash(0);
+    __syncthreads();
+    for (int block = first_block; block <= last_block; ++block) {
+        const int buffer = (block - first_block) & 1;
+        if (block < last_block) fetch(block + 1);
         const int base = block * PAGE;
-        const int lo = valid ? my_first - base : PAGE;
-        const int hi = valid ? my_pos - base : -1;
-        attend_page<HD>(c, k_pages + at, v_pages + at, head_dim, scale_log2, lo, hi, pos_hi - base);
+        if (rows > 0 && base <= wave_hi) {      // a wave whose rows all lie before this page has nothing to add
+            const uint16_t* kt = lds + (size_t)buffer * (k_elems + v_elems);
+            attend_page<HD>(c, kt, kt + k_elems, head_dim, scale_log2, valid ? my_first - base : PAGE,
+                            valid ? my_pos - base : -1, pos_hi - base, k_stride, v_stride);
+        }
+        if (block < last_block) stash(buffer ^ 1);
+        __syncthreads();
     }
     float l = c.l;
     l += __shfl_xor(l, 16, 64);
@@ -253,7 +302,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) void attention_decode_split_kerne
         const size_t at = ((size_t)page * num_kv_heads + kvh) * PAGE * head_dim;
         const int base = block * PAGE;
         attend_page<HD>(c, k_pages + at, v_pages + at, head_dim, scale_log2, valid ? first - base : PAGE,
-                        valid ? pos - base : -1, pos - base);
+                        valid ? pos - base : -1, pos - base, head_dim, PAGE);
     }
     float l = c.l;
     l += __shfl_xor(l, 16, 64);
@@ -344,22 +393,32 @@ static int check_common(const char* name, int rows, int num_heads, int num_kv_he
         else { CALL(256); }                 \
     } while (0)
 
-// bfloat16 q [rows][heads * head_dim] -> out (same shape). tile_seg / tile_row0 [tiles].
+// bfloat16 q [rows][heads * head_dim] -> out (same shape). tile_seg / tile_row0 [tiles]: tiles of
+// up to 64 rows that never span two segments.
 extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_pages, const void* v_pages,
                                     const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                                     const int32_t* tile_row0, int tiles, const int32_t* seg_row0,
                                     const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim,
                                     float scale, int window, int page_size, int num_pages, void* stream) {
     if (check_common("attention_prefill", rows, num_heads, num_kv_heads, head_dim, page_size, window, num_pages, table_stride)) return -1;
-    FW_REQUIRE(num_heads / num_kv_heads <= 16, "attention_prefill: at most 16 query heads per kv head, got %d", num_heads / num_kv_heads);
-    FW_REQUIRE(tiles >= 0 && tiles <= rows && num_kv_heads <= 65535, "attention_prefill: %d tiles for %d rows", tiles, rows);
+    FW_REQUIRE(tiles >= 0 && tiles <= rows && num_heads <= 65535, "attention_prefill: %d tiles for %d rows", tiles, rows);
     if (rows == 0 || tiles == 0) return 0;
-    dim3 grid(tiles, num_kv_heads);
-    const int threads = 64 * (num_heads / num_kv_heads);
+    dim3 grid(tiles, num_heads);
+    const int lds_bytes = 2 * (PAGE * (head_dim + KV_PAD) + head_dim * (PAGE + KV_PAD)) * 2;
 #define CALL(HD)                                                                                                   \
-    attention_prefill_kernel<HD><<<grid, threads, 0, (hipStream_t)stream>>>(                                        \
-        (const uint16_t*)q, (uint16_t*)out, (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table,        \
-        table_stride, tile_seg, tile_row0, seg_row0, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window)
+    {                                                                                                              \
+        static int configured = 0;                                                                                 \
+        if (lds_bytes > configured) {                                                                              \
+            hipError_t status = hipFuncSetAttribute((const void*)attention_prefill_kernel<HD>,                     \
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);        \
+            FW_REQUIRE(status == hipSuccess, "attention_prefill: cannot reserve %d bytes of LDS", lds_bytes);      \
+            configured = lds_bytes;                                                                                \
+        }                                                                                                          \
+        attention_prefill_kernel<HD><<<grid, 256, lds_bytes, (hipStream_t)stream>>>(                                \
+            (const uint16_t*)q, (uint16_t*)out, (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table,    \
+            table_stride, tile_seg, tile_row0, seg_row0, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, \
+            window);                                                                                               \
+    }
     FW_BY_HEAD_DIM(head_dim, CALL);
 #undef CALL
     FW_LAUNCH_CHECK("attention_prefill");

@@ -87,8 +87,8 @@ int fw_attention_generic(const void* q, void* out, int dtype, const void* k_page
                          int num_pages, void* stream);
 
 // The same attention on the matrix cores, bfloat16 only, head_dim a multiple of 16 up to 256.
-// Prompt portions: rows are cut into tiles of 16 that never span two segments (tile_seg,
-// tile_row0); at most 16 query heads per kv head.
+// Prompt portions: rows are cut into tiles of up to 64 that never span two segments (tile_seg,
+// tile_row0).
 int fw_attention_prefill(const void* q, void* out, const void* k_pages, const void* v_pages,
                          const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                          const int32_t* tile_row0, int tiles, const int32_t* seg_row0, const int32_t* row_pos,

@@ -84,7 +84,7 @@ class StepContext:
         self.host_seg_row0 = seg_row0
         self.host_seg_slot = seg_slot
 
-        tile_seg, tile_row0 = ops.query_tiles(seg_row0)        # tiles of 16 rows for the prompt attention kernel
+        tile_seg, tile_row0 = ops.query_tiles(seg_row0)        # tiles of up to 64 rows for the prompt attention kernel
         tables = [cache.block_table_rows(g, self.requests) for g in range(len(cache.groups))]
         pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows,
                                                           tile_seg, tile_row0)]

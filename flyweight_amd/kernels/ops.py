@@ -422,12 +422,15 @@ def gemm_decode(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
 DECODE_SPLIT_PAGES = 4
 
 
+QUERY_TILE = 64
+
+
 def query_tiles(seg_row0):
-    """Cuts the rows of each segment into tiles of 16 that never span two segments:
+    """Cuts the rows of each segment into tiles of up to 64 that never span two segments:
     (segment of each tile, first row of each tile), as lists."""
     tile_seg, tile_row0 = [], []
     for seg in range(len(seg_row0) - 1):
-        for row in range(seg_row0[seg], seg_row0[seg + 1], 16):
+        for row in range(seg_row0[seg], seg_row0[seg + 1], QUERY_TILE):
             tile_seg.append(seg)
             tile_row0.append(row)
     return tile_seg, tile_row0
@@ -495,7 +498,7 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
     if fast and ctx.all_decode:
         return attention_decode(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                                 ctx.row_pos, scale, ctx.max_context, window)
-    if fast and num_heads // num_kv_heads <= 16:
+    if fast:
         return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.tile_seg,
                                  ctx.tile_row0, ctx.seg_row0, ctx.row_pos, scale, window)
     return attention_generic(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
