@@ -3,8 +3,8 @@
 //
 // A workgroup of four waves computes a 128 x 128 tile; each wave a 64 x 64 quarter as 2 x 2
 // MFMA tiles. Both operands are k-contiguous, so a 128 x 64 slab of each is copied per
-// iteration: global -> registers (requested before the multiply of the current slab) -> LDS
-// (after it), two LDS buffers, one barrier per iteration. LDS rows are padded from 128 to
+// iteration: global -> registers (requested two slabs ahead of the one being multiplied) ->
+// LDS (one slab ahead), two LDS buffers, one barrier per iteration. LDS rows are padded from 128 to
 // 144 bytes so that the 16-byte operand reads of 16 consecutive rows fall into different
 // banks. Workgroups are numbered so that each XCD (every eighth workgroup id) works on a
 // compact group of tiles and finds its operands in its own L2.
@@ -91,15 +91,26 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    // the next slab is on its way from global memory while the current one is multiplied
-    u32x4 ra0[4], rw0[W_CHUNKS];
+    // Two slabs are on their way from global memory while a third is multiplied: what limits
+    // this kernel is the latency of those loads times the bytes in flight per compute unit.
+    // The two register sets are named apart (not indexed) so that they stay in registers.
+    u32x4 ra0[4], rw0[W_CHUNKS], ra1[4], rw1[W_CHUNKS];
     const u32x4 zero = {0u, 0u, 0u, 0u};
     auto fetch = [&](u32x4 (&ra)[4], u32x4 (&rw)[W_CHUNKS], int k0) {
+        // Every load is issued unconditionally (past the end of K from column 0, then dropped):
+        // a branch around a load would make the compiler wait for ALL loads at the next wait.
         const bool ok = k0 + kc < K;                    // K is a multiple of 8
+        const int from = ok ? k0 : 0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ra[i] = ok ? *reinterpret_cast<const u32x4*>(a_src[i] + k0) : zero;
+        for (int i = 0; i < 4; ++i) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(a_src[i] + from);
+            ra[i] = ok ? v : zero;
+        }
 #pragma unroll
-        for (int i = 0; i < W_CHUNKS; ++i) rw[i] = ok ? *reinterpret_cast<const u32x4*>(w_src[i] + k0) : zero;
+        for (int i = 0; i < W_CHUNKS; ++i) {
+            const u32x4 v = *reinterpret_cast<const u32x4*>(w_src[i] + from);
+            rw[i] = ok ? v : zero;
+        }
     };
     auto stash = [&](const u32x4 (&ra)[4], const u32x4 (&rw)[W_CHUNKS], int buffer) {
         unsigned char* base = lds + buffer * (A_SLAB + W_SLAB);
@@ -136,16 +147,38 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
         }
     };
 
+    // slab s travels: global -> register set s % 2 (requested while slab s - 2 is multiplied)
+    // -> LDS buffer s % 2 (stored while slab s - 1 is multiplied) -> multiplied. The steady
+    // state has no branches, so the compiler can count exactly which loads it must wait for.
     const int steps = (K + TK - 1) / TK;
+    int step = 0;
     fetch(ra0, rw0, 0);
+    fetch(ra1, rw1, TK);                                // past the end: zeros
     stash(ra0, rw0, 0);
     __syncthreads();
-    for (int step = 0; step < steps; ++step) {
-        const int buffer = step & 1;
-        if (step + 1 < steps) fetch(ra0, rw0, (step + 1) * TK);
-        multiply(buffer);
-        if (step + 1 < steps) stash(ra0, rw0, buffer ^ 1);
+    while (step + 3 < steps) {
+        fetch(ra0, rw0, (step + 2) * TK);
+        multiply(0);
+        stash(ra1, rw1, 1);
         __syncthreads();
+        fetch(ra1, rw1, (step + 3) * TK);
+        multiply(1);
+        stash(ra0, rw0, 0);
+        __syncthreads();
+        step += 2;
+    }
+    // at most three slabs are left: slab `step` is in buffer 0, slab step + 1 in set 1
+    if (step + 2 < steps) fetch(ra0, rw0, (step + 2) * TK);
+    multiply(0);
+    if (step + 1 < steps) {
+        stash(ra1, rw1, 1);
+        __syncthreads();
+        multiply(1);
+        if (step + 2 < steps) {
+            stash(ra0, rw0, 0);
+            __syncthreads();
+            multiply(0);
+        }
     }
 
     // D layout of the 32x32 product: lane holds column lane % 32; register r is row
