@@ -44,11 +44,18 @@ int fw_gemm_mfma(const void* a, const void* w, const float* bias, void* out, int
 // up rows], out bfloat16 [M][N]; 3: gated short convolution of single-token segments, w = [B rows;
 // C rows; x rows] of N channels each, state [slots][N][kernel_size - 1] read and shifted.
 // fw_gemm_decode_fits says whether a shape is taken (1) or must go to separate kernels (0).
+// The accumulating epilogue can also leave what the NEXT norm needs: next_activations bfloat16
+// [M][N] = x_new * w_next and next_squares [fw_gemm_decode_accumulate_tiles(N)][16], per-tile sums
+// of x_new^2 of every row. A later call takes them with prologue 2 (a = those activations,
+// squares/squares_tiles = those sums, eps) and applies the row's scale in its epilogue.
 int fw_gemm_decode(int prologue, const void* a, const float* norm_weight, const int32_t* row_index, float eps,
                    int one_centered, const void* w, const float* bias, void* out, int out_dtype, int epilogue,
                    int M, int N, int K, const float* taps, const float* conv_bias, float* state,
-                   const int32_t* seg_slot, int kernel_size, void* stream);
+                   const int32_t* seg_slot, int kernel_size, const float* next_norm_weight,
+                   int next_one_centered, void* next_activations, float* next_squares, const float* squares,
+                   int squares_tiles, void* stream);
 int fw_gemm_decode_fits(int M, int N, int K, int epilogue);
+int fw_gemm_decode_accumulate_tiles(int N);
 
 // out[r][i] = silu(gu[r][i]) * gu[r][I + i]; the input may be float32 beside a bfloat16 output
 int fw_swiglu(const void* gate_up, int in_dtype, void* out, int out_dtype, int rows, int intermediate,

@@ -12,9 +12,14 @@
 //             as it goes (rounded to bfloat16 before the scale instead of after it: the same
 //             relative rounding), adds up x^2 of what it reads, and the row's r multiplies the
 //             sums in the epilogue;
+//             or "pre-normed": the kernel that last added to the residual stream (the
+//             accumulating epilogue below) also left bf16(x * w_next) and, per tile of features,
+//             the sum of x^2 of every row; this kernel reads those as plain bfloat16 activations
+//             and forms the row's r from the partial sums, so the norm costs almost nothing;
 //  product    W streams once from global memory straight into v_mfma_f32_16x16x32_bf16
 //             operands, K split over the waves of the workgroup in chunks of 128;
-//  epilogue   store | add into the float32 residual stream | SwiGLU (tiles: gate, up) |
+//  epilogue   store | add into the float32 residual stream (optionally leaving the pre-normed
+//             activations for the next norm, see above) | SwiGLU (tiles: gate, up) |
 //             gated short convolution for single-token segments (tiles: B, C, x of the same
 //             channels; reads and shifts the request's state; see shortconv.hip).
 //
@@ -50,6 +55,14 @@ struct DecodeGemmArgs {
     float* state;               // [slots][N][kernel_size - 1]
     const int32_t* seg_slot;    // [M]
     int kernel_size;
+    // accumulating epilogue: what the next norm will need (all null: nothing is left)
+    const float* next_norm_weight;  // [N]
+    int next_one_centered;
+    uint16_t* next_activations;     // bfloat16 [M][N] = x_new * (w_next or 1 + w_next)
+    float* next_squares;            // [tiles][16]: sum over the tile's features of x_new^2 per row
+    // pre-normed prologue
+    const float* squares;           // [squares_tiles][16], left by the kernel above
+    int squares_tiles;
 };
 
 __device__ __forceinline__ float dg_silu(float g) {
@@ -67,12 +80,27 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
     constexpr bool TILED = EPI == DG_SWIGLU || EPI == DG_CONV;    // the tiles of a workgroup are kinds of one feature
 
     const bool a_ok = r16 < M;
-    const int a_index = a_ok ? (PRO == 1 && p.row_index ? p.row_index[r16] : r16) : 0;
+    const int a_index = a_ok ? (PRO == 1 && p.row_index ? p.row_index[r16] : r16) : 0;     // (pre-normed rows are never gathered)
     const uint16_t* a_bf16 = static_cast<const uint16_t*>(p.a) + (size_t)a_index * K + g * 8;
     const float* a_f32 = static_cast<const float*>(p.a) + (size_t)a_index * K + g * 8;
     const float* norm_w = p.norm_weight + g * 8;
     const float one = p.one_centered ? 1.0f : 0.0f;
 
+    float prepared_square = 0.0f;
+    if (PRO == 2 && r16 < M) {
+        // This lane's share of the partial sums of x^2 that the rows' producer left: the waves
+        // and the four lanes of a row split the tiles in a fixed order, four loads in flight;
+        // the shares meet in the epilogue like the norm prologue's own.
+        const float* from = p.squares + r16;
+        float part[4] = {0.f, 0.f, 0.f, 0.f};
+        int t = wave * 4 + g;
+        const int step = WAVES * 4;
+        for (; t + 3 * step < p.squares_tiles; t += 4 * step)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) part[u] += from[(size_t)(t + u * step) * 16];
+        for (; t < p.squares_tiles; t += step) part[0] += from[(size_t)t * 16];
+        prepared_square = (part[0] + part[1]) + (part[2] + part[3]);
+    }
     for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
         const uint16_t* w_row[RT];
         bool w_ok[RT];
@@ -92,29 +120,36 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
             bf16x8 wf[RT][4], af[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
+                // Every load is issued unconditionally (a run past the end of K, or of a row that
+                // does not exist, is read from a valid place and dropped): a branch around a load
+                // would make the compiler wait for all loads in flight at the next wait.
                 const int k = k0 + j * 32;
                 const bool ok = k + g * 8 < K;          // K is a multiple of 8: a run of 8 is in or out as a whole
+                const int from = ok ? k : 0;
+                const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
-                    wf[rt][j] = (ok && w_ok[rt]) ? *reinterpret_cast<const bf16x8*>(w_row[rt] + k) : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-                if (PRO == 0) {
-                    af[j] = (ok && a_ok) ? *reinterpret_cast<const bf16x8*>(a_bf16 + k) : bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                for (int rt = 0; rt < RT; ++rt) {
+                    const bf16x8 v = *reinterpret_cast<const bf16x8*>(w_row[rt] + from);
+                    wf[rt][j] = (ok && w_ok[rt]) ? v : none;
+                }
+                if (PRO != 1) {
+                    const bf16x8 v = *reinterpret_cast<const bf16x8*>(a_bf16 + from);
+                    af[j] = (ok && a_ok) ? v : none;
                 } else {
-                    u32x4 packed = {0u, 0u, 0u, 0u};
-                    if (ok && a_ok) {
-                        const f32x4 lo = *reinterpret_cast<const f32x4*>(a_f32 + k);
-                        const f32x4 hi = *reinterpret_cast<const f32x4*>(a_f32 + k + 4);
-                        const f32x4 wl = *reinterpret_cast<const f32x4*>(norm_w + k);
-                        const f32x4 wh = *reinterpret_cast<const f32x4*>(norm_w + k + 4);
+                    const f32x4 lo = *reinterpret_cast<const f32x4*>(a_f32 + from);
+                    const f32x4 hi = *reinterpret_cast<const f32x4*>(a_f32 + from + 4);
+                    const f32x4 wl = *reinterpret_cast<const f32x4*>(norm_w + from);
+                    const f32x4 wh = *reinterpret_cast<const f32x4*>(norm_w + from + 4);
+                    const float keep = (ok && a_ok) ? 1.0f : 0.0f;
+                    u32x4 packed;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) square += lo[e] * lo[e] + hi[e] * hi[e];
+                    for (int e = 0; e < 4; ++e) square += keep * (lo[e] * lo[e] + hi[e] * hi[e]);
 #pragma unroll
-                        for (int e = 0; e < 2; ++e) {
-                            packed[e] = (uint32_t)float_to_bf16_bits(lo[2 * e] * (one + wl[2 * e])) |
-                                        ((uint32_t)float_to_bf16_bits(lo[2 * e + 1] * (one + wl[2 * e + 1])) << 16);
-                            packed[2 + e] = (uint32_t)float_to_bf16_bits(hi[2 * e] * (one + wh[2 * e])) |
-                                            ((uint32_t)float_to_bf16_bits(hi[2 * e + 1] * (one + wh[2 * e + 1])) << 16);
-                        }
+                    for (int e = 0; e < 2; ++e) {
+                        packed[e] = (uint32_t)float_to_bf16_bits(keep * lo[2 * e] * (one + wl[2 * e])) |
+                                    ((uint32_t)float_to_bf16_bits(keep * lo[2 * e + 1] * (one + wl[2 * e + 1])) << 16);
+                        packed[2 + e] = (uint32_t)float_to_bf16_bits(keep * hi[2 * e] * (one + wh[2 * e])) |
+                                        ((uint32_t)float_to_bf16_bits(keep * hi[2 * e + 1] * (one + wh[2 * e + 1])) << 16);
                     }
                     af[j] = __builtin_bit_cast(bf16x8, packed);
                 }
@@ -130,7 +165,8 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) partial[wave][rt][lane][r] = acc[rt][r];
-        if (PRO == 1) {
+        if (PRO == 2) square = prepared_square;
+        if (PRO != 0) {
             // this wave's share of sum x^2 of row r16: over the four k groups
             square += __shfl_xor(square, 16, 64);
             square += __shfl_xor(square, 32, 64);
@@ -144,29 +180,38 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
         const bool mine = m < M && !(ROWS == 8 && g >= 2);
         const int n0 = tile * ROWS;
         float inv = 1.0f;
-        if (PRO == 1 && mine) {
+        if (PRO != 0 && mine) {
             float total = 0.0f;
             for (int v = 0; v < WAVES; ++v) total += squares[v][m];
             inv = rsqrtf(total / (float)K + p.eps);
         }
         if (!TILED) {
-            if (mine) {
-                for (int rt = wave; rt < RT; rt += WAVES) {
-                    float total[4] = {0.f, 0.f, 0.f, 0.f};
-                    for (int v = 0; v < WAVES; ++v)
+            for (int rt = wave; rt < RT; rt += WAVES) {
+                float total[4] = {0.f, 0.f, 0.f, 0.f};
+                for (int v = 0; v < WAVES; ++v)
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) total[r] += partial[v][rt][lane][r];
+                    for (int r = 0; r < 4; ++r) total[r] += partial[v][rt][lane][r];
+                float row_square = 0.0f;
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int n = n0 + g * 4 + r + rt * ROWS * num_tiles;
-                        if (n >= N) continue;
-                        float value = total[r] * inv;
-                        if (p.bias) value += p.bias[n];
-                        TO* out = static_cast<TO*>(p.out);
-                        const size_t at = (size_t)m * N + n;
-                        if (EPI == DG_ACCUMULATE) value += load_as_float(out, at);
-                        store_from_float(out, at, value);
+                for (int r = 0; r < 4; ++r) {
+                    const int n = n0 + g * 4 + r + rt * ROWS * num_tiles;
+                    if (!mine || n >= N) continue;
+                    float value = total[r] * inv;
+                    if (p.bias) value += p.bias[n];
+                    TO* out = static_cast<TO*>(p.out);
+                    const size_t at = (size_t)m * N + n;
+                    if (EPI == DG_ACCUMULATE) value += load_as_float(out, at);
+                    store_from_float(out, at, value);
+                    if (EPI == DG_ACCUMULATE && p.next_activations) {
+                        const float w = p.next_norm_weight[n] + (p.next_one_centered ? 1.0f : 0.0f);
+                        p.next_activations[at] = float_to_bf16_bits(value * w);
+                        row_square += value * value;
                     }
+                }
+                if (EPI == DG_ACCUMULATE && p.next_squares) {       // RT is 1 here: wave 0, every lane
+                    row_square += __shfl_xor(row_square, 16, 64);
+                    row_square += __shfl_xor(row_square, 32, 64);
+                    if (g == 0) p.next_squares[(size_t)tile * 16 + m] = m < M ? row_square : 0.0f;
                 }
             }
         } else if (wave == 0 && mine) {
@@ -223,19 +268,25 @@ static int launch(const DecodeGemmArgs& args, hipStream_t stream) {
 }
 
 // prologue 0: a bfloat16 [M][K]; 1: RMS norm of float32 rows (norm_weight, eps, one_centered,
-// optional row_index). epilogue 0: store out_dtype [M][N]; 1: float32 out += ; 2: SwiGLU, w =
+// optional row_index); 2: a bfloat16 [M][K] = x * w left by an accumulating call together with
+// `squares` [squares_tiles][16], the row's scale is formed from those. epilogue 0: store out_dtype [M][N]; 1: float32 out += ; 2: SwiGLU, w =
 // [gate rows; up rows], out bfloat16 [M][N]; 3: gated short convolution, w = [B rows; C rows; x
 // rows] of N channels each, out_dtype [M][N], state updated.
 extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_weight, const int32_t* row_index,
                               float eps, int one_centered, const void* w, const float* bias, void* out,
                               int out_dtype, int epilogue, int M, int N, int K, const float* taps,
                               const float* conv_bias, float* state, const int32_t* seg_slot, int kernel_size,
-                              void* stream) {
+                              const float* next_norm_weight, int next_one_centered, void* next_activations,
+                              float* next_squares, const float* squares, int squares_tiles, void* stream) {
     FW_REQUIRE(M >= 1 && M <= 16, "gemm_decode: takes 1..16 rows, got %d", M);
     FW_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_decode: K (%d) must be a positive multiple of 8, N (%d) positive", K, N);
-    FW_REQUIRE(prologue == 0 || prologue == 1, "gemm_decode: unknown prologue %d", prologue);
+    FW_REQUIRE(prologue >= 0 && prologue <= 2, "gemm_decode: unknown prologue %d", prologue);
+    FW_REQUIRE(prologue != 2 || (squares != nullptr && squares_tiles >= 1 && eps > 0.0f), "gemm_decode: the pre-normed prologue needs the partial sums of squares and eps");
+    FW_REQUIRE((next_activations == nullptr) == (next_squares == nullptr) && (next_activations == nullptr) == (next_norm_weight == nullptr),
+               "gemm_decode: the next norm's weight, activations and sums of squares come together");
+    FW_REQUIRE(next_activations == nullptr || epilogue == DG_ACCUMULATE, "gemm_decode: only the accumulating product prepares the next norm");
     FW_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemm_decode: unknown epilogue %d", epilogue);
-    FW_REQUIRE(prologue == 0 || (norm_weight != nullptr && eps > 0.0f), "gemm_decode: the norm prologue needs its weight and eps");
+    FW_REQUIRE(prologue != 1 || (norm_weight != nullptr && eps > 0.0f), "gemm_decode: the norm prologue needs its weight and eps");
     FW_REQUIRE(epilogue != DG_ACCUMULATE || out_dtype == FW_F32, "gemm_decode: accumulation needs a float32 destination");
     FW_REQUIRE(epilogue != DG_ACCUMULATE || prologue == 0, "gemm_decode: the accumulating product takes bfloat16 activations");
     FW_REQUIRE(epilogue != DG_SWIGLU || out_dtype == FW_BF16, "gemm_decode: SwiGLU stores bfloat16");
@@ -249,6 +300,9 @@ extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_wei
     args.w = (const uint16_t*)w; args.bias = bias; args.out = out; args.M = M; args.N = N; args.K = K;
     args.tile_stride = (epilogue == DG_SWIGLU || epilogue == DG_CONV) ? N : 0;
     args.taps = taps; args.conv_bias = conv_bias; args.state = state; args.seg_slot = seg_slot; args.kernel_size = kernel_size;
+    args.next_norm_weight = next_norm_weight; args.next_one_centered = next_one_centered;
+    args.next_activations = (uint16_t*)next_activations; args.next_squares = next_squares;
+    args.squares = squares; args.squares_tiles = squares_tiles;
     hipStream_t s = (hipStream_t)stream;
     const bool narrow = N < 256 * 16;       // fewer than one 16-feature tile per compute unit: use 8-feature tiles
     int status = -2;
@@ -259,15 +313,18 @@ extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_wei
     } else if (epilogue == DG_STORE) {
 #define DG_STORE_CASE(RT, ROWS)                                                                     \
     if (prologue == 1) { if (out_dtype == FW_F32) DG_TRY(RT, 8, ROWS, 1, DG_STORE, float); else DG_TRY(RT, 8, ROWS, 1, DG_STORE, bf16_t); } \
+    else if (prologue == 2) { if (out_dtype == FW_F32) DG_TRY(RT, 8, ROWS, 2, DG_STORE, float); else DG_TRY(RT, 8, ROWS, 2, DG_STORE, bf16_t); } \
     else { if (out_dtype == FW_F32) DG_TRY(RT, 8, ROWS, 0, DG_STORE, float); else DG_TRY(RT, 8, ROWS, 0, DG_STORE, bf16_t); }
         if (N >= 16384) { DG_STORE_CASE(2, 16) } else if (narrow) { DG_STORE_CASE(1, 8) } else { DG_STORE_CASE(1, 16) }
 #undef DG_STORE_CASE
     } else if (epilogue == DG_SWIGLU) {
         if (prologue == 1) { if (narrow) DG_TRY(2, 8, 8, 1, DG_SWIGLU, bf16_t); else DG_TRY(2, 8, 16, 1, DG_SWIGLU, bf16_t); }
+        else if (prologue == 2) { if (narrow) DG_TRY(2, 8, 8, 2, DG_SWIGLU, bf16_t); else DG_TRY(2, 8, 16, 2, DG_SWIGLU, bf16_t); }
         else { if (narrow) DG_TRY(2, 8, 8, 0, DG_SWIGLU, bf16_t); else DG_TRY(2, 8, 16, 0, DG_SWIGLU, bf16_t); }
     } else {
 #define DG_CONV_CASE(ROWS)                                                                          \
     if (prologue == 1) { if (out_dtype == FW_F32) DG_TRY(3, 8, ROWS, 1, DG_CONV, float); else DG_TRY(3, 8, ROWS, 1, DG_CONV, bf16_t); } \
+    else if (prologue == 2) { if (out_dtype == FW_F32) DG_TRY(3, 8, ROWS, 2, DG_CONV, float); else DG_TRY(3, 8, ROWS, 2, DG_CONV, bf16_t); } \
     else { if (out_dtype == FW_F32) DG_TRY(3, 8, ROWS, 0, DG_CONV, float); else DG_TRY(3, 8, ROWS, 0, DG_CONV, bf16_t); }
         if (narrow) { DG_CONV_CASE(8) } else { DG_CONV_CASE(16) }
 #undef DG_CONV_CASE
@@ -276,6 +333,13 @@ extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_wei
     if (status != 0) return -1;
     FW_LAUNCH_CHECK("gemm_decode");
     return 0;
+}
+
+// How many tiles of features the accumulating product of this shape uses (the first extent of
+// the sums of squares it leaves for the next norm).
+extern "C" int fw_gemm_decode_accumulate_tiles(int N) {
+    const bool narrow = N < 256 * 16;
+    return fw_ceil_div(N, narrow ? 8 : 16);
 }
 
 // Whether fw_gemm_decode takes this shape (the caller falls back to separate kernels if not).

@@ -97,8 +97,14 @@ class CausalLM:
         """Runs the rows of ``ctx`` through every scheduled layer; returns float32 logits
         [wanted, vocab] for ``ctx.want_rows`` (None when nothing is wanted)."""
         x = ops.embed_rows(self.embedding, ctx.token_ids)
-        for entry in self.spec.schedule:
+        schedule = self.spec.schedule
+        ctx.prepared = None
+        for at, entry in enumerate(schedule):
+            # the norm that reads the residual after this layer, for the layer's last product
+            following = self.layers[schedule[at + 1].layer] if at + 1 < len(schedule) else None
+            ctx.norm_after_block = getattr(following, "mixer_norm", None)
             self.layers[entry.layer].forward(x, ctx, ctx.cache_view(cache, entry))
+        ctx.prepared = ctx.norm_after_block = None
         if ctx.num_wanted == 0:
             return None
         return self.head.forward(LazyNorm(self.final_norm, x, ctx, row_index=ctx.want_rows), out_dtype=torch.float32)

@@ -370,13 +370,20 @@ def gemm_decode(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
                 row_index: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
                 accumulate_into: Optional[torch.Tensor] = None, taps: Optional[torch.Tensor] = None,
                 conv_bias: Optional[torch.Tensor] = None, state: Optional[torch.Tensor] = None,
-                seg_slot: Optional[torch.Tensor] = None) -> torch.Tensor:
+                seg_slot: Optional[torch.Tensor] = None, squares: Optional[torch.Tensor] = None,
+                next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False):
     """One kernel for (optional RMS norm of float32 rows) -> product with bfloat16 ``w`` -> epilogue.
     With ``norm_weight`` ``a`` holds float32 rows (gathered through ``row_index`` if given), else
-    bfloat16 activations. See fw_gemm_decode in fw_kernels.h for the epilogues."""
-    _dev(a, w, bias, norm_weight, row_index, accumulate_into, taps, conv_bias, state, seg_slot)
+    bfloat16 activations. With ``next_norm_weight`` the accumulating epilogue also leaves what
+    the norm after it needs, and the call returns (activations x * w_next, sums of squares);
+    a later call takes those as ``a`` and ``squares`` (with ``eps``) and skips the norm's
+    arithmetic. See fw_gemm_decode in fw_kernels.h for the epilogues."""
+    _dev(a, w, bias, norm_weight, row_index, accumulate_into, taps, conv_bias, state, seg_slot, squares, next_norm_weight)
     _want(w, torch.bfloat16, "w")
     normed = norm_weight is not None
+    if squares is not None and (normed or squares.dtype != torch.float32 or squares.dim() != 2 or squares.shape[1] != 16
+                                or not squares.is_contiguous()):
+        raise KernelError("gemm_decode: sums of squares are float32 [tiles, 16] and replace the norm")
     rows = row_index.numel() if (normed and row_index is not None) else a.shape[0]
     K = a.shape[1]
     tiles = {EPILOGUE_SWIGLU: 2, EPILOGUE_CONV: 3}.get(epilogue, 1)
@@ -412,10 +419,20 @@ def gemm_decode(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
     else:
         out_dtype = out_dtype or torch.bfloat16
         target = torch.empty((rows, N), dtype=out_dtype, device=a.device)
+    next_activations = next_squares = None
+    if next_norm_weight is not None:
+        if epilogue != EPILOGUE_ACCUMULATE or next_norm_weight.dtype != torch.float32 or next_norm_weight.shape != (N,):
+            raise KernelError("gemm_decode: only the accumulating product prepares the next norm, whose weight is float32 [N]")
+        next_activations = torch.empty((rows, N), dtype=torch.bfloat16, device=a.device)
+        next_squares = torch.empty((library().fw_gemm_decode_accumulate_tiles(N), 16), dtype=torch.float32, device=a.device)
+    prologue = 1 if normed else (2 if squares is not None else 0)
     _check(library().fw_gemm_decode(
-        int(normed), _p(a), _p(norm_weight), _p(row_index), ctypes.c_float(eps), int(one_centered), _p(w), _p(bias),
+        prologue, _p(a), _p(norm_weight), _p(row_index), ctypes.c_float(eps), int(one_centered), _p(w), _p(bias),
         _p(target), _code(out_dtype), int(epilogue), rows, N, K, _p(taps), _p(conv_bias), _p(state), _p(seg_slot),
-        int(kernel_size), _stream()))
+        int(kernel_size), _p(next_norm_weight), int(next_one_centered), _p(next_activations), _p(next_squares),
+        _p(squares), 0 if squares is None else squares.shape[0], _stream()))
+    if next_norm_weight is not None:
+        return next_activations, next_squares
     return target
 
 

@@ -86,7 +86,7 @@ class GQAttention(Mixer):
         self.q_norm_weight = tensors[self._name("q_norm")] if self.qk_norm else None
         self.k_norm_weight = tensors[self._name("k_norm")] if self.qk_norm else None
 
-    def forward(self, h, residual, ctx, cache) -> None:
+    def forward(self, h, residual, ctx, cache):
         qkv = self.qkv.forward(h, out_dtype=torch.float32)      # normed, rotated and rounded once, below
         cos, sin = ctx.position_tables(self.position)
         q = ops.qk_norm_rope_kv_write(
@@ -95,4 +95,4 @@ class GQAttention(Mixer):
             ctx.row_seg, ctx.row_pos, write_kv=cache.writes)
         attended = ops.attention(q, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
                                  cache.block_table, ctx, self.scale, int(self.window or 0))
-        self.out.accumulate(attended, residual)
+        return self.out.accumulate(attended, residual, then=getattr(ctx, "upcoming_norm", None))

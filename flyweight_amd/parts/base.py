@@ -66,12 +66,16 @@ class Mixer(Part):
     def cache_need(self):
         return None
 
-    def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx, cache) -> None:
+    def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx, cache):
+        """Adds the mixer's output to ``residual`` in place. May return what its last product
+        prepared for ``ctx.upcoming_norm`` (``Linear.accumulate(..., then=...)``); returning
+        None is always right."""
         raise NotImplementedError
 
 
 class FeedForward(Part):
-    def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx) -> None:
+    def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx):
+        """Adds to ``residual`` in place; the return value is as for a mixer."""
         raise NotImplementedError
 
 

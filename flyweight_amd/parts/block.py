@@ -46,8 +46,13 @@ class PreNormResidualBlock:
 
     def forward(self, x, ctx, cache) -> None:
         """``x`` [rows, hidden] float32 is updated in place."""
-        # a part that can take the norm into its own first kernel gets it unevaluated
-        h = LazyNorm(self.mixer_norm, x, ctx)
-        self.mixer.forward(h if getattr(self.mixer, "accepts_lazy_norm", False) else h.tensor(), x, ctx, cache)
-        h = LazyNorm(self.ffn_norm, x, ctx)
-        self.ffn.forward(h if getattr(self.ffn, "accepts_lazy_norm", False) else h.tensor(), x, ctx)
+        # A part that can take the norm into its own first kernel gets it unevaluated. A part is
+        # told which norm reads the residual after it (ctx.upcoming_norm) and may return what its
+        # last product prepared for that norm; a part that returns nothing costs a plain norm.
+        h = LazyNorm(self.mixer_norm, x, ctx, prepared=getattr(ctx, "prepared", None))
+        ctx.upcoming_norm = self.ffn_norm
+        prepared = self.mixer.forward(h if getattr(self.mixer, "accepts_lazy_norm", False) else h.tensor(), x, ctx, cache)
+        h = LazyNorm(self.ffn_norm, x, ctx, prepared=prepared)
+        ctx.upcoming_norm = getattr(ctx, "norm_after_block", None)
+        ctx.prepared = self.ffn.forward(h if getattr(self.ffn, "accepts_lazy_norm", False) else h.tensor(), x, ctx)
+        ctx.upcoming_norm = None

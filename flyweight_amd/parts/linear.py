@@ -5,7 +5,8 @@ stream in the kernel's epilogue, so the residual sum never leaves float32; ``swi
 ``short_conv`` finish the product with that part's arithmetic. Which kernel runs is chosen
 here from the operand types and the number of rows: for up to 16 rows of a bfloat16 model one
 fused kernel takes the RMS norm before the product (handed over as a :class:`LazyNorm`) and
-the epilogue after it; otherwise the norm runs on its own and the skinny, tiled or generic
+the epilogue after it, and the product that adds to the residual stream prepares the norm
+that follows; otherwise the norm runs on its own and the skinny, tiled or generic
 product follows.
 """
 
@@ -16,7 +17,7 @@ from typing import Optional, Union
 import torch
 
 from ..kernels import ops
-from .norm import LazyNorm
+from .norm import LazyNorm, Prepared
 
 Input = Union[torch.Tensor, LazyNorm]
 
@@ -47,11 +48,15 @@ class Linear:
         if not isinstance(a, LazyNorm):
             return {}
         weight, eps, one_centered = a.rms_parameters()
+        if a.prepared is not None:
+            return {"squares": a.prepared.squares, "eps": eps}
         return {"norm_weight": weight, "eps": eps, "one_centered": one_centered, "row_index": a.row_index}
 
     @staticmethod
     def _rows_of(a: Input) -> torch.Tensor:
-        return a.x if isinstance(a, LazyNorm) else a
+        if not isinstance(a, LazyNorm):
+            return a
+        return a.prepared.activations if a.prepared is not None else a.x
 
     @staticmethod
     def _tensor_of(a: Input) -> torch.Tensor:
@@ -65,11 +70,21 @@ class Linear:
                                    **self._norm_arguments(a))
         return ops.gemm(self._tensor_of(a), self.weight, self.bias, out_dtype=out_dtype)
 
-    def accumulate(self, a: torch.Tensor, residual: torch.Tensor) -> None:
+    def accumulate(self, a: torch.Tensor, residual: torch.Tensor, then=None) -> Optional[Prepared]:
+        """residual += a . W^T. ``then`` names the norm that will read the residual next, if the
+        caller knows it and this is the last change before it: the fused kernel then leaves that
+        norm's work behind (returned; None when it did not)."""
         if self._fused(a, self.out_features, ops.EPILOGUE_ACCUMULATE):
+            parameters = then.rms_parameters() if hasattr(then, "rms_parameters") else None
+            if parameters is not None and parameters[0].shape == (self.out_features,) and then.dtype == torch.bfloat16:
+                activations, squares = ops.gemm_decode(
+                    a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias, accumulate_into=residual,
+                    next_norm_weight=parameters[0], next_one_centered=parameters[2])
+                return Prepared(then, activations, squares)
             ops.gemm_decode(a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias, accumulate_into=residual)
-            return
+            return None
         ops.gemm(a, self.weight, self.bias, accumulate_into=residual)
+        return None
 
     def swiglu(self, a: Input) -> torch.Tensor:
         """The weight holds gate rows then up rows: silu(a . gate^T) * (a . up^T)."""

@@ -12,13 +12,28 @@ from ..weights.loader import TensorDecl
 from .base import Norm, register_norm
 
 
+class Prepared:
+    """What the product that last added to the residual stream left for the norm after it:
+    ``activations`` bfloat16 [rows, size] = x * w of that norm and ``squares`` [tiles, 16],
+    partial sums of x^2 per row, from which a product's kernel forms the row's 1/rms itself."""
+
+    def __init__(self, norm: Norm, activations: torch.Tensor, squares: torch.Tensor):
+        self.norm, self.activations, self.squares = norm, activations, squares
+
+
 class LazyNorm:
     """A norm that has not run yet: the rows ``x`` (optionally gathered through ``row_index``)
     and the norm to apply. A product that can apply an RMS norm in its own kernel takes it as
-    it is (``rms_parameters``); anything else calls ``tensor()``, which runs the norm once."""
+    it is (``rms_parameters``, or ``prepared`` when the rows' producer already did most of it);
+    anything else calls ``tensor()``, which runs the norm once."""
 
-    def __init__(self, norm: Norm, x: torch.Tensor, ctx, row_index: Optional[torch.Tensor] = None):
+    def __init__(self, norm: Norm, x: torch.Tensor, ctx, row_index: Optional[torch.Tensor] = None,
+                 prepared: Optional[Prepared] = None):
         self.norm, self.x, self.ctx, self.row_index = norm, x, ctx, row_index
+        # only what was made for this very norm and these rows counts
+        ok = prepared is not None and prepared.norm is norm and row_index is None \
+            and prepared.activations.shape == x.shape
+        self.prepared = prepared if ok else None
         self._tensor = None
 
     @property

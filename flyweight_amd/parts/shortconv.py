@@ -59,13 +59,12 @@ class ShortConv(Mixer):
         self.taps = tensors[p + "conv.weight"].reshape(self.hidden, self.kernel_size).contiguous()
         self.conv_bias = tensors[p + "conv.bias"] if self.bias else None
 
-    def forward(self, h, residual, ctx, cache) -> None:
+    def forward(self, h, residual, ctx, cache):
         if ctx.all_decode:      # single-token segments: norm, in_proj, convolution and state shift in one kernel
             gated = self.in_proj.short_conv_decode(h, self.taps, self.conv_bias, cache.state, ctx.seg_slot, self.dtype)
             if gated is not None:
-                self.out_proj.accumulate(gated, residual)
-                return
+                return self.out_proj.accumulate(gated, residual, then=getattr(ctx, "upcoming_norm", None))
         bcx = self.in_proj.forward(h, out_dtype=torch.float32)  # B * x and the taps' sum stay in float32
         gated = ops.shortconv(bcx, self.taps, self.conv_bias, cache.state, ctx.row_seg, ctx.seg_row0, ctx.seg_slot,
                               ctx.num_segments, out_dtype=self.dtype)
-        self.out_proj.accumulate(gated, residual)
+        return self.out_proj.accumulate(gated, residual, then=getattr(ctx, "upcoming_norm", None))

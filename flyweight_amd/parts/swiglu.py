@@ -46,6 +46,6 @@ class SwiGLU(FeedForward):
         self.gate_up = Linear(torch.cat([gate, up], dim=0))
         self.down = Linear(tensors[self._name("down")])
 
-    def forward(self, h, residual, ctx) -> None:
+    def forward(self, h, residual, ctx):
         # the activation is formed from float32 sums and rounded once
-        self.down.accumulate(self.gate_up.swiglu(h), residual)
+        return self.down.accumulate(self.gate_up.swiglu(h), residual, then=getattr(ctx, "upcoming_norm", None))

@@ -584,6 +584,55 @@ def test_fused_decode_product_with_the_convolution_epilogue(ops, M, H, L, with_b
     close(dev_state, want_state2, torch.float32, 4.0)
 
 
+@pytest.mark.parametrize("M", [1, 6, 16])
+@pytest.mark.parametrize("H,N,one_centered", [(72, 80, False), (200, 96, True), (4104, 144, False), (2048, 6144, True)])
+def test_fused_decode_product_prepares_the_next_norm(ops, M, H, N, one_centered):
+    """The product that adds to the residual stream leaves x * w of the norm after it and sums
+    of squares per tile; the next product takes both instead of norming itself. Checked: what
+    is left, and the next product (every epilogue that may follow) against a plain norm."""
+    K = 136
+    a = as_dev(gen(M, K, seed=1), torch.bfloat16)
+    w_out = as_dev(gen(H, K, seed=2, scale=K ** -0.5), torch.bfloat16)
+    residual = gen(M, H, seed=3, scale=2).float().to(DEV)
+    norm_w = (0.1 * gen(H, seed=4) + (0 if one_centered else 1)).float()
+    eps = 1e-5
+    x_new = residual.cpu().double() + back(a) @ back(w_out).T
+    activations, squares = ops.gemm_decode(a, w_out, ops.EPILOGUE_ACCUMULATE, accumulate_into=residual,
+                                           next_norm_weight=norm_w.to(DEV), next_one_centered=one_centered)
+    close(residual, x_new, torch.float32, 2.0)
+    x_kernel = residual.cpu().double()               # the float32 values the kernel squared and scaled
+    scale = norm_w.double() + (1 if one_centered else 0)
+    assert activations.dtype == torch.bfloat16 and squares.shape[1] == 16
+    assert torch.equal(activations.cpu(), (x_kernel.float() * scale.float()).to(torch.bfloat16))
+    total = squares.cpu().double().sum(0)
+    assert float((total[:M] - (x_kernel ** 2).sum(-1)).abs().max()) <= 1e-5 * float((x_kernel ** 2).sum(-1).max())
+    assert float(total[M:].abs().max()) == 0.0 if M < 16 else True
+    # the following product: rows as the kernel forms them are activations * 1/rms
+    inv = 1.0 / torch.sqrt((x_kernel ** 2).mean(-1, keepdim=True) + eps)
+    h = activations.cpu().double() * inv
+    w = as_dev(gen(N, H, seed=5, scale=H ** -0.5), torch.bfloat16)
+    want = h @ back(w).T
+    got = ops.gemm_decode(activations, w, ops.EPILOGUE_STORE, squares=squares, eps=eps, out_dtype=torch.float32)
+    close(got, want, torch.float32, 2.0)
+    fused = ops.gemm_decode(residual, w, ops.EPILOGUE_STORE, norm_weight=norm_w.to(DEV), eps=eps, one_centered=one_centered,
+                            out_dtype=torch.float32)
+    close(got, fused.cpu().double(), torch.float32, 2.0)        # the norm done in the product's own prologue agrees
+    half = N // 2
+    got = ops.gemm_decode(activations, w, ops.EPILOGUE_SWIGLU, squares=squares, eps=eps)
+    close(got, F.silu(want[:, :half]) * want[:, half:], torch.bfloat16, 0.4)
+    if N % 3 == 0:
+        C, L = N // 3, 3
+        taps, state = gen(C, L, seed=6).float(), gen(M, C, L - 1, seed=7).float()
+        slots = torch.arange(M - 1, -1, -1, dtype=torch.int32)
+        segments = [(i, 1, int(slots[i])) for i in range(M)]
+        want_out, want_state = conv_reference(want, taps.double(), None, state.double(), segments)
+        dev_state = state.to(DEV)
+        got = ops.gemm_decode(activations, w, ops.EPILOGUE_CONV, squares=squares, eps=eps, taps=taps.to(DEV), state=dev_state,
+                              seg_slot=slots.to(DEV), out_dtype=torch.float32)
+        close(got, want_out, torch.float32, 4.0)
+        close(dev_state, want_state, torch.float32, 4.0)
+
+
 def test_fused_decode_product_limits(ops):
     from flyweight_amd.kernels.ops import KernelError
     assert not ops.gemm_decode_fits(17, 64, 64, ops.EPILOGUE_STORE) and not ops.gemm_decode_fits(4, 64, 68, ops.EPILOGUE_STORE)
