@@ -11,6 +11,15 @@
 
 // ---- error channel: every entry point returns 0 or -1 and leaves a message ---------
 void fw_set_error(const char* format, ...);
+// A workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every global
+// load in flight (its fence covers global memory), which empties a prefetch pipeline at each
+// barrier; use this one where waves hand data to each other through LDS alone.
+__device__ __forceinline__ void fw_lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 #define FW_REQUIRE(cond, ...)                    \
     do {                                         \
         if (!(cond)) {                           \

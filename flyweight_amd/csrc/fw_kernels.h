@@ -4,6 +4,7 @@
 // checked on the host before anything is launched; a kernel never runs on operands it
 // was not written for.
 #pragma once
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -37,6 +38,14 @@ int fw_gemm_skinny(const void* a, const void* w, const float* bias, void* out, i
                    int M, int N, int K, void* stream);
 int fw_gemm_mfma(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                  int M, int N, int K, void* stream);
+// The same product for 1..64 rows with K split over workgroups, so that a is not re-read by every
+// few features (decode steps of 17..64 requests). fw_gemm_medium_plan says what a shape needs:
+// bytes of workspace (0: none) and int32 counters (0: none) that are zero before the first call;
+// the kernel leaves them zero. Calls that overlap on one device need their own of both.
+int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* workspace_bytes, int* counters);
+int fw_gemm_medium(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
+                   int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
+                   int counters_len, void* stream);
 
 // Fused product for decode steps of up to 16 rows. prologue 0: a is bfloat16 [M][K]; 1: a is
 // float32 rows, RMS-normed with norm_weight/eps (rows gathered through row_index if given) inside

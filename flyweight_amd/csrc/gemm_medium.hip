@@ -1,0 +1,361 @@
+// Matrix product for a few dozen rows: out[M][N] = a[M][K] . w[N][K]^T, M <= 64, bfloat16 operands,
+// float32 accumulation on the matrix cores. This is the decode step of 17..64 requests (and any
+// short batch): still bound by reading W once from HBM, but a is now large enough (up to 1 MB)
+// that re-reading it from L2 in every workgroup of a few features would cost several times the
+// traffic of W itself. So the work is cut the other way:
+//
+//  * a workgroup (4 waves) owns 64 or 32 consecutive features and a slice of K; with few
+//    features the slices of K go to different workgroups (blockIdx.y) so that every compute unit
+//    still streams its share of W;
+//  * W goes from global memory straight into MFMA operand registers (lane (n, g) of the 16x16x32
+//    instruction holds k = 8g..8g+7 of feature n), four chunks of 64 k in flight per wave;
+//  * a is staged through LDS once per workgroup (two buffers, one barrier per chunk), also
+//    four chunks ahead in registers, and read from there as MFMA operands by every wave;
+//  * partial sums over K: inside a workgroup through LDS in wave order; between workgroups
+//    through a float32 workspace that the LAST workgroup of a tile to arrive (a ticket from an
+//    atomic counter) sums in slice order, so the result does not depend on timing. The counter
+//    is left at zero again. Nobody waits for anybody.
+//
+// Every global load is unconditional (addresses clamped into the operands, a zeroed outside
+// the slice on its way to LDS): a branch around a load, or arithmetic right behind it, makes
+// the compiler wait for loads in flight. The barriers order LDS traffic only, for the same reason.
+// Epilogues as in the other products: store, add into the float32 residual stream, SwiGLU.
+// The reference has no counterpart for this batch size: its decode projections are
+// one-warp-per-row vector kernels run per request (native/include/flyweight_v2_qwen_kernels.hpp:855-941).
+#include "fw_common.h"
+#include "fw_kernels.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+#define GM_THREADS 256
+#define GM_DEPTH 4      // chunks in flight
+#define GM_PAD 8        // bfloat16 elements between LDS rows: spreads the rows over the banks
+
+enum { GM_STORE = 0, GM_ACCUMULATE = 1, GM_SWIGLU = 2 };
+
+struct MediumArgs {
+    const uint16_t* a;
+    const uint16_t* w;
+    const float* bias;
+    void* out;
+    int M, N, K;            // N: output features (for SwiGLU w has 2N rows: gate, then up)
+    int k_per_split;        // a multiple of the workgroup's chunk
+    int splits;
+    float* partials;        // [splits][tiles][kinds * MT][FW][64][4]
+    int* counters;          // [tiles], zero between calls
+};
+
+__device__ __forceinline__ float gm_silu(float g) {
+    if (g >= 0.0f) return g / (1.0f + __expf(-g));
+    const float e = __expf(g);
+    return g * e / (1.0f + e);
+}
+
+// MT: tiles of 16 rows of a. FW: waves side by side over features (4: 64 features, no split of
+// K inside the workgroup; 2: 32 features, the two halves of a 128-k chunk go to wave pairs).
+template <int MT, int FW, int MODE, typename TO>
+__global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArgs p) {
+    constexpr int KP = 4 / FW;                  // parts of K inside the workgroup
+    constexpr int CHUNK = 64 * KP;              // k per iteration of the workgroup
+    constexpr int KINDS = MODE == GM_SWIGLU ? 2 : 1;
+    constexpr int SEG = CHUNK / 8;              // 16-byte pieces per row of a chunk of a
+    constexpr int PIECES = MT * 16 * SEG;       // pieces per chunk of a
+    constexpr int AP = (PIECES + GM_THREADS - 1) / GM_THREADS;
+    constexpr int STRIDE = CHUNK + GM_PAD;
+    __shared__ __attribute__((aligned(16))) uint16_t a_lds[2][MT * 16][STRIDE];
+    __shared__ float k_parts[KP > 1 ? KP - 1 : 1][KP > 1 ? FW : 1][KP > 1 ? KINDS * MT : 1][KP > 1 ? 64 : 1][4];
+    __shared__ int ticket_shared;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
+    const int ft = wave % FW, kp = wave / FW;
+    const int M = p.M, N = p.N, K = p.K;
+    const int tile = blockIdx.x, tiles = gridDim.x;
+    const int n0 = tile * 16 * FW;
+    const int k_begin = blockIdx.y * p.k_per_split;
+    const int k_end = min(K, k_begin + p.k_per_split);
+    const int chunks = (k_end - k_begin + CHUNK - 1) / CHUNK;
+    const int iterations = (chunks + GM_DEPTH - 1) / GM_DEPTH * GM_DEPTH;
+
+    const int feature = n0 + 16 * ft + r16;
+    const uint16_t* w_row[KINDS];
+#pragma unroll
+    for (int kind = 0; kind < KINDS; ++kind) w_row[kind] = p.w + (size_t)((feature < N ? feature : 0) + kind * N) * K;
+    const uint16_t* a_piece[AP];
+    int piece_row[AP], piece_k[AP];
+#pragma unroll
+    for (int i = 0; i < AP; ++i) {
+        const int q = threadIdx.x + i * GM_THREADS;
+        piece_row[i] = q / SEG;
+        piece_k[i] = (q % SEG) * 8;
+        a_piece[i] = p.a + (size_t)min(piece_row[i], M - 1) * K;
+    }
+
+    bf16x8 wf[GM_DEPTH][KINDS][2], areg[GM_DEPTH][AP];
+    f32x4 acc[KINDS][MT];
+#pragma unroll
+    for (int kind = 0; kind < KINDS; ++kind)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[kind][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // Nothing is done to a loaded value before the chunk is used (a select right behind a load
+    // would wait for it at once): W comes from a clamped address as it is, and the rows of a are
+    // zeroed outside the slice when they move to LDS, three chunks after their load.
+    auto load = [&](const int d, const int c) {
+        const int k0 = k_begin + c * CHUNK;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int k = k0 + kp * 64 + ks * 32 + g * 8;
+#pragma unroll
+            for (int kind = 0; kind < KINDS; ++kind)
+                wf[d][kind][ks] = *reinterpret_cast<const bf16x8*>(w_row[kind] + (k < k_end ? k : 0));
+        }
+#pragma unroll
+        for (int i = 0; i < AP; ++i) {
+            const int k = k0 + piece_k[i];
+            areg[d][i] = *reinterpret_cast<const bf16x8*>(a_piece[i] + (k < k_end ? k : 0));
+        }
+    };
+    auto stage = [&](const int d, const int buffer, const int c) {
+        const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < AP; ++i)
+            if (PIECES % GM_THREADS == 0 || piece_row[i] < MT * 16) {
+                // K and the slices are multiples of 8: a run of 8 is inside or outside as a whole
+                const bool inside = k_begin + c * CHUNK + piece_k[i] < k_end;
+                *reinterpret_cast<bf16x8*>(&a_lds[buffer][piece_row[i]][piece_k[i]]) = inside ? areg[d][i] : none;
+            }
+    };
+    auto multiply = [&](const int d, const int buffer) {
+        bf16x8 af[2][MT];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                af[ks][mt] = *reinterpret_cast<const bf16x8*>(&a_lds[buffer][mt * 16 + r16][kp * 64 + ks * 32 + g * 8]);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int kind = 0; kind < KINDS; ++kind)
+                    acc[kind][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[d][kind][ks], af[ks][mt], acc[kind][mt], 0, 0, 0);
+    };
+
+#pragma unroll
+    for (int d = 0; d < GM_DEPTH; ++d) load(d, d);
+    stage(0, 0, 0);
+    fw_lds_barrier();
+    for (int c0 = 0; c0 < iterations; c0 += GM_DEPTH) {
+#pragma unroll
+        for (int d = 0; d < GM_DEPTH; ++d) {
+            // chunk c0 + d: its W is in register set d, its a in LDS buffer d % 2; the next chunk's a
+            // waits in register set d + 1 and moves to the other buffer; set d is then refilled
+            multiply(d, d & 1);
+            stage((d + 1) % GM_DEPTH, (d + 1) & 1, c0 + d + 1);
+            load(d, c0 + d + GM_DEPTH);
+            fw_lds_barrier();       // LDS only: the loads just issued stay in flight
+        }
+    }
+
+    // the parts of K inside the workgroup meet in LDS, in wave order
+    if (KP > 1) {
+        if (kp > 0)
+#pragma unroll
+            for (int kind = 0; kind < KINDS; ++kind)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) k_parts[kp > 0 ? kp - 1 : 0][ft][kind * MT + mt][lane][r] = acc[kind][mt][r];
+        __syncthreads();
+        if (kp == 0)
+            for (int part = 0; part < KP - 1; ++part)
+#pragma unroll
+                for (int kind = 0; kind < KINDS; ++kind)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[kind][mt][r] += k_parts[part][ft][kind * MT + mt][lane][r];
+    }
+
+    // The slices of K of different workgroups meet in the workspace; the last to arrive sums them.
+    // The partial sums are written and read with device-scope accesses, which go past the caches
+    // that workgroups on different dies do not share, so no cache has to be written back or
+    // dropped as a whole (what a device-wide fence does): a wave waits for its own stores to be
+    // acknowledged, the workgroup meets, then one thread takes the ticket.
+    if (p.splits > 1) {
+        float* mine = p.partials + ((((size_t)blockIdx.y * tiles + tile) * (KINDS * MT) * FW + ft) * 64 + lane) * 4;
+        if (kp == 0)
+#pragma unroll
+            for (int kind = 0; kind < KINDS; ++kind)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        __hip_atomic_store(mine + (size_t)(kind * MT + mt) * FW * 256 + r, acc[kind][mt][r], __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (threadIdx.x == 0)
+            ticket_shared = __hip_atomic_fetch_add(&p.counters[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (ticket_shared != p.splits - 1) return;
+        if (kp == 0) {
+#pragma unroll
+            for (int kind = 0; kind < KINDS; ++kind)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[kind][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int split = 0; split < p.splits; ++split) {
+                const float* theirs = p.partials + ((((size_t)split * tiles + tile) * (KINDS * MT) * FW + ft) * 64 + lane) * 4;
+                float v[KINDS * MT][4];
+#pragma unroll
+                for (int t = 0; t < KINDS * MT; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        v[t][r] = __hip_atomic_load(theirs + (size_t)t * FW * 256 + r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                for (int kind = 0; kind < KINDS; ++kind)
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) acc[kind][mt][r] += v[kind * MT + mt][r];
+            }
+        }
+        if (threadIdx.x == 0) __hip_atomic_store(&p.counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (kp != 0) return;
+
+    // D layout of the 16x16 product: lane holds features 4 * (lane / 16) + r of the wave's tile
+    // for row lane % 16 of a
+    const int n_first = n0 + 16 * ft + 4 * g;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + r16;
+        if (m >= M) continue;
+        float value[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int n = n_first + r;
+            if (MODE == GM_SWIGLU) {
+                value[r] = gm_silu(acc[0][mt][r]) * acc[1][mt][r];
+            } else {
+                value[r] = acc[0][mt][r] + ((p.bias && n < N) ? p.bias[n] : 0.0f);
+            }
+        }
+        TO* out = static_cast<TO*>(p.out);
+        const size_t at = (size_t)m * N + n_first;
+        if (n_first + 3 < N && (N & 3) == 0) {
+            if constexpr (sizeof(TO) == 4) {
+                f32x4* to = reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.out) + at);
+                f32x4 v = {value[0], value[1], value[2], value[3]};
+                if (MODE == GM_ACCUMULATE) {
+                    const f32x4 old = *to;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] += old[r];
+                }
+                *to = v;
+            } else {
+                uint2 packed;
+                packed.x = (uint32_t)float_to_bf16_bits(value[0]) | ((uint32_t)float_to_bf16_bits(value[1]) << 16);
+                packed.y = (uint32_t)float_to_bf16_bits(value[2]) | ((uint32_t)float_to_bf16_bits(value[3]) << 16);
+                *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.out) + at) = packed;
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if (n_first + r >= N) continue;
+                float v = value[r];
+                if (MODE == GM_ACCUMULATE) v += load_as_float(out, at + r);
+                store_from_float(out, at + r, v);
+            }
+        }
+    }
+}
+
+// ----- host side ---------------------------------------------------------------------------
+struct MediumPlan {
+    int mt, fw, tiles, splits, k_per_split;
+    size_t workspace_bytes;
+};
+
+static MediumPlan medium_plan(int M, int N, int K, int mode) {
+    MediumPlan plan;
+    plan.mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+    const int kinds = mode == GM_SWIGLU ? 2 : 1;
+    if (fw_ceil_div(N, 64) >= 384) {            // enough tiles of 64 features for every compute unit
+        plan.fw = 4;
+        plan.tiles = fw_ceil_div(N, 64);
+        plan.splits = 1;
+        plan.k_per_split = fw_ceil_div(K, 64) * 64;
+    } else {
+        plan.fw = 2;
+        plan.tiles = fw_ceil_div(N, 32);
+        const int chunk = 128;
+        int splits = (256 + plan.tiles / 2) / plan.tiles;           // about one workgroup per compute unit
+        const int most = K / (2 * chunk) > 1 ? K / (2 * chunk) : 1; // at least two chunks per slice
+        splits = splits < 1 ? 1 : (splits > most ? most : splits);
+        if (splits > 16) splits = 16;
+        plan.k_per_split = fw_ceil_div(fw_ceil_div(K, splits), chunk) * chunk;
+        plan.splits = fw_ceil_div(K, plan.k_per_split);
+    }
+    plan.workspace_bytes = plan.splits > 1
+        ? (size_t)plan.splits * plan.tiles * kinds * plan.mt * plan.fw * 64 * 4 * sizeof(float) : 0;
+    return plan;
+}
+
+// What fw_gemm_medium needs for a shape: bytes of workspace (0: none) and the number of int32
+// counters (0: none); the counters must be zero before the first call and are left zero.
+extern "C" int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* workspace_bytes, int* counters) {
+    FW_REQUIRE(M >= 1 && M <= 64 && N > 0 && K > 0, "gemm_medium: takes 1..64 rows, got M %d N %d K %d", M, N, K);
+    const MediumPlan plan = medium_plan(M, N, K, mode);
+    *workspace_bytes = plan.workspace_bytes;
+    *counters = plan.splits > 1 ? plan.tiles : 0;
+    return 0;
+}
+
+template <int MT, int FW>
+static void medium_launch(const MediumArgs& args, int out_dtype, int mode, dim3 grid, hipStream_t stream) {
+    if (mode == GM_SWIGLU) gemm_medium_kernel<MT, FW, GM_SWIGLU, bf16_t><<<grid, GM_THREADS, 0, stream>>>(args);
+    else if (mode == GM_ACCUMULATE) gemm_medium_kernel<MT, FW, GM_ACCUMULATE, float><<<grid, GM_THREADS, 0, stream>>>(args);
+    else if (out_dtype == FW_F32) gemm_medium_kernel<MT, FW, GM_STORE, float><<<grid, GM_THREADS, 0, stream>>>(args);
+    else gemm_medium_kernel<MT, FW, GM_STORE, bf16_t><<<grid, GM_THREADS, 0, stream>>>(args);
+}
+
+// mode 0: out = a . w^T (+ bias) stored as out_dtype; 1: out (float32) += a . w^T (+ bias);
+// 2: w is [2 * N][K] (gate rows, then up rows); out [M][N] bfloat16 = silu(gate) * up.
+// workspace / counters: as fw_gemm_medium_plan says for this shape. Calls that overlap on one
+// device must not share counters or workspace.
+extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
+                              int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
+                              int counters_len, void* stream) {
+    FW_REQUIRE(M >= 1 && M <= 64, "gemm_medium: takes 1..64 rows, got %d", M);
+    FW_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_medium: K (%d) must be a positive multiple of 8, N (%d) positive", K, N);
+    FW_REQUIRE(mode >= 0 && mode <= 2, "gemm_medium: unknown mode %d", mode);
+    FW_REQUIRE(mode != GM_ACCUMULATE || out_dtype == FW_F32, "gemm_medium: accumulation needs a float32 destination");
+    FW_REQUIRE(mode != GM_SWIGLU || (out_dtype == FW_BF16 && bias == nullptr), "gemm_medium: SwiGLU stores bfloat16 and takes no bias");
+    FW_REQUIRE(out_dtype == FW_F32 || out_dtype == FW_BF16, "gemm_medium: unknown out dtype %d", out_dtype);
+    FW_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)out % 16 == 0) && ((uintptr_t)workspace % 16 == 0),
+               "gemm_medium: operands must be 16-byte aligned");
+    const MediumPlan plan = medium_plan(M, N, K, mode);
+    FW_REQUIRE(plan.splits == 1 || (workspace != nullptr && workspace_bytes >= plan.workspace_bytes && counters != nullptr &&
+                                    counters_len >= plan.tiles),
+               "gemm_medium: this shape needs %zu bytes of workspace and %d counters", plan.workspace_bytes, plan.tiles);
+    FW_REQUIRE(plan.tiles <= 65535 * 16 && plan.splits <= 65535, "gemm_medium: too many tiles");
+    MediumArgs args;
+    args.a = (const uint16_t*)a; args.w = (const uint16_t*)w; args.bias = bias; args.out = out;
+    args.M = M; args.N = N; args.K = K; args.k_per_split = plan.k_per_split; args.splits = plan.splits;
+    args.partials = (float*)workspace; args.counters = counters;
+    const dim3 grid(plan.tiles, plan.splits);
+    hipStream_t s = (hipStream_t)stream;
+    if (plan.fw == 4) {
+        if (plan.mt == 1) medium_launch<1, 4>(args, out_dtype, mode, grid, s);
+        else if (plan.mt == 2) medium_launch<2, 4>(args, out_dtype, mode, grid, s);
+        else medium_launch<4, 4>(args, out_dtype, mode, grid, s);
+    } else {
+        if (plan.mt == 1) medium_launch<1, 2>(args, out_dtype, mode, grid, s);
+        else if (plan.mt == 2) medium_launch<2, 2>(args, out_dtype, mode, grid, s);
+        else medium_launch<4, 2>(args, out_dtype, mode, grid, s);
+    }
+    FW_LAUNCH_CHECK("gemm_medium");
+    return 0;
+}

@@ -67,6 +67,7 @@ class CausalLM:
 
     def bind(self, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device: torch.device) -> None:
         self.dtype, self.device = dtype, device
+        ops.prepare_device(device)
         self.embedding = tensors[self.spec.embedding_name]
         head = self.embedding if self.spec.lm_head_name is None else tensors[self.spec.lm_head_name]
         self.head = Linear(head)

@@ -299,13 +299,52 @@ def fill_zero(t: torch.Tensor) -> None:
 
 
 def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int) -> None:
-    """bfloat16 operands on the matrix cores: the skinny kernel for up to 64 rows, the tiled one beyond."""
+    """bfloat16 operands on the matrix cores: the skinny kernel for up to 16 rows, the medium one
+    (K split over workgroups) for up to 64, the tiled one beyond."""
     M, K = a.shape
+    if SKINNY_MAX_ROWS < M <= MEDIUM_MAX_ROWS:
+        gemm_medium_into(a, w, bias, target, out_code, mode, N)
+        return
     entry = library().fw_gemm_skinny if M <= SKINNY_MAX_ROWS else library().fw_gemm_mfma
     _check(entry(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K, _stream()))
 
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 16
+MEDIUM_MAX_ROWS = 64
+_MEDIUM_COUNTERS = {}
+
+
+def _medium_counters(device: torch.device, count: int) -> torch.Tensor:
+    """Zeroed int32 counters for the medium product's tickets, one set per device: the kernel
+    leaves them at zero, and calls on one device follow each other in stream order (work on
+    several streams of one device at once would need a set per stream)."""
+    have = _MEDIUM_COUNTERS.get(device.index)
+    if have is None or have.numel() < count:
+        if torch.cuda.is_current_stream_capturing():
+            raise KernelError("gemm_medium: its counters must exist before a graph is captured (prepare_device)")
+        have = torch.zeros(max(count, 8192), dtype=torch.int32, device=device)
+        _MEDIUM_COUNTERS[device.index] = have
+    return have
+
+
+def prepare_device(device: torch.device) -> None:
+    """Allocates what kernels keep between calls on this device; a model does this when its
+    weights arrive, so that nothing is allocated for the first time inside a graph capture."""
+    _medium_counters(torch.device(device), 0)
+
+
+def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int) -> None:
+    """The product for 1..64 rows with K split over workgroups (fw_gemm_medium)."""
+    M, K = a.shape
+    need_bytes, need_counters = ctypes.c_size_t(0), ctypes.c_int(0)
+    _check(library().fw_gemm_medium_plan(M, N, K, mode, ctypes.byref(need_bytes), ctypes.byref(need_counters)))
+    workspace = counters = None
+    if need_bytes.value:
+        workspace = torch.empty(need_bytes.value // 4, dtype=torch.float32, device=a.device)
+        counters = _medium_counters(a.device, need_counters.value)
+    _check(library().fw_gemm_medium(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K, _p(workspace),
+                                    ctypes.c_size_t(need_bytes.value), _p(counters),
+                                    0 if counters is None else counters.numel(), _stream()))
 
 
 def _fast_ok(a: torch.Tensor, w: torch.Tensor) -> bool:

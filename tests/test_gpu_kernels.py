@@ -363,9 +363,39 @@ def test_fast_gemm_rows_do_not_depend_on_the_batch(ops):
     whole = ops.gemm(a, w, out_dtype=torch.float32)
     assert torch.equal(ops.gemm(a[100:230].contiguous(), w, out_dtype=torch.float32), whole[100:230])
     few = ops.gemm(a[:40].contiguous(), w, out_dtype=torch.float32)
-    assert torch.equal(ops.gemm(a[7:8].contiguous(), w, out_dtype=torch.float32)[0], few[7])
-    # the decode and the prompt kernel sum in different orders: equal up to float32 rounding
+    assert torch.equal(ops.gemm(a[7:30].contiguous(), w, out_dtype=torch.float32), few[7:30])
+    fewer = ops.gemm(a[:12].contiguous(), w, out_dtype=torch.float32)
+    assert torch.equal(ops.gemm(a[7:8].contiguous(), w, out_dtype=torch.float32)[0], fewer[7])
+    # the kernels for few, some and many rows sum in different orders: equal up to float32 rounding
     close(few, whole[:40].cpu().double(), torch.float32, 2.0)
+    close(fewer, whole[:12].cpu().double(), torch.float32, 2.0)
+
+
+@pytest.mark.parametrize("M", [17, 33, 48, 64])
+@pytest.mark.parametrize("N,K", [(64, 4096), (96, 520), (2048, 8192), (6144, 2048), (25000, 72)])
+def test_medium_gemm_splits_k_over_workgroups(ops, M, N, K):
+    """Few features and a long K: slices of K go to different workgroups and the last one to
+    arrive sums them in slice order. Twice in a row (the tickets are left at zero), every
+    epilogue, and bitwise the same whichever workgroup came last."""
+    a = as_dev(gen(M, K), torch.bfloat16)
+    w = as_dev(gen(N, K, seed=1, scale=K ** -0.5), torch.bfloat16)
+    bias = gen(N, seed=2).float().to(DEV)
+    want = back(a) @ back(w).T
+    first = ops.gemm(a, w, bias, out_dtype=torch.float32)
+    close(first, want + bias.cpu().double(), torch.float32, 2.0)
+    for _ in range(3):
+        assert torch.equal(ops.gemm(a, w, bias, out_dtype=torch.float32), first)
+    # other rows through the same workspace: nothing of the call before may be seen again
+    for seed in (7, 8):
+        other = as_dev(gen(M, K, seed=seed), torch.bfloat16)
+        close(ops.gemm(other, w, out_dtype=torch.float32), back(other) @ back(w).T, torch.float32, 2.0)
+    close(ops.gemm(a, w), want, torch.bfloat16, 0.4)
+    residual = gen(M, N, seed=3).float().to(DEV)
+    before = residual.cpu().double()
+    ops.gemm(a, w, accumulate_into=residual)
+    close(residual, before + want, torch.float32, 2.0)
+    half = N // 2
+    close(ops.gemm_swiglu(a, w), F.silu(want[:, :half]) * want[:, half:], torch.bfloat16, 0.4)
 
 
 # ----- attention on the matrix cores -------------------------------------------------------------
