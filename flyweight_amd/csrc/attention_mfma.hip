@@ -169,9 +169,9 @@ __device__ __forceinline__ void load_query(Columns<HD>& c, const uint16_t* __res
 
 // ---- prompt portions ---------------------------------------------------------------------------
 // grid (tiles of 64 query rows, heads); four waves, 16 rows each, all of one head. The pages of
-// the kv head are copied global -> registers -> LDS one page ahead of the one being worked on
-// (two LDS buffers, one barrier per page), so that the copy hides behind the softmax
-// arithmetic. tile_seg / tile_row0: the segment of each tile and its first row (a tile never
+// the kv head are copied global -> registers (two pages ahead) -> LDS (one page ahead of the
+// one being worked on; two LDS buffers, one barrier per page), so that the copy hides behind the
+// softmax arithmetic. tile_seg / tile_row0: the segment of each tile and its first row (a tile never
 // spans two segments). LDS rows are padded by 16 bytes against bank conflicts.
 #define KV_PAD 8
 template <int HD>
@@ -185,7 +185,8 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     const int k_elems = PAGE * k_stride, v_elems = head_dim * v_stride;
     uint16_t* lds = reinterpret_cast<uint16_t*>(lds_raw);      // [buffer][K tile | V tile]
 
-    const int tile = blockIdx.x, head = blockIdx.y;
+    // the last tiles of a long prompt see the most keys: they start first, the short ones fill in behind
+    const int tile = gridDim.x - 1 - blockIdx.x, head = blockIdx.y;
     const int kvh = head / (num_heads / num_kv_heads);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, g = lane >> 4;
     const int seg = tile_seg[tile];
@@ -207,22 +208,25 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     const int32_t* table = block_table + (size_t)seg * table_stride;
     const size_t page_elems = (size_t)PAGE * head_dim;
 
-    // the copy: a page's K is 64 rows of head_dim, its V head_dim rows of 64; runs of 16 bytes
-    const int k_runs = PAGE * head_dim / 8, v_runs = head_dim * PAGE / 8;        // equal
+    // the copy: a page's K is 64 rows of head_dim, its V head_dim rows of 64; runs of 16 bytes.
+    // Loads are unconditional (a run or a page past the end is read from a valid place again and
+    // never used) and the barriers order LDS traffic only, so that the pages requested stay in
+    // flight while the page before them is worked on.
+    const int k_runs = PAGE * head_dim / 8;                                      // as many for V
     constexpr int MAX_RUNS = HD * PAGE / 8 / 256;                                // per thread, per operand
-    u32x4 hold_k[MAX_RUNS], hold_v[MAX_RUNS];
-    auto fetch = [&](int block) {
-        const size_t at = ((size_t)table[block] * num_kv_heads + kvh) * page_elems;
+    const int first_block = tile_first / PAGE, last_block = pos_hi / PAGE;
+    u32x4 hold_k0[MAX_RUNS], hold_v0[MAX_RUNS], hold_k1[MAX_RUNS], hold_v1[MAX_RUNS];
+    auto fetch = [&](u32x4 (&hold_k)[MAX_RUNS], u32x4 (&hold_v)[MAX_RUNS], int block) {
+        const size_t at = ((size_t)table[block < last_block ? block : last_block] * num_kv_heads + kvh) * page_elems;
 #pragma unroll
         for (int u = 0; u < MAX_RUNS; ++u) {
             const int run = tid + u * 256;
-            if (run < k_runs) {
-                hold_k[u] = *reinterpret_cast<const u32x4*>(k_pages + at + (size_t)run * 8);
-                hold_v[u] = *reinterpret_cast<const u32x4*>(v_pages + at + (size_t)run * 8);
-            }
+            const size_t from = at + (size_t)(run < k_runs ? run : 0) * 8;
+            hold_k[u] = *reinterpret_cast<const u32x4*>(k_pages + from);
+            hold_v[u] = *reinterpret_cast<const u32x4*>(v_pages + from);
         }
     };
-    auto stash = [&](int buffer) {
+    auto stash = [&](const u32x4 (&hold_k)[MAX_RUNS], const u32x4 (&hold_v)[MAX_RUNS], int buffer) {
         uint16_t* kt = lds + (size_t)buffer * (k_elems + v_elems);
         uint16_t* vt = kt + k_elems;
         const int k_per_row = head_dim / 8;
@@ -235,22 +239,33 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
             }
         }
     };
-
-    const int first_block = tile_first / PAGE, last_block = pos_hi / PAGE;
-    fetch(first_block);
-    stash(0);
-    __syncthreads();
-    for (int block = first_block; block <= last_block; ++block) {
-        const int buffer = (block - first_block) & 1;
-        if (block < last_block) fetch(block + 1);
+    auto attend = [&](int block, int buffer) {
         const int base = block * PAGE;
         if (rows > 0 && base <= wave_hi) {      // a wave whose rows all lie before this page has nothing to add
             const uint16_t* kt = lds + (size_t)buffer * (k_elems + v_elems);
             attend_page<HD>(c, kt, kt + k_elems, head_dim, scale_log2, valid ? my_first - base : PAGE,
                             valid ? my_pos - base : -1, pos_hi - base, k_stride, v_stride);
         }
-        if (block < last_block) stash(buffer ^ 1);
-        __syncthreads();
+    };
+
+    // page b travels: global -> register set (b - first) % 2, requested two pages ahead -> LDS
+    // buffer (b - first) % 2, stored while page b - 1 is worked on -> attended
+    fetch(hold_k0, hold_v0, first_block);
+    fetch(hold_k1, hold_v1, first_block + 1);
+    stash(hold_k0, hold_v0, 0);
+    fw_lds_barrier();
+    for (int block = first_block; block <= last_block; block += 2) {
+        fetch(hold_k0, hold_v0, block + 2);
+        __builtin_amdgcn_sched_barrier(0);      // keep the requests ahead of the work they overlap
+        attend(block, 0);
+        stash(hold_k1, hold_v1, 1);
+        fw_lds_barrier();
+        if (block + 1 > last_block) break;
+        fetch(hold_k1, hold_v1, block + 3);
+        __builtin_amdgcn_sched_barrier(0);
+        attend(block + 1, 1);
+        stash(hold_k0, hold_v0, 0);
+        fw_lds_barrier();
     }
     float l = c.l;
     l += __shfl_xor(l, 16, 64);

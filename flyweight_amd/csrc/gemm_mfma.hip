@@ -97,25 +97,20 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
     u32x4 ra0[4], rw0[W_CHUNKS], ra1[4], rw1[W_CHUNKS];
     const u32x4 zero = {0u, 0u, 0u, 0u};
     auto fetch = [&](u32x4 (&ra)[4], u32x4 (&rw)[W_CHUNKS], int k0) {
-        // Every load is issued unconditionally (past the end of K from column 0, then dropped):
-        // a branch around a load would make the compiler wait for ALL loads at the next wait.
-        const bool ok = k0 + kc < K;                    // K is a multiple of 8
-        const int from = ok ? k0 : 0;
+        // Every load is issued unconditionally (past the end of K from column 0) and nothing
+        // touches the value until it moves to LDS: a branch around a load, or arithmetic right
+        // behind it, would make the compiler wait for loads in flight.
+        const int from = k0 + kc < K ? k0 : 0;          // K is a multiple of 8
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const u32x4 v = *reinterpret_cast<const u32x4*>(a_src[i] + from);
-            ra[i] = ok ? v : zero;
-        }
+        for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const u32x4*>(a_src[i] + from);
 #pragma unroll
-        for (int i = 0; i < W_CHUNKS; ++i) {
-            const u32x4 v = *reinterpret_cast<const u32x4*>(w_src[i] + from);
-            rw[i] = ok ? v : zero;
-        }
+        for (int i = 0; i < W_CHUNKS; ++i) rw[i] = *reinterpret_cast<const u32x4*>(w_src[i] + from);
     };
-    auto stash = [&](const u32x4 (&ra)[4], const u32x4 (&rw)[W_CHUNKS], int buffer) {
+    auto stash = [&](const u32x4 (&ra)[4], const u32x4 (&rw)[W_CHUNKS], int buffer, int k0) {
         unsigned char* base = lds + buffer * (A_SLAB + W_SLAB);
+        const bool ok = k0 + kc < K;                    // a past the end of K is zero; W may then be anything finite
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(base + lds_at[i]) = ra[i];
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<u32x4*>(base + lds_at[i]) = ok ? ra[i] : zero;
 #pragma unroll
         for (int i = 0; i < W_CHUNKS; ++i) *reinterpret_cast<u32x4*>(base + A_SLAB + lds_at[i]) = rw[i];
     };
@@ -152,31 +147,34 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
     // state has no branches, so the compiler can count exactly which loads it must wait for.
     const int steps = (K + TK - 1) / TK;
     int step = 0;
+    // The barriers order LDS traffic only: the loads just requested stay in flight across them.
     fetch(ra0, rw0, 0);
-    fetch(ra1, rw1, TK);                                // past the end: zeros
-    stash(ra0, rw0, 0);
-    __syncthreads();
+    fetch(ra1, rw1, TK);                                // past the end: dropped when stored
+    stash(ra0, rw0, 0, 0);
+    fw_lds_barrier();
     while (step + 3 < steps) {
         fetch(ra0, rw0, (step + 2) * TK);
+        __builtin_amdgcn_sched_barrier(0);              // keep the requests ahead of the work they overlap
         multiply(0);
-        stash(ra1, rw1, 1);
-        __syncthreads();
+        stash(ra1, rw1, 1, (step + 1) * TK);
+        fw_lds_barrier();
         fetch(ra1, rw1, (step + 3) * TK);
+        __builtin_amdgcn_sched_barrier(0);
         multiply(1);
-        stash(ra0, rw0, 0);
-        __syncthreads();
+        stash(ra0, rw0, 0, (step + 2) * TK);
+        fw_lds_barrier();
         step += 2;
     }
     // at most three slabs are left: slab `step` is in buffer 0, slab step + 1 in set 1
     if (step + 2 < steps) fetch(ra0, rw0, (step + 2) * TK);
     multiply(0);
     if (step + 1 < steps) {
-        stash(ra1, rw1, 1);
-        __syncthreads();
+        stash(ra1, rw1, 1, (step + 1) * TK);
+        fw_lds_barrier();
         multiply(1);
         if (step + 2 < steps) {
-            stash(ra0, rw0, 0);
-            __syncthreads();
+            stash(ra0, rw0, 0, (step + 2) * TK);
+            fw_lds_barrier();
             multiply(0);
         }
     }

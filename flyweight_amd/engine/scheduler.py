@@ -58,6 +58,15 @@ class Request:
     def tokens(self) -> List[int]:
         return self.prompt + self.generated
 
+    def tokens_from(self, first: int, count: int) -> List[int]:
+        """tokens[first:first + count] without joining the two lists."""
+        end, split = first + count, len(self.prompt)
+        if end <= split:
+            return self.prompt[first:end]
+        if first >= split:
+            return self.generated[first - split:end - split]
+        return self.prompt[first:] + self.generated[:end - split]
+
     @property
     def remaining(self) -> int:
         return len(self.prompt) + len(self.generated) - self.computed
@@ -77,10 +86,23 @@ class StepPlan:
     failed: List[Request] = field(default_factory=list)
     admitted: List[Request] = field(default_factory=list)
     cancelled: List[Request] = field(default_factory=list)
+    num_tokens: int = 0
+    _planned: set = field(default_factory=set)      # ids of the requests that have a segment
 
-    @property
-    def num_tokens(self) -> int:
-        return sum(len(s.tokens) for s in self.segments)
+    def add(self, segment: PlannedSegment) -> None:
+        self.segments.append(segment)
+        self.num_tokens += len(segment.tokens)
+        self._planned.add(segment.request.id)
+
+    def drop(self, request: Request) -> None:
+        if request.id not in self._planned:
+            return
+        self.num_tokens -= sum(len(s.tokens) for s in self.segments if s.request is request)
+        self.segments = [s for s in self.segments if s.request is not request]
+        self._planned.discard(request.id)
+
+    def has(self, request: Request) -> bool:
+        return request.id in self._planned
 
 
 class Scheduler:
@@ -148,8 +170,7 @@ class Scheduler:
         plan.failed.append(request)
 
     def _preempt(self, victim: Request, plan: StepPlan) -> None:
-        for segment in [s for s in plan.segments if s.request is victim]:
-            plan.segments.remove(segment)
+        plan.drop(victim)
         self._evict(victim)
         victim.preemptions += 1
         self.preemptions += 1
@@ -185,7 +206,7 @@ class Scheduler:
 
     def _plan_once(self, plan: StepPlan) -> None:
         cache = self.cache
-        planned = lambda request: any(s.request is request for s in plan.segments)     # noqa: E731
+        planned = plan.has
 
         # 1. decode rows, oldest first; make room by preempting the newest
         for request in list(self.running):
@@ -201,7 +222,7 @@ class Scheduler:
             if not request.live:
                 continue
             cache.reserve(request.id, request.computed + 1)
-            plan.segments.append(PlannedSegment(request, [request.tokens[request.computed]], True))
+            plan.add(PlannedSegment(request, request.tokens_from(request.computed, 1), True))
 
         # 2. portions of prompts of running requests, oldest first
         for request in list(self.running):
@@ -243,8 +264,7 @@ class Scheduler:
         if portion < 1:
             return
         self.cache.reserve(request.id, request.computed + portion)
-        tokens = request.tokens[request.computed:request.computed + portion]
-        plan.segments.append(PlannedSegment(request, tokens, portion == request.remaining))
+        plan.add(PlannedSegment(request, request.tokens_from(request.computed, portion), portion == request.remaining))
 
     # ----- after the step ---------------------------------------------------------------
     def complete(self, plan: StepPlan, sampled: Dict[int, int]) -> List[Tuple[int, int, int]]:
