@@ -10,23 +10,83 @@ has no such state.
 Lifetime of a request: ``admit`` (takes a slot, zeroes its state) -> per step ``reserve``
 (maps pages for the tokens the step will append; all or nothing) and ``commit`` (the new
 length; a windowed group gives back the pages its window has passed) -> ``release``
-(everything back to the pools). The reference reserves one contiguous arena per slot for
+(everything back to the pools). The bookkeeping is the host library's (C++,
+``csrc/host/cache.hpp``); this class is its Python face and owns the tensors. The reference reserves one contiguous arena per slot for
 the whole context instead (native/src/v2_runtime.cpp:20700-20758) and zeroes it on reset
 (:20437-20451).
 """
 
 from __future__ import annotations
 
-from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Mapping, Optional, Sequence, Tuple
+import ctypes
+from dataclasses import dataclass
+from typing import Dict, Hashable, Iterator, List, Mapping, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
+from .. import host
 from .needs import FixedState, PagedKV
 from .pages import CacheAccountingError, OutOfPages, PagePool, SlotPool
 
-NO_PAGE = -1
+NO_PAGE = host.NO_PAGE
+_FIRST_NAMED_ID = 1 << 62       # ids of requests whose key is not a small non-negative integer
+
+
+class _Tables(Mapping):
+    """The block tables of one page group: request -> page per block (NO_PAGE once given back)."""
+
+    def __init__(self, manager: "CacheManager", group: int):
+        self._manager, self._group = manager, group
+
+    def __getitem__(self, request: Hashable) -> List[int]:
+        manager = self._manager
+        if request not in manager.requests:
+            raise KeyError(request)
+        native = manager._id(request)
+        capacity = manager.max_pages_per_request
+        pages = host.ints(capacity)
+        count = manager._lib.fwh_cache_table(manager._native, native, self._group, pages, capacity)
+        if count < 0:
+            raise KeyError(request)
+        return list(pages[:count])
+
+    def __iter__(self) -> Iterator[Hashable]:
+        return iter(self._manager.requests)
+
+    def __len__(self) -> int:
+        return len(self._manager.requests)
+
+
+class _LiveRequests(Mapping):
+    """The live requests: key -> (slot, length)."""
+
+    def __init__(self, manager: "CacheManager"):
+        self._manager = manager
+
+    def _keys(self) -> List[Hashable]:
+        manager = self._manager
+        capacity = manager.max_requests
+        found = host.ids(capacity)
+        count = manager._lib.fwh_cache_live(manager._native, found, capacity)
+        return [manager._key(found[i]) for i in range(count)]
+
+    def __contains__(self, request) -> bool:
+        manager = self._manager
+        native = manager._id(request, create=False)
+        return native is not None and bool(manager._lib.fwh_cache_is_live(manager._native, native))
+
+    def __getitem__(self, request: Hashable) -> Tuple[int, int]:
+        if request not in self:
+            raise KeyError(request)
+        return self._manager.slot_of(request), self._manager.length_of(request)
+
+    def __iter__(self) -> Iterator[Hashable]:
+        return iter(self._keys())
+
+    def __len__(self) -> int:
+        manager = self._manager
+        return manager._lib.fwh_cache_live(manager._native, host.ids(0), 0)
 
 
 @dataclass
@@ -35,13 +95,7 @@ class PageGroup:
     need: PagedKV
     entries: List[int]
     pool: PagePool
-    tables: Dict[Hashable, List[int]] = field(default_factory=dict)   # request -> page per block (NO_PAGE if given back)
-
-
-@dataclass
-class _Request:
-    slot: int
-    length: int = 0
+    tables: Mapping
 
 
 class CacheManager:
@@ -59,23 +113,31 @@ class CacheManager:
         self.groups: List[PageGroup] = []
         self.entry_group: Dict[int, int] = {}
         self.state_entries: Dict[int, FixedState] = {}
-        by_key: Dict[Tuple, PageGroup] = {}
+        grouped: Dict[Tuple, Tuple[PagedKV, List[int]]] = {}
         for entry in sorted(needs):
             need = needs[entry]
             if isinstance(need, PagedKV):
-                group = by_key.get(need.group_key())
-                if group is None:
-                    group = PageGroup(need.group_key(), need, [], PagePool(num_pages))
-                    by_key[need.group_key()] = group
-                    self.groups.append(group)
-                group.entries.append(entry)
-                self.entry_group[entry] = self.groups.index(group)
+                grouped.setdefault(need.group_key(), (need, []))[1].append(entry)
+                self.entry_group[entry] = list(grouped).index(need.group_key())
             elif isinstance(need, FixedState):
                 self.state_entries[entry] = need
             elif need is not None:
                 raise TypeError(f"cache entry {entry}: unknown need {need!r}")
-        self.slots = SlotPool(max_requests)
-        self.requests: Dict[Hashable, _Request] = {}
+        # the bookkeeping lives in the host library
+        self._lib = host.library()
+        windows = (ctypes.c_int * max(len(grouped), 1))(*[int(need.window or 0) for need, _ in grouped.values()])
+        self._native = self._lib.fwh_cache_create(len(grouped), windows, num_pages, max_requests, page_size,
+                                                  self.max_pages_per_request)
+        if not self._native:
+            raise ValueError(host.last_error())
+        for index, (key, (need, entries)) in enumerate(grouped.items()):
+            pool = PagePool(borrowed=self._lib.fwh_cache_group_pool(self._native, index), owner=self)
+            self.groups.append(PageGroup(key, need, entries, pool, _Tables(self, index)))
+        self.slots = SlotPool(borrowed=self._lib.fwh_cache_slot_pool(self._native), owner=self)
+        self.requests = _LiveRequests(self)
+        self._ids: Dict[Hashable, int] = {}         # keys that are not small integers -> ids of the host library
+        self._keys: Dict[int, Hashable] = {}
+        self._next_named = _FIRST_NAMED_ID
         # storage
         self.k_pages: Dict[int, torch.Tensor] = {}
         self.v_pages: Dict[int, torch.Tensor] = {}
@@ -90,26 +152,47 @@ class CacheManager:
             for entry, need in self.state_entries.items():
                 self.state[entry] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
 
+    def __del__(self):
+        if getattr(self, "_native", None):
+            self._lib.fwh_cache_destroy(self._native)
+            self._native = None
+
+    # ----- request keys ---------------------------------------------------------------------
+    def _id(self, request: Hashable, create: bool = True) -> Optional[int]:
+        """The host library names requests by 64-bit integers: a small non-negative integer key
+        is its own id (the scheduler's ids are such), any other key gets one of its own."""
+        if isinstance(request, (int, np.integer)) and not isinstance(request, bool) and 0 <= int(request) < _FIRST_NAMED_ID:
+            return int(request)
+        found = self._ids.get(request)
+        if found is None and create:
+            found = self._ids[request] = self._next_named
+            self._keys[found] = request
+            self._next_named += 1
+        return found
+
+    def _key(self, native: int) -> Hashable:
+        return self._keys.get(native, native)
+
+    def _forget(self, request: Hashable) -> None:
+        native = self._ids.pop(request, None)
+        if native is not None:
+            self._keys.pop(native, None)
+
+    @property
+    def native_handle(self):
+        """The host library's cache object (for the scheduler, which lives beside it)."""
+        return self._native
+
     # ----- sizes ------------------------------------------------------------------------
     def pages_for(self, tokens: int) -> int:
         return (tokens + self.page_size - 1) // self.page_size
 
-    def _first_needed_block(self, group: PageGroup, length: int) -> int:
-        """Blocks before this one hold only keys the window has passed once the sequence
-        is ``length`` tokens long (the next query sits at position ``length``)."""
-        if group.need.window is None:
-            return 0
-        first_key = max(0, length - group.need.window + 1)
-        return first_key // self.page_size
-
     def pages_missing(self, request: Hashable, new_length: int) -> Dict[int, int]:
         """Per group: pages a reservation up to ``new_length`` would have to take."""
-        missing = {}
-        blocks = self.pages_for(new_length)
-        for index, group in enumerate(self.groups):
-            table = group.tables.get(request, [])
-            missing[index] = max(0, blocks - len(table))
-        return missing
+        native = self._id(request, create=False)
+        out = host.ints(len(self.groups))
+        self._lib.fwh_cache_pages_missing(self._native, -1 if native is None else native, int(new_length), out)
+        return {index: out[index] for index in range(len(self.groups))}
 
     def can_reserve(self, request: Hashable, new_length: int, spare: int = 0) -> bool:
         if self.pages_for(new_length) > self.max_pages_per_request:
@@ -124,88 +207,79 @@ class CacheManager:
     def admit(self, request: Hashable) -> int:
         if request in self.requests:
             raise CacheAccountingError(f"request {request!r} is already live")
-        slot = self.slots.alloc()
-        self.requests[request] = _Request(slot)
-        for group in self.groups:
-            group.tables[request] = []
-        for tensor in self.state.values():
-            tensor[slot].zero_()
+        slot = self._lib.fwh_cache_admit(self._native, self._id(request))
+        if slot == host.OUT_OF_PAGES:
+            raise OutOfPages("out of request slots")
+        if slot < 0:
+            raise CacheAccountingError(host.last_error())
+        self.zero_slot(slot)
         return slot
 
+    def zero_slot(self, slot: int) -> None:
+        """A slot's state starts at zero for the request that takes it."""
+        for tensor in self.state.values():
+            tensor[slot].zero_()
+
     def slot_of(self, request: Hashable) -> int:
-        return self.requests[request].slot
+        slot = self._lib.fwh_cache_slot_of(self._native, self._live_id(request))
+        if slot < 0:
+            raise KeyError(request)
+        return slot
 
     def length_of(self, request: Hashable) -> int:
-        return self.requests[request].length
+        length = self._lib.fwh_cache_length_of(self._native, self._live_id(request))
+        if length < 0:
+            raise KeyError(request)
+        return length
+
+    def _live_id(self, request: Hashable) -> int:
+        native = self._id(request, create=False)
+        if native is None:
+            raise KeyError(f"request {request!r} is not live")
+        return native
 
     def reserve(self, request: Hashable, new_length: int) -> None:
         """Map pages for positions < new_length in every group, or raise OutOfPages and
         change nothing."""
         if request not in self.requests:
             raise KeyError(f"request {request!r} is not live")
-        if self.pages_for(new_length) > self.max_pages_per_request:
-            raise OutOfPages(f"request {request!r} would need {self.pages_for(new_length)} pages; "
-                             f"a block table holds {self.max_pages_per_request}")
-        missing = self.pages_missing(request, new_length)
-        for g, count in missing.items():
-            if self.groups[g].pool.free_count < count:
-                raise OutOfPages(f"out of cache pages: request {request!r} needs {count} more, "
-                                 f"{self.groups[g].pool.free_count} free")
-        for g, count in missing.items():
-            group = self.groups[g]
-            table = group.tables[request]
-            for _ in range(count):
-                table.append(group.pool.alloc())
+        status = self._lib.fwh_cache_reserve(self._native, self._id(request), int(new_length))
+        if status == host.OUT_OF_PAGES:
+            raise OutOfPages(host.last_error().replace(f"request {self._id(request)} ", f"request {request!r} "))
+        if status < 0:
+            raise CacheAccountingError(host.last_error())
 
     def commit(self, request: Hashable, new_length: int) -> None:
-        state = self.requests[request]
-        if new_length < state.length:
-            raise ValueError("a sequence does not shrink")
-        state.length = new_length
-        for group in self.groups:
-            table = group.tables[request]
-            for block in range(min(self._first_needed_block(group, new_length), len(table))):
-                if table[block] != NO_PAGE:
-                    group.pool.free(table[block])
-                    table[block] = NO_PAGE
+        if request not in self.requests:
+            raise KeyError(request)
+        if self._lib.fwh_cache_commit(self._native, self._id(request), int(new_length)) < 0:
+            raise ValueError(host.last_error())
 
     def release(self, request: Hashable) -> None:
         if request not in self.requests:
             raise CacheAccountingError(f"request {request!r} is released but not live")
-        state = self.requests.pop(request)
-        for group in self.groups:
-            for page in group.tables.pop(request):
-                if page != NO_PAGE:
-                    group.pool.free(page)
-        self.slots.free(state.slot)
+        if self._lib.fwh_cache_release(self._native, self._id(request)) < 0:
+            raise CacheAccountingError(host.last_error())
+        self._forget(request)
 
     # ----- views for the step function ---------------------------------------------------
     def block_table_rows(self, group_index: int, requests: Sequence[Hashable], stride: Optional[int] = None) -> np.ndarray:
-        group = self.groups[group_index]
-        stride = stride or max([len(group.tables[r]) for r in requests] + [1])
-        rows = np.full((len(requests), stride), 0, dtype=np.int32)
+        natives = host.ids(len(requests))
         for i, request in enumerate(requests):
-            table = group.tables[request]
-            # a page that was given back is never read (the window has passed it); any valid id will do
-            rows[i, :len(table)] = [p if p != NO_PAGE else 0 for p in table]
+            natives[i] = self._live_id(request)
+        if stride is None:
+            stride = max([self.pages_for(self.length_of(r)) for r in requests] +
+                         [len(self.groups[group_index].tables[r]) for r in requests] + [1])
+        rows = np.zeros((len(requests), stride), dtype=np.int32)
+        if self._lib.fwh_cache_fill_tables(self._native, group_index, natives, len(requests), stride, rows.ctypes.data) < 0:
+            raise CacheAccountingError(host.last_error())
         return rows
 
     # ----- accounting -------------------------------------------------------------------
     def check_invariants(self) -> None:
         """No page lost, none held twice; slots likewise."""
-        for group in self.groups:
-            held = [p for table in group.tables.values() for p in table if p != NO_PAGE]
-            if len(held) != len(set(held)):
-                raise CacheAccountingError("a page is held by two block tables")
-            if len(held) != group.pool.in_use:
-                raise CacheAccountingError(f"{group.pool.in_use} pages are out of the pool but tables hold {len(held)}")
-            if any(not group.pool.is_held(p) for p in held):
-                raise CacheAccountingError("a block table holds a page the pool believes free")
-            if set(group.tables) != set(self.requests):
-                raise CacheAccountingError("block tables and live requests differ")
-        slots = [r.slot for r in self.requests.values()]
-        if len(slots) != len(set(slots)) or len(slots) != self.slots.num_slots - self.slots.free_count:
-            raise CacheAccountingError("slot accounting is off")
+        if self._lib.fwh_cache_check(self._native) < 0:
+            raise CacheAccountingError(host.last_error())
 
     def stats(self) -> Dict[str, int]:
         return {

@@ -1,14 +1,15 @@
-"""Page pool, block tables and state slots: the bookkeeping of the cache, host side.
+"""Page pool and state slots: Python faces of the host library's LIFO pools.
 
 A page holds ``page_size`` consecutive tokens of one sequence. The pool is a LIFO stack
 of free page ids, so a page given back is the next one handed out; a sequence's block
 table maps token t to page ``table[t // page_size]``. Same operations as the reference's
-(unwired) primitive: native/src/paged_kv.h:133-204 (pool, ensure/truncate/release).
+(unwired) primitive: native/src/paged_kv.h:133-204 (pool, ensure/truncate/release). The
+bookkeeping itself is C++ (``csrc/host/cache.hpp``).
 """
 
 from __future__ import annotations
 
-from typing import List
+from .. import host
 
 
 class OutOfPages(RuntimeError):
@@ -19,64 +20,76 @@ class CacheAccountingError(AssertionError):
     """A page or slot was freed twice, or freed without being held."""
 
 
-class PagePool:
-    def __init__(self, num_pages: int):
-        if num_pages <= 0:
-            raise ValueError("a page pool needs at least one page")
-        self.num_pages = num_pages
-        self._free: List[int] = list(range(num_pages - 1, -1, -1))   # pop() hands out page 0 first
-        self._held = [False] * num_pages
-        self.peak_in_use = 0
+class _Pool:
+    """A pool of the host library: its own (``size``) or one that lives inside a cache
+    (``borrowed`` handle, freed with the cache)."""
+
+    _empty_message = "out of cache pages"
+    _what = "page"
+
+    def __init__(self, size: int = 0, borrowed=None, owner=None):
+        self._lib = host.library()
+        self._owner = owner                 # keeps the cache alive while its pool is looked at
+        if borrowed is not None:
+            self._handle, self._owned = borrowed, False
+        else:
+            if size <= 0:
+                raise ValueError(f"a {self._what} pool needs at least one {self._what}")
+            self._handle, self._owned = self._lib.fwh_pool_create(size), True
+
+    def __del__(self):
+        if getattr(self, "_owned", False) and self._handle:
+            self._lib.fwh_pool_destroy(self._handle)
+            self._handle = None
+
+    @property
+    def size(self) -> int:
+        return self._lib.fwh_pool_size(self._handle)
 
     @property
     def free_count(self) -> int:
-        return len(self._free)
+        return self._lib.fwh_pool_free_count(self._handle)
 
     @property
     def in_use(self) -> int:
-        return self.num_pages - len(self._free)
-
-    def alloc(self) -> int:
-        if not self._free:
-            raise OutOfPages("out of cache pages")
-        page = self._free.pop()
-        self._held[page] = True
-        self.peak_in_use = max(self.peak_in_use, self.in_use)
-        return page
-
-    def free(self, page: int) -> None:
-        if not 0 <= page < self.num_pages or not self._held[page]:
-            raise CacheAccountingError(f"page {page} is freed but not held")
-        self._held[page] = False
-        self._free.append(page)
-
-    def is_held(self, page: int) -> bool:
-        return self._held[page]
-
-
-class SlotPool:
-    """Slots of fixed-size per-request state; also a LIFO stack."""
-
-    def __init__(self, num_slots: int):
-        if num_slots <= 0:
-            raise ValueError("a slot pool needs at least one slot")
-        self.num_slots = num_slots
-        self._free: List[int] = list(range(num_slots - 1, -1, -1))
-        self._held = [False] * num_slots
+        return self.size - self.free_count
 
     @property
-    def free_count(self) -> int:
-        return len(self._free)
+    def peak_in_use(self) -> int:
+        return self._lib.fwh_pool_peak(self._handle)
 
     def alloc(self) -> int:
-        if not self._free:
-            raise OutOfPages("out of request slots")
-        slot = self._free.pop()
-        self._held[slot] = True
-        return slot
+        got = self._lib.fwh_pool_alloc(self._handle)
+        if got < 0:
+            raise OutOfPages(self._empty_message)
+        return got
 
-    def free(self, slot: int) -> None:
-        if not 0 <= slot < self.num_slots or not self._held[slot]:
-            raise CacheAccountingError(f"slot {slot} is freed but not held")
-        self._held[slot] = False
-        self._free.append(slot)
+    def free(self, index: int) -> None:
+        if self._lib.fwh_pool_free(self._handle, int(index)) < 0:
+            raise CacheAccountingError(f"{self._what} {index} is freed but not held")
+
+    def is_held(self, index: int) -> bool:
+        return bool(self._lib.fwh_pool_is_held(self._handle, int(index)))
+
+
+class PagePool(_Pool):
+    def __init__(self, num_pages: int = 0, borrowed=None, owner=None):
+        super().__init__(num_pages, borrowed, owner)
+
+    @property
+    def num_pages(self) -> int:
+        return self.size
+
+
+class SlotPool(_Pool):
+    """Slots of fixed-size per-request state; also a LIFO stack."""
+
+    _empty_message = "out of request slots"
+    _what = "slot"
+
+    def __init__(self, num_slots: int = 0, borrowed=None, owner=None):
+        super().__init__(num_slots, borrowed, owner)
+
+    @property
+    def num_slots(self) -> int:
+        return self.size

@@ -1,0 +1,211 @@
+// The cache's bookkeeping: LIFO pools, block tables per page group, state slots.
+// Same operations as the reference's (unwired) paging primitive, native/src/paged_kv.h:133-204
+// (pool, ensure / truncate / release), grown by page groups with a window and by slots.
+#pragma once
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace fwh {
+
+struct OutOfPages : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+struct AccountingError : std::logic_error {
+    using std::logic_error::logic_error;
+};
+
+class Pool {
+public:
+    explicit Pool(int size) : held_(size, 0) {
+        if (size <= 0) throw std::invalid_argument("a pool needs at least one entry");
+        free_.reserve(size);
+        for (int id = size - 1; id >= 0; --id) free_.push_back(id);      // id 0 is handed out first
+    }
+    int size() const { return (int)held_.size(); }
+    int free_count() const { return (int)free_.size(); }
+    int in_use() const { return size() - free_count(); }
+    int peak() const { return peak_; }
+    bool is_held(int id) const { return id >= 0 && id < size() && held_[id]; }
+    int alloc() {
+        if (free_.empty()) throw OutOfPages("out of cache pages");
+        const int id = free_.back();
+        free_.pop_back();
+        held_[id] = 1;
+        if (in_use() > peak_) peak_ = in_use();
+        return id;
+    }
+    void free(int id) {
+        if (!is_held(id)) throw AccountingError("id " + std::to_string(id) + " is freed but not held");
+        held_[id] = 0;
+        free_.push_back(id);
+    }
+
+private:
+    std::vector<int> free_;
+    std::vector<char> held_;
+    int peak_ = 0;
+};
+
+constexpr int NO_PAGE = -1;
+
+struct Group {
+    int window;                                             // 0: every key is kept
+    Pool pool;
+    std::unordered_map<int64_t, std::vector<int>> tables;   // request -> page per block (NO_PAGE once given back)
+    Group(int window_, int pages) : window(window_), pool(pages) {}
+};
+
+struct Live {
+    int slot;
+    int length = 0;
+};
+
+class Cache {
+public:
+    Cache(const std::vector<int>& windows, int num_pages, int max_requests, int page_size, int max_pages_per_request)
+        : page_size_(page_size), num_pages_(num_pages), max_requests_(max_requests),
+          max_pages_per_request_(max_pages_per_request > 0 ? max_pages_per_request : num_pages), slots_(max_requests) {
+        if (page_size <= 0 || num_pages <= 0) throw std::invalid_argument("page size and page count must be positive");
+        groups_.reserve(windows.size());
+        for (int window : windows) groups_.emplace_back(window, num_pages);
+    }
+
+    int page_size() const { return page_size_; }
+    int num_pages() const { return num_pages_; }
+    int max_requests() const { return max_requests_; }
+    int max_pages_per_request() const { return max_pages_per_request_; }
+    int num_groups() const { return (int)groups_.size(); }
+    Group& group(int g) { return groups_.at(g); }
+    Pool& slots() { return slots_; }
+    const std::unordered_map<int64_t, Live>& live() const { return live_; }
+
+    int pages_for(int tokens) const { return (tokens + page_size_ - 1) / page_size_; }
+
+    // Blocks before this one hold only keys the window has passed once the sequence is
+    // `length` tokens long (the next query sits at position `length`).
+    int first_needed_block(const Group& group, int length) const {
+        if (group.window <= 0) return 0;
+        const int first_key = length - group.window + 1 > 0 ? length - group.window + 1 : 0;
+        return first_key / page_size_;
+    }
+
+    bool is_live(int64_t request) const { return live_.count(request) != 0; }
+    const Live& of(int64_t request) const {
+        auto it = live_.find(request);
+        if (it == live_.end()) throw std::out_of_range("request " + std::to_string(request) + " is not live");
+        return it->second;
+    }
+
+    // pages a reservation up to new_length would take from group g
+    int pages_missing(int64_t request, int new_length, int g) const {
+        const Group& group = groups_[g];
+        auto it = group.tables.find(request);
+        const int have = it == group.tables.end() ? 0 : (int)it->second.size();
+        const int blocks = pages_for(new_length);
+        return blocks > have ? blocks - have : 0;
+    }
+    bool fits(int64_t request, int new_length) const {
+        if (pages_for(new_length) > max_pages_per_request_) return false;
+        for (int g = 0; g < num_groups(); ++g)
+            if (groups_[g].pool.free_count() < pages_missing(request, new_length, g)) return false;
+        return true;
+    }
+    // free pages of the tightest group
+    int free_pages() const {
+        int least = 1 << 30;
+        for (const Group& group : groups_) least = group.pool.free_count() < least ? group.pool.free_count() : least;
+        return least;
+    }
+
+    int admit(int64_t request) {
+        if (is_live(request)) throw AccountingError("request " + std::to_string(request) + " is already live");
+        if (slots_.free_count() == 0) throw OutOfPages("out of request slots");
+        const int slot = slots_.alloc();
+        live_[request] = Live{slot, 0};
+        for (Group& group : groups_) group.tables[request] = {};
+        return slot;
+    }
+    // Maps pages for positions < new_length in every group, or throws and changes nothing.
+    void reserve(int64_t request, int new_length) {
+        of(request);
+        if (pages_for(new_length) > max_pages_per_request_)
+            throw OutOfPages("request " + std::to_string(request) + " would need " + std::to_string(pages_for(new_length)) +
+                             " pages; a block table holds " + std::to_string(max_pages_per_request_));
+        for (int g = 0; g < num_groups(); ++g) {
+            const int missing = pages_missing(request, new_length, g);
+            if (groups_[g].pool.free_count() < missing)
+                throw OutOfPages("out of cache pages: request " + std::to_string(request) + " needs " + std::to_string(missing) +
+                                 " more, " + std::to_string(groups_[g].pool.free_count()) + " free");
+        }
+        for (int g = 0; g < num_groups(); ++g) {
+            Group& group = groups_[g];
+            std::vector<int>& table = group.tables[request];
+            for (int missing = pages_missing(request, new_length, g); missing > 0; --missing) table.push_back(group.pool.alloc());
+        }
+    }
+    void commit(int64_t request, int new_length) {
+        Live& state = live_.at(request);
+        if (new_length < state.length) throw std::invalid_argument("a sequence does not shrink");
+        state.length = new_length;
+        for (Group& group : groups_) {
+            std::vector<int>& table = group.tables[request];
+            const int passed = first_needed_block(group, new_length);
+            for (int block = 0; block < passed && block < (int)table.size(); ++block)
+                if (table[block] != NO_PAGE) {
+                    group.pool.free(table[block]);
+                    table[block] = NO_PAGE;
+                }
+        }
+    }
+    void release(int64_t request) {
+        auto it = live_.find(request);
+        if (it == live_.end()) throw AccountingError("request " + std::to_string(request) + " is released but not live");
+        for (Group& group : groups_) {
+            auto table = group.tables.find(request);
+            for (int page : table->second)
+                if (page != NO_PAGE) group.pool.free(page);
+            group.tables.erase(table);
+        }
+        slots_.free(it->second.slot);
+        live_.erase(it);
+    }
+
+    // No page lost, none held twice; slots likewise.
+    void check() const {
+        for (const Group& group : groups_) {
+            std::vector<char> seen(num_pages_, 0);
+            int held = 0;
+            for (const auto& entry : group.tables) {
+                if (!live_.count(entry.first)) throw AccountingError("block tables and live requests differ");
+                for (int page : entry.second) {
+                    if (page == NO_PAGE) continue;
+                    if (seen[page]) throw AccountingError("a page is held by two block tables");
+                    if (!group.pool.is_held(page)) throw AccountingError("a block table holds a page the pool believes free");
+                    seen[page] = 1;
+                    ++held;
+                }
+            }
+            if (group.tables.size() != live_.size()) throw AccountingError("block tables and live requests differ");
+            if (held != group.pool.in_use())
+                throw AccountingError(std::to_string(group.pool.in_use()) + " pages are out of the pool but tables hold " +
+                                      std::to_string(held));
+        }
+        std::vector<char> slot_seen(max_requests_, 0);
+        for (const auto& entry : live_) {
+            if (slot_seen[entry.second.slot] || !slots_.is_held(entry.second.slot)) throw AccountingError("slot accounting is off");
+            slot_seen[entry.second.slot] = 1;
+        }
+        if ((int)live_.size() != slots_.in_use()) throw AccountingError("slot accounting is off");
+    }
+
+private:
+    int page_size_, num_pages_, max_requests_, max_pages_per_request_;
+    std::vector<Group> groups_;
+    Pool slots_;
+    std::unordered_map<int64_t, Live> live_;
+};
+
+}  // namespace fwh

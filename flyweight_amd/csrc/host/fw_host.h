@@ -1,0 +1,86 @@
+// Host side of the engine behind a flat C ABI: the cache's bookkeeping (page pools, block
+// tables, state slots) and the continuous-batching scheduler. Nothing here touches the GPU; the
+// Python package holds the tensors and launches the kernels, and asks this library who holds
+// which page and what the next step runs. Built with the host compiler alone.
+//
+// Conventions: a request is a 64-bit id chosen by the caller. Functions return >= 0 on success
+// and a negative code on error, with the text in fwh_last_error() (per thread). FWH_OUT_OF_PAGES
+// is the one expected failure: nothing was changed.
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FWH_ERROR (-1)
+#define FWH_OUT_OF_PAGES (-2)
+#define FWH_NO_PAGE (-1)
+
+const char* fwh_last_error(void);
+int fwh_abi_version(void);
+
+// ---- a LIFO pool of page (or slot) ids: the id given back last is handed out next ---------------
+void* fwh_pool_create(int size);
+void fwh_pool_destroy(void* pool);
+int fwh_pool_alloc(void* pool);                 // id, or FWH_OUT_OF_PAGES
+int fwh_pool_free(void* pool, int id);          // FWH_ERROR if the id is not held
+int fwh_pool_size(void* pool);
+int fwh_pool_free_count(void* pool);
+int fwh_pool_peak(void* pool);                  // most ids out at any time
+int fwh_pool_is_held(void* pool, int id);
+
+// ---- the cache: page groups (window 0: every key is kept), block tables, slots --------------------
+void* fwh_cache_create(int num_groups, const int* windows, int num_pages, int max_requests, int page_size,
+                       int max_pages_per_request);
+void fwh_cache_destroy(void* cache);
+void* fwh_cache_group_pool(void* cache, int group);     // borrowed: lives as long as the cache
+void* fwh_cache_slot_pool(void* cache);
+int fwh_cache_admit(void* cache, int64_t request);      // the slot; FWH_OUT_OF_PAGES when no slot is free
+int fwh_cache_reserve(void* cache, int64_t request, int new_length);    // all groups or nothing
+int fwh_cache_commit(void* cache, int64_t request, int new_length);     // windowed groups give pages back
+int fwh_cache_release(void* cache, int64_t request);
+int fwh_cache_is_live(void* cache, int64_t request);
+int fwh_cache_slot_of(void* cache, int64_t request);
+int fwh_cache_length_of(void* cache, int64_t request);
+int fwh_cache_pages_missing(void* cache, int64_t request, int new_length, int* per_group);
+int fwh_cache_table(void* cache, int64_t request, int group, int* pages, int capacity);     // its length
+// rows of block tables for a batch: pages given back read as page 0 (they are never looked at)
+int fwh_cache_fill_tables(void* cache, int group, const int64_t* requests, int count, int stride, int* rows);
+int fwh_cache_live(void* cache, int64_t* requests, int capacity);       // how many are live
+int fwh_cache_check(void* cache);                       // no page lost, held twice or free while held
+
+// ---- the scheduler ---------------------------------------------------------------------------------
+// Event kinds as the reference numbers them (native/include/flyweight_v2.h:413-417).
+#define FWH_EVENT_TOKEN 0
+#define FWH_EVENT_FINISHED 1
+#define FWH_EVENT_ERROR 2
+#define FWH_EVENT_PREFILL 3
+
+void* fwh_scheduler_create(void* cache, int max_positions, int max_batch_tokens, int chunk_size, int max_live,
+                           int max_queued);
+void fwh_scheduler_destroy(void* scheduler);
+int64_t fwh_scheduler_submit(void* scheduler, const int* prompt, int prompt_len, int max_new_tokens,
+                             const int* stop_tokens, int num_stop);    // the request's id (>= 1)
+int fwh_scheduler_cancel(void* scheduler, int64_t request);            // 1 if it was still going
+int fwh_scheduler_has_work(void* scheduler);
+int fwh_scheduler_preemptions(void* scheduler);
+int fwh_scheduler_queue(void* scheduler, int which, int64_t* requests, int capacity);   // 0 waiting, 1 running
+// Plans the next step (reserving its pages) and keeps the plan until the next call.
+// counts: segments, tokens, preempted, failed, admitted, cancelled.
+int fwh_scheduler_schedule(void* scheduler, int counts[6]);
+int fwh_plan_segments(void* scheduler, int64_t* requests, int* num_tokens, int* wants_logits, int* tokens);
+int fwh_plan_list(void* scheduler, int which, int64_t* requests);      // 0 preempted, 1 failed, 2 admitted, 3 cancelled
+// After the step: the token drawn for every segment that wanted logits. Events (request, token or
+// progress, kind) come back; returns their number (at most 2 per segment plus failed and cancelled).
+int fwh_scheduler_complete(void* scheduler, const int64_t* requests, const int* tokens, int count,
+                           int64_t* event_requests, int* event_values, int* event_kinds, int capacity);
+// info: computed, live, finished, cancelled, admitted_at, preemptions, prompt length, generated length, max_new_tokens
+int fwh_request_info(void* scheduler, int64_t request, int info[9]);
+int fwh_request_generated(void* scheduler, int64_t request, int* tokens, int capacity);
+const char* fwh_request_error(void* scheduler, int64_t request);       // "" if none
+int fwh_scheduler_forget(void* scheduler, int64_t request);            // drops a finished request's record
+
+#ifdef __cplusplus
+}
+#endif

@@ -16,15 +16,19 @@ request that cannot fit alone ends with an error. The reference has no pages to 
 (a slot reserves the whole context, native/src/v2_runtime.cpp:33578-33609) and visits tasks
 round-robin, one prompt chunk or one token per visit (:33730-33787).
 
-This file decides; it runs nothing. It needs only the cache manager's bookkeeping.
+The decisions are made by the host library (C++, ``csrc/host/scheduler.hpp``) on the cache's
+own bookkeeping; this file is its Python face: it keeps what only Python needs of a request
+(sampling configuration, random stream) and turns plans and events into objects. It decides;
+it runs nothing.
 """
 
 from __future__ import annotations
 
-import collections
+import ctypes
 from dataclasses import dataclass, field
-from typing import Deque, Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Dict, List, Optional, Sequence, Tuple
 
+from .. import host
 from ..cache import CacheManager
 from ..sampling import GREEDY, SamplingConfig, make_rng
 
@@ -37,39 +41,59 @@ class SchedulerError(ValueError):
     pass
 
 
-@dataclass
 class Request:
-    id: int
-    prompt: List[int]
-    max_new_tokens: int
-    sampling: SamplingConfig = GREEDY
-    stop_tokens: Tuple[int, ...] = ()
-    generated: List[int] = field(default_factory=list)
-    computed: int = 0               # tokens whose keys/values/state are in the cache
-    live: bool = False
-    finished: bool = False
-    cancelled: bool = False
-    error: Optional[str] = None
-    admitted_at: int = -1           # admission counter: larger = more recent
-    preemptions: int = 0
-    rng: object = None
+    """A request as Python sees it: what was submitted, and a view of its progress, which the
+    host library keeps."""
+
+    def __init__(self, scheduler: "Scheduler", request_id: int, prompt: List[int], max_new_tokens: int,
+                 sampling: SamplingConfig, stop_tokens: Tuple[int, ...]):
+        self._scheduler = scheduler
+        self.id = request_id
+        self.prompt = prompt
+        self.max_new_tokens = max_new_tokens
+        self.sampling = sampling
+        self.stop_tokens = stop_tokens
+        self.rng = make_rng(sampling.seed, request_id)
+
+    def _info(self) -> List[int]:
+        out = host.ints(9)
+        scheduler = self._scheduler
+        if scheduler._lib.fwh_request_info(scheduler._native, self.id, out) < 0:
+            raise SchedulerError(host.last_error())
+        return list(out)
+
+    computed = property(lambda self: self._info()[0])       # tokens whose keys/values/state are in the cache
+    live = property(lambda self: bool(self._info()[1]))
+    finished = property(lambda self: bool(self._info()[2]))
+    cancelled = property(lambda self: bool(self._info()[3]))
+    admitted_at = property(lambda self: self._info()[4])    # admission counter: larger = more recent
+    preemptions = property(lambda self: self._info()[5])
+
+    @property
+    def generated(self) -> List[int]:
+        scheduler = self._scheduler
+        count = self._info()[7]
+        out = host.ints(count)
+        scheduler._lib.fwh_request_generated(scheduler._native, self.id, out, count)
+        return list(out[:count])
+
+    @property
+    def error(self) -> Optional[str]:
+        scheduler = self._scheduler
+        text = scheduler._lib.fwh_request_error(scheduler._native, self.id).decode("utf-8", "replace")
+        return text or None
 
     @property
     def tokens(self) -> List[int]:
         return self.prompt + self.generated
 
-    def tokens_from(self, first: int, count: int) -> List[int]:
-        """tokens[first:first + count] without joining the two lists."""
-        end, split = first + count, len(self.prompt)
-        if end <= split:
-            return self.prompt[first:end]
-        if first >= split:
-            return self.generated[first - split:end - split]
-        return self.prompt[first:] + self.generated[:end - split]
-
     @property
     def remaining(self) -> int:
-        return len(self.prompt) + len(self.generated) - self.computed
+        info = self._info()
+        return info[6] + info[7] - info[0]
+
+    def __repr__(self) -> str:
+        return f"Request({self.id}, prompt of {len(self.prompt)}, max_new_tokens={self.max_new_tokens})"
 
 
 @dataclass
@@ -87,22 +111,7 @@ class StepPlan:
     admitted: List[Request] = field(default_factory=list)
     cancelled: List[Request] = field(default_factory=list)
     num_tokens: int = 0
-    _planned: set = field(default_factory=set)      # ids of the requests that have a segment
-
-    def add(self, segment: PlannedSegment) -> None:
-        self.segments.append(segment)
-        self.num_tokens += len(segment.tokens)
-        self._planned.add(segment.request.id)
-
-    def drop(self, request: Request) -> None:
-        if request.id not in self._planned:
-            return
-        self.num_tokens -= sum(len(s.tokens) for s in self.segments if s.request is request)
-        self.segments = [s for s in self.segments if s.request is not request]
-        self._planned.discard(request.id)
-
-    def has(self, request: Request) -> bool:
-        return request.id in self._planned
+    serial: int = 0         # plans are completed in the order they were made, each once
 
 
 class Scheduler:
@@ -115,12 +124,18 @@ class Scheduler:
         self.max_batch_tokens = max_batch_tokens
         self.chunk_size = chunk_size
         self.max_live = min(max_live or cache.max_requests, cache.max_requests)
-        self.waiting: Deque[Request] = collections.deque()
-        self.running: List[Request] = []        # in admission order, oldest first
         self.requests: Dict[int, Request] = {}
-        self._next_id = 1
-        self._admissions = 0
-        self.preemptions = 0
+        self._lib = host.library()
+        self._native = self._lib.fwh_scheduler_create(cache.native_handle, max_positions, max_batch_tokens, chunk_size,
+                                                      self.max_live, MAX_QUEUED)
+        if not self._native:
+            raise SchedulerError(host.last_error())
+        self._serial = 0
+
+    def __del__(self):
+        if getattr(self, "_native", None):
+            self._lib.fwh_scheduler_destroy(self._native)
+            self._native = None
 
     # ----- submitting -------------------------------------------------------------------
     def submit(self, prompt: Sequence[int], max_new_tokens: int, sampling: SamplingConfig = GREEDY,
@@ -128,167 +143,81 @@ class Scheduler:
         """Validation as the reference's task submit (native/src/v2_runtime.cpp:32502-32520):
         a prompt, room for prompt + output in the context, a bounded queue."""
         prompt = [int(t) for t in prompt]
-        if not prompt:
-            raise SchedulerError("the prompt is empty")
-        if max_new_tokens < 1:
-            raise SchedulerError("max_tokens must be at least 1")
-        if len(prompt) + max_new_tokens > self.max_positions:
-            raise SchedulerError(f"prompt ({len(prompt)}) + max_tokens ({max_new_tokens}) exceeds the context "
-                                 f"of {self.max_positions}")
-        if len(self.waiting) >= MAX_QUEUED:
-            raise SchedulerError(f"the queue holds {MAX_QUEUED} requests already")
-        request = Request(id=self._next_id, prompt=prompt, max_new_tokens=int(max_new_tokens), sampling=sampling,
-                          stop_tokens=tuple(int(t) for t in stop_tokens))
-        request.rng = make_rng(sampling.seed, request.id)
-        self._next_id += 1
-        self.requests[request.id] = request
-        self.waiting.append(request)
+        stop = tuple(int(t) for t in stop_tokens)
+        request_id = self._lib.fwh_scheduler_submit(self._native, (ctypes.c_int * max(len(prompt), 1))(*prompt), len(prompt),
+                                                    int(max_new_tokens), (ctypes.c_int * max(len(stop), 1))(*stop), len(stop))
+        if request_id < 0:
+            raise SchedulerError(host.last_error())
+        request = Request(self, request_id, prompt, int(max_new_tokens), sampling, stop)
+        self.requests[request_id] = request
         return request
 
     def cancel(self, request_id: int) -> bool:
-        request = self.requests.get(request_id)
-        if request is None or request.finished:
+        if request_id not in self.requests:
             return False
-        request.cancelled = True
-        return True
+        return bool(self._lib.fwh_scheduler_cancel(self._native, int(request_id)))
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self._lib.fwh_scheduler_has_work(self._native))
+
+    @property
+    def preemptions(self) -> int:
+        return self._lib.fwh_scheduler_preemptions(self._native)
+
+    def _queue(self, which: int) -> List[Request]:
+        count = self._lib.fwh_scheduler_queue(self._native, which, host.ids(0), 0)
+        out = host.ids(count)
+        self._lib.fwh_scheduler_queue(self._native, which, out, count)
+        return [self.requests[out[i]] for i in range(count)]
+
+    waiting = property(lambda self: self._queue(0))
+    running = property(lambda self: self._queue(1))         # in admission order, oldest first
 
     # ----- planning ---------------------------------------------------------------------
-    def _evict(self, request: Request) -> None:
-        self.cache.release(request.id)
-        request.live = False
-        request.computed = 0
-        self.running.remove(request)
-
-    def _fail(self, request: Request, message: str, plan: StepPlan) -> None:
-        if request.live:
-            self._evict(request)
-        request.error = message
-        request.finished = True
-        plan.failed.append(request)
-
-    def _preempt(self, victim: Request, plan: StepPlan) -> None:
-        plan.drop(victim)
-        self._evict(victim)
-        victim.preemptions += 1
-        self.preemptions += 1
-        self.waiting.appendleft(victim)
-        plan.preempted.append(victim)
-
-    def _fits(self, request: Request, new_length: int) -> bool:
-        cache = self.cache
-        if cache.pages_for(new_length) > cache.max_pages_per_request:
-            return False
-        return all(cache.groups[g].pool.free_count >= n for g, n in cache.pages_missing(request.id, new_length).items())
-
     def schedule(self) -> StepPlan:
-        plan = StepPlan()
-        # cancelled requests leave first
-        for request in [r for r in self.running if r.cancelled]:
-            self._evict(request)
-            request.finished = True
-            plan.cancelled.append(request)
-        for request in [r for r in self.waiting if r.cancelled]:
-            self.waiting.remove(request)
-            request.finished = True
-            plan.cancelled.append(request)
-        while True:
-            self._plan_once(plan)
-            if plan.segments or not self.running:
-                return plan
-            # every running request waits for pages and none can move
-            if len(self.running) == 1:
-                self._fail(self.running[0], "out of cache pages: the request does not fit even alone", plan)
-            else:
-                self._preempt(self.running[-1], plan)
-
-    def _plan_once(self, plan: StepPlan) -> None:
+        """Plans the next step and reserves its pages. The slots of the requests admitted in it
+        start at zero."""
+        counts = host.ints(6)
+        if self._lib.fwh_scheduler_schedule(self._native, counts) < 0:
+            raise SchedulerError(host.last_error())
+        segments, tokens = counts[0], counts[1]
+        self._serial += 1
+        plan = StepPlan(num_tokens=tokens, serial=self._serial)
+        if segments:
+            owners, lengths, wants, flat = host.ids(segments), host.ints(segments), host.ints(segments), host.ints(tokens)
+            self._lib.fwh_plan_segments(self._native, owners, lengths, wants, flat)
+            flat, at = list(flat[:tokens]), 0
+            for i in range(segments):
+                plan.segments.append(PlannedSegment(self.requests[owners[i]], flat[at:at + lengths[i]], bool(wants[i])))
+                at += lengths[i]
+        for which, target in enumerate((plan.preempted, plan.failed, plan.admitted, plan.cancelled)):
+            if counts[2 + which]:
+                out = host.ids(counts[2 + which])
+                self._lib.fwh_plan_list(self._native, which, out)
+                target.extend(self.requests[out[i]] for i in range(counts[2 + which]))
         cache = self.cache
-        planned = plan.has
-
-        # 1. decode rows, oldest first; make room by preempting the newest
-        for request in list(self.running):
-            if not request.live or request.remaining != 1 or planned(request):
-                continue
-            if plan.num_tokens >= self.max_batch_tokens:
-                break
-            while request.live and not self._fits(request, request.computed + 1):
-                if len(self.running) == 1:
-                    self._fail(request, "out of cache pages: the request does not fit even alone", plan)
-                else:
-                    self._preempt(self.running[-1], plan)       # may be the request itself, if it is the newest
-            if not request.live:
-                continue
-            cache.reserve(request.id, request.computed + 1)
-            plan.add(PlannedSegment(request, request.tokens_from(request.computed, 1), True))
-
-        # 2. portions of prompts of running requests, oldest first
-        for request in list(self.running):
-            if request.remaining < 1 or planned(request):
-                continue
-            if plan.num_tokens >= self.max_batch_tokens:
-                break
-            self._plan_portion(request, plan)
-
-        # 3. admissions, in queue order, while everything a first portion needs is there;
-        #    none in a step in which somebody had to give way
-        while (self.waiting and not plan.preempted and plan.num_tokens < self.max_batch_tokens
-               and len(self.running) < self.max_live and cache.slots.free_count > 0):
-            request = self.waiting[0]
-            total = len(request.prompt) + request.max_new_tokens
-            limit = min(cache.max_pages_per_request, cache.num_pages)
-            if cache.groups and cache.pages_for(total) > limit:
-                self.waiting.popleft()
-                self._fail(request, f"the request needs {cache.pages_for(total)} cache pages for {total} tokens; "
-                                    f"the pool holds {limit}", plan)
-                continue
-            portion = min(request.remaining, self.chunk_size, self.max_batch_tokens - plan.num_tokens)
-            if any(group.pool.free_count < cache.pages_for(portion) for group in cache.groups):
-                break
-            self.waiting.popleft()
-            cache.admit(request.id)
-            request.live = True
-            request.admitted_at = self._admissions
-            self._admissions += 1
-            self.running.append(request)
-            plan.admitted.append(request)
-            self._plan_portion(request, plan)
-
-    def _plan_portion(self, request: Request, plan: StepPlan) -> None:
-        portion = min(request.remaining, self.chunk_size, self.max_batch_tokens - plan.num_tokens)
-        # shrink to what the pool can hold right now; a portion may be cut anywhere
-        while portion >= 1 and not self._fits(request, request.computed + portion):
-            portion -= (request.computed + portion) % self.cache.page_size or self.cache.page_size
-        if portion < 1:
-            return
-        self.cache.reserve(request.id, request.computed + portion)
-        plan.add(PlannedSegment(request, request.tokens_from(request.computed, portion), portion == request.remaining))
+        for request in plan.admitted:
+            if request.id in cache.requests:
+                cache.zero_slot(cache.slot_of(request.id))
+        return plan
 
     # ----- after the step ---------------------------------------------------------------
     def complete(self, plan: StepPlan, sampled: Dict[int, int]) -> List[Tuple[int, int, int]]:
         """``sampled``: request id -> token drawn from the logits of its last row. Returns
         events (request id, token or progress, kind)."""
-        events: List[Tuple[int, int, int]] = []
-        for request in plan.failed:
-            events.append((request.id, 0, EVENT_ERROR))
-        for request in plan.cancelled:
-            events.append((request.id, len(request.generated), EVENT_FINISHED))
-        for segment in plan.segments:
-            request = segment.request
-            request.computed += len(segment.tokens)
-            self.cache.commit(request.id, request.computed)
-            if not segment.wants_logits:
-                events.append((request.id, request.computed, EVENT_PREFILL))
-                continue
-            token = int(sampled[request.id])
-            request.generated.append(token)
-            events.append((request.id, token, EVENT_TOKEN))
-            done = (token in request.stop_tokens or len(request.generated) >= request.max_new_tokens
-                    or len(request.prompt) + len(request.generated) >= self.max_positions)
-            if done:
-                self._evict(request)
-                request.finished = True
-                events.append((request.id, len(request.generated), EVENT_FINISHED))
-        return events
+        if plan.serial != self._serial:
+            raise SchedulerError("only the plan made last can be completed, and only once")
+        self._serial += 1
+        wanting = [s.request.id for s in plan.segments if s.wants_logits]
+        missing = [r for r in wanting if r not in sampled]
+        if missing:
+            raise KeyError(missing[0])
+        owners = (ctypes.c_int64 * max(len(wanting), 1))(*wanting)
+        drawn = (ctypes.c_int * max(len(wanting), 1))(*[int(sampled[r]) for r in wanting])
+        capacity = 2 * len(plan.segments) + len(plan.failed) + len(plan.cancelled) + 1
+        event_owner, event_value, event_kind = host.ids(capacity), host.ints(capacity), host.ints(capacity)
+        count = self._lib.fwh_scheduler_complete(self._native, owners, drawn, len(wanting), event_owner, event_value,
+                                                 event_kind, capacity)
+        if count < 0:
+            raise SchedulerError(host.last_error())
+        return [(event_owner[i], event_value[i], event_kind[i]) for i in range(count)]

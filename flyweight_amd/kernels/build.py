@@ -1,4 +1,5 @@
-"""Builds the gfx950 kernel library from ``csrc/*.hip`` with hipcc.
+"""Builds the gfx950 kernel library from ``csrc/*.hip`` with hipcc, and the host library
+(cache bookkeeping and scheduler, ``csrc/host/*.cpp``) with the host compiler.
 
 The library is built in-tree (``csrc/_build/libflyweight_hip.so``) so that it travels
 with the source tree; when the tree is not writable it is built under the temporary
@@ -143,5 +144,78 @@ def ensure_built() -> str:
         raise
 
 
+# ----- the host library: no GPU code, built with the host compiler alone -------------------------
+HOST_DIR = os.path.join(CSRC, "host")
+HOST_LIB_NAME = "libflyweight_host.so"
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+
+
+def _host_fingerprint() -> str:
+    digest = hashlib.sha256()
+    for name in sorted(os.listdir(HOST_DIR)):
+        if name.endswith((".cpp", ".hpp", ".h")):
+            digest.update(name.encode())
+            with open(os.path.join(HOST_DIR, name), "rb") as handle:
+                digest.update(handle.read())
+    digest.update(" ".join(HOST_FLAGS).encode())
+    return digest.hexdigest()
+
+
+def _host_compiler() -> str:
+    for name in ("g++", "c++", "clang++"):
+        found = shutil.which(name)
+        if found:
+            return found
+    return _hipcc()
+
+
+def find_host_library(require_current: bool = True) -> Optional[str]:
+    wanted = _host_fingerprint() if require_current else None
+    for folder in build_dirs():
+        lib = os.path.join(folder, HOST_LIB_NAME)
+        stamp = os.path.join(folder, "host.stamp")
+        if not os.path.isfile(lib):
+            continue
+        if wanted is None:
+            return lib
+        if os.path.isfile(stamp):
+            with open(stamp, "r", encoding="utf-8") as handle:
+                if handle.read().strip() == wanted:
+                    return lib
+    return None
+
+
+def build_host(verbose: bool = True) -> str:
+    folder = _writable_dir()
+    started = time.time()
+    units = sorted(os.path.join(HOST_DIR, f) for f in os.listdir(HOST_DIR) if f.endswith(".cpp"))
+    lib = os.path.join(folder, HOST_LIB_NAME)
+    partial = lib + f".{os.getpid()}.tmp"
+    result = subprocess.run([_host_compiler(), *HOST_FLAGS, "-o", partial, *units], capture_output=True, text=True)
+    if result.returncode != 0:
+        raise RuntimeError(f"building {HOST_LIB_NAME} failed:\n{result.stderr}")
+    os.replace(partial, lib)
+    with open(os.path.join(folder, "host.stamp"), "w", encoding="utf-8") as handle:
+        handle.write(_host_fingerprint())
+    if verbose:
+        _say(f"built {lib} in {time.time() - started:.0f} s")
+    return lib
+
+
+def ensure_host_built() -> str:
+    lib = find_host_library(require_current=True)
+    if lib is not None:
+        return lib
+    try:
+        return build_host()
+    except RuntimeError:
+        stale = find_host_library(require_current=False)
+        if stale is not None:
+            _say(f"warning: could not rebuild; loading {stale}, which is older than the sources")
+            return stale
+        raise
+
+
 if __name__ == "__main__":
     build()
+    build_host()
