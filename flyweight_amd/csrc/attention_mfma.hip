@@ -5,7 +5,7 @@
 // waves per workgroup sharing the pages through LDS). For decode
 // a column is one of the query heads that share the kv head, and the keys are split between
 // workgroups in runs of SPLIT_PAGES pages whose partial results (running maximum, sum and
-// unnormalised output) a second kernel merges in order.
+// unnormalised output) the workgroup that finishes last merges in the order of the keys.
 //
 // The products are formed transposed so that nothing has to change lanes between them:
 //   S^T[key][col] = K[key][d] . Q^T[d][col]        (v_mfma_f32_16x16x32_bf16, k = d)
@@ -285,15 +285,19 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 // grid (rows, kv heads * head tiles, splits); four waves, each takes one page of the split's
 // SPLIT_PAGES, and their results are merged in LDS in the order of the keys. Columns are the
 // query heads of the kv group (16 per head tile). partial [rows][heads][max_splits][head_dim + 4]:
-// unnormalised output, then maximum and sum; a split with nothing to do writes nothing.
+// unnormalised output, then maximum and sum; a split with nothing to do writes nothing and takes
+// no ticket. The last workgroup of a (row, kv head, head tile) to arrive merges what the others
+// left; the only workgroup of a short row writes the result at once.
 template <int HD>
 __global__ __launch_bounds__(64 * SPLIT_PAGES) void attention_decode_split_kernel(
-    const uint16_t* __restrict__ q, float* __restrict__ partial, const uint16_t* __restrict__ k_pages,
+    const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* partial, int* tickets,
+    const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ row_seg, const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads,
     int head_dim, float scale_log2, int window, int max_splits) {
     __shared__ f32x4 shared_o[SPLIT_PAGES][HD / 16][64];
     __shared__ float shared_m[SPLIT_PAGES][16], shared_l[SPLIT_PAGES][16];
+    __shared__ int ticket_shared;
     const int row = blockIdx.x, split = blockIdx.z;
     const int group = num_heads / num_kv_heads;
     const int head_tiles = (group + 15) / 16;
@@ -329,61 +333,90 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) void attention_decode_split_kerne
         shared_l[wave][col] = l;
     }
     __syncthreads();
-    if (wave != 0 || !valid) return;
-    float m = NEG_BIG;
+    // how many workgroups work on this row: those whose first page holds a visible key
+    const int row_splits = (last_block - first / PAGE + 1 + SPLIT_PAGES - 1) / SPLIT_PAGES;
+    const int stride = PART_STRIDE(head_dim);
+    if (wave == 0 && valid) {
+        float m = NEG_BIG;
 #pragma unroll
-    for (int w = 0; w < SPLIT_PAGES; ++w) m = fmaxf(m, shared_m[w][col]);
-    float total = 0.0f, weight[SPLIT_PAGES];
+        for (int w = 0; w < SPLIT_PAGES; ++w) m = fmaxf(m, shared_m[w][col]);
+        float total = 0.0f, weight[SPLIT_PAGES];
 #pragma unroll
-    for (int w = 0; w < SPLIT_PAGES; ++w) {
-        weight[w] = exp2f(shared_m[w][col] - m);        // a wave without a page has l = 0 and o = 0
-        total += weight[w] * shared_l[w][col];
-    }
-    float* dest = partial + (((size_t)row * num_heads + head) * max_splits + split) * PART_STRIDE(head_dim);
+        for (int w = 0; w < SPLIT_PAGES; ++w) {
+            weight[w] = exp2f(shared_m[w][col] - m);        // a wave without a page has l = 0 and o = 0
+            total += weight[w] * shared_l[w][col];
+        }
+        float* dest = partial + (((size_t)row * num_heads + head) * max_splits + split) * stride;
+        uint16_t* final_dest = out + ((size_t)row * num_heads + head) * head_dim;
 #pragma unroll
-    for (int t = 0; t < HD / 16; ++t) {
-        if (t * 16 >= head_dim) break;
-        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < HD / 16; ++t) {
+            if (t * 16 >= head_dim) break;
+            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int w = 0; w < SPLIT_PAGES; ++w) sum += weight[w] * shared_o[w][t][lane];
-        *reinterpret_cast<f32x4*>(dest + t * 16 + g * 4) = sum;
-    }
-    if (g == 0) {
-        dest[head_dim] = m;
-        dest[head_dim + 1] = total;
-    }
-}
-
-// grid (rows, heads): merges the splits of one (row, head) in order of the keys.
-__global__ __launch_bounds__(64) void attention_decode_merge_kernel(
-    const float* __restrict__ partial, uint16_t* __restrict__ out, const int32_t* __restrict__ row_pos, int num_heads,
-    int head_dim, int window, int max_splits) {
-    const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-    const int pos = row_pos[row];
-    const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
-    const int blocks = pos / PAGE - first / PAGE + 1;
-    const int splits = (blocks + SPLIT_PAGES - 1) / SPLIT_PAGES;
-    const float* source = partial + ((size_t)row * num_heads + head) * max_splits * PART_STRIDE(head_dim);
-    float m = NEG_BIG;
-    for (int s = 0; s < splits; ++s) m = fmaxf(m, source[(size_t)s * PART_STRIDE(head_dim) + head_dim]);
-    float total = 0.0f;
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < splits; ++s) {
-        const float* part = source + (size_t)s * PART_STRIDE(head_dim);
-        const float weight = exp2f(part[head_dim] - m);
-        total += weight * part[head_dim + 1];
+            for (int w = 0; w < SPLIT_PAGES; ++w) sum += weight[w] * shared_o[w][t][lane];
+            if (row_splits == 1) {
+                // the only workgroup of its row: the result is final
+                const float inv = 1.0f / total;
+                u32x2 packed = {pack_bf16(sum[0] * inv, sum[1] * inv), pack_bf16(sum[2] * inv, sum[3] * inv)};
+                *reinterpret_cast<u32x2*>(final_dest + t * 16 + g * 4) = packed;
+            } else {
+                // device-scope stores: they pass the caches that workgroups on other dies do not share
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int d = lane + 64 * j;
-            if (d < head_dim) acc[j] += weight * part[d];
+                for (int r = 0; r < 4; ++r)
+                    __hip_atomic_store(dest + t * 16 + g * 4 + r, sum[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        if (g == 0 && row_splits > 1) {
+            __hip_atomic_store(dest + head_dim, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(dest + head_dim + 1, total, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-    const float inv = 1.0f / total;
-    uint16_t* dest = out + ((size_t)row * num_heads + head) * head_dim;
+    if (row_splits == 1) return;
+    // The workgroup of a (row, kv head) that arrives last merges the parts, in the order of the keys:
+    // every wave waits for its own stores to be acknowledged, the workgroup meets, one thread
+    // takes the ticket. Nobody waits for another workgroup. The ticket counter is left at zero.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    int* ticket = tickets + (size_t)row * gridDim.y + blockIdx.y;
+    if (threadIdx.x == 0) ticket_shared = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (ticket_shared != row_splits - 1) return;
+    if (threadIdx.x == 0) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int columns = group - head_tile * 16 < 16 ? group - head_tile * 16 : 16;
+    for (int item = threadIdx.x; item < columns * head_dim; item += 64 * SPLIT_PAGES) {
+        const int merged_head = kvh * group + head_tile * 16 + item / head_dim, d = item % head_dim;
+        const float* source = partial + ((size_t)row * num_heads + merged_head) * max_splits * stride;
+        // eight parts are requested at a time (past the last one: the last one again, not used)
+        auto part_at = [&](int sp, int offset) {
+            const int clamped = sp < row_splits ? sp : row_splits - 1;
+            return __hip_atomic_load(source + (size_t)clamped * stride + offset, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        };
+        float m = NEG_BIG;
+        for (int sp0 = 0; sp0 < row_splits; sp0 += 8) {
+            float ms[8];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int d = lane + 64 * j;
-        if (d < head_dim) dest[d] = float_to_bf16_bits(acc[j] * inv);
+            for (int u = 0; u < 8; ++u) ms[u] = part_at(sp0 + u, head_dim);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) m = fmaxf(m, ms[u]);
+        }
+        float total = 0.0f, acc = 0.0f;
+        for (int sp0 = 0; sp0 < row_splits; sp0 += 8) {
+            float ms[8], ls[8], vs[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                ms[u] = part_at(sp0 + u, head_dim);
+                ls[u] = part_at(sp0 + u, head_dim + 1);
+                vs[u] = part_at(sp0 + u, d);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (sp0 + u >= row_splits) break;
+                const float weight = exp2f(ms[u] - m);
+                total += weight * ls[u];
+                acc += weight * vs[u];
+            }
+        }
+        out[((size_t)row * num_heads + merged_head) * head_dim + d] = float_to_bf16_bits(acc / total);
     }
 }
 
@@ -442,9 +475,11 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
 
 // One row per request. partial: float32 workspace of rows * heads * max_splits * (head_dim + 4).
 // max_context: no row's position reaches it (the caller knows; the kernel cannot check);
-// max_splits must cover the keys such a row sees, in runs of 4 pages.
+// max_splits must cover the keys such a row sees, in runs of 4 pages. tickets: rows * kv heads *
+// ceil(group / 16) int32 counters, zero before the first call and left zero; calls that overlap on
+// one device need their own (and their own workspace).
 extern "C" int fw_attention_decode(const void* q, void* out, float* partial, int max_splits, int max_context,
-                                   const void* k_pages,
+                                   int* tickets, int tickets_len, const void* k_pages,
                                    const void* v_pages, const int32_t* block_table, int table_stride,
                                    const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                                    int num_kv_heads, int head_dim, float scale, int window, int page_size,
@@ -464,16 +499,15 @@ extern "C" int fw_attention_decode(const void* q, void* out, float* partial, int
     const int group = num_heads / num_kv_heads;
     const int head_tiles = (group + 15) / 16;
     FW_REQUIRE(rows <= 1 << 20 && num_kv_heads * head_tiles <= 65535 && num_heads <= 65535, "attention_decode: grid too large");
+    FW_REQUIRE(max_splits == 1 || (tickets != nullptr && (long long)tickets_len >= (long long)rows * num_kv_heads * head_tiles),
+               "attention_decode: %d rows need %d ticket counters", rows, rows * num_kv_heads * head_tiles);
     dim3 grid(rows, num_kv_heads * head_tiles, max_splits);
 #define CALL(HD)                                                                                                   \
     attention_decode_split_kernel<HD><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                                        \
-        (const uint16_t*)q, partial, (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table, table_stride, \
-        row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits)
+        (const uint16_t*)q, (uint16_t*)out, partial, tickets, (const uint16_t*)k_pages, (const uint16_t*)v_pages, \
+        block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits)
     FW_BY_HEAD_DIM(head_dim, CALL);
 #undef CALL
-    FW_LAUNCH_CHECK("attention_decode_split");
-    attention_decode_merge_kernel<<<dim3(rows, num_heads), 64, 0, (hipStream_t)stream>>>(
-        partial, (uint16_t*)out, row_pos, num_heads, head_dim, window, max_splits);
-    FW_LAUNCH_CHECK("attention_decode_merge");
+    FW_LAUNCH_CHECK("attention_decode");
     return 0;
 }

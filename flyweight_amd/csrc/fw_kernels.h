@@ -42,10 +42,13 @@ int fw_gemm_mfma(const void* a, const void* w, const float* bias, void* out, int
 // few features (decode steps of 17..64 requests). fw_gemm_medium_plan says what a shape needs:
 // bytes of workspace (0: none) and int32 counters (0: none) that are zero before the first call;
 // the kernel leaves them zero. Calls that overlap on one device need their own of both.
-int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* workspace_bytes, int* counters);
+// The accumulating product of up to 16 rows can leave what the norm after it needs, as
+// fw_gemm_decode does (next_activations [M][N] bfloat16, next_squares [squares_rows][16]).
+int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* workspace_bytes, int* counters, int* squares_rows);
 int fw_gemm_medium(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                    int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
-                   int counters_len, void* stream);
+                   int counters_len, const float* next_norm_weight, int next_one_centered,
+                   void* next_activations, float* next_squares, void* stream);
 
 // Fused product for decode steps of up to 16 rows. prologue 0: a is bfloat16 [M][K]; 1: a is
 // float32 rows, RMS-normed with norm_weight/eps (rows gathered through row_index if given) inside
@@ -111,10 +114,12 @@ int fw_attention_prefill(const void* q, void* out, const void* k_pages, const vo
                          int rows, int num_heads, int num_kv_heads, int head_dim, float scale, int window,
                          int page_size, int num_pages, void* stream);
 // Decode (one row per request): the keys are split between workgroups in runs of 4 pages and
-// merged in order. partial: float32 workspace [rows][heads][max_splits][head_dim + 4];
-// max_context: an upper bound on position + 1 of every row, known to the caller.
+// merged in order by the workgroup that finishes last. partial: float32 workspace
+// [rows][heads][max_splits][head_dim + 4]; max_context: an upper bound on position + 1 of every
+// row, known to the caller; tickets: rows * kv_heads * ceil(heads / kv_heads / 16) int32 counters,
+// zero before the first call and left zero.
 int fw_attention_decode(const void* q, void* out, float* partial, int max_splits, int max_context,
-                        const void* k_pages, const void* v_pages, const int32_t* block_table, int table_stride,
+                        int* tickets, int tickets_len, const void* k_pages, const void* v_pages, const int32_t* block_table, int table_stride,
                         const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
                         int head_dim, float scale, int window, int page_size, int num_pages, void* stream);
 

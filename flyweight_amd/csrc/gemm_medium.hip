@@ -44,6 +44,11 @@ struct MediumArgs {
     int splits;
     float* partials;        // [splits][tiles][kinds * MT][FW][64][4]
     int* counters;          // [tiles], zero between calls
+    // accumulating product of up to 16 rows: what the norm after it will need (all null: nothing)
+    const float* next_norm_weight;  // [N]
+    int next_one_centered;
+    uint16_t* next_activations;     // bfloat16 [M][N] = x_new * (w_next or 1 + w_next)
+    float* next_squares;            // [tiles * FW][16]: this wave's sum of x_new^2 per row
 };
 
 __device__ __forceinline__ float gm_silu(float g) {
@@ -228,46 +233,69 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
     // D layout of the 16x16 product: lane holds features 4 * (lane / 16) + r of the wave's tile
     // for row lane % 16 of a
     const int n_first = n0 + 16 * ft + 4 * g;
+    const bool whole = n_first + 3 < N && (N & 3) == 0;     // four features in one aligned piece
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + r16;
-        if (m >= M) continue;
-        float value[4];
+        const bool mine = m < M;
+        const size_t at = (size_t)(mine ? m : 0) * N + n_first;
+        float v[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int n = n_first + r;
-            if (MODE == GM_SWIGLU) {
-                value[r] = gm_silu(acc[0][mt][r]) * acc[1][mt][r];
+            if (MODE == GM_SWIGLU) v[r] = gm_silu(acc[0][mt][r]) * acc[1][mt][r];
+            else v[r] = acc[0][mt][r] + ((p.bias && n < N) ? p.bias[n] : 0.0f);
+        }
+        if (mine) {
+            if constexpr (sizeof(TO) == 4) {
+                float* to = reinterpret_cast<float*>(p.out) + at;
+                if (whole) {
+                    f32x4 packed = {v[0], v[1], v[2], v[3]};
+                    if (MODE == GM_ACCUMULATE) {
+                        const f32x4 old = *reinterpret_cast<const f32x4*>(to);
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) packed[r] = v[r] = v[r] + old[r];
+                    }
+                    *reinterpret_cast<f32x4*>(to) = packed;
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (n_first + r >= N) continue;
+                        if (MODE == GM_ACCUMULATE) v[r] += to[r];
+                        to[r] = v[r];
+                    }
+                }
             } else {
-                value[r] = acc[0][mt][r] + ((p.bias && n < N) ? p.bias[n] : 0.0f);
+                uint16_t* to = reinterpret_cast<uint16_t*>(p.out) + at;
+                if (whole) {
+                    uint2 packed;
+                    packed.x = (uint32_t)float_to_bf16_bits(v[0]) | ((uint32_t)float_to_bf16_bits(v[1]) << 16);
+                    packed.y = (uint32_t)float_to_bf16_bits(v[2]) | ((uint32_t)float_to_bf16_bits(v[3]) << 16);
+                    *reinterpret_cast<uint2*>(to) = packed;
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (n_first + r < N) to[r] = float_to_bf16_bits(v[r]);
+                }
             }
         }
-        TO* out = static_cast<TO*>(p.out);
-        const size_t at = (size_t)m * N + n_first;
-        if (n_first + 3 < N && (N & 3) == 0) {
-            if constexpr (sizeof(TO) == 4) {
-                f32x4* to = reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p.out) + at);
-                f32x4 v = {value[0], value[1], value[2], value[3]};
-                if (MODE == GM_ACCUMULATE) {
-                    const f32x4 old = *to;
+        // what the norm after this addition needs (decode steps of up to 16 rows): x * w of that
+        // norm in bfloat16, and this wave's sum of x^2 per row; the product that follows forms the
+        // row's 1/rms from those sums
+        if (MODE == GM_ACCUMULATE && MT == 1 && p.next_activations) {
+            float row_square = 0.0f;
+            if (mine)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) v[r] += old[r];
+                for (int r = 0; r < 4; ++r) {
+                    const int n = n_first + r;
+                    if (n >= N) continue;
+                    const float w = p.next_norm_weight[n] + (p.next_one_centered ? 1.0f : 0.0f);
+                    p.next_activations[at + r] = float_to_bf16_bits(v[r] * w);
+                    row_square += v[r] * v[r];
                 }
-                *to = v;
-            } else {
-                uint2 packed;
-                packed.x = (uint32_t)float_to_bf16_bits(value[0]) | ((uint32_t)float_to_bf16_bits(value[1]) << 16);
-                packed.y = (uint32_t)float_to_bf16_bits(value[2]) | ((uint32_t)float_to_bf16_bits(value[3]) << 16);
-                *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p.out) + at) = packed;
-            }
-        } else {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                if (n_first + r >= N) continue;
-                float v = value[r];
-                if (MODE == GM_ACCUMULATE) v += load_as_float(out, at + r);
-                store_from_float(out, at + r, v);
-            }
+            row_square += __shfl_xor(row_square, 16, 64);
+            row_square += __shfl_xor(row_square, 32, 64);
+            if (g == 0) p.next_squares[((size_t)tile * FW + ft) * 16 + r16] = row_square;
         }
     }
 }
@@ -277,6 +305,7 @@ struct MediumPlan {
     int mt, fw, tiles, splits, k_per_split;
     size_t workspace_bytes;
 };
+
 
 static MediumPlan medium_plan(int M, int N, int K, int mode) {
     MediumPlan plan;
@@ -303,13 +332,15 @@ static MediumPlan medium_plan(int M, int N, int K, int mode) {
     return plan;
 }
 
-// What fw_gemm_medium needs for a shape: bytes of workspace (0: none) and the number of int32
-// counters (0: none); the counters must be zero before the first call and are left zero.
-extern "C" int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* workspace_bytes, int* counters) {
+// What fw_gemm_medium needs for a shape: bytes of workspace (0: none), the number of int32
+// counters (0: none; they must be zero before the first call and are left zero), and how many
+// rows of 16 the sums of squares for the next norm take.
+extern "C" int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* workspace_bytes, int* counters, int* squares_rows) {
     FW_REQUIRE(M >= 1 && M <= 64 && N > 0 && K > 0, "gemm_medium: takes 1..64 rows, got M %d N %d K %d", M, N, K);
     const MediumPlan plan = medium_plan(M, N, K, mode);
     *workspace_bytes = plan.workspace_bytes;
     *counters = plan.splits > 1 ? plan.tiles : 0;
+    *squares_rows = plan.tiles * plan.fw;       // first extent of the sums of squares left for the next norm
     return 0;
 }
 
@@ -327,7 +358,8 @@ static void medium_launch(const MediumArgs& args, int out_dtype, int mode, dim3 
 // device must not share counters or workspace.
 extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                               int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
-                              int counters_len, void* stream) {
+                              int counters_len, const float* next_norm_weight, int next_one_centered,
+                              void* next_activations, float* next_squares, void* stream) {
     FW_REQUIRE(M >= 1 && M <= 64, "gemm_medium: takes 1..64 rows, got %d", M);
     FW_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_medium: K (%d) must be a positive multiple of 8, N (%d) positive", K, N);
     FW_REQUIRE(mode >= 0 && mode <= 2, "gemm_medium: unknown mode %d", mode);
@@ -336,6 +368,10 @@ extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, v
     FW_REQUIRE(out_dtype == FW_F32 || out_dtype == FW_BF16, "gemm_medium: unknown out dtype %d", out_dtype);
     FW_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0) && ((uintptr_t)out % 16 == 0) && ((uintptr_t)workspace % 16 == 0),
                "gemm_medium: operands must be 16-byte aligned");
+    FW_REQUIRE((next_activations == nullptr) == (next_squares == nullptr) && (next_activations == nullptr) == (next_norm_weight == nullptr),
+               "gemm_medium: the next norm's weight, activations and sums of squares come together");
+    FW_REQUIRE(next_activations == nullptr || (mode == GM_ACCUMULATE && M <= 16),
+               "gemm_medium: only the accumulating product of up to 16 rows prepares the next norm");
     const MediumPlan plan = medium_plan(M, N, K, mode);
     FW_REQUIRE(plan.splits == 1 || (workspace != nullptr && workspace_bytes >= plan.workspace_bytes && counters != nullptr &&
                                     counters_len >= plan.tiles),
@@ -345,6 +381,8 @@ extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, v
     args.a = (const uint16_t*)a; args.w = (const uint16_t*)w; args.bias = bias; args.out = out;
     args.M = M; args.N = N; args.K = K; args.k_per_split = plan.k_per_split; args.splits = plan.splits;
     args.partials = (float*)workspace; args.counters = counters;
+    args.next_norm_weight = next_norm_weight; args.next_one_centered = next_one_centered;
+    args.next_activations = (uint16_t*)next_activations; args.next_squares = next_squares;
     const dim3 grid(plan.tiles, plan.splits);
     hipStream_t s = (hipStream_t)stream;
     if (plan.fw == 4) {

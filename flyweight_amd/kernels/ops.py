@@ -322,14 +322,15 @@ _MEDIUM_COUNTERS = {}
 
 
 def _medium_counters(device: torch.device, count: int) -> torch.Tensor:
-    """Zeroed int32 counters for the medium product's tickets, one set per device: the kernel
+    """Zeroed int32 counters for the tickets of the kernels whose last workgroup finishes the
+    work of the others (the medium product, decode attention), one set per device: each kernel
     leaves them at zero, and calls on one device follow each other in stream order (work on
     several streams of one device at once would need a set per stream)."""
     have = _MEDIUM_COUNTERS.get(device.index)
     if have is None or have.numel() < count:
         if torch.cuda.is_current_stream_capturing():
             raise KernelError("gemm_medium: its counters must exist before a graph is captured (prepare_device)")
-        have = torch.zeros(max(count, 8192), dtype=torch.int32, device=device)
+        have = torch.zeros(max(count, 65536), dtype=torch.int32, device=device)
         _MEDIUM_COUNTERS[device.index] = have
     return have
 
@@ -340,18 +341,29 @@ def prepare_device(device: torch.device) -> None:
     _medium_counters(torch.device(device), 0)
 
 
-def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int) -> None:
-    """The product for 1..64 rows with K split over workgroups (fw_gemm_medium)."""
+def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int,
+                     next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False):
+    """The product for 1..64 rows with K split over workgroups (fw_gemm_medium). With
+    ``next_norm_weight`` (accumulating product of up to 16 rows) returns what the norm after it
+    needs: (activations x * w_next, sums of squares)."""
     M, K = a.shape
-    need_bytes, need_counters = ctypes.c_size_t(0), ctypes.c_int(0)
-    _check(library().fw_gemm_medium_plan(M, N, K, mode, ctypes.byref(need_bytes), ctypes.byref(need_counters)))
-    workspace = counters = None
+    need_bytes, need_counters, squares_rows = ctypes.c_size_t(0), ctypes.c_int(0), ctypes.c_int(0)
+    _check(library().fw_gemm_medium_plan(M, N, K, mode, ctypes.byref(need_bytes), ctypes.byref(need_counters),
+                                         ctypes.byref(squares_rows)))
+    workspace = counters = next_activations = next_squares = None
     if need_bytes.value:
         workspace = torch.empty(need_bytes.value // 4, dtype=torch.float32, device=a.device)
         counters = _medium_counters(a.device, need_counters.value)
+    if next_norm_weight is not None:
+        next_activations = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
+        next_squares = torch.empty((squares_rows.value, 16), dtype=torch.float32, device=a.device)
     _check(library().fw_gemm_medium(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K, _p(workspace),
                                     ctypes.c_size_t(need_bytes.value), _p(counters),
-                                    0 if counters is None else counters.numel(), _stream()))
+                                    0 if counters is None else counters.numel(), _p(next_norm_weight),
+                                    int(next_one_centered), _p(next_activations), _p(next_squares), _stream()))
+    if next_norm_weight is not None:
+        return next_activations, next_squares
+    return None
 
 
 def _fast_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -405,6 +417,7 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
 # ---- fused products for decode steps of up to 16 rows --------------------------------------------
 EPILOGUE_STORE, EPILOGUE_ACCUMULATE, EPILOGUE_SWIGLU, EPILOGUE_CONV = 0, 1, 2, 3
 DECODE_MAX_ROWS = 16
+LONG_K = 4096
 
 
 def gemm_decode_fits(rows: int, features: int, k: int, epilogue: int) -> bool:
@@ -466,9 +479,14 @@ def gemm_decode(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
         out_dtype = out_dtype or torch.bfloat16
         target = torch.empty((rows, N), dtype=out_dtype, device=a.device)
     next_activations = next_squares = None
+    if next_norm_weight is not None and (epilogue != EPILOGUE_ACCUMULATE or next_norm_weight.dtype != torch.float32
+                                         or next_norm_weight.shape != (N,)):
+        raise KernelError("gemm_decode: only the accumulating product prepares the next norm, whose weight is float32 [N]")
+    if epilogue == EPILOGUE_ACCUMULATE and K >= LONG_K and N <= 4096:
+        # few features and a long K: the kernel that splits K over workgroups streams W faster
+        left = gemm_medium_into(a, w, bias, target, F32, 1, N, next_norm_weight, next_one_centered)
+        return target if left is None else left
     if next_norm_weight is not None:
-        if epilogue != EPILOGUE_ACCUMULATE or next_norm_weight.dtype != torch.float32 or next_norm_weight.shape != (N,):
-            raise KernelError("gemm_decode: only the accumulating product prepares the next norm, whose weight is float32 [N]")
         next_activations = torch.empty((rows, N), dtype=torch.bfloat16, device=a.device)
         next_squares = torch.empty((library().fw_gemm_decode_accumulate_tiles(N), 16), dtype=torch.float32, device=a.device)
     prologue = 1 if normed else (2 if squares is not None else 0)
@@ -545,8 +563,11 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
     splits = decode_splits(max_context, window)
     partial = torch.empty((rows, num_heads, splits, head_dim + 4), dtype=torch.float32, device=q.device)
     out = torch.empty_like(q)
+    group = num_heads // num_kv_heads
+    tickets = _medium_counters(q.device, rows * num_kv_heads * ((group + 15) // 16))
     _check(library().fw_attention_decode(
-        _p(q), _p(out), _p(partial), splits, int(max_context), _p(k_pages), _p(v_pages), _p(block_table),
+        _p(q), _p(out), _p(partial), splits, int(max_context), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages),
+        _p(block_table),
         block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale),
         int(window), PAGE_SIZE, pages, _stream()))
     return out

@@ -477,7 +477,7 @@ def test_attention_decode_on_the_matrix_cores(ops, nh, nkv, hd, window):
         partial = torch.empty(rows * nh * (hd + 4), device=DEV)
         status = ops.library().fw_attention_decode(
             ctypes.c_void_p(q.data_ptr()), ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(partial.data_ptr()), 1, 100000,
-            ctypes.c_void_p(k_pages.data_ptr()), ctypes.c_void_p(v_pages.data_ptr()), ctypes.c_void_p(d(table).data_ptr()),
+            None, 0, ctypes.c_void_p(k_pages.data_ptr()), ctypes.c_void_p(v_pages.data_ptr()), ctypes.c_void_p(d(table).data_ptr()),
             table.shape[1], ctypes.c_void_p(d(np.arange(rows)).data_ptr()), ctypes.c_void_p(d(positions).data_ptr()), rows, nh,
             nkv, hd, ctypes.c_float(scale), 0, 64, 40, None)
         ops._check(status)
@@ -615,12 +615,13 @@ def test_fused_decode_product_with_the_convolution_epilogue(ops, M, H, L, with_b
 
 
 @pytest.mark.parametrize("M", [1, 6, 16])
-@pytest.mark.parametrize("H,N,one_centered", [(72, 80, False), (200, 96, True), (4104, 144, False), (2048, 6144, True)])
-def test_fused_decode_product_prepares_the_next_norm(ops, M, H, N, one_centered):
+@pytest.mark.parametrize("H,N,one_centered,K", [(72, 80, False, 136), (200, 96, True, 136), (4104, 144, False, 136),
+                                                 (2048, 6144, True, 136), (2048, 96, False, 8192), (104, 96, True, 4104)])
+def test_fused_decode_product_prepares_the_next_norm(ops, M, H, N, one_centered, K):
     """The product that adds to the residual stream leaves x * w of the norm after it and sums
     of squares per tile; the next product takes both instead of norming itself. Checked: what
-    is left, and the next product (every epilogue that may follow) against a plain norm."""
-    K = 136
+    is left, and the next product (every epilogue that may follow) against a plain norm. With a
+    long K the accumulating product is the one that splits K over workgroups."""
     a = as_dev(gen(M, K, seed=1), torch.bfloat16)
     w_out = as_dev(gen(H, K, seed=2, scale=K ** -0.5), torch.bfloat16)
     residual = gen(M, H, seed=3, scale=2).float().to(DEV)
