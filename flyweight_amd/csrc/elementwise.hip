@@ -216,10 +216,42 @@ extern "C" int fw_topk_rows(const float* logits, float* values, int32_t* ids, in
     return 0;
 }
 
-extern "C" int fw_argmax_rows(const float* logits, int32_t* ids, int rows, int vocab, void* stream) {
-    FW_REQUIRE(rows >= 0 && vocab > 0, "argmax_rows: bad sizes rows=%d vocab=%d", rows, vocab);
+// Argmax in two steps, so that a few rows of a wide vocabulary still fill the chip: grid (parts,
+// rows) finds the best key of each part of a row, then one wave per row finds the best of those.
+// Keys order by value, then by the lower id, so the result does not depend on the cut.
+#define ARGMAX_PARTS 64
+__global__ __launch_bounds__(256) void argmax_parts_kernel(const float* __restrict__ logits,
+                                                           unsigned long long* __restrict__ best_of_part, int vocab) {
+    __shared__ unsigned long long scratch[16];
+    const int part = blockIdx.x, row = blockIdx.y;
+    const int per_part = (vocab + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
+    const int begin = part * per_part, end = begin + per_part < vocab ? begin + per_part : vocab;
+    const float* source = logits + (size_t)row * vocab;
+    unsigned long long best = 0;
+    for (int i = begin + threadIdx.x; i < end; i += blockDim.x) {
+        const unsigned long long key = candidate_key(source[i], i);
+        if (key > best) best = key;
+    }
+    best = block_max_u64(best, scratch);
+    if (threadIdx.x == 0) best_of_part[(size_t)row * ARGMAX_PARTS + part] = best;
+}
+
+__global__ __launch_bounds__(64) void argmax_finish_kernel(const unsigned long long* __restrict__ best_of_part,
+                                                           int32_t* __restrict__ ids) {
+    const int row = blockIdx.x;
+    unsigned long long best = best_of_part[(size_t)row * ARGMAX_PARTS + threadIdx.x];     // 64 parts, 64 lanes
+    best = wave_max_u64(best);
+    if (threadIdx.x == 0) ids[row] = (int)(0xffffffffu - (uint32_t)(best & 0xffffffffull));
+}
+
+// workspace: rows * 64 64-bit words (the best key of each part of each row)
+extern "C" int fw_argmax_rows(const float* logits, int32_t* ids, void* workspace, int rows, int vocab, void* stream) {
+    FW_REQUIRE(rows >= 0 && rows <= 65535 && vocab > 0, "argmax_rows: bad sizes rows=%d vocab=%d", rows, vocab);
     if (rows == 0) return 0;
-    topk_rows_kernel<<<rows, 1024, 0, (hipStream_t)stream>>>(logits, nullptr, ids, vocab, 1);
+    FW_REQUIRE(workspace != nullptr && (uintptr_t)workspace % 8 == 0, "argmax_rows: needs an 8-byte aligned workspace");
+    argmax_parts_kernel<<<dim3(ARGMAX_PARTS, rows), 256, 0, (hipStream_t)stream>>>(logits, (unsigned long long*)workspace, vocab);
+    FW_LAUNCH_CHECK("argmax_rows (parts)");
+    argmax_finish_kernel<<<rows, 64, 0, (hipStream_t)stream>>>((const unsigned long long*)workspace, ids);
     FW_LAUNCH_CHECK("argmax_rows");
     return 0;
 }

@@ -286,7 +286,8 @@ def argmax_rows(logits: torch.Tensor) -> torch.Tensor:
     _want(logits, torch.float32, "logits")
     rows, vocab = logits.shape
     ids = torch.empty((rows,), dtype=torch.int32, device=logits.device)
-    _check(library().fw_argmax_rows(_p(logits), _p(ids), rows, vocab, _stream()))
+    workspace = torch.empty((max(rows, 1), 64), dtype=torch.int64, device=logits.device)       # best key of each part
+    _check(library().fw_argmax_rows(_p(logits), _p(ids), _p(workspace), rows, vocab, _stream()))
     return ids
 
 
