@@ -165,6 +165,9 @@ public:
     std::vector<Event> complete(const std::unordered_map<int64_t, int>& sampled) {
         std::vector<Event> events;
         Plan& plan = plan_;
+        for (const Segment& segment : plan.segments)       // nothing changes unless every token is there
+            if (segment.wants_logits && !sampled.count(segment.request->id))
+                throw SchedulerError("no token was handed over for request " + std::to_string(segment.request->id));
         for (Request* request : plan.failed) events.push_back({request->id, 0, EVENT_ERROR});
         for (Request* request : plan.cancelled) events.push_back({request->id, (int)request->generated.size(), EVENT_FINISHED});
         for (const Segment& segment : plan.segments) {
@@ -175,10 +178,7 @@ public:
                 events.push_back({request->id, request->computed, EVENT_PREFILL});
                 continue;
             }
-            auto drawn = sampled.find(request->id);
-            if (drawn == sampled.end())
-                throw SchedulerError("no token was handed over for request " + std::to_string(request->id));
-            const int token = drawn->second;
+            const int token = sampled.find(request->id)->second;
             request->generated.push_back(token);
             events.push_back({request->id, token, EVENT_TOKEN});
             const bool stop = std::find(request->stop_tokens.begin(), request->stop_tokens.end(), token) != request->stop_tokens.end();
