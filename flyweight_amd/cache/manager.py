@@ -249,6 +249,38 @@ class CacheManager:
         if status < 0:
             raise CacheAccountingError(host.last_error())
 
+    # ----- a whole step at once (one call into the host library each) ------------------------------
+    def _natives(self, requests: Sequence[Hashable]):
+        natives = host.ids(len(requests))
+        for i, request in enumerate(requests):
+            native = self._id(request, create=False)
+            natives[i] = -1 if native is None else native
+        return natives
+
+    def describe(self, requests: Sequence[Hashable]) -> Tuple[List[int], List[int]]:
+        """(lengths, slots) of live requests; KeyError names the first one that is not live."""
+        count = len(requests)
+        lengths, slots = host.ints(count), host.ints(count)
+        if self._lib.fwh_cache_describe(self._native, self._natives(requests), count, lengths, slots) < 0:
+            raise KeyError(next((r for r in requests if r not in self.requests), host.last_error()))
+        return list(lengths[:count]), list(slots[:count])
+
+    def reserve_all(self, requests: Sequence[Hashable], new_lengths: Sequence[int]) -> None:
+        """The reservations of a whole step: all of them, or OutOfPages and nothing changed."""
+        count = len(requests)
+        status = self._lib.fwh_cache_reserve_batch(self._native, self._natives(requests),
+                                                   (ctypes.c_int * max(count, 1))(*[int(n) for n in new_lengths]), count)
+        if status == host.OUT_OF_PAGES:
+            raise OutOfPages(host.last_error())
+        if status < 0:
+            raise KeyError(host.last_error())
+
+    def commit_all(self, requests: Sequence[Hashable], new_lengths: Sequence[int]) -> None:
+        count = len(requests)
+        if self._lib.fwh_cache_commit_batch(self._native, self._natives(requests),
+                                            (ctypes.c_int * max(count, 1))(*[int(n) for n in new_lengths]), count) < 0:
+            raise ValueError(host.last_error())
+
     def commit(self, request: Hashable, new_length: int) -> None:
         if request not in self.requests:
             raise KeyError(request)

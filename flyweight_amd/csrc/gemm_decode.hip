@@ -81,9 +81,10 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
 
     const bool a_ok = r16 < M;
     const int a_index = a_ok ? (PRO == 1 && p.row_index ? p.row_index[r16] : r16) : 0;     // (pre-normed rows are never gathered)
-    const uint16_t* a_bf16 = static_cast<const uint16_t*>(p.a) + (size_t)a_index * K + g * 8;
-    const float* a_f32 = static_cast<const float*>(p.a) + (size_t)a_index * K + g * 8;
-    const float* norm_w = p.norm_weight + g * 8;
+    // pointers to the rows; the column (k + 8 g) is added at each load so that it can be clamped
+    const uint16_t* a_bf16 = static_cast<const uint16_t*>(p.a) + (size_t)a_index * K;
+    const float* a_f32 = static_cast<const float*>(p.a) + (size_t)a_index * K;
+    const float* norm_w = p.norm_weight;
     const float one = p.one_centered ? 1.0f : 0.0f;
 
     float prepared_square = 0.0f;
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
             const int feature = tile * ROWS + (ROWS == 16 ? r16 : (r16 & 7));
             const int n = TILED ? feature + rt * p.tile_stride : feature + rt * ROWS * num_tiles;
             w_ok[rt] = TILED ? feature < N : n < N;
-            w_row[rt] = p.w + (size_t)(w_ok[rt] ? n : 0) * K + g * 8;
+            w_row[rt] = p.w + (size_t)(w_ok[rt] ? n : 0) * K;
         }
         f32x4 acc[RT];
 #pragma unroll
@@ -125,7 +126,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
                 // would make the compiler wait for all loads in flight at the next wait.
                 const int k = k0 + j * 32;
                 const bool ok = k + g * 8 < K;          // K is a multiple of 8: a run of 8 is in or out as a whole
-                const int from = ok ? k : 0;
+                const int from = ok ? k + g * 8 : 0;    // columns 0..7 always exist
                 const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {

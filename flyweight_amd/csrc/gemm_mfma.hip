@@ -61,7 +61,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
 
-    // what this thread copies: runs of 16 bytes at (row tid / 8 + 32 i, k 8 * (tid % 8))
+    // what this thread copies: runs of 16 bytes at (row tid / 8 + 32 i, k 8 * (tid % 8)); the
+    // pointers are to the rows, the column is added at each load so that it can be clamped
     const uint16_t* a_src[4];
     const uint16_t* w_src[W_CHUNKS];
     int lds_at[4];
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
         const int row = (tid >> 3) + 32 * i;
         int am = m0 + row;
         am = am < M ? am : M - 1;                       // rows past the end are computed and dropped
-        a_src[i] = a + (size_t)am * K + kc;
+        a_src[i] = a + (size_t)am * K;
         lds_at[i] = row * ROW_BYTES + (tid & 7) * 16;
         if (i < W_CHUNKS) {
             int wr;
@@ -79,7 +80,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
             else wr = n0 + row;
             const int limit = MODE == MF_SWIGLU ? (row < BN / 2 ? N : up_offset + N) : N;
             wr = wr < limit ? wr : limit - 1;
-            w_src[i] = w + (size_t)wr * K + kc;
+            w_src[i] = w + (size_t)wr * K;
         }
     }
 
@@ -100,7 +101,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
         // Every load is issued unconditionally (past the end of K from column 0) and nothing
         // touches the value until it moves to LDS: a branch around a load, or arithmetic right
         // behind it, would make the compiler wait for loads in flight.
-        const int from = k0 + kc < K ? k0 : 0;          // K is a multiple of 8
+        const int from = k0 + kc < K ? k0 + kc : 0;     // K is a multiple of 8: columns 0..7 always exist
 #pragma unroll
         for (int i = 0; i < 4; ++i) ra[i] = *reinterpret_cast<const u32x4*>(a_src[i] + from);
 #pragma unroll

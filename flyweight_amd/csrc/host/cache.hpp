@@ -146,6 +146,22 @@ public:
             for (int missing = pages_missing(request, new_length, g); missing > 0; --missing) table.push_back(group.pool.alloc());
         }
     }
+    // The reservations of a whole step: all of them, or OutOfPages and nothing changed.
+    void reserve_batch(const int64_t* requests, const int* new_lengths, int count) {
+        std::vector<int> needed(groups_.size(), 0);
+        for (int i = 0; i < count; ++i) {
+            of(requests[i]);
+            if (pages_for(new_lengths[i]) > max_pages_per_request_)
+                throw OutOfPages("request " + std::to_string(requests[i]) + " would need " + std::to_string(pages_for(new_lengths[i])) +
+                                 " pages; a block table holds " + std::to_string(max_pages_per_request_));
+            for (int g = 0; g < num_groups(); ++g) needed[g] += pages_missing(requests[i], new_lengths[i], g);
+        }
+        for (int g = 0; g < num_groups(); ++g)
+            if (groups_[g].pool.free_count() < needed[g])
+                throw OutOfPages("out of cache pages: the step needs " + std::to_string(needed[g]) + " more, " +
+                                 std::to_string(groups_[g].pool.free_count()) + " free");
+        for (int i = 0; i < count; ++i) reserve(requests[i], new_lengths[i]);
+    }
     void commit(int64_t request, int new_length) {
         Live& state = live_.at(request);
         if (new_length < state.length) throw std::invalid_argument("a sequence does not shrink");

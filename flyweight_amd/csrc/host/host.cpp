@@ -114,6 +114,29 @@ int fwh_cache_fill_tables(void* cache, int group, const int64_t* requests, int c
         return 0;
     });
 }
+int fwh_cache_describe(void* cache, const int64_t* requests, int count, int* lengths, int* slots) {
+    return guarded([&] {
+        fwh::Cache* c = cache_of(cache);
+        for (int i = 0; i < count; ++i) {
+            const fwh::Live& live = c->of(requests[i]);
+            lengths[i] = live.length;
+            slots[i] = live.slot;
+        }
+        return 0;
+    });
+}
+int fwh_cache_reserve_batch(void* cache, const int64_t* requests, const int* new_lengths, int count) {
+    return guarded([&] {
+        cache_of(cache)->reserve_batch(requests, new_lengths, count);
+        return 0;
+    });
+}
+int fwh_cache_commit_batch(void* cache, const int64_t* requests, const int* new_lengths, int count) {
+    return guarded([&] {
+        for (int i = 0; i < count; ++i) cache_of(cache)->commit(requests[i], new_lengths[i]);
+        return 0;
+    });
+}
 int fwh_cache_live(void* cache, int64_t* requests, int capacity) {
     int n = 0;
     for (const auto& entry : cache_of(cache)->live()) {

@@ -32,47 +32,64 @@ class StepEntry:
     want: Sequence[int] = ()       # places among ``tokens`` whose logits are asked for
 
 
+def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int, max_positions: int):
+    """What a step may not bring: no entries, an unknown or repeated request, no tokens, a token
+    outside the vocabulary, a place outside the entry, a sequence past the model's limit.
+    Returns the requests' current lengths and slots (one call into the host library)."""
+    if not entries:
+        raise StepError("a step needs at least one entry")
+    requests = [entry.request for entry in entries]
+    if len(set(requests)) != len(requests):
+        seen = set()
+        for request in requests:
+            if request in seen:
+                raise StepError(f"request {request!r} appears twice in one step")
+            seen.add(request)
+    try:
+        lengths, slots = cache.describe(requests)
+    except KeyError as error:
+        raise StepError(f"request {error.args[0]!r} was not admitted") from None
+    for entry, start in zip(entries, lengths):
+        n = len(entry.tokens)
+        if n < 1:
+            raise StepError(f"request {entry.request!r} brings no tokens")
+        if start + n > max_positions:
+            raise StepError(f"request {entry.request!r} would reach {start + n} tokens; the model's limit is {max_positions}")
+        low, high = (min(entry.tokens), max(entry.tokens)) if n > 1 else (entry.tokens[0], entry.tokens[0])
+        if not (0 <= int(low) and int(high) < vocab_size):
+            bad = next(t for t in entry.tokens if not 0 <= int(t) < vocab_size)
+            raise StepError(f"token id {bad} of request {entry.request!r} is outside the vocabulary (0..{vocab_size - 1})")
+        for place in entry.want:
+            if not 0 <= int(place) < n:
+                raise StepError(f"request {entry.request!r} wants logits at place {place} of {n} tokens")
+    return lengths, slots
+
+
 class StepContext:
     """The batch as the kernels see it: per-row and per-segment index arrays on the
     device (one upload), block tables per page group, and per-step tables of the position
     encodings."""
 
     def __init__(self, entries: Sequence[StepEntry], cache: CacheManager, device: torch.device, vocab_size: int,
-                 max_positions: int):
-        if not entries:
-            raise StepError("a step needs at least one entry")
-        seen = set()
+                 max_positions: int, described=None):
+        """``described``: (lengths, slots) of the entries' requests if the caller has checked the
+        entries already (``check_entries``)."""
+        starts, slots = described if described is not None else check_entries(entries, cache, vocab_size, max_positions)
         tokens: List[int] = []
         row_pos: List[int] = []
         row_seg: List[int] = []
         seg_row0: List[int] = [0]
-        seg_slot: List[int] = []
+        seg_slot: List[int] = list(slots)
         want_rows: List[int] = []
-        self.requests: List[Hashable] = []
+        self.requests: List[Hashable] = [entry.request for entry in entries]
         self.new_lengths: List[int] = []
-        for seg, entry in enumerate(entries):
-            if entry.request in seen:
-                raise StepError(f"request {entry.request!r} appears twice in one step")
-            seen.add(entry.request)
+        for seg, (entry, start) in enumerate(zip(entries, starts)):
             n = len(entry.tokens)
-            if n < 1:
-                raise StepError(f"request {entry.request!r} brings no tokens")
-            start = cache.length_of(entry.request)
-            if start + n > max_positions:
-                raise StepError(f"request {entry.request!r} would reach {start + n} tokens; the model's limit is {max_positions}")
-            for t in entry.tokens:
-                if not 0 <= int(t) < vocab_size:
-                    raise StepError(f"token id {t} of request {entry.request!r} is outside the vocabulary (0..{vocab_size - 1})")
-            for place in entry.want:
-                if not 0 <= int(place) < n:
-                    raise StepError(f"request {entry.request!r} wants logits at place {place} of {n} tokens")
-                want_rows.append(len(tokens) + int(place))
+            want_rows.extend(len(tokens) + int(place) for place in entry.want)
             tokens.extend(int(t) for t in entry.tokens)
             row_pos.extend(range(start, start + n))
             row_seg.extend([seg] * n)
             seg_row0.append(len(tokens))
-            seg_slot.append(cache.slot_of(entry.request))
-            self.requests.append(entry.request)
             self.new_lengths.append(start + n)
         self.num_rows = len(tokens)
         self.num_segments = len(entries)
@@ -134,18 +151,24 @@ class StepContext:
         self._position_tables = {}
         return self
 
-    def refresh(self, entries: Sequence[StepEntry], cache: CacheManager) -> None:
+    def refresh(self, entries: Sequence[StepEntry], cache: CacheManager, described=None) -> None:
         """Writes this step's tokens, positions, slots and block tables and uploads them."""
         host = self._host
         self.requests = [e.request for e in entries]
-        starts = [cache.length_of(r) for r in self.requests]
+        starts, slots = described if described is not None else cache.describe(self.requests)
+        uploaded = getattr(self, "_uploaded", None)
+        if uploaded is not None:
+            uploaded.synchronize()      # the pinned buffer is still being read until the last upload has run
         self.new_lengths = [s + 1 for s in starts]
         host[0][:] = [int(e.tokens[0]) for e in entries]
         host[1][:] = starts
-        host[4][:] = [cache.slot_of(r) for r in self.requests]
+        host[4][:] = slots
         for g in range(len(cache.groups)):
             host[8 + g][:] = cache.block_table_rows(g, self.requests, stride=self._table_stride).reshape(-1)
         self.device_buffer.copy_(self.host_buffer, non_blocking=True)
+        if uploaded is None:
+            uploaded = self._uploaded = torch.cuda.Event()
+        uploaded.record()
 
     def position_tables(self, part):
         key = part.key()
@@ -201,50 +224,18 @@ class Stepper:
         OutOfPages, having changed nothing, when the cache cannot hold the new tokens."""
         cache = self.cache
         spec = self.model.spec
-        if not entries:
-            raise StepError("a step needs at least one entry")
-        seen = set()
-        for entry in entries:
-            if entry.request not in cache.requests:
-                raise StepError(f"request {entry.request!r} was not admitted")
-            if entry.request in seen:
-                raise StepError(f"request {entry.request!r} appears twice in one step")
-            seen.add(entry.request)
-            if len(entry.tokens) < 1:
-                raise StepError(f"request {entry.request!r} brings no tokens")
-            if cache.length_of(entry.request) + len(entry.tokens) > spec.max_positions:
-                raise StepError(f"request {entry.request!r} would reach "
-                                f"{cache.length_of(entry.request) + len(entry.tokens)} tokens; the model's limit is "
-                                f"{spec.max_positions}")
-            for t in entry.tokens:
-                if not 0 <= int(t) < spec.vocab_size:
-                    raise StepError(f"token id {t} of request {entry.request!r} is outside the vocabulary "
-                                    f"(0..{spec.vocab_size - 1})")
-            for place in entry.want:
-                if not 0 <= int(place) < len(entry.tokens):
-                    raise StepError(f"request {entry.request!r} wants logits at place {place} of {len(entry.tokens)} tokens")
+        described = check_entries(entries, cache, spec.vocab_size, spec.max_positions)
+        requests = [entry.request for entry in entries]
+        new_lengths = [start + len(entry.tokens) for entry, start in zip(entries, described[0])]
         # reserve everything first so that a failure leaves no request half-served
-        needed = {g: 0 for g in range(len(cache.groups))}
-        for entry in entries:
-            new_length = cache.length_of(entry.request) + len(entry.tokens)
-            if cache.pages_for(new_length) > cache.max_pages_per_request:
-                raise OutOfPages(f"request {entry.request!r} would need {cache.pages_for(new_length)} pages; "
-                                 f"a block table holds {cache.max_pages_per_request}")
-            for g, count in cache.pages_missing(entry.request, new_length).items():
-                needed[g] += count
-        for g, count in needed.items():
-            if cache.groups[g].pool.free_count < count:
-                raise OutOfPages(f"out of cache pages: the step needs {count} more, {cache.groups[g].pool.free_count} free")
-        for entry in entries:
-            cache.reserve(entry.request, cache.length_of(entry.request) + len(entry.tokens))
+        cache.reserve_all(requests, new_lengths)
         if self.use_graphs and all(len(entry.tokens) == 1 for entry in entries):
             captured = self._captured_decode(len(entries))
             if captured is not None:
-                return self._replay(captured, entries)
-        ctx = StepContext(entries, cache, self.device, self.model.spec.vocab_size, self.model.spec.max_positions)
+                return self._replay(captured, entries, described)
+        ctx = StepContext(entries, cache, self.device, spec.vocab_size, spec.max_positions, described=described)
         logits = self.model.forward(ctx, cache)
-        for request, length in zip(ctx.requests, ctx.new_lengths):
-            cache.commit(request, length)
+        cache.commit_all(ctx.requests, ctx.new_lengths)
         self.steps += 1
         self.tokens_run += ctx.num_rows
         return logits
@@ -267,10 +258,10 @@ class Stepper:
         self._graphs[batch] = captured
         return captured
 
-    def _replay(self, captured: "_CapturedDecode", entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def _replay(self, captured: "_CapturedDecode", entries: Sequence[StepEntry], described=None) -> Optional[torch.Tensor]:
         cache = self.cache
         ctx = captured.ctx
-        ctx.refresh(entries, cache)
+        ctx.refresh(entries, cache, described)
         if captured.graph is None:
             # record the step once; recording runs nothing, the replay below does
             side = torch.cuda.Stream()
@@ -283,8 +274,7 @@ class Stepper:
             captured.graph = graph
         captured.graph.replay()
         self.graph_replays += 1
-        for request, length in zip(ctx.requests, ctx.new_lengths):
-            cache.commit(request, length)
+        cache.commit_all(ctx.requests, ctx.new_lengths)
         self.steps += 1
         self.tokens_run += ctx.num_rows
         wanted = [i for i, entry in enumerate(entries) if len(entry.want)]
