@@ -48,8 +48,17 @@ struct MediumArgs {
     const float* next_norm_weight;  // [N]
     int next_one_centered;
     uint16_t* next_activations;     // bfloat16 [M][N] = x_new * (w_next or 1 + w_next)
-    float* next_squares;            // [tiles * FW][16]: this wave's sum of x_new^2 per row
+    float* next_squares;            // [tiles * FW][row stride]: this wave's sum of x_new^2 per row (rows >= M: unspecified)
+    // prepared activations: a = x * w of an RMS norm, left by an accumulating product together with
+    // these sums; the rows' 1/rms is formed here and applied to the sums of the product
+    const float* squares;           // [squares_rows][row stride]
+    int squares_rows;
+    float eps;
 };
+
+// rows of the sums of squares are 16 wide for up to 16 rows of a (the fused decode product's
+// layout), 64 wide beyond
+__host__ __device__ inline int gm_square_stride(int M) { return M <= 16 ? 16 : 64; }
 
 __device__ __forceinline__ float gm_silu(float g) {
     if (g >= 0.0f) return g / (1.0f + __expf(-g));
@@ -71,10 +80,25 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
     __shared__ __attribute__((aligned(16))) uint16_t a_lds[2][MT * 16][STRIDE];
     __shared__ float k_parts[KP > 1 ? KP - 1 : 1][KP > 1 ? FW : 1][KP > 1 ? KINDS * MT : 1][KP > 1 ? 64 : 1][4];
     __shared__ int ticket_shared;
+    __shared__ float square_parts[GM_THREADS], inv_rows[64];
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
     const int ft = wave % FW, kp = wave / FW;
     const int M = p.M, N = p.N, K = p.K;
+    // prepared activations: this thread's share of the sums of squares of one row, requested first
+    const int square_stride = gm_square_stride(M);
+    float square_share = 0.0f;
+    if (p.squares) {
+        const int row = threadIdx.x % square_stride, part = threadIdx.x / square_stride, parts = GM_THREADS / square_stride;
+        const float* from = p.squares + row;
+        float share[4] = {0.f, 0.f, 0.f, 0.f};
+        int e = part;
+        for (; e + 3 * parts < p.squares_rows; e += 4 * parts)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) share[u] += from[(size_t)(e + u * parts) * square_stride];
+        for (; e < p.squares_rows; e += parts) share[0] += from[(size_t)e * square_stride];
+        square_share = (share[0] + share[1]) + (share[2] + share[3]);
+    }
     const int tile = blockIdx.x, tiles = gridDim.x;
     const int n0 = tile * 16 * FW;
     const int k_begin = blockIdx.y * p.k_per_split;
@@ -150,7 +174,14 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
 #pragma unroll
     for (int d = 0; d < GM_DEPTH; ++d) load(d, d);
     stage(0, 0, 0);
+    if (p.squares) square_parts[threadIdx.x] = square_share;
     fw_lds_barrier();
+    if (p.squares && threadIdx.x < square_stride) {
+        // the shares of a row meet in a fixed order; read in the epilogue, many barriers from here
+        float total = 0.0f;
+        for (int part = 0; part < GM_THREADS / square_stride; ++part) total += square_parts[part * square_stride + threadIdx.x];
+        inv_rows[threadIdx.x] = rsqrtf(total / (float)K + p.eps);
+    }
     for (int c0 = 0; c0 < iterations; c0 += GM_DEPTH) {
 #pragma unroll
         for (int d = 0; d < GM_DEPTH; ++d) {
@@ -240,11 +271,12 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
         const bool mine = m < M;
         const size_t at = (size_t)(mine ? m : 0) * N + n_first;
         float v[4];
+        const float inv = p.squares ? inv_rows[mine ? m : 0] : 1.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int n = n_first + r;
-            if (MODE == GM_SWIGLU) v[r] = gm_silu(acc[0][mt][r]) * acc[1][mt][r];
-            else v[r] = acc[0][mt][r] + ((p.bias && n < N) ? p.bias[n] : 0.0f);
+            if (MODE == GM_SWIGLU) v[r] = gm_silu(acc[0][mt][r] * inv) * (acc[1][mt][r] * inv);
+            else v[r] = acc[0][mt][r] * inv + ((p.bias && n < N) ? p.bias[n] : 0.0f);
         }
         if (mine) {
             if constexpr (sizeof(TO) == 4) {
@@ -279,10 +311,9 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
                 }
             }
         }
-        // what the norm after this addition needs (decode steps of up to 16 rows): x * w of that
-        // norm in bfloat16, and this wave's sum of x^2 per row; the product that follows forms the
-        // row's 1/rms from those sums
-        if (MODE == GM_ACCUMULATE && MT == 1 && p.next_activations) {
+        // what the norm after this addition needs: x * w of that norm in bfloat16, and this wave's
+        // sum of x^2 per row; the product that follows forms the row's 1/rms from those sums
+        if (MODE == GM_ACCUMULATE && p.next_activations) {
             float row_square = 0.0f;
             if (mine)
 #pragma unroll
@@ -295,7 +326,7 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
                 }
             row_square += __shfl_xor(row_square, 16, 64);
             row_square += __shfl_xor(row_square, 32, 64);
-            if (g == 0) p.next_squares[((size_t)tile * FW + ft) * 16 + r16] = row_square;
+            if (g == 0) p.next_squares[((size_t)tile * FW + ft) * square_stride + m] = row_square;
         }
     }
 }
@@ -340,7 +371,7 @@ extern "C" int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* worksp
     const MediumPlan plan = medium_plan(M, N, K, mode);
     *workspace_bytes = plan.workspace_bytes;
     *counters = plan.splits > 1 ? plan.tiles : 0;
-    *squares_rows = plan.tiles * plan.fw;       // first extent of the sums of squares left for the next norm
+    *squares_rows = plan.tiles * plan.fw;       // first extent of the sums of squares left for the next norm (the second: 16 for M <= 16, else 64)
     return 0;
 }
 
@@ -359,7 +390,8 @@ static void medium_launch(const MediumArgs& args, int out_dtype, int mode, dim3 
 extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                               int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
                               int counters_len, const float* next_norm_weight, int next_one_centered,
-                              void* next_activations, float* next_squares, void* stream) {
+                              void* next_activations, float* next_squares, const float* squares, int squares_rows,
+                              float eps, void* stream) {
     FW_REQUIRE(M >= 1 && M <= 64, "gemm_medium: takes 1..64 rows, got %d", M);
     FW_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_medium: K (%d) must be a positive multiple of 8, N (%d) positive", K, N);
     FW_REQUIRE(mode >= 0 && mode <= 2, "gemm_medium: unknown mode %d", mode);
@@ -370,8 +402,8 @@ extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, v
                "gemm_medium: operands must be 16-byte aligned");
     FW_REQUIRE((next_activations == nullptr) == (next_squares == nullptr) && (next_activations == nullptr) == (next_norm_weight == nullptr),
                "gemm_medium: the next norm's weight, activations and sums of squares come together");
-    FW_REQUIRE(next_activations == nullptr || (mode == GM_ACCUMULATE && M <= 16),
-               "gemm_medium: only the accumulating product of up to 16 rows prepares the next norm");
+    FW_REQUIRE(next_activations == nullptr || mode == GM_ACCUMULATE, "gemm_medium: only the accumulating product prepares the next norm");
+    FW_REQUIRE(squares == nullptr || (squares_rows >= 1 && eps > 0.0f), "gemm_medium: prepared activations come with their sums of squares and eps");
     const MediumPlan plan = medium_plan(M, N, K, mode);
     FW_REQUIRE(plan.splits == 1 || (workspace != nullptr && workspace_bytes >= plan.workspace_bytes && counters != nullptr &&
                                     counters_len >= plan.tiles),
@@ -383,6 +415,7 @@ extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, v
     args.partials = (float*)workspace; args.counters = counters;
     args.next_norm_weight = next_norm_weight; args.next_one_centered = next_one_centered;
     args.next_activations = (uint16_t*)next_activations; args.next_squares = next_squares;
+    args.squares = squares; args.squares_rows = squares_rows; args.eps = eps;
     const dim3 grid(plan.tiles, plan.splits);
     hipStream_t s = (hipStream_t)stream;
     if (plan.fw == 4) {

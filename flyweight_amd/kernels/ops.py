@@ -343,10 +343,12 @@ def prepare_device(device: torch.device) -> None:
 
 
 def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int,
-                     next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False):
+                     next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False,
+                     squares: Optional[torch.Tensor] = None, eps: float = 0.0):
     """The product for 1..64 rows with K split over workgroups (fw_gemm_medium). With
-    ``next_norm_weight`` (accumulating product of up to 16 rows) returns what the norm after it
-    needs: (activations x * w_next, sums of squares)."""
+    ``squares`` ``a`` holds prepared activations (x * w of an RMS norm) and the rows' 1/rms is
+    formed from those sums. With ``next_norm_weight`` (accumulating product) returns what the
+    norm after it needs: (activations x * w_next, sums of squares)."""
     M, K = a.shape
     need_bytes, need_counters, squares_rows = ctypes.c_size_t(0), ctypes.c_int(0), ctypes.c_int(0)
     _check(library().fw_gemm_medium_plan(M, N, K, mode, ctypes.byref(need_bytes), ctypes.byref(need_counters),
@@ -355,16 +357,53 @@ def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tenso
     if need_bytes.value:
         workspace = torch.empty(need_bytes.value // 4, dtype=torch.float32, device=a.device)
         counters = _medium_counters(a.device, need_counters.value)
+    stride = 16 if M <= DECODE_MAX_ROWS else 64
     if next_norm_weight is not None:
         next_activations = torch.empty((M, N), dtype=torch.bfloat16, device=a.device)
-        next_squares = torch.empty((squares_rows.value, 16), dtype=torch.float32, device=a.device)
+        next_squares = torch.empty((squares_rows.value, stride), dtype=torch.float32, device=a.device)
+    if squares is not None and (squares.dtype != torch.float32 or squares.dim() != 2 or squares.shape[1] != stride
+                                or not squares.is_contiguous()):
+        raise KernelError(f"gemm_medium: sums of squares for {M} rows are float32 [n, {stride}]")
     _check(library().fw_gemm_medium(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K, _p(workspace),
                                     ctypes.c_size_t(need_bytes.value), _p(counters),
                                     0 if counters is None else counters.numel(), _p(next_norm_weight),
-                                    int(next_one_centered), _p(next_activations), _p(next_squares), _stream()))
+                                    int(next_one_centered), _p(next_activations), _p(next_squares), _p(squares),
+                                    0 if squares is None else squares.shape[0], ctypes.c_float(eps), _stream()))
     if next_norm_weight is not None:
         return next_activations, next_squares
     return None
+
+
+def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Optional[torch.Tensor] = None,
+                out_dtype: Optional[torch.dtype] = None, accumulate_into: Optional[torch.Tensor] = None,
+                squares: Optional[torch.Tensor] = None, eps: float = 0.0,
+                next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False):
+    """The medium product with the fused decode product's conventions (EPILOGUE_STORE /
+    ACCUMULATE / SWIGLU): returns the output, or for an accumulation with ``next_norm_weight``
+    what the norm after it needs."""
+    _dev(a, w, bias, accumulate_into, squares, next_norm_weight)
+    _want(a, torch.bfloat16, "a")
+    _want(w, torch.bfloat16, "w")
+    M, K = a.shape
+    kinds = 2 if epilogue == EPILOGUE_SWIGLU else 1
+    if not 1 <= M <= MEDIUM_MAX_ROWS or w.shape[1] != K or w.shape[0] % kinds or K % 8 or epilogue not in (0, 1, 2):
+        raise KernelError(f"gemm_medium: a is {tuple(a.shape)}, w is {tuple(w.shape)}, epilogue {epilogue}")
+    N = w.shape[0] // kinds
+    if bias is not None and (bias.dtype != torch.float32 or bias.shape != (w.shape[0],)):
+        raise KernelError("gemm_medium: bias must be float32, one entry per row of w")
+    if next_norm_weight is not None and (epilogue != EPILOGUE_ACCUMULATE or next_norm_weight.dtype != torch.float32
+                                         or next_norm_weight.shape != (N,)):
+        raise KernelError("gemm_medium: only the accumulating product prepares the next norm, whose weight is float32 [N]")
+    if epilogue == EPILOGUE_ACCUMULATE:
+        _want(accumulate_into, torch.float32, "accumulate_into")
+        if accumulate_into.shape != (M, N):
+            raise KernelError(f"gemm_medium: destination is {tuple(accumulate_into.shape)}, expected {(M, N)}")
+        left = gemm_medium_into(a, w, bias, accumulate_into, F32, 1, N, next_norm_weight, next_one_centered, squares, eps)
+        return accumulate_into if left is None else left
+    out_dtype = torch.bfloat16 if epilogue == EPILOGUE_SWIGLU else (out_dtype or torch.bfloat16)
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    gemm_medium_into(a, w, bias, out, _code(out_dtype), epilogue, N, squares=squares, eps=eps)
+    return out
 
 
 def _fast_ok(a: torch.Tensor, w: torch.Tensor) -> bool:

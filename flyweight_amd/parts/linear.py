@@ -62,9 +62,28 @@ class Linear:
     def _tensor_of(a: Input) -> torch.Tensor:
         return a.tensor() if isinstance(a, LazyNorm) else a
 
+    def _medium(self, a: Input) -> bool:
+        """17..64 rows of a bfloat16 model: the product that splits K over workgroups, which
+        takes prepared activations and prepares the next norm as the fused decode product does."""
+        if self.weight.dtype != torch.bfloat16 or a.dtype != torch.bfloat16 or self.in_features % 8:
+            return False
+        rows = a.rows if isinstance(a, LazyNorm) else a.shape[0]
+        if not ops.DECODE_MAX_ROWS < rows <= ops.MEDIUM_MAX_ROWS:
+            return False
+        return not isinstance(a, LazyNorm) or a.prepared is not None
+
+    @staticmethod
+    def _prepared_arguments(a: Input) -> dict:
+        if not isinstance(a, LazyNorm):
+            return {}
+        return {"squares": a.prepared.squares, "eps": a.rms_parameters()[1]}
+
     # ----- products -----------------------------------------------------------------------
     def forward(self, a: Input, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         out_dtype = out_dtype or a.dtype
+        if self._medium(a):
+            return ops.gemm_medium(self._rows_of(a), self.weight, ops.EPILOGUE_STORE, bias=self.bias, out_dtype=out_dtype,
+                                   **self._prepared_arguments(a))
         if self._fused(a, self.out_features, ops.EPILOGUE_STORE):
             return ops.gemm_decode(self._rows_of(a), self.weight, ops.EPILOGUE_STORE, bias=self.bias, out_dtype=out_dtype,
                                    **self._norm_arguments(a))
@@ -74,9 +93,19 @@ class Linear:
         """residual += a . W^T. ``then`` names the norm that will read the residual next, if the
         caller knows it and this is the last change before it: the fused kernel then leaves that
         norm's work behind (returned; None when it did not)."""
+        parameters = then.rms_parameters() if hasattr(then, "rms_parameters") else None
+        if parameters is not None and (parameters[0].shape != (self.out_features,) or then.dtype != torch.bfloat16):
+            parameters = None
+        if self._medium(a):
+            if parameters is not None:
+                activations, squares = ops.gemm_medium(a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias,
+                                                       accumulate_into=residual, next_norm_weight=parameters[0],
+                                                       next_one_centered=parameters[2])
+                return Prepared(then, activations, squares)
+            ops.gemm_medium(a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias, accumulate_into=residual)
+            return None
         if self._fused(a, self.out_features, ops.EPILOGUE_ACCUMULATE):
-            parameters = then.rms_parameters() if hasattr(then, "rms_parameters") else None
-            if parameters is not None and parameters[0].shape == (self.out_features,) and then.dtype == torch.bfloat16:
+            if parameters is not None:
                 activations, squares = ops.gemm_decode(
                     a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias, accumulate_into=residual,
                     next_norm_weight=parameters[0], next_one_centered=parameters[2])
@@ -88,6 +117,8 @@ class Linear:
 
     def swiglu(self, a: Input) -> torch.Tensor:
         """The weight holds gate rows then up rows: silu(a . gate^T) * (a . up^T)."""
+        if self.bias is None and self._medium(a):
+            return ops.gemm_medium(self._rows_of(a), self.weight, ops.EPILOGUE_SWIGLU, **self._prepared_arguments(a))
         if self.bias is None and self._fused(a, self.out_features // 2, ops.EPILOGUE_SWIGLU):
             return ops.gemm_decode(self._rows_of(a), self.weight, ops.EPILOGUE_SWIGLU, out_dtype=torch.bfloat16,
                                    **self._norm_arguments(a))

@@ -664,6 +664,45 @@ def test_fused_decode_product_prepares_the_next_norm(ops, M, H, N, one_centered,
         close(dev_state, want_state, torch.float32, 4.0)
 
 
+@pytest.mark.parametrize("M", [17, 40, 64])
+@pytest.mark.parametrize("H,N,K,one_centered", [(72, 80, 136, False), (2048, 6144, 8192, True), (4104, 144, 64, False)])
+def test_medium_product_prepares_and_takes_the_next_norm(ops, M, H, N, K, one_centered):
+    """The same hand-over as in the fused decode product, for 17..64 rows: the accumulating
+    product leaves x * w and sums of squares (rows 64 wide), the next product takes them."""
+    a = as_dev(gen(M, K, seed=1), torch.bfloat16)
+    w_out = as_dev(gen(H, K, seed=2, scale=K ** -0.5), torch.bfloat16)
+    residual = gen(M, H, seed=3, scale=2).float().to(DEV)
+    norm_w = (0.1 * gen(H, seed=4) + (0 if one_centered else 1)).float()
+    eps = 1e-5
+    x_new = residual.cpu().double() + back(a) @ back(w_out).T
+    activations, squares = ops.gemm_medium(a, w_out, ops.EPILOGUE_ACCUMULATE, accumulate_into=residual,
+                                           next_norm_weight=norm_w.to(DEV), next_one_centered=one_centered)
+    close(residual, x_new, torch.float32, 2.0)
+    x_kernel = residual.cpu().double()
+    scale = norm_w.double() + (1 if one_centered else 0)
+    assert squares.shape[1] == 64
+    assert torch.equal(activations.cpu(), (x_kernel.float() * scale.float()).to(torch.bfloat16))
+    total = squares.cpu().double().sum(0)
+    assert float((total[:M] - (x_kernel ** 2).sum(-1)).abs().max()) <= 1e-5 * float((x_kernel ** 2).sum(-1).max())
+    inv = 1.0 / torch.sqrt((x_kernel ** 2).mean(-1, keepdim=True) + eps)
+    h = activations.cpu().double() * inv
+    w = as_dev(gen(N, H, seed=5, scale=H ** -0.5), torch.bfloat16)
+    bias = gen(N, seed=6).float().to(DEV)
+    want = h @ back(w).T
+    got = ops.gemm_medium(activations, w, ops.EPILOGUE_STORE, squares=squares, eps=eps, out_dtype=torch.float32, bias=bias)
+    close(got, want + bias.cpu().double(), torch.float32, 2.0)
+    # against a plain norm kernel followed by the plain product: one more rounding (the norm's output)
+    normed = ops.rmsnorm_rows(residual, norm_w.to(DEV), eps, torch.bfloat16, one_centered=one_centered)
+    close(ops.gemm(normed, w, out_dtype=torch.float32), want, torch.bfloat16, 1.0)
+    half = N // 2
+    got = ops.gemm_medium(activations, w, ops.EPILOGUE_SWIGLU, squares=squares, eps=eps)
+    close(got, F.silu(want[:, :half]) * want[:, half:], torch.bfloat16, 0.4)
+    other = gen(M, N, seed=7).float().to(DEV)
+    before = other.cpu().double()
+    ops.gemm_medium(activations, w, ops.EPILOGUE_ACCUMULATE, accumulate_into=other, squares=squares, eps=eps)
+    close(other, before + want, torch.float32, 2.0)
+
+
 def test_fused_decode_product_limits(ops):
     from flyweight_amd.kernels.ops import KernelError
     assert not ops.gemm_decode_fits(17, 64, 64, ops.EPILOGUE_STORE) and not ops.gemm_decode_fits(4, 64, 68, ops.EPILOGUE_STORE)
