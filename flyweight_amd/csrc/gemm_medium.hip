@@ -315,15 +315,25 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
         // sum of x^2 per row; the product that follows forms the row's 1/rms from those sums
         if (MODE == GM_ACCUMULATE && p.next_activations) {
             float row_square = 0.0f;
-            if (mine)
+            if (mine) {
+                const float one = p.next_one_centered ? 1.0f : 0.0f;
+                if (whole) {
+                    const f32x4 w = *reinterpret_cast<const f32x4*>(p.next_norm_weight + n_first);
+                    uint2 packed;
+                    packed.x = (uint32_t)float_to_bf16_bits(v[0] * (w[0] + one)) | ((uint32_t)float_to_bf16_bits(v[1] * (w[1] + one)) << 16);
+                    packed.y = (uint32_t)float_to_bf16_bits(v[2] * (w[2] + one)) | ((uint32_t)float_to_bf16_bits(v[3] * (w[3] + one)) << 16);
+                    *reinterpret_cast<uint2*>(p.next_activations + at) = packed;
+                    row_square = (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
+                } else {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int n = n_first + r;
-                    if (n >= N) continue;
-                    const float w = p.next_norm_weight[n] + (p.next_one_centered ? 1.0f : 0.0f);
-                    p.next_activations[at + r] = float_to_bf16_bits(v[r] * w);
-                    row_square += v[r] * v[r];
+                    for (int r = 0; r < 4; ++r) {
+                        const int n = n_first + r;
+                        if (n >= N) continue;
+                        p.next_activations[at + r] = float_to_bf16_bits(v[r] * (p.next_norm_weight[n] + one));
+                        row_square += v[r] * v[r];
+                    }
                 }
+            }
             row_square += __shfl_xor(row_square, 16, 64);
             row_square += __shfl_xor(row_square, 32, 64);
             if (g == 0) p.next_squares[((size_t)tile * FW + ft) * square_stride + m] = row_square;
