@@ -38,6 +38,11 @@ int fw_gemm_skinny(const void* a, const void* w, const float* bias, void* out, i
                    int M, int N, int K, void* stream);
 int fw_gemm_mfma(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                  int M, int N, int K, void* stream);
+// The prompt product with 256 x 256 tiles, for shapes that give enough of them to fill the chip
+// (fw_gemm_mfma_big_tiles says how many).
+int fw_gemm_mfma_big(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
+                     int M, int N, int K, void* stream);
+int fw_gemm_mfma_big_tiles(int mode, int M, int N, int K);     // 0: the kernel does not take the shape
 // The same product for 1..64 rows with K split over workgroups, so that a is not re-read by every
 // few features (decode steps of 17..64 requests). fw_gemm_medium_plan says what a shape needs:
 // bytes of workspace (0: none) and int32 counters (0: none) that are zero before the first call;

@@ -313,12 +313,18 @@ def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out
     if SKINNY_MAX_ROWS < M <= MEDIUM_MAX_ROWS:
         gemm_medium_into(a, w, bias, target, out_code, mode, N)
         return
-    entry = library().fw_gemm_skinny if M <= SKINNY_MAX_ROWS else library().fw_gemm_mfma
+    if M <= SKINNY_MAX_ROWS:
+        entry = library().fw_gemm_skinny
+    elif library().fw_gemm_mfma_big_tiles(mode, M, N, K) >= BIG_TILES_MIN:
+        entry = library().fw_gemm_mfma_big      # enough 256 x 256 tiles to fill the chip
+    else:
+        entry = library().fw_gemm_mfma
     _check(entry(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K, _stream()))
 
 
 SKINNY_MAX_ROWS = 16
 MEDIUM_MAX_ROWS = 64
+BIG_TILES_MIN = 192      # 256 x 256 tiles from which the large-tile prompt product is used (256 compute units)
 _MEDIUM_COUNTERS = {}
 
 

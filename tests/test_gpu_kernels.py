@@ -357,6 +357,26 @@ def test_fast_gemm_every_epilogue(ops, M, N, K):
         close(ops.gemm_swiglu(a, w), act, torch.bfloat16, 0.4)
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 6144, 96), (1500, 8200, 160), (4000, 3100, 64)])
+def test_large_tile_prompt_product(ops, M, N, K):
+    """Shapes with at least 192 tiles of 256 x 256 go to the large-tile kernel: every epilogue,
+    edges in both directions, few and many slabs."""
+    assert ops.library().fw_gemm_mfma_big_tiles(0, M, N, K) >= ops.BIG_TILES_MIN and not ops.library().fw_gemm_mfma_big_tiles(0, M, N, K + 8)
+    a = as_dev(gen(M, K), torch.bfloat16)
+    w = as_dev(gen(N, K, seed=1, scale=K ** -0.5), torch.bfloat16)
+    bias = gen(N, seed=2).float().to(DEV)
+    want = back(a) @ back(w).T
+    close(ops.gemm(a, w, bias, out_dtype=torch.float32), want + bias.cpu().double(), torch.float32, 2.0)
+    close(ops.gemm(a, w), want, torch.bfloat16, 0.4)
+    residual = gen(M, N, seed=3).float().to(DEV)
+    before = residual.cpu().double()
+    ops.gemm(a, w, accumulate_into=residual)
+    close(residual, before + want, torch.float32, 2.0)
+    if N % 2 == 0 and ops.library().fw_gemm_mfma_big_tiles(2, M, N // 2, K) >= ops.BIG_TILES_MIN:
+        half = N // 2
+        close(ops.gemm_swiglu(a, w), F.silu(want[:, :half]) * want[:, half:], torch.bfloat16, 0.4)
+
+
 def test_fast_gemm_rows_do_not_depend_on_the_batch(ops):
     a = as_dev(gen(300, 256), torch.bfloat16)
     w = as_dev(gen(200, 256, seed=1), torch.bfloat16)
