@@ -237,11 +237,13 @@ static int launch(const void* a, const void* w, const float* bias, void* out, in
 }
 
 // Narrow outputs take 64-feature tiles when 128-feature ones would give at most one workgroup
-// per compute unit (measured at 2,048 rows: 2048 features 42 vs 51 us, 3072 features 63 vs 49 us).
+// per compute unit (measured at 2,048 rows: 2048 features 42 vs 51 us, 3072 features 63 vs 49 us);
+// with a long K and exactly one 128-feature tile per compute unit the wider tile wins again (less
+// traffic per flop: 2,048 features, K 8,192: 111 vs 126 us).
 template <int MODE, typename TO>
 static int launch_by_width(const void* a, const void* w, const float* bias, void* out, int M, int N, int K, hipStream_t stream) {
     const long long tiles128 = (long long)fw_ceil_div(M, TM) * fw_ceil_div(N, TN);
-    if (tiles128 <= 256) return launch<MODE, 64, TO>(a, w, bias, out, M, N, K, stream);
+    if (tiles128 < 256 || (tiles128 == 256 && K < 4096)) return launch<MODE, 64, TO>(a, w, bias, out, M, N, K, stream);
     return launch<MODE, 128, TO>(a, w, bias, out, M, N, K, stream);
 }
 
