@@ -35,6 +35,13 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     return (uint32_t)float_to_bf16_bits(lo) | ((uint32_t)float_to_bf16_bits(hi) << 16);
 }
+// the same in one instruction (v_cvt_pk_bf16_f32, round to nearest even)
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+__device__ __forceinline__ uint32_t pack_bf16_pair(float lo, float hi) {
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
 
 // State of one wave: 16 columns, HD channels (HD a multiple of 32; channels >= head_dim are zero).
 template <int HD>
@@ -53,8 +60,7 @@ __device__ __forceinline__ void attend_page(Columns<HD>& c, const uint16_t* __re
                                             int lo, int hi, int last_written, int k_stride, int v_stride) {
     const int lane = threadIdx.x & 63;
     const int i16 = lane & 15, g = lane >> 4;
-    // all key loads of the page are issued before the first product; with the 64-channel
-    // instantiation (the measured case) the values too: they do not depend on the scores
+    // all key loads of the page are issued before the first product
     bf16x8 kf[4][HD / 32];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
@@ -65,19 +71,6 @@ __device__ __forceinline__ void attend_page(Columns<HD>& c, const uint16_t* __re
             if (dc * 32 + g * 8 < head_dim) kf[kt][dc] = *reinterpret_cast<const bf16x8*>(key + dc * 32);
         }
     }
-    constexpr bool EARLY_V = HD == 64;
-    u32x2 vearly[EARLY_V ? 2 : 1][EARLY_V ? HD / 16 : 1][2];
-    if (EARLY_V) {
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int t = 0; t < HD / 16; ++t) {
-                if (t * 16 >= head_dim) break;
-                const uint16_t* value = v_page + (size_t)(t * 16 + i16) * v_stride + kb * 32 + g * 4;
-                vearly[kb][t][0] = *reinterpret_cast<const u32x2*>(value);
-                vearly[kb][t][1] = *reinterpret_cast<const u32x2*>(value + 16);
-            }
-    }
     f32x4 s[4];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
@@ -86,22 +79,36 @@ __device__ __forceinline__ void attend_page(Columns<HD>& c, const uint16_t* __re
         for (int dc = 0; dc < HD / 32; ++dc)
             s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kt][dc], c.q[dc], s[kt], 0, 0, 0);
     }
-    // mask, then the running maximum of this column: over this lane's 16 scores, then over
-    // the four lanes that share the column
+    // The running maximum of this column: over this lane's 16 scores, then over the four lanes
+    // that share the column. A page of which every key counts for every column of the wave (all
+    // but the pages on the diagonal, at a window's edge, and a sequence's last) needs no mask.
+    const bool full = __all(lo <= 0 && hi >= PAGE - 1) && last_written >= PAGE - 1;
     float page_max = NEG_BIG;
+    if (full) {
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
+        for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int key = kt * 16 + g * 4 + r;
-            const float v = (key >= lo && key <= hi) ? s[kt][r] * scale_log2 : NEG_BIG;
-            s[kt][r] = v;
-            page_max = fmaxf(page_max, v);
-        }
+            for (int r = 0; r < 4; ++r) {
+                s[kt][r] *= scale_log2;
+                page_max = fmaxf(page_max, s[kt][r]);
+            }
+    } else {
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = kt * 16 + g * 4 + r;
+                const float v = (key >= lo && key <= hi) ? s[kt][r] * scale_log2 : NEG_BIG;
+                s[kt][r] = v;
+                page_max = fmaxf(page_max, v);
+            }
+    }
     page_max = fmaxf(page_max, __shfl_xor(page_max, 16, 64));
     page_max = fmaxf(page_max, __shfl_xor(page_max, 32, 64));
     const float new_max = fmaxf(c.m, page_max);
-    const float alpha = exp2f(c.m - new_max);
+    // the hardware's 2^x: arguments are <= 0 here, and one far below (a first page, a masked key
+    // against a real maximum) gives 0
+    const float alpha = __builtin_amdgcn_exp2f(c.m - new_max);
     c.m = new_max;
     float sum = 0.0f;
     uint32_t p[4][2];
@@ -110,15 +117,18 @@ __device__ __forceinline__ void attend_page(Columns<HD>& c, const uint16_t* __re
         float e[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            e[r] = s[kt][r] > 0.5f * NEG_BIG ? exp2f(s[kt][r] - new_max) : 0.0f;
+            e[r] = __builtin_amdgcn_exp2f(s[kt][r] - new_max);
+            if (!full) e[r] = s[kt][r] > 0.5f * NEG_BIG ? e[r] : 0.0f;     // a column that has seen no key yet: maximum NEG_BIG too
             sum += e[r];
         }
-        p[kt][0] = pack_bf16(e[0], e[1]);
-        p[kt][1] = pack_bf16(e[2], e[3]);
+        p[kt][0] = pack_bf16_pair(e[0], e[1]);
+        p[kt][1] = pack_bf16_pair(e[2], e[3]);
     }
     c.l = c.l * alpha + sum;
+    if (__any(alpha != 1.0f)) {         // the maximum of some column rose (seldom after the first pages)
 #pragma unroll
-    for (int t = 0; t < HD / 16; ++t) c.o[t] *= alpha;
+        for (int t = 0; t < HD / 16; ++t) c.o[t] *= alpha;
+    }
     const bool partial_page = last_written < PAGE - 1;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
@@ -128,15 +138,9 @@ __device__ __forceinline__ void attend_page(Columns<HD>& c, const uint16_t* __re
 #pragma unroll
         for (int t = 0; t < HD / 16; ++t) {
             if (t * 16 >= head_dim) break;
-            u32x2 va, vb;
-            if (EARLY_V) {
-                va = vearly[kb][t][0];
-                vb = vearly[kb][t][1];
-            } else {
-                const uint16_t* value = v_page + (size_t)(t * 16 + i16) * v_stride;
-                va = *reinterpret_cast<const u32x2*>(value + key_a);
-                vb = *reinterpret_cast<const u32x2*>(value + key_b);
-            }
+            const uint16_t* value = v_page + (size_t)(t * 16 + i16) * v_stride;
+            u32x2 va = *reinterpret_cast<const u32x2*>(value + key_a);
+            u32x2 vb = *reinterpret_cast<const u32x2*>(value + key_b);
             if (partial_page) {
                 // keep keys <= last_written only: two keys per 32-bit word, low half first
                 auto keep = [&](uint32_t word, int first_key) -> uint32_t {
@@ -243,8 +247,10 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
         const int base = block * PAGE;
         if (rows > 0 && base <= wave_hi) {      // a wave whose rows all lie before this page has nothing to add
             const uint16_t* kt = lds + (size_t)buffer * (k_elems + v_elems);
-            attend_page<HD>(c, kt, kt + k_elems, head_dim, scale_log2, valid ? my_first - base : PAGE,
-                            valid ? my_pos - base : -1, pos_hi - base, k_stride, v_stride);
+            // a lane without a row computes along with the bounds of the tile's first row (nothing of
+            // it is stored): a page that is whole for the rows is then whole for the wave
+            attend_page<HD>(c, kt, kt + k_elems, head_dim, scale_log2, my_first - base, my_pos - base, pos_hi - base,
+                            k_stride, v_stride);
         }
     };
 
@@ -320,8 +326,9 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) void attention_decode_split_kerne
         const int page = block_table[(size_t)row_seg[row] * table_stride + block];
         const size_t at = ((size_t)page * num_kv_heads + kvh) * PAGE * head_dim;
         const int base = block * PAGE;
-        attend_page<HD>(c, k_pages + at, v_pages + at, head_dim, scale_log2, valid ? first - base : PAGE,
-                        valid ? pos - base : -1, pos - base, head_dim, PAGE);
+        // a lane without a head computes along (q = 0, nothing of it is stored)
+        attend_page<HD>(c, k_pages + at, v_pages + at, head_dim, scale_log2, first - base, pos - base, pos - base,
+                        head_dim, PAGE);
     }
     float l = c.l;
     l += __shfl_xor(l, 16, 64);
