@@ -32,6 +32,18 @@ SHAPE = dict(
 PROMPT = 2048
 CONTEXT = 4096
 
+# The two serving workloads BASELINE.json names beside the headline (configs[3] and configs[4]);
+# run with --workload, they print one JSON line of their own.
+SHAPE_350M = dict(SHAPE, hidden_size=1024, num_attention_heads=16, intermediate_size=6656, max_position_embeddings=33280)
+SHAPE_2P6B = dict(SHAPE, num_hidden_layers=30, intermediate_size=10752, max_position_embeddings=9216,
+                  full_attn_idxs=[2, 6, 10, 14, 18, 21, 24, 27])
+WORKLOADS = {
+    # 64 requests with 32,768-token prompts in portions of 2,048, 256 new tokens each: the cache is the load
+    "long-context": dict(shape=SHAPE_350M, name="LFM2-350M shape", requests=64, prompt=(32768, 32768), output=(256, 256)),
+    # 128 requests, prompts of 64..8,192 tokens and 128..1,024 new tokens, under continuous batching
+    "mixed": dict(shape=SHAPE_2P6B, name="LFM2-2.6B shape", requests=128, prompt=(64, 8192), output=(128, 1024)),
+}
+
 
 def log(text: str) -> None:
     print(f"[bench] {text}", file=sys.stderr, flush=True)
@@ -120,6 +132,63 @@ def prefill_run(torch, model, config, repeats: int = 3):
     return best
 
 
+def serving_run(torch, workload: str, requests: int, seed: int = 0) -> dict:
+    """Submits every request of a workload at once and steps the engine until all are done."""
+    import numpy as np
+    from flyweight_amd import Model, Runtime
+    from flyweight_amd.config import config_from_dict
+    spec = WORKLOADS[workload]
+    config = config_from_dict(spec["shape"])
+    log(f"building the {spec['name']} with random bfloat16 weights")
+    model = Model.random(config, seed=0, dtype="bfloat16")
+    rng = np.random.default_rng(seed)
+    prompts = rng.integers(spec["prompt"][0], spec["prompt"][1] + 1, requests).tolist()
+    outputs = rng.integers(spec["output"][0], spec["output"][1] + 1, requests).tolist()
+    context = max(p + o for p, o in zip(prompts, outputs))
+    pages = sum((p + o + 63) // 64 for p, o in zip(prompts, outputs))
+    # a step holds 2,048 tokens: the decoded tokens of the running requests first, portions of prompts in the rest
+    runtime = Runtime(model, context_limit=context, parallel_sequences=requests, num_pages=pages,
+                      max_batch_tokens=PROMPT, prefill_rows=PROMPT).prepare()
+    # a short request first: every kernel and library is loaded before the clock starts
+    runtime.generate(rng.integers(0, config.vocab_size, 100).tolist(), 4)
+    for prompt, output in zip(prompts, outputs):
+        runtime.task_submit(rng.integers(0, config.vocab_size, prompt).tolist(), output)
+    log(f"{requests} requests, {sum(prompts)} prompt tokens, {sum(outputs)} tokens to generate")
+    generated = finished = steps = 0
+    torch.cuda.synchronize()
+    began = last = time.perf_counter()
+    while runtime.scheduler.has_work():
+        events = runtime.engine_step()
+        steps += 1
+        generated += sum(1 for e in events if e[2] == 0)
+        finished += sum(1 for e in events if e[2] == 1)
+        errors = [e for e in events if e[2] == 2]
+        assert not errors, f"a request failed: {runtime.task_error(errors[0][0])}"
+        if time.perf_counter() - last > 20.0:
+            last = time.perf_counter()
+            log(f"step {steps}: {generated} tokens generated, {finished} requests finished")
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - began
+    assert finished == requests and generated == sum(outputs), (finished, generated)
+    info = runtime.info
+    preemptions = info["preemptions"]
+    runtime.close()
+    return {
+        "metric": f"tokens/s, prompt and generated ({workload} workload, {spec['name']})",
+        "value": round((sum(prompts) + generated) / elapsed, 1), "unit": "tokens/s", "n_gpus": 1,
+        "generated_per_s": round(generated / elapsed, 1), "seconds": round(elapsed, 3), "steps": steps,
+        "steps_with_prompt_tokens": {"count": info["prefill_calls"], "seconds": round(info["prefill_ns"] * 1e-9, 3)},
+        "decode_only_steps": {"count": steps - info["prefill_calls"], "seconds": round(info["decode_ns"] * 1e-9, 3)},
+        "higher_is_better": True, "dtype": "bf16", "data": "synthetic: seeded uniform token ids and lengths, random-init weights",
+        "config": {"model": spec["name"], "layers": config.num_hidden_layers, "hidden": config.hidden_size,
+                   "heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
+                   "head_dim": config.head_dim, "ff_dim": config.ff_dim, "vocab": config.vocab_size,
+                   "attention_layers": len(config.full_attn_idxs), "requests": requests,
+                   "prompt_tokens": sum(prompts), "generated_tokens": generated, "longest_context": context,
+                   "portion": PROMPT, "cache_pages": pages, "preemptions": preemptions},
+    }
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -128,6 +197,9 @@ def main() -> int:
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
     parser.add_argument("--only", choices=("decode", "prefill"), help="run one phase and print no JSON (for profiling)")
+    parser.add_argument("--workload", choices=("headline",) + tuple(WORKLOADS), default="headline",
+                        help="headline: the LFM2-1.2B decode and prefill figures; the others: a whole serving run")
+    parser.add_argument("--requests", type=int, help="requests of a serving workload (default: as the workload names)")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for {args.gpus})", flush=True)
@@ -140,6 +212,9 @@ def main() -> int:
     from flyweight_amd import Model
     from flyweight_amd.config import config_from_dict
 
+    if args.workload != "headline":
+        print(json.dumps(serving_run(torch, args.workload, args.requests or WORKLOADS[args.workload]["requests"])), flush=True)
+        return 0
     config = config_from_dict(SHAPE)
     log("building the LFM2-1.2B shape with random bfloat16 weights")
     model = Model.random(config, seed=0, dtype="bfloat16")

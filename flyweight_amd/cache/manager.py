@@ -300,8 +300,7 @@ class CacheManager:
         for i, request in enumerate(requests):
             natives[i] = self._live_id(request)
         if stride is None:
-            stride = max([self.pages_for(self.length_of(r)) for r in requests] +
-                         [len(self.groups[group_index].tables[r]) for r in requests] + [1])
+            stride = max(self._lib.fwh_cache_longest_table(self._native, group_index, natives, len(requests)), 1)
         rows = np.zeros((len(requests), stride), dtype=np.int32)
         if self._lib.fwh_cache_fill_tables(self._native, group_index, natives, len(requests), stride, rows.ctypes.data) < 0:
             raise CacheAccountingError(host.last_error())

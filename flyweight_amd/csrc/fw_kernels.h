@@ -43,6 +43,14 @@ int fw_gemm_mfma(const void* a, const void* w, const float* bias, void* out, int
 int fw_gemm_mfma_big(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                      int M, int N, int K, void* stream);
 int fw_gemm_mfma_big_tiles(int mode, int M, int N, int K);     // 0: the kernel does not take the shape
+// fw_gemm_mfma with K cut into slices for products with fewer tiles than compute units (a few
+// hundred rows, a narrow output). fw_gemm_mfma_split_plan says what a shape needs: bytes of
+// workspace and int32 counters that are zero before the first call and are left zero (both 0: the
+// shape is not cut, use fw_gemm_mfma). Calls that overlap on one device need their own of both.
+int fw_gemm_mfma_split_plan(int mode, int M, int N, int K, size_t* workspace_bytes, int* counters);
+int fw_gemm_mfma_split(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
+                       int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
+                       int counters_len, void* stream);
 // The same product for 1..64 rows with K split over workgroups, so that a is not re-read by every
 // few features (decode steps of 17..64 requests). fw_gemm_medium_plan says what a shape needs:
 // bytes of workspace (0: none) and int32 counters (0: none) that are zero before the first call;

@@ -47,6 +47,7 @@ int fwh_cache_pages_missing(void* cache, int64_t request, int new_length, int* p
 int fwh_cache_table(void* cache, int64_t request, int group, int* pages, int capacity);     // its length
 // rows of block tables for a batch: pages given back read as page 0 (they are never looked at)
 int fwh_cache_fill_tables(void* cache, int group, const int64_t* requests, int count, int stride, int* rows);
+int fwh_cache_longest_table(void* cache, int group, const int64_t* requests, int count);     // blocks of the longest of these tables
 // for a whole batch: lengths and slots (FWH_ERROR names the first request that is not live);
 // reservations for all or for none; the new lengths
 int fwh_cache_describe(void* cache, const int64_t* requests, int count, int* lengths, int* slots);

@@ -114,6 +114,18 @@ int fwh_cache_fill_tables(void* cache, int group, const int64_t* requests, int c
         return 0;
     });
 }
+int fwh_cache_longest_table(void* cache, int group, const int64_t* requests, int count) {
+    return guarded([&] {
+        const auto& tables = cache_of(cache)->group(group).tables;
+        int longest = 0;
+        for (int i = 0; i < count; ++i) {
+            auto it = tables.find(requests[i]);
+            if (it == tables.end()) throw std::out_of_range("request " + std::to_string(requests[i]) + " has no block table");
+            longest = (int)it->second.size() > longest ? (int)it->second.size() : longest;
+        }
+        return longest;
+    });
+}
 int fwh_cache_describe(void* cache, const int64_t* requests, int count, int* lengths, int* slots) {
     return guarded([&] {
         fwh::Cache* c = cache_of(cache);

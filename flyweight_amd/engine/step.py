@@ -75,9 +75,9 @@ class StepContext:
         """``described``: (lengths, slots) of the entries' requests if the caller has checked the
         entries already (``check_entries``)."""
         starts, slots = described if described is not None else check_entries(entries, cache, vocab_size, max_positions)
-        tokens: List[int] = []
-        row_pos: List[int] = []
-        row_seg: List[int] = []
+        # per-row arrays are put together from one numpy piece per entry: a prompt portion has
+        # thousands of rows, and a Python loop over them would take longer than some kernels
+        token_parts, pos_parts, seg_parts = [], [], []
         seg_row0: List[int] = [0]
         seg_slot: List[int] = list(slots)
         want_rows: List[int] = []
@@ -85,18 +85,22 @@ class StepContext:
         self.new_lengths: List[int] = []
         for seg, (entry, start) in enumerate(zip(entries, starts)):
             n = len(entry.tokens)
-            want_rows.extend(len(tokens) + int(place) for place in entry.want)
-            tokens.extend(int(t) for t in entry.tokens)
-            row_pos.extend(range(start, start + n))
-            row_seg.extend([seg] * n)
-            seg_row0.append(len(tokens))
+            want_rows.extend(seg_row0[-1] + int(place) for place in entry.want)
+            token_parts.append(np.asarray(entry.tokens, dtype=np.int32))
+            pos_parts.append(np.arange(start, start + n, dtype=np.int32))
+            seg_parts.append(np.full(n, seg, dtype=np.int32))
+            seg_row0.append(seg_row0[-1] + n)
             self.new_lengths.append(start + n)
+        tokens = np.concatenate(token_parts)
+        row_pos = np.concatenate(pos_parts)
+        row_seg = np.concatenate(seg_parts)
         self.num_rows = len(tokens)
         self.num_segments = len(entries)
         self.num_wanted = len(want_rows)
         self.all_decode = self.num_rows == self.num_segments
         self.max_context = max(self.new_lengths)
         self.device = device
+        # the same on the host, for parts that plan their work there
         self.host_row_pos = row_pos
         self.host_seg_row0 = seg_row0
         self.host_seg_slot = seg_slot

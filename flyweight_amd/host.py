@@ -40,6 +40,7 @@ _SIGNATURES = {
     "fwh_cache_pages_missing": (c_int, [c_void_p, c_int64, c_int, _INTS]),
     "fwh_cache_table": (c_int, [c_void_p, c_int64, c_int, _INTS, c_int]),
     "fwh_cache_fill_tables": (c_int, [c_void_p, c_int, _IDS, c_int, c_int, c_void_p]),
+    "fwh_cache_longest_table": (c_int, [c_void_p, c_int, _IDS, c_int]),
     "fwh_cache_describe": (c_int, [c_void_p, _IDS, c_int, _INTS, _INTS]),
     "fwh_cache_reserve_batch": (c_int, [c_void_p, _IDS, _INTS, c_int]),
     "fwh_cache_commit_batch": (c_int, [c_void_p, _IDS, _INTS, c_int]),

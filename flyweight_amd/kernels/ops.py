@@ -308,16 +308,25 @@ def fill_zero(t: torch.Tensor) -> None:
 
 def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int) -> None:
     """bfloat16 operands on the matrix cores: the skinny kernel for up to 16 rows, the medium one
-    (K split over workgroups) for up to 64, the tiled one beyond."""
+    (K split over workgroups) for up to 64, the tiled ones beyond (large tiles where they fill the
+    chip, K cut into slices where even the small tiles are too few)."""
     M, K = a.shape
     if SKINNY_MAX_ROWS < M <= MEDIUM_MAX_ROWS:
         gemm_medium_into(a, w, bias, target, out_code, mode, N)
         return
     if M <= SKINNY_MAX_ROWS:
         entry = library().fw_gemm_skinny
-    elif library().fw_gemm_mfma_big_tiles(mode, M, N, K) >= BIG_TILES_MIN:
+    elif M > BIG_MIN_ROWS and library().fw_gemm_mfma_big_tiles(mode, M, N, K) >= BIG_TILES_MIN:
         entry = library().fw_gemm_mfma_big      # enough 256 x 256 tiles to fill the chip
     else:
+        need_bytes, need_counters = ctypes.c_size_t(0), ctypes.c_int(0)
+        _check(library().fw_gemm_mfma_split_plan(mode, M, N, K, ctypes.byref(need_bytes), ctypes.byref(need_counters)))
+        if need_bytes.value:                    # fewer tiles than compute units: K is cut into slices
+            workspace = torch.empty(need_bytes.value // 4, dtype=torch.float32, device=a.device)
+            counters = _medium_counters(a.device, need_counters.value)
+            _check(library().fw_gemm_mfma_split(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K, _p(workspace),
+                                                ctypes.c_size_t(need_bytes.value), _p(counters), counters.numel(), _stream()))
+            return
         entry = library().fw_gemm_mfma
     _check(entry(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K, _stream()))
 
@@ -325,6 +334,7 @@ def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out
 SKINNY_MAX_ROWS = 16
 MEDIUM_MAX_ROWS = 64
 BIG_TILES_MIN = 192      # 256 x 256 tiles from which the large-tile prompt product is used (256 compute units)
+BIG_MIN_ROWS = 128       # up to here a 256-row tile would be at least half empty (the head at 128 rows: 110 vs 78 us)
 _MEDIUM_COUNTERS = {}
 
 

@@ -377,6 +377,35 @@ def test_large_tile_prompt_product(ops, M, N, K):
         close(ops.gemm_swiglu(a, w), F.silu(want[:, :half]) * want[:, half:], torch.bfloat16, 0.4)
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 2048, 2048), (128, 2048, 8192), (130, 104, 1032), (200, 3072, 2048), (300, 2500, 520),
+                                   (1000, 200, 4096)])
+def test_tiled_product_cuts_k_into_slices(ops, M, N, K):
+    """More than 64 rows but fewer tiles than compute units: K goes to several workgroups and the
+    last one of a tile to arrive adds the slices in their order. Every epilogue, edges in rows,
+    features and K, twice in a row (the tickets are left at zero), and bitwise the same whichever
+    workgroup came last."""
+    import ctypes
+    need_bytes, need_counters = ctypes.c_size_t(0), ctypes.c_int(0)
+    assert ops.library().fw_gemm_mfma_split_plan(0, M, N, K, ctypes.byref(need_bytes), ctypes.byref(need_counters)) == 0
+    assert need_bytes.value > 0 and need_counters.value > 0, "the shape is meant to be cut"
+    a = as_dev(gen(M, K), torch.bfloat16)
+    w = as_dev(gen(N, K, seed=1, scale=K ** -0.5), torch.bfloat16)
+    bias = gen(N, seed=2).float().to(DEV)
+    want = back(a) @ back(w).T
+    first = ops.gemm(a, w, bias, out_dtype=torch.float32)
+    close(first, want + bias.cpu().double(), torch.float32, 2.0)
+    for _ in range(3):
+        assert torch.equal(ops.gemm(a, w, bias, out_dtype=torch.float32), first)
+    close(ops.gemm(a, w), want, torch.bfloat16, 0.4)
+    residual = gen(M, N, seed=3).float().to(DEV)
+    before = residual.cpu().double()
+    ops.gemm(a, w, accumulate_into=residual)
+    close(residual, before + want, torch.float32, 2.0)
+    if N % 2 == 0:
+        half = N // 2
+        close(ops.gemm_swiglu(a, w), F.silu(want[:, :half]) * want[:, half:], torch.bfloat16, 0.4)
+
+
 def test_fast_gemm_rows_do_not_depend_on_the_batch(ops):
     a = as_dev(gen(300, 256), torch.bfloat16)
     w = as_dev(gen(200, 256, seed=1), torch.bfloat16)
