@@ -20,6 +20,19 @@ __device__ __forceinline__ void fw_lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Lets the matrix pipe finish what was issued before control goes on. Inside one basic block the
+// compiler keeps a product and the first read of its result far enough apart; where the read is
+// the target of a taken branch it has been seen one instruction behind the product, reading the
+// registers the product writes last before they were written (seen in the attention kernel with
+// head sizes below the template's: two of four components stale). Called once behind a loop of
+// products, before branches that lead to code reading the accumulators. 24 wait states cover the
+// longest product (16 passes).
+__device__ __forceinline__ void fw_mfma_drain() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 15\n\ts_nop 7");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 #define FW_REQUIRE(cond, ...)                    \
     do {                                         \
         if (!(cond)) {                           \

@@ -122,12 +122,14 @@ int fw_attention_generic(const void* q, void* out, int dtype, const void* k_page
 
 // The same attention on the matrix cores, bfloat16 only, head_dim a multiple of 16 up to 256.
 // Prompt portions: rows are cut into tiles of up to 64 that never span two segments (tile_seg,
-// tile_row0).
+// tile_row0). heads_together: how many query heads of a kv group one workgroup takes, reading
+// the keys and values once for all of them (1, or 4 up to head_dim 64); 0: 4 where the group has
+// as many and every compute unit still gets a workgroup, else 1.
 int fw_attention_prefill(const void* q, void* out, const void* k_pages, const void* v_pages,
                          const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                          const int32_t* tile_row0, int tiles, const int32_t* seg_row0, const int32_t* row_pos,
                          int rows, int num_heads, int num_kv_heads, int head_dim, float scale, int window,
-                         int page_size, int num_pages, void* stream);
+                         int page_size, int num_pages, int heads_together, void* stream);
 // Decode (one row per request): the keys are split between workgroups in runs of 4 pages and
 // merged in order by the workgroup that finishes last. partial: float32 workspace
 // [rows][heads][max_splits][head_dim + 4]; max_context: an upper bound on position + 1 of every

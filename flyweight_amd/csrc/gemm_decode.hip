@@ -161,6 +161,7 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
                 for (int rt = 0; rt < RT; ++rt)
                     acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][j], af[j], acc[rt], 0, 0, 0);
         }
+        fw_mfma_drain();     // the loop is left by a branch; the accumulators are read next
 
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)

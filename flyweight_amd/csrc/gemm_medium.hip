@@ -193,6 +193,7 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
             fw_lds_barrier();       // LDS only: the loads just issued stay in flight
         }
     }
+    fw_mfma_drain();     // branches follow that lead to code reading the accumulators
 
     // the parts of K inside the workgroup meet in LDS, in wave order
     if (KP > 1) {

@@ -189,6 +189,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(
             multiply(0);
         }
     }
+    fw_mfma_drain();     // the branches below lead to code that reads the accumulators
 
     // The slices of K meet in the workspace: [slice][tile][accumulator register][thread]. The
     // sums are written and read with device-scope accesses (past the caches that workgroups on

@@ -224,6 +224,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         __builtin_amdgcn_sched_barrier(0);
     }
 #undef FW_INTERLEAVE
+    fw_mfma_drain();     // branches follow that lead to code reading the accumulators
 
     // D layout of the 32x32 product: lane holds column lane % 32; register r is row
     // 8 * (r / 4) + 4 * (lane / 32) + r % 4

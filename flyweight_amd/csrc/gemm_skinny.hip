@@ -93,6 +93,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
                 for (int mt = 0; mt < MT; ++mt)
                     acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[rt][j], af[mt][j], acc[rt][mt], 0, 0, 0);
     }
+    fw_mfma_drain();     // the loop is left by a branch; the accumulators are read next
 
     // partial sums meet in LDS; wave `t % WAVES` finishes tile t
 #pragma unroll

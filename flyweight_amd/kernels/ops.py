@@ -582,7 +582,9 @@ def decode_splits(max_context: int, window: int = 0) -> int:
 
 def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                       v_pages: torch.Tensor, block_table: torch.Tensor, tile_seg: torch.Tensor, tile_row0: torch.Tensor,
-                      seg_row0: torch.Tensor, row_pos: torch.Tensor, scale: float, window: int = 0) -> torch.Tensor:
+                      seg_row0: torch.Tensor, row_pos: torch.Tensor, scale: float, window: int = 0,
+                      heads_together: int = 0) -> torch.Tensor:
+    """``heads_together``: query heads of a kv group per workgroup (1, or 4 up to head_dim 64), 0: the kernel's choice."""
     _dev(q, k_pages, v_pages, block_table, tile_seg, tile_row0, seg_row0, row_pos)
     _want(q, torch.bfloat16, "q")
     rows = q.shape[0]
@@ -598,7 +600,7 @@ def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     _check(library().fw_attention_prefill(
         _p(q), _p(out), _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(tile_seg), _p(tile_row0),
         tile_seg.numel(), _p(seg_row0), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale),
-        int(window), PAGE_SIZE, pages, _stream()))
+        int(window), PAGE_SIZE, pages, int(heads_together), _stream()))
     return out
 
 

@@ -496,6 +496,34 @@ def test_attention_prefill_on_the_matrix_cores(ops, nh, nkv, hd, window):
     close(generic, want, torch.bfloat16)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 1, 16, 0), (3, 1, 48, 0), (12, 2, 64, 0), (32, 8, 64, 0), (8, 2, 32, 70)])
+def test_attention_prefill_takes_four_heads_of_a_group_together(ops, nh, nkv, hd, window):
+    """One workgroup reads a page once for four query heads of the kv group: whole runs of four,
+    a group of three (one head idle), a group of six (a run of four and one of two), head sizes
+    below the kernel's, a window. Against the reference and bitwise against one head at a time."""
+    lengths = [150, 200, 64, 65, 33]
+    starts = [0, 120, 63, 64, 16]
+    keys, values, table, k_pages, v_pages = _mfma_setup(nh, nkv, hd, lengths, num_pages=14, seed=5)
+    counts = [n - s for n, s in zip(lengths, starts)]
+    seg_row0 = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    row_pos = np.concatenate([np.arange(s, n) for s, n in zip(starts, lengths)]).astype(np.int32)
+    row_seg = np.concatenate([np.full(c, i) for i, c in enumerate(counts)]).astype(np.int32)
+    tile_seg, tile_row0 = ops.query_tiles(seg_row0.tolist())
+    rows = int(seg_row0[-1])
+    q = as_dev(gen(rows, nh * hd, seed=4), torch.bfloat16)
+    scale = 1 / math.sqrt(hd)
+    d = lambda a: torch.tensor(np.asarray(a, dtype=np.int32), device=DEV)       # noqa: E731
+    run = lambda together: ops.attention_prefill(q, nh, nkv, hd, k_pages, v_pages, d(table), d(tile_seg), d(tile_row0),  # noqa: E731
+                                                 d(seg_row0), d(row_pos), scale, window, heads_together=together)
+    four = run(4)
+    want = torch.stack([attention_reference(back(q)[r].reshape(nh, hd), keys[row_seg[r]], values[row_seg[r]], int(row_pos[r]),
+                                            scale, window, nh // nkv).reshape(-1) for r in range(rows)])
+    close(four, want, torch.bfloat16)
+    assert torch.equal(four, run(1))
+    with pytest.raises(ops.KernelError, match="heads together"):
+        run(2)
+
+
 @pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (3, 1, 48, 0), (6, 3, 80, 0), (32, 8, 64, 0), (2, 2, 128, 0),
                                               (20, 1, 256, 0), (4, 2, 32, 300), (4, 4, 64, 64), (2, 1, 64, 1)])
 def test_attention_decode_on_the_matrix_cores(ops, nh, nkv, hd, window):
