@@ -55,19 +55,22 @@ struct Columns {
 // group over the same rows): the keys and values are read once for all of them. `lo`/`hi`: the
 // keys of this page that this lane's column may see are those with lo <= key <= hi
 // (page-relative; hi < 0: none). `last_written`: keys beyond it hold whatever an earlier owner of
-// the page left, and are zeroed before they meet P = 0.
+// the page left, and are zeroed before they meet P = 0: here if CLEAN_V, else the caller has done
+// it (the prompt kernel does when it copies a page to LDS).
 //
 // The softmax arithmetic (one exponential per score on the quarter-rate unit) takes more issue
-// cycles than the matrix products take on their pipe, so the work is laid out in phases without
-// branches between them, each over all heads: the compiler can then let the products of one head
-// run behind the arithmetic of another. FULL: every key of the page counts for every column of
-// the wave (all pages but those on the diagonal, at a window's edge, and a sequence's last): no
+// cycles than the matrix products take on their pipe, so the work is laid out in phases, each
+// over all heads, with one short branch (the mask) that touches nothing but the scores: the
+// compiler can then let the products of one head run behind the arithmetic of another, and the
+// accumulators stay where they are (a join of two paths that both write them costs a register
+// move per accumulator and page). A page of which every key counts for every column of the wave
+// (all pages but those on the diagonal, at a window's edge, and a sequence's last) skips the
 // mask. The scale is folded into the exponent's argument: the maximum is taken over the raw
 // scores (the scale is positive) and kept scaled.
-template <int HD, int NH, bool FULL>
-__device__ __forceinline__ void attend_page_as(Columns<HD> (&c)[NH], const uint16_t* __restrict__ k_page,
-                                               const uint16_t* __restrict__ v_page, int head_dim, float scale_log2,
-                                               int lo, int hi, int last_written, int k_stride, int v_stride) {
+template <int HD, int NH, bool CLEAN_V>
+__device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t* __restrict__ k_page,
+                                            const uint16_t* __restrict__ v_page, int head_dim, float scale_log2,
+                                            int lo, int hi, int last_written, int k_stride, int v_stride) {
     const int lane = threadIdx.x & 63;
     const int i16 = lane & 15, g = lane >> 4;
     // all key loads of the page are issued before the first product
@@ -92,6 +95,18 @@ __device__ __forceinline__ void attend_page_as(Columns<HD> (&c)[NH], const uint1
             for (int dc = 0; dc < HD / 32; ++dc)
                 s[h][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kt][dc], c[h].q[dc], s[h][kt], 0, 0, 0);
         }
+    const bool full = __all(lo <= 0 && hi >= PAGE - 1) && last_written >= PAGE - 1;
+    if (!full) {
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = kt * 16 + g * 4 + r;
+                const bool seen = key >= lo && key <= hi;
+#pragma unroll
+                for (int h = 0; h < NH; ++h) s[h][kt][r] = seen ? s[h][kt][r] : NEG_BIG;
+            }
+    }
     // the running maximum of each column: over this lane's 16 scores, then over the four lanes
     // that share the column
     float alpha[NH], shift[NH];
@@ -102,23 +117,20 @@ __device__ __forceinline__ void attend_page_as(Columns<HD> (&c)[NH], const uint1
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                if (!FULL) {
-                    const int key = kt * 16 + g * 4 + r;
-                    s[h][kt][r] = (key >= lo && key <= hi) ? s[h][kt][r] : NEG_BIG;
-                }
-                page_max = fmaxf(page_max, s[h][kt][r]);
-            }
+            for (int r = 0; r < 4; ++r) page_max = fmaxf(page_max, s[h][kt][r]);
         page_max = fmaxf(page_max, __shfl_xor(page_max, 16, 64));
         page_max = fmaxf(page_max, __shfl_xor(page_max, 32, 64));
         // a column that has seen no key yet keeps NEG_BIG (the raw maximum times the scale would overflow)
-        const float new_max = fmaxf(c[h].m, page_max > 0.5f * NEG_BIG ? page_max * scale_log2 : NEG_BIG);
+        const bool any_key = page_max > 0.5f * NEG_BIG;
+        const float new_max = fmaxf(c[h].m, any_key ? page_max * scale_log2 : NEG_BIG);
         // the hardware's 2^x: arguments are <= 0 here, and one far below (a first page, a masked key
         // against a real maximum) gives 0
         alpha[h] = __builtin_amdgcn_exp2f(c[h].m - new_max);
         rose |= alpha[h] != 1.0f;
         c[h].m = new_max;
-        shift[h] = -new_max;
+        // a masked score (NEG_BIG) times the scale is far below any maximum: its exponential is 0.
+        // A column without any key so far (maximum NEG_BIG) subtracts nothing, so that the same holds.
+        shift[h] = new_max > 0.5f * NEG_BIG ? -new_max : 0.0f;
     }
     if (__any(rose)) {          // the maximum of some column rose (seldom after the first pages)
 #pragma unroll
@@ -136,7 +148,6 @@ __device__ __forceinline__ void attend_page_as(Columns<HD> (&c)[NH], const uint1
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 e[r] = __builtin_amdgcn_exp2f(fmaf(s[h][kt][r], scale_log2, shift[h]));
-                if (!FULL) e[r] = s[h][kt][r] > 0.5f * NEG_BIG ? e[r] : 0.0f;   // masked, also where the column's maximum is NEG_BIG too
                 sum += e[r];
             }
             p[h][kt][0] = pack_bf16_pair(e[0], e[1]);
@@ -144,7 +155,6 @@ __device__ __forceinline__ void attend_page_as(Columns<HD> (&c)[NH], const uint1
         }
         c[h].l = c[h].l * alpha[h] + sum;
     }
-    const bool partial_page = last_written < PAGE - 1;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
         bf16x8 pf[NH];
@@ -154,6 +164,12 @@ __device__ __forceinline__ void attend_page_as(Columns<HD> (&c)[NH], const uint1
             pf[h] = __builtin_bit_cast(bf16x8, pw);
         }
         const int key_a = kb * 32 + g * 4, key_b = key_a + 16;
+        // keys <= last_written are kept: two keys per 32-bit word, the low half first. Without branches:
+        // one between the load of V and the product would put every product into a block of its own.
+        auto kept = [&](int first_key) -> uint32_t {
+            return first_key + 1 <= last_written ? 0xffffffffu : (first_key <= last_written ? 0xffffu : 0u);
+        };
+        const uint32_t keep_a0 = kept(key_a), keep_a1 = kept(key_a + 2), keep_b0 = kept(key_b), keep_b1 = kept(key_b + 2);
         // Every channel tile of the template is computed, those past head_dim from the last real
         // channel again (their output is never stored): a branch around a matrix product whose
         // result is read right behind the branch is not safe. The compiler spaces a product and
@@ -167,35 +183,15 @@ __device__ __forceinline__ void attend_page_as(Columns<HD> (&c)[NH], const uint1
             const uint16_t* value = v_page + (size_t)channel * v_stride;
             u32x2 va = *reinterpret_cast<const u32x2*>(value + key_a);
             u32x2 vb = *reinterpret_cast<const u32x2*>(value + key_b);
-            if (partial_page) {
-                // keep keys <= last_written only: two keys per 32-bit word, low half first
-                auto keep = [&](uint32_t word, int first_key) -> uint32_t {
-                    if (first_key + 1 <= last_written) return word;
-                    if (first_key <= last_written) return word & 0xffffu;
-                    return 0u;
-                };
-                va = u32x2{keep(va[0], key_a), keep(va[1], key_a + 2)};
-                vb = u32x2{keep(vb[0], key_b), keep(vb[1], key_b + 2)};
-            }
             u32x4 vw = {va[0], va[1], vb[0], vb[1]};
+            if (CLEAN_V) vw = u32x4{va[0] & keep_a0, va[1] & keep_a1, vb[0] & keep_b0, vb[1] & keep_b1};
             const bf16x8 vf = __builtin_bit_cast(bf16x8, vw);
 #pragma unroll
             for (int h = 0; h < NH; ++h) c[h].o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[h], c[h].o[t], 0, 0, 0);
         }
     }
-    // for the same reason the last products have left the pipe before control leaves this
-    // function (the caller joins two variants of it and may read the output at once)
+    // for the same reason the last products have left the pipe before control leaves this function
     fw_mfma_drain();
-}
-
-template <int HD, int NH>
-__device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t* __restrict__ k_page,
-                                            const uint16_t* __restrict__ v_page, int head_dim, float scale_log2,
-                                            int lo, int hi, int last_written, int k_stride, int v_stride) {
-    if (__all(lo <= 0 && hi >= PAGE - 1) && last_written >= PAGE - 1)
-        attend_page_as<HD, NH, true>(c, k_page, v_page, head_dim, scale_log2, lo, hi, last_written, k_stride, v_stride);
-    else
-        attend_page_as<HD, NH, false>(c, k_page, v_page, head_dim, scale_log2, lo, hi, last_written, k_stride, v_stride);
 }
 
 template <int HD>
@@ -282,16 +278,28 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
             hold_v[u] = *reinterpret_cast<const u32x4*>(v_pages + from);
         }
     };
-    auto stash = [&](const u32x4 (&hold_k)[MAX_RUNS], const u32x4 (&hold_v)[MAX_RUNS], int buffer) {
+    // The values of keys past the last one written (only in the tile's last page) are zeroed on
+    // their way to LDS: whatever an earlier owner of the page left there must not meet P = 0.
+    auto stash = [&](const u32x4 (&hold_k)[MAX_RUNS], const u32x4 (&hold_v)[MAX_RUNS], int buffer, int block) {
         uint16_t* kt = lds + (size_t)buffer * (k_elems + v_elems);
         uint16_t* vt = kt + k_elems;
         const int k_per_row = head_dim / 8;
+        const int last_written = pos_hi - block * PAGE;         // < 0 for a page past the end: never attended
 #pragma unroll
         for (int u = 0; u < MAX_RUNS; ++u) {
             const int run = tid + u * 256;
             if (run < k_runs) {
                 *reinterpret_cast<u32x4*>(kt + (run / k_per_row) * k_stride + (run % k_per_row) * 8) = hold_k[u];
-                *reinterpret_cast<u32x4*>(vt + (run / 8) * v_stride + (run % 8) * 8) = hold_v[u];
+                u32x4 v = hold_v[u];
+                if (last_written < PAGE - 1) {
+                    const int key0 = (run % 8) * 8;             // this run: keys key0 .. key0 + 7 of one channel
+#pragma unroll
+                    for (int word = 0; word < 4; ++word) {
+                        const int first_key = key0 + 2 * word;
+                        v[word] &= first_key + 1 <= last_written ? 0xffffffffu : (first_key <= last_written ? 0xffffu : 0u);
+                    }
+                }
+                *reinterpret_cast<u32x4*>(vt + (run / 8) * v_stride + (run % 8) * 8) = v;
             }
         }
     };
@@ -301,7 +309,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
             const uint16_t* kt = lds + (size_t)buffer * (k_elems + v_elems);
             // a lane without a row computes along with the bounds of the tile's first row (nothing of
             // it is stored): a page that is whole for the rows is then whole for the wave
-            attend_page<HD, NH>(c, kt, kt + k_elems, head_dim, scale_log2, my_first - base, my_pos - base, pos_hi - base,
+            attend_page<HD, NH, false>(c, kt, kt + k_elems, head_dim, scale_log2, my_first - base, my_pos - base, pos_hi - base,
                             k_stride, v_stride);
         }
     };
@@ -310,19 +318,19 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     // buffer (b - first) % 2, stored while page b - 1 is worked on -> attended
     fetch(hold_k0, hold_v0, first_block);
     fetch(hold_k1, hold_v1, first_block + 1);
-    stash(hold_k0, hold_v0, 0);
+    stash(hold_k0, hold_v0, 0, first_block);
     fw_lds_barrier();
     for (int block = first_block; block <= last_block; block += 2) {
         fetch(hold_k0, hold_v0, block + 2);
         __builtin_amdgcn_sched_barrier(0);      // keep the requests ahead of the work they overlap
         attend(block, 0);
-        stash(hold_k1, hold_v1, 1);
+        stash(hold_k1, hold_v1, 1, block + 1);
         fw_lds_barrier();
         if (block + 1 > last_block) break;
         fetch(hold_k1, hold_v1, block + 3);
         __builtin_amdgcn_sched_barrier(0);
         attend(block + 1, 1);
-        stash(hold_k0, hold_v0, 0);
+        stash(hold_k0, hold_v0, 0, block + 2);
         fw_lds_barrier();
     }
 #pragma unroll
@@ -383,7 +391,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) void attention_decode_split_kerne
         const size_t at = ((size_t)page * num_kv_heads + kvh) * PAGE * head_dim;
         const int base = block * PAGE;
         // a lane without a head computes along (q = 0, nothing of it is stored)
-        attend_page<HD, 1>(columns_of_wave, k_pages + at, v_pages + at, head_dim, scale_log2, first - base, pos - base, pos - base,
+        attend_page<HD, 1, true>(columns_of_wave, k_pages + at, v_pages + at, head_dim, scale_log2, first - base, pos - base, pos - base,
                         head_dim, PAGE);
     }
     float l = c.l;
