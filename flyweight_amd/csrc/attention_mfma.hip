@@ -56,7 +56,9 @@ struct Columns {
 // keys of this page that this lane's column may see are those with lo <= key <= hi
 // (page-relative; hi < 0: none). `last_written`: keys beyond it hold whatever an earlier owner of
 // the page left, and are zeroed before they meet P = 0: here if CLEAN_V, else the caller has done
-// it (the prompt kernel does when it copies a page to LDS).
+// it (the prompt kernel does when it copies a page to LDS). K_PADDED: a key's row holds HD channels,
+// those past head_dim zero (the prompt kernel's LDS tile), so every lane loads; else the lanes past
+// head_dim take zeros without loading.
 //
 // The softmax arithmetic (one exponential per score on the quarter-rate unit) takes more issue
 // cycles than the matrix products take on their pipe, so the work is laid out in phases, each
@@ -67,7 +69,7 @@ struct Columns {
 // (all pages but those on the diagonal, at a window's edge, and a sequence's last) skips the
 // mask. The scale is folded into the exponent's argument: the maximum is taken over the raw
 // scores (the scale is positive) and kept scaled.
-template <int HD, int NH, bool CLEAN_V>
+template <int HD, int NH, bool CLEAN_V, bool K_PADDED>
 __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t* __restrict__ k_page,
                                             const uint16_t* __restrict__ v_page, int head_dim, float scale_log2,
                                             int lo, int hi, int last_written, int k_stride, int v_stride) {
@@ -80,8 +82,12 @@ __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t
         const uint16_t* key = k_page + (size_t)(kt * 16 + i16) * k_stride + g * 8;
 #pragma unroll
         for (int dc = 0; dc < HD / 32; ++dc) {
-            kf[kt][dc] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-            if (dc * 32 + g * 8 < head_dim) kf[kt][dc] = *reinterpret_cast<const bf16x8*>(key + dc * 32);
+            if (K_PADDED) {
+                kf[kt][dc] = *reinterpret_cast<const bf16x8*>(key + dc * 32);
+            } else {
+                kf[kt][dc] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (dc * 32 + g * 8 < head_dim) kf[kt][dc] = *reinterpret_cast<const bf16x8*>(key + dc * 32);
+            }
         }
     }
     // scores of all heads
@@ -118,8 +124,7 @@ __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) page_max = fmaxf(page_max, s[h][kt][r]);
-        page_max = fmaxf(page_max, __shfl_xor(page_max, 16, 64));
-        page_max = fmaxf(page_max, __shfl_xor(page_max, 32, 64));
+        page_max = fw_quad_max(page_max);
         // a column that has seen no key yet keeps NEG_BIG (the raw maximum times the scale would overflow)
         const bool any_key = page_max > 0.5f * NEG_BIG;
         const float new_max = fmaxf(c[h].m, any_key ? page_max * scale_log2 : NEG_BIG);
@@ -226,9 +231,18 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     const int32_t* __restrict__ tile_seg, const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ seg_row0,
     const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, float scale_log2, int window) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-    const int k_stride = head_dim + KV_PAD, v_stride = PAGE + KV_PAD;
+    // a key's row in LDS holds HD channels, those past head_dim zero: every lane loads its operand
+    constexpr int k_stride = HD + KV_PAD;
+    const int v_stride = PAGE + KV_PAD;
     const int k_elems = PAGE * k_stride, v_elems = head_dim * v_stride;
     uint16_t* lds = reinterpret_cast<uint16_t*>(lds_raw);      // [buffer][K tile | V tile]
+    if (head_dim < HD) {
+        const int runs_per_row = (HD - head_dim) / 8;          // head_dim is a multiple of 16
+        for (int run = threadIdx.x; run < 2 * PAGE * runs_per_row; run += 256) {
+            const int buffer = run / (PAGE * runs_per_row), row = run / runs_per_row % PAGE, at = run % runs_per_row;
+            *reinterpret_cast<u32x4*>(lds + (size_t)buffer * (k_elems + v_elems) + row * k_stride + head_dim + at * 8) = u32x4{0u, 0u, 0u, 0u};
+        }
+    }
 
     // the last tiles of a long prompt see the most keys: they start first, the short ones fill in behind
     const int tile = gridDim.x - 1 - blockIdx.x;
@@ -268,14 +282,21 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     constexpr int MAX_RUNS = HD * PAGE / 8 / 256;                                // per thread, per operand
     const int first_block = tile_first / PAGE, last_block = pos_hi / PAGE;
     u32x4 hold_k0[MAX_RUNS], hold_v0[MAX_RUNS], hold_k1[MAX_RUNS], hold_v1[MAX_RUNS];
+    // what a thread copies of every page: fixed offsets, so that a page's address is a scalar
+    // base plus these (no vector arithmetic per page; the registers that receive a page are
+    // otherwise borrowed for it, and giving them back means waiting for loads still in flight)
+    uint32_t run_offset[MAX_RUNS];
+#pragma unroll
+    for (int u = 0; u < MAX_RUNS; ++u) run_offset[u] = (uint32_t)(tid + u * 256 < k_runs ? tid + u * 256 : 0) * 8u;
     auto fetch = [&](u32x4 (&hold_k)[MAX_RUNS], u32x4 (&hold_v)[MAX_RUNS], int block) {
-        const size_t at = ((size_t)table[block < last_block ? block : last_block] * num_kv_heads + kvh) * page_elems;
+        const int page = __builtin_amdgcn_readfirstlane(table[block < last_block ? block : last_block]);
+        const size_t at = ((size_t)page * num_kv_heads + kvh) * page_elems;
+        const uint16_t* k_from = k_pages + at;
+        const uint16_t* v_from = v_pages + at;
 #pragma unroll
         for (int u = 0; u < MAX_RUNS; ++u) {
-            const int run = tid + u * 256;
-            const size_t from = at + (size_t)(run < k_runs ? run : 0) * 8;
-            hold_k[u] = *reinterpret_cast<const u32x4*>(k_pages + from);
-            hold_v[u] = *reinterpret_cast<const u32x4*>(v_pages + from);
+            hold_k[u] = *reinterpret_cast<const u32x4*>(k_from + run_offset[u]);
+            hold_v[u] = *reinterpret_cast<const u32x4*>(v_from + run_offset[u]);
         }
     };
     // The values of keys past the last one written (only in the tile's last page) are zeroed on
@@ -309,7 +330,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
             const uint16_t* kt = lds + (size_t)buffer * (k_elems + v_elems);
             // a lane without a row computes along with the bounds of the tile's first row (nothing of
             // it is stored): a page that is whole for the rows is then whole for the wave
-            attend_page<HD, NH, false>(c, kt, kt + k_elems, head_dim, scale_log2, my_first - base, my_pos - base, pos_hi - base,
+            attend_page<HD, NH, false, true>(c, kt, kt + k_elems, head_dim, scale_log2, my_first - base, my_pos - base, pos_hi - base,
                             k_stride, v_stride);
         }
     };
@@ -335,9 +356,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
     }
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
-        float l = c[h].l;
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
+        const float l = fw_quad_sum(c[h].l);
         if (!valid || first_in_group + h >= group) continue;
         const float inv = 1.0f / l;
         uint16_t* dest = out + ((size_t)my_row * num_heads + kvh * group + first_in_group + h) * head_dim;
@@ -391,12 +410,10 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) void attention_decode_split_kerne
         const size_t at = ((size_t)page * num_kv_heads + kvh) * PAGE * head_dim;
         const int base = block * PAGE;
         // a lane without a head computes along (q = 0, nothing of it is stored)
-        attend_page<HD, 1, true>(columns_of_wave, k_pages + at, v_pages + at, head_dim, scale_log2, first - base, pos - base, pos - base,
+        attend_page<HD, 1, true, false>(columns_of_wave, k_pages + at, v_pages + at, head_dim, scale_log2, first - base, pos - base, pos - base,
                         head_dim, PAGE);
     }
-    float l = c.l;
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    const float l = fw_quad_sum(c.l);
 #pragma unroll
     for (int t = 0; t < HD / 16; ++t) shared_o[wave][t][lane] = c.o[t];
     if (g == 0) {
@@ -535,9 +552,9 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
         heads_together = most_together == 4 && group >= 4 && (long long)tiles * num_kv_heads * ((group + 3) / 4) >= 256 ? 4 : 1;
     dim3 grid(tiles, num_kv_heads * ((group + heads_together - 1) / heads_together));
     FW_REQUIRE(grid.y <= 65535, "attention_prefill: too many heads");
-    const int lds_bytes = 2 * (PAGE * (head_dim + KV_PAD) + head_dim * (PAGE + KV_PAD)) * 2;
 #define LAUNCH(HD, NH)                                                                                             \
     {                                                                                                              \
+        const int lds_bytes = 2 * (PAGE * (HD + KV_PAD) + head_dim * (PAGE + KV_PAD)) * 2;                         \
         static int configured = 0;                                                                                 \
         if (lds_bytes > configured) {                                                                              \
             hipError_t status = hipFuncSetAttribute((const void*)attention_prefill_kernel<HD, NH>,                 \

@@ -20,6 +20,44 @@ __device__ __forceinline__ void fw_lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Reductions over the four lanes l, l ^ 16, l ^ 32, l ^ 48 of a wave (every lane gets the result)
+// with the row-swap instructions of gfx950 instead of two trips through the LDS crossbar
+// (__shfl_xor). v_permlane16_swap exchanges rows 1 and 3 of its first register with rows 0 and 2
+// of its second; v_permlane32_swap the upper half of the first with the lower half of the second.
+// Given one value in two registers, the two results of a swap are the two partners of a lane.
+// The second copy is made opaque: given one value twice the compiler may name one register
+// twice, and the instruction then swaps rows inside that register. The results are taken as
+// scalars before they are reinterpreted (a bit cast straight from the builtin's vector result
+// lost its second element at compile time).
+__device__ __forceinline__ void fw_quad_partners16(float x, float& mine, float& partner) {
+    uint32_t u = __float_as_uint(x), copy = u;
+    asm volatile("" : "+v"(copy));
+    const auto swapped = __builtin_amdgcn_permlane16_swap(u, copy, false, false);
+    const uint32_t first = swapped[0], second = swapped[1];
+    mine = __uint_as_float(first);
+    partner = __uint_as_float(second);
+}
+__device__ __forceinline__ void fw_quad_partners32(float x, float& mine, float& partner) {
+    uint32_t u = __float_as_uint(x), copy = u;
+    asm volatile("" : "+v"(copy));
+    const auto swapped = __builtin_amdgcn_permlane32_swap(u, copy, false, false);
+    const uint32_t first = swapped[0], second = swapped[1];
+    mine = __uint_as_float(first);
+    partner = __uint_as_float(second);
+}
+__device__ __forceinline__ float fw_quad_max(float x) {
+    float a, b;
+    fw_quad_partners16(x, a, b);
+    fw_quad_partners32(fmaxf(a, b), a, b);
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float fw_quad_sum(float x) {
+    float a, b;
+    fw_quad_partners16(x, a, b);
+    fw_quad_partners32(a + b, a, b);
+    return a + b;
+}
+
 // Lets the matrix pipe finish what was issued before control goes on. Inside one basic block the
 // compiler keeps a product and the first read of its result far enough apart; where the read is
 // the target of a taken branch it has been seen one instruction behind the product, reading the
