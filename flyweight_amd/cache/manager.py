@@ -250,35 +250,42 @@ class CacheManager:
             raise CacheAccountingError(host.last_error())
 
     # ----- a whole step at once (one call into the host library each) ------------------------------
-    def _natives(self, requests: Sequence[Hashable]):
+    # ``natives``: what ``natives_of`` gave for the same requests, so that a step that makes
+    # several of these calls translates its request keys once.
+    def natives_of(self, requests: Sequence[Hashable]):
+        """The host library's ids of these requests (-1 for one it has never seen), as a C array."""
+        small = _FIRST_NAMED_ID
+        if all(type(r) is int and 0 <= r < small for r in requests):
+            return (ctypes.c_int64 * max(len(requests), 1))(*requests)
         natives = host.ids(len(requests))
         for i, request in enumerate(requests):
             native = self._id(request, create=False)
             natives[i] = -1 if native is None else native
         return natives
 
-    def describe(self, requests: Sequence[Hashable]) -> Tuple[List[int], List[int]]:
+    def describe(self, requests: Sequence[Hashable], natives=None) -> Tuple[List[int], List[int]]:
         """(lengths, slots) of live requests; KeyError names the first one that is not live."""
         count = len(requests)
         lengths, slots = host.ints(count), host.ints(count)
-        if self._lib.fwh_cache_describe(self._native, self._natives(requests), count, lengths, slots) < 0:
+        natives = self.natives_of(requests) if natives is None else natives
+        if self._lib.fwh_cache_describe(self._native, natives, count, lengths, slots) < 0:
             raise KeyError(next((r for r in requests if r not in self.requests), host.last_error()))
-        return list(lengths[:count]), list(slots[:count])
+        return lengths[:count], slots[:count]
 
-    def reserve_all(self, requests: Sequence[Hashable], new_lengths: Sequence[int]) -> None:
+    def reserve_all(self, requests: Sequence[Hashable], new_lengths: Sequence[int], natives=None) -> None:
         """The reservations of a whole step: all of them, or OutOfPages and nothing changed."""
         count = len(requests)
-        status = self._lib.fwh_cache_reserve_batch(self._native, self._natives(requests),
-                                                   (ctypes.c_int * max(count, 1))(*[int(n) for n in new_lengths]), count)
+        natives = self.natives_of(requests) if natives is None else natives
+        status = self._lib.fwh_cache_reserve_batch(self._native, natives, (ctypes.c_int * max(count, 1))(*new_lengths), count)
         if status == host.OUT_OF_PAGES:
             raise OutOfPages(host.last_error())
         if status < 0:
             raise KeyError(host.last_error())
 
-    def commit_all(self, requests: Sequence[Hashable], new_lengths: Sequence[int]) -> None:
+    def commit_all(self, requests: Sequence[Hashable], new_lengths: Sequence[int], natives=None) -> None:
         count = len(requests)
-        if self._lib.fwh_cache_commit_batch(self._native, self._natives(requests),
-                                            (ctypes.c_int * max(count, 1))(*[int(n) for n in new_lengths]), count) < 0:
+        natives = self.natives_of(requests) if natives is None else natives
+        if self._lib.fwh_cache_commit_batch(self._native, natives, (ctypes.c_int * max(count, 1))(*new_lengths), count) < 0:
             raise ValueError(host.last_error())
 
     def commit(self, request: Hashable, new_length: int) -> None:
@@ -295,14 +302,17 @@ class CacheManager:
         self._forget(request)
 
     # ----- views for the step function ---------------------------------------------------
-    def block_table_rows(self, group_index: int, requests: Sequence[Hashable], stride: Optional[int] = None) -> np.ndarray:
-        natives = host.ids(len(requests))
-        for i, request in enumerate(requests):
-            natives[i] = self._live_id(request)
+    def block_table_rows(self, group_index: int, requests: Sequence[Hashable], stride: Optional[int] = None,
+                         natives=None) -> np.ndarray:
+        if natives is None:
+            natives = self.natives_of(requests)
         if stride is None:
             stride = max(self._lib.fwh_cache_longest_table(self._native, group_index, natives, len(requests)), 1)
         rows = np.zeros((len(requests), stride), dtype=np.int32)
         if self._lib.fwh_cache_fill_tables(self._native, group_index, natives, len(requests), stride, rows.ctypes.data) < 0:
+            for request in requests:
+                if request not in self.requests:
+                    raise KeyError(f"request {request!r} is not live")
             raise CacheAccountingError(host.last_error())
         return rows
 

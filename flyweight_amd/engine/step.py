@@ -35,7 +35,8 @@ class StepEntry:
 def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int, max_positions: int):
     """What a step may not bring: no entries, an unknown or repeated request, no tokens, a token
     outside the vocabulary, a place outside the entry, a sequence past the model's limit.
-    Returns the requests' current lengths and slots (one call into the host library)."""
+    Returns the requests' current lengths and slots (one call into the host library) and the
+    host library's ids of the requests, for the step's further calls."""
     if not entries:
         raise StepError("a step needs at least one entry")
     requests = [entry.request for entry in entries]
@@ -45,10 +46,25 @@ def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size:
             if request in seen:
                 raise StepError(f"request {request!r} appears twice in one step")
             seen.add(request)
+    natives = cache.natives_of(requests)
     try:
-        lengths, slots = cache.describe(requests)
+        lengths, slots = cache.describe(requests, natives)
     except KeyError as error:
         raise StepError(f"request {error.args[0]!r} was not admitted") from None
+    if all(len(entry.tokens) == 1 for entry in entries):
+        # a decode step: the same checks without a loop over the entries' fields
+        tokens = [entry.tokens[0] for entry in entries]
+        if max(lengths) + 1 > max_positions:
+            entry, start = next((e, s) for e, s in zip(entries, lengths) if s + 1 > max_positions)
+            raise StepError(f"request {entry.request!r} would reach {start + 1} tokens; the model's limit is {max_positions}")
+        if not (0 <= int(min(tokens)) and int(max(tokens)) < vocab_size):
+            entry = next(e for e in entries if not 0 <= int(e.tokens[0]) < vocab_size)
+            raise StepError(f"token id {entry.tokens[0]} of request {entry.request!r} is outside the vocabulary (0..{vocab_size - 1})")
+        for entry in entries:
+            for place in entry.want:
+                if int(place) != 0:
+                    raise StepError(f"request {entry.request!r} wants logits at place {place} of 1 tokens")
+        return lengths, slots, natives
     for entry, start in zip(entries, lengths):
         n = len(entry.tokens)
         if n < 1:
@@ -62,7 +78,7 @@ def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size:
         for place in entry.want:
             if not 0 <= int(place) < n:
                 raise StepError(f"request {entry.request!r} wants logits at place {place} of {n} tokens")
-    return lengths, slots
+    return lengths, slots, natives
 
 
 class StepContext:
@@ -74,7 +90,7 @@ class StepContext:
                  max_positions: int, described=None):
         """``described``: (lengths, slots) of the entries' requests if the caller has checked the
         entries already (``check_entries``)."""
-        starts, slots = described if described is not None else check_entries(entries, cache, vocab_size, max_positions)
+        starts, slots, natives = described if described is not None else check_entries(entries, cache, vocab_size, max_positions)
         # per-row arrays are put together from one numpy piece per entry: a prompt portion has
         # thousands of rows, and a Python loop over them would take longer than some kernels
         token_parts, pos_parts, seg_parts = [], [], []
@@ -106,7 +122,7 @@ class StepContext:
         self.host_seg_slot = seg_slot
 
         tile_seg, tile_row0 = ops.query_tiles(seg_row0)        # tiles of up to 64 rows for the prompt attention kernel
-        tables = [cache.block_table_rows(g, self.requests) for g in range(len(cache.groups))]
+        tables = [cache.block_table_rows(g, self.requests, natives=natives) for g in range(len(cache.groups))]
         pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows,
                                                           tile_seg, tile_row0)]
         pieces += [t.reshape(-1) for t in tables]
@@ -159,7 +175,11 @@ class StepContext:
         """Writes this step's tokens, positions, slots and block tables and uploads them."""
         host = self._host
         self.requests = [e.request for e in entries]
-        starts, slots = described if described is not None else cache.describe(self.requests)
+        if described is not None:
+            starts, slots, natives = described
+        else:
+            natives = cache.natives_of(self.requests)
+            starts, slots = cache.describe(self.requests, natives)
         uploaded = getattr(self, "_uploaded", None)
         if uploaded is not None:
             uploaded.synchronize()      # the pinned buffer is still being read until the last upload has run
@@ -168,7 +188,7 @@ class StepContext:
         host[1][:] = starts
         host[4][:] = slots
         for g in range(len(cache.groups)):
-            host[8 + g][:] = cache.block_table_rows(g, self.requests, stride=self._table_stride).reshape(-1)
+            host[8 + g][:] = cache.block_table_rows(g, self.requests, stride=self._table_stride, natives=natives).reshape(-1)
         self.device_buffer.copy_(self.host_buffer, non_blocking=True)
         if uploaded is None:
             uploaded = self._uploaded = torch.cuda.Event()
@@ -232,14 +252,14 @@ class Stepper:
         requests = [entry.request for entry in entries]
         new_lengths = [start + len(entry.tokens) for entry, start in zip(entries, described[0])]
         # reserve everything first so that a failure leaves no request half-served
-        cache.reserve_all(requests, new_lengths)
+        cache.reserve_all(requests, new_lengths, described[2])
         if self.use_graphs and all(len(entry.tokens) == 1 for entry in entries):
             captured = self._captured_decode(len(entries))
             if captured is not None:
                 return self._replay(captured, entries, described)
         ctx = StepContext(entries, cache, self.device, spec.vocab_size, spec.max_positions, described=described)
         logits = self.model.forward(ctx, cache)
-        cache.commit_all(ctx.requests, ctx.new_lengths)
+        cache.commit_all(ctx.requests, ctx.new_lengths, described[2])
         self.steps += 1
         self.tokens_run += ctx.num_rows
         return logits
@@ -278,7 +298,7 @@ class Stepper:
             captured.graph = graph
         captured.graph.replay()
         self.graph_replays += 1
-        cache.commit_all(ctx.requests, ctx.new_lengths)
+        cache.commit_all(ctx.requests, ctx.new_lengths, None if described is None else described[2])
         self.steps += 1
         self.tokens_run += ctx.num_rows
         wanted = [i for i, entry in enumerate(entries) if len(entry.want)]
