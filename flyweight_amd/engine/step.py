@@ -115,6 +115,12 @@ class StepContext:
         self.num_wanted = len(want_rows)
         self.all_decode = self.num_rows == self.num_segments
         self.max_context = max(self.new_lengths)
+        # segments of one token that a mixed step begins with (a scheduler puts the decoded tokens
+        # first): mixers may give them to their decode kernels. Their rows and query tiles are 0 .. n - 1.
+        self.decode_prefix = 0
+        if not self.all_decode:
+            while len(entries[self.decode_prefix].tokens) == 1:
+                self.decode_prefix += 1
         self.device = device
         # the same on the host, for parts that plan their work there
         self.host_row_pos = row_pos
@@ -145,6 +151,7 @@ class StepContext:
         self = cls.__new__(cls)
         self.num_rows = self.num_segments = self.num_wanted = batch
         self.all_decode = True
+        self.decode_prefix = 0
         self.max_context = max_context          # bounds the split-key grid, not the result
         self.device = device
         self.host_row_pos = self.host_seg_row0 = self.host_seg_slot = None     # not for captured steps

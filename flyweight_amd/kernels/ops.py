@@ -583,8 +583,9 @@ def decode_splits(max_context: int, window: int = 0) -> int:
 def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                       v_pages: torch.Tensor, block_table: torch.Tensor, tile_seg: torch.Tensor, tile_row0: torch.Tensor,
                       seg_row0: torch.Tensor, row_pos: torch.Tensor, scale: float, window: int = 0,
-                      heads_together: int = 0) -> torch.Tensor:
-    """``heads_together``: query heads of a kv group per workgroup (1, or 4 up to head_dim 64), 0: the kernel's choice."""
+                      heads_together: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``heads_together``: query heads of a kv group per workgroup (1, or 4 up to head_dim 64), 0: the
+    kernel's choice. Only the rows of the given tiles are written (into ``out`` if given)."""
     _dev(q, k_pages, v_pages, block_table, tile_seg, tile_row0, seg_row0, row_pos)
     _want(q, torch.bfloat16, "q")
     rows = q.shape[0]
@@ -596,7 +597,10 @@ def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_pos.numel() < rows or tile_seg.numel() != tile_row0.numel():
         raise KernelError("attention: batch index arrays are inconsistent")
-    out = torch.empty_like(q)
+    if out is None:
+        out = torch.empty_like(q)
+    elif out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
+        raise KernelError("attention: out must be like q")
     _check(library().fw_attention_prefill(
         _p(q), _p(out), _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(tile_seg), _p(tile_row0),
         tile_seg.numel(), _p(seg_row0), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale),
@@ -606,7 +610,7 @@ def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
 
 def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                      v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
-                     scale: float, max_context: int, window: int = 0) -> torch.Tensor:
+                     scale: float, max_context: int, window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One row per request; ``max_context`` bounds position + 1 of every row (the host knows it)."""
     _dev(q, k_pages, v_pages, block_table, row_seg, row_pos)
     _want(q, torch.bfloat16, "q")
@@ -620,7 +624,10 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
         raise KernelError("attention: batch index arrays are too short")
     splits = decode_splits(max_context, window)
     partial = torch.empty((rows, num_heads, splits, head_dim + 4), dtype=torch.float32, device=q.device)
-    out = torch.empty_like(q)
+    if out is None:
+        out = torch.empty_like(q)
+    elif out.shape != q.shape or out.dtype != q.dtype or not out.is_contiguous():
+        raise KernelError("attention: out must be like q")
     group = num_heads // num_kv_heads
     tickets = _medium_counters(q.device, rows * num_kv_heads * ((group + 15) // 16))
     _check(library().fw_attention_decode(
@@ -633,15 +640,24 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
 
 def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
               v_pages: torch.Tensor, block_table: torch.Tensor, ctx, scale: float, window: int = 0) -> torch.Tensor:
-    """bfloat16 with a head size in steps of 16 runs on the matrix cores (the split-key
-    decode kernel when every segment is one row, the tiled one otherwise); float32 and
-    everything else on the generic kernel."""
+    """bfloat16 with a head size in steps of 16 runs on the matrix cores: the split-key decode
+    kernel for segments of one row (all of them, or those a mixed step begins with: a single row
+    would hold a 64-row tile of the prompt kernel and walk its whole context alone), the tiled
+    kernel for the rest; float32 and everything else on the generic kernel."""
     fast = q.dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= MAX_HEAD_DIM
     if fast and ctx.all_decode:
         return attention_decode(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                                 ctx.row_pos, scale, ctx.max_context, window)
     if fast:
-        return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.tile_seg,
-                                 ctx.tile_row0, ctx.seg_row0, ctx.row_pos, scale, window)
+        single = getattr(ctx, "decode_prefix", 0)       # leading segments of one row: rows and tiles 0 .. single - 1
+        if single == 0:
+            return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.tile_seg,
+                                     ctx.tile_row0, ctx.seg_row0, ctx.row_pos, scale, window)
+        out = torch.empty_like(q)
+        attention_decode(q[:single], num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
+                         ctx.row_pos, scale, ctx.max_context, window, out=out[:single])
+        return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table,
+                                 ctx.tile_seg[single:], ctx.tile_row0[single:], ctx.seg_row0, ctx.row_pos, scale, window,
+                                 out=out)
     return attention_generic(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                              ctx.row_pos, scale, window)

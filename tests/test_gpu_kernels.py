@@ -496,6 +496,36 @@ def test_attention_prefill_on_the_matrix_cores(ops, nh, nkv, hd, window):
     close(generic, want, torch.bfloat16)
 
 
+@pytest.mark.parametrize("window", [0, 50])
+def test_attention_gives_the_leading_single_rows_of_a_mixed_step_to_the_decode_kernel(ops, window):
+    """A step that begins with decoded tokens and goes on with portions of prompts: the single rows
+    in front go through the split-key kernel, everything else (a single row further back too)
+    through the tiled one, and both write one output."""
+    from types import SimpleNamespace
+    nh, nkv, hd = 8, 2, 64
+    lengths = [131, 6, 57, 71, 300]
+    starts = [130, 5, 20, 70, 290]
+    keys, values, table, k_pages, v_pages = _mfma_setup(nh, nkv, hd, lengths, num_pages=16, seed=9)
+    counts = [n - s for n, s in zip(lengths, starts)]
+    seg_row0 = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    row_pos = np.concatenate([np.arange(s, n) for s, n in zip(starts, lengths)]).astype(np.int32)
+    row_seg = np.concatenate([np.full(c, i) for i, c in enumerate(counts)]).astype(np.int32)
+    tile_seg, tile_row0 = ops.query_tiles(seg_row0.tolist())
+    rows = int(seg_row0[-1])
+    q = as_dev(gen(rows, nh * hd, seed=8), torch.bfloat16)
+    scale = 1 / math.sqrt(hd)
+    d = lambda a: torch.tensor(np.asarray(a, dtype=np.int32), device=DEV)       # noqa: E731
+    ctx = SimpleNamespace(all_decode=False, decode_prefix=2, max_context=max(lengths), row_seg=d(row_seg), row_pos=d(row_pos),
+                          tile_seg=d(tile_seg), tile_row0=d(tile_row0), seg_row0=d(seg_row0))
+    mixed = ops.attention(q, nh, nkv, hd, k_pages, v_pages, d(table), ctx, scale, window)
+    want = torch.stack([attention_reference(back(q)[r].reshape(nh, hd), keys[row_seg[r]], values[row_seg[r]], int(row_pos[r]),
+                                            scale, window, nh // nkv).reshape(-1) for r in range(rows)])
+    close(mixed, want, torch.bfloat16)
+    ctx.decode_prefix = 0
+    tiled = ops.attention(q, nh, nkv, hd, k_pages, v_pages, d(table), ctx, scale, window)
+    assert torch.equal(mixed[2:], tiled[2:])        # the rows of the tiled kernel do not depend on who else it serves
+
+
 @pytest.mark.parametrize("nh,nkv,hd,window", [(4, 1, 16, 0), (3, 1, 48, 0), (12, 2, 64, 0), (32, 8, 64, 0), (8, 2, 32, 70)])
 def test_attention_prefill_takes_four_heads_of_a_group_together(ops, nh, nkv, hd, window):
     """One workgroup reads a page once for four query heads of the kv group: whole runs of four,
