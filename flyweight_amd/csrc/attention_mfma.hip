@@ -214,7 +214,9 @@ __device__ __forceinline__ void load_query(Columns<HD>& c, const uint16_t* __res
 }
 
 // ---- prompt portions ---------------------------------------------------------------------------
-// grid (tiles of 64 query rows, kv heads * runs of NH query heads of a kv group); four waves, 16
+// A workgroup per (tile of 64 query rows, kv head, run of NH query heads of its group), numbered
+// tile by tile in the order the caller lists the tiles (those that see the most keys first: the
+// short ones then fill in behind, whatever head they belong to); four waves, 16
 // rows each, every wave with the same NH heads: a page's keys and values are read once for all
 // of them (from global memory and from LDS), which is what a long context is bound by. Fewer
 // heads per workgroup give more and shorter workgroups, which evens out a short causal prompt.
@@ -244,10 +246,10 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
         }
     }
 
-    // the last tiles of a long prompt see the most keys: they start first, the short ones fill in behind
-    const int tile = gridDim.x - 1 - blockIdx.x;
     const int group = num_heads / num_kv_heads, runs = (group + NH - 1) / NH;
-    const int kvh = blockIdx.y / runs, first_in_group = (blockIdx.y % runs) * NH;
+    const int per_tile = num_kv_heads * runs;
+    const int tile = blockIdx.x / per_tile, of_tile = blockIdx.x % per_tile;
+    const int kvh = of_tile / runs, first_in_group = (of_tile % runs) * NH;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 15, g = lane >> 4;
     const int seg = tile_seg[tile];
     const int tile_first_row = tile_row0[tile];
@@ -530,11 +532,13 @@ static int check_common(const char* name, int rows, int num_heads, int num_kv_he
     } while (0)
 
 // bfloat16 q [rows][heads * head_dim] -> out (same shape). tile_seg / tile_row0 [tiles]: tiles of
-// up to 64 rows that never span two segments. heads_together: query heads of a kv group that one
-// workgroup takes (1, or 4 up to head_dim 64), or 0: chosen here: 4 where the group has as many
-// and that still gives every compute unit a workgroup (measured at 2,048 rows, 32 heads in 8
-// groups, head_dim 64: 94 vs 110 us from position 0, 1.18 vs 1.47 ms behind 30,720 tokens; at
-// 512 rows 29 vs 17 us; two together never beat one).
+// up to 64 rows that never span two segments, in any order (workgroups start in that order: list
+// the tiles that see the most keys first). heads_together: query heads of a kv group that one
+// workgroup takes (1, or 4 up to head_dim 64). Four read a page once for four heads (1.09 vs
+// 1.27 ms for 2,048 rows behind 30,720 tokens, 32 heads in 8 groups, head_dim 64), one gives four
+// times as many workgroups to even out tiles of unequal length (58 vs 81 us for the same rows
+// from position 0; equal behind 6,144 tokens). The caller, who knows the positions, says which;
+// 0: chosen here from the shape alone: 4 where that still leaves every compute unit four workgroups.
 extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_pages, const void* v_pages,
                                     const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                                     const int32_t* tile_row0, int tiles, const int32_t* seg_row0,
@@ -549,9 +553,10 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
     if (rows == 0 || tiles == 0) return 0;
     const int group = num_heads / num_kv_heads;
     if (heads_together == 0)
-        heads_together = most_together == 4 && group >= 4 && (long long)tiles * num_kv_heads * ((group + 3) / 4) >= 256 ? 4 : 1;
-    dim3 grid(tiles, num_kv_heads * ((group + heads_together - 1) / heads_together));
-    FW_REQUIRE(grid.y <= 65535, "attention_prefill: too many heads");
+        heads_together = most_together == 4 && group >= 4 && (long long)tiles * num_kv_heads * ((group + 3) / 4) >= 1024 ? 4 : 1;
+    const long long blocks = (long long)tiles * num_kv_heads * ((group + heads_together - 1) / heads_together);
+    FW_REQUIRE(blocks < (1ll << 31), "attention_prefill: too many tiles and heads");
+    dim3 grid((unsigned)blocks);
 #define LAUNCH(HD, NH)                                                                                             \
     {                                                                                                              \
         const int lds_bytes = 2 * (PAGE * (HD + KV_PAD) + head_dim * (PAGE + KV_PAD)) * 2;                         \

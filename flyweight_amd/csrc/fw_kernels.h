@@ -122,9 +122,10 @@ int fw_attention_generic(const void* q, void* out, int dtype, const void* k_page
 
 // The same attention on the matrix cores, bfloat16 only, head_dim a multiple of 16 up to 256.
 // Prompt portions: rows are cut into tiles of up to 64 that never span two segments (tile_seg,
-// tile_row0). heads_together: how many query heads of a kv group one workgroup takes, reading
-// the keys and values once for all of them (1, or 4 up to head_dim 64); 0: 4 where the group has
-// as many and every compute unit still gets a workgroup, else 1.
+// tile_row0), in any order: workgroups start in the order of the tiles, so the caller lists those
+// that see the most keys first. heads_together: how many query heads of a kv group one workgroup takes, reading
+// the keys and values once for all of them (1, or 4 up to head_dim 64: 4 pays behind a long
+// context, 1 evens out a short causal prompt); 0: chosen from the shape alone.
 int fw_attention_prefill(const void* q, void* out, const void* k_pages, const void* v_pages,
                          const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                          const int32_t* tile_row0, int tiles, const int32_t* seg_row0, const int32_t* row_pos,

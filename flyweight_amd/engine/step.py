@@ -128,6 +128,16 @@ class StepContext:
         self.host_seg_slot = seg_slot
 
         tile_seg, tile_row0 = ops.query_tiles(seg_row0)        # tiles of up to 64 rows for the prompt attention kernel
+        # Workgroups start in the order of the tiles: those that see the most keys go first, the short
+        # ones fill in behind. The tiles of the leading single rows stay in front (mixers may hand
+        # those rows to their decode kernels and skip their tiles).
+        if len(tile_seg) - self.decode_prefix > 1:
+            tile_seg, tile_row0 = np.asarray(tile_seg, dtype=np.int32), np.asarray(tile_row0, dtype=np.int32)
+            tile_end = np.minimum(tile_row0 + ops.QUERY_TILE, np.asarray(seg_row0, dtype=np.int32)[tile_seg + 1])
+            keys_seen = row_pos[tile_end - 1].astype(np.int64)
+            keys_seen[:self.decode_prefix] = np.iinfo(np.int64).max
+            order = np.argsort(-keys_seen, kind="stable")
+            tile_seg, tile_row0 = tile_seg[order], tile_row0[order]
         tables = [cache.block_table_rows(g, self.requests, natives=natives) for g in range(len(cache.groups))]
         pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows,
                                                           tile_seg, tile_row0)]

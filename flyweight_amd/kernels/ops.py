@@ -650,14 +650,20 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                                 ctx.row_pos, scale, ctx.max_context, window)
     if fast:
         single = getattr(ctx, "decode_prefix", 0)       # leading segments of one row: rows and tiles 0 .. single - 1
+        # four query heads of a kv group per workgroup pay where the rows sit behind a long context
+        # (a page is read once for the four); from the start of a prompt one head per workgroup
+        # gives more and shorter workgroups, which evens out the causal triangle
+        rows = q.shape[0] - single
+        keys = min(window, ctx.max_context) if window else ctx.max_context      # the most keys a row can see
+        together = 4 if head_dim <= 64 and num_heads // num_kv_heads >= 4 and keys >= 4 * rows else 0
         if single == 0:
             return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.tile_seg,
-                                     ctx.tile_row0, ctx.seg_row0, ctx.row_pos, scale, window)
+                                     ctx.tile_row0, ctx.seg_row0, ctx.row_pos, scale, window, heads_together=together)
         out = torch.empty_like(q)
         attention_decode(q[:single], num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                          ctx.row_pos, scale, ctx.max_context, window, out=out[:single])
         return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table,
                                  ctx.tile_seg[single:], ctx.tile_row0[single:], ctx.seg_row0, ctx.row_pos, scale, window,
-                                 out=out)
+                                 heads_together=together, out=out)
     return attention_generic(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                              ctx.row_pos, scale, window)
