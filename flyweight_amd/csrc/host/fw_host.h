@@ -81,6 +81,19 @@ int fwh_plan_list(void* scheduler, int which, int64_t* requests);      // 0 pree
 // progress, kind) come back; returns their number (at most 2 per segment plus failed and cancelled).
 int fwh_scheduler_complete(void* scheduler, const int64_t* requests, const int* tokens, int count,
                            int64_t* event_requests, int* event_values, int* event_kinds, int capacity);
+// A decode step planned and finished without a list per request on the caller's side. If the plan
+// made last is one token for each of its requests, each wanting logits, and nothing else happened
+// in it (nobody admitted, preempted, failed or cancelled), fwh_plan_fill_decode writes what a
+// captured decode step uploads: the tokens, the positions they get (the requests' lengths), the
+// requests' slots, and for every page group the rows of the block tables ([group][row][stride],
+// group_stride ints apart); returns the number of rows, or FWH_NOT_DECODE_ONLY and writes nothing.
+// fwh_scheduler_complete_ordered is fwh_scheduler_complete with the tokens given in the order
+// of the plan's segments that wanted logits.
+#define FWH_NOT_DECODE_ONLY (-3)
+int fwh_plan_fill_decode(void* scheduler, int capacity, int* tokens, int* positions, int* slots, int table_stride,
+                         int* tables, int group_stride);
+int fwh_scheduler_complete_ordered(void* scheduler, const int* tokens, int count, int64_t* event_requests,
+                                   int* event_values, int* event_kinds, int capacity);
 // info: computed, live, finished, cancelled, admitted_at, preemptions, prompt length, generated length, max_new_tokens
 int fwh_request_info(void* scheduler, int64_t request, int info[9]);
 int fwh_request_generated(void* scheduler, int64_t request, int* tokens, int capacity);

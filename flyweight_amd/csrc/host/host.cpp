@@ -239,6 +239,59 @@ int fwh_scheduler_complete(void* scheduler, const int64_t* requests, const int* 
         return (int)events.size();
     });
 }
+int fwh_plan_fill_decode(void* scheduler, int capacity, int* tokens, int* positions, int* slots, int table_stride,
+                         int* tables, int group_stride) {
+    return guarded([&] {
+        fwh::Scheduler* s = scheduler_of(scheduler);
+        const fwh::Plan& plan = s->plan();
+        if (plan.segments.empty() || !plan.preempted.empty() || !plan.failed.empty() || !plan.admitted.empty() ||
+            !plan.cancelled.empty() || (int)plan.segments.size() > capacity)
+            return FWH_NOT_DECODE_ONLY;
+        for (const fwh::Segment& segment : plan.segments)
+            if (segment.count != 1 || !segment.wants_logits) return FWH_NOT_DECODE_ONLY;
+        fwh::Cache& cache = s->cache();
+        const int rows = (int)plan.segments.size();
+        for (int g = 0; g < cache.num_groups(); ++g)
+            for (const fwh::Segment& segment : plan.segments)
+                if ((int)cache.group(g).tables.at(segment.request->id).size() > table_stride)
+                    throw std::length_error("a block table is longer than the row it is copied to");
+        for (int i = 0; i < rows; ++i) {
+            const fwh::Request* request = plan.segments[i].request;
+            tokens[i] = request->token_at(plan.segments[i].first);
+            positions[i] = plan.segments[i].first;
+            slots[i] = cache.of(request->id).slot;
+            for (int g = 0; g < cache.num_groups(); ++g) {
+                const std::vector<int>& table = cache.group(g).tables.at(request->id);
+                int* row = tables + (size_t)g * group_stride + (size_t)i * table_stride;
+                // a page that was given back is never read (the window has passed it); any valid id will do
+                for (int b = 0; b < table_stride; ++b) row[b] = b < (int)table.size() && table[b] != fwh::NO_PAGE ? table[b] : 0;
+            }
+        }
+        return rows;
+    });
+}
+int fwh_scheduler_complete_ordered(void* scheduler, const int* tokens, int count, int64_t* event_requests,
+                                   int* event_values, int* event_kinds, int capacity) {
+    return guarded([&] {
+        fwh::Scheduler* s = scheduler_of(scheduler);
+        std::unordered_map<int64_t, int> sampled;
+        int given = 0;
+        for (const fwh::Segment& segment : s->plan().segments)
+            if (segment.wants_logits) {
+                if (given >= count) throw fwh::SchedulerError("fewer tokens were handed over than the plan's segments want");
+                sampled[segment.request->id] = tokens[given++];
+            }
+        if (given != count) throw fwh::SchedulerError("more tokens were handed over than the plan's segments want");
+        const std::vector<fwh::Event> events = s->complete(sampled);
+        if ((int)events.size() > capacity) throw std::length_error("the event buffer is too small");
+        for (size_t i = 0; i < events.size(); ++i) {
+            event_requests[i] = events[i].request;
+            event_values[i] = events[i].value;
+            event_kinds[i] = events[i].kind;
+        }
+        return (int)events.size();
+    });
+}
 int fwh_request_info(void* scheduler, int64_t request, int info[9]) {
     return guarded([&] {
         const fwh::Request* r = scheduler_of(scheduler)->find(request);

@@ -134,6 +134,7 @@ public:
     const std::deque<Request*>& waiting() const { return waiting_; }
     const std::vector<Request*>& running() const { return running_; }
     const Plan& plan() const { return plan_; }
+    Cache& cache() { return *cache_; }
 
     const Plan& schedule() {
         plan_.clear();

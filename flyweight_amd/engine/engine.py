@@ -15,6 +15,7 @@ from typing import Callable, Dict, Hashable, List, Optional, Sequence, Tuple
 import torch
 
 from ..cache import OutOfPages
+from ..kernels import ops
 from ..sampling import GREEDY, SamplingConfig, sample_rows
 from .model import CausalLM, load_model, parse_dtype
 from .scheduler import (EVENT_ERROR, EVENT_FINISHED, EVENT_PREFILL, EVENT_TOKEN, Request, Scheduler,
@@ -175,7 +176,22 @@ class Runtime:
         scheduler = self.scheduler
         if not scheduler.has_work():
             return []
-        plan = scheduler.schedule()
+        counts = scheduler.plan_next()
+        # A plain decode step (one token for every request of the plan, every token the most likely
+        # one, nothing else happened) that a captured step serves goes from the scheduler's plan to
+        # the upload buffer and back without an object per request.
+        if counts[0] and counts[0] == counts[1] and not any(counts[2:6]) and scheduler.all_greedy:
+            captured = self.stepper.captured_step(counts[0])
+            if captured is not None:
+                began = time.perf_counter_ns()
+                logits = self.stepper.replay_planned(captured, scheduler)
+                if logits is not None:
+                    tokens = ops.argmax_rows(logits).cpu().numpy()
+                    self._counters["steps"] += 1
+                    self._counters["decode_calls"] += counts[0]
+                    self._counters["decode_ns"] += time.perf_counter_ns() - began
+                    return scheduler.complete_ordered(tokens)
+        plan = scheduler.read_plan(counts)
         for request in plan.failed:
             self._errors[request.id] = request.error or "failed"
         sampled: Dict[int, int] = {}

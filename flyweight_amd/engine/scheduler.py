@@ -131,6 +131,7 @@ class Scheduler:
         if not self._native:
             raise SchedulerError(host.last_error())
         self._serial = 0
+        self._drawing = set()       # unfinished requests whose tokens are drawn, not taken as the most likely
 
     def __del__(self):
         if getattr(self, "_native", None):
@@ -150,6 +151,8 @@ class Scheduler:
             raise SchedulerError(host.last_error())
         request = Request(self, request_id, prompt, int(max_new_tokens), sampling, stop)
         self.requests[request_id] = request
+        if not sampling.greedy:
+            self._drawing.add(request_id)
         return request
 
     def cancel(self, request_id: int) -> bool:
@@ -177,11 +180,62 @@ class Scheduler:
     def schedule(self) -> StepPlan:
         """Plans the next step and reserves its pages. The slots of the requests admitted in it
         start at zero."""
+        return self.read_plan(self.plan_next())
+
+    # The two halves of ``schedule``, for a caller that can serve a plain decode step without
+    # an object per request: ``plan_next`` makes the plan in the host library and says how large
+    # it is; ``fill_decode`` writes such a step's batch straight into a captured step's upload
+    # buffer and ``complete_ordered`` finishes it; ``read_plan`` gives any plan as objects.
+    def plan_next(self):
+        """Plans the next step (pages reserved); returns its counts: segments, tokens,
+        preempted, failed, admitted, cancelled."""
         counts = host.ints(6)
         if self._lib.fwh_scheduler_schedule(self._native, counts) < 0:
             raise SchedulerError(host.last_error())
-        segments, tokens = counts[0], counts[1]
         self._serial += 1
+        return counts
+
+    @property
+    def all_greedy(self) -> bool:
+        return not self._drawing
+
+    def fill_decode(self, capacity: int, tokens, positions, slots, table_stride: int, tables, group_stride: int) -> int:
+        """If the plan made last is one token for each of its requests and nothing else, writes
+        the step's tokens, positions, slots and block-table rows to these int32 arrays (numpy
+        views of a pinned buffer) and returns the number of rows; -1 otherwise."""
+        rows = self._lib.fwh_plan_fill_decode(self._native, int(capacity), tokens.ctypes.data, positions.ctypes.data,
+                                              slots.ctypes.data, int(table_stride),
+                                              tables.ctypes.data if tables is not None else None, int(group_stride))
+        if rows == host.NOT_DECODE_ONLY:
+            return -1
+        if rows < 0:
+            raise SchedulerError(host.last_error())
+        return rows
+
+    def complete_ordered(self, tokens) -> List[Tuple[int, int, int]]:
+        """``complete`` for the plan made last, the tokens (int32 numpy array) in the order of
+        its segments that wanted logits."""
+        self._serial += 1
+        count = int(tokens.shape[0])
+        capacity = 2 * count + 1
+        event_owner, event_value, event_kind = host.ids(capacity), host.ints(capacity), host.ints(capacity)
+        made = self._lib.fwh_scheduler_complete_ordered(self._native, tokens.ctypes.data_as(ctypes.POINTER(ctypes.c_int)), count,
+                                                        event_owner, event_value, event_kind, capacity)
+        if made < 0:
+            raise SchedulerError(host.last_error())
+        return self._events(event_owner, event_value, event_kind, made)
+
+    def _events(self, owners, values, kinds, count: int) -> List[Tuple[int, int, int]]:
+        events = list(zip(owners[:count], values[:count], kinds[:count]))
+        if self._drawing:
+            for owner, _, kind in events:
+                if kind in (1, 2):
+                    self._drawing.discard(owner)
+        return events
+
+    def read_plan(self, counts) -> StepPlan:
+        """The plan made last (by ``plan_next``) as objects."""
+        segments, tokens = counts[0], counts[1]
         plan = StepPlan(num_tokens=tokens, serial=self._serial)
         if segments:
             owners, lengths, wants, flat = host.ids(segments), host.ints(segments), host.ints(segments), host.ints(tokens)
@@ -220,4 +274,4 @@ class Scheduler:
                                                  event_kind, capacity)
         if count < 0:
             raise SchedulerError(host.last_error())
-        return [(event_owner[i], event_value[i], event_kind[i]) for i in range(count)]
+        return self._events(event_owner, event_value, event_kind, count)

@@ -197,19 +197,44 @@ class StepContext:
         else:
             natives = cache.natives_of(self.requests)
             starts, slots = cache.describe(self.requests, natives)
-        uploaded = getattr(self, "_uploaded", None)
-        if uploaded is not None:
-            uploaded.synchronize()      # the pinned buffer is still being read until the last upload has run
+        self.wait_uploaded()
         self.new_lengths = [s + 1 for s in starts]
         host[0][:] = [int(e.tokens[0]) for e in entries]
         host[1][:] = starts
         host[4][:] = slots
         for g in range(len(cache.groups)):
             host[8 + g][:] = cache.block_table_rows(g, self.requests, stride=self._table_stride, natives=natives).reshape(-1)
+        self.upload()
+
+    def wait_uploaded(self) -> None:
+        """The pinned buffer is still being read until the last upload has run: wait for it
+        before the buffer is written again."""
+        uploaded = getattr(self, "_uploaded", None)
+        if uploaded is not None:
+            uploaded.synchronize()
+
+    def upload(self) -> None:
         self.device_buffer.copy_(self.host_buffer, non_blocking=True)
-        if uploaded is None:
-            uploaded = self._uploaded = torch.cuda.Event()
-        uploaded.record()
+        if getattr(self, "_uploaded", None) is None:
+            self._uploaded = torch.cuda.Event()
+        self._uploaded.record()
+
+    def fill_from(self, scheduler) -> bool:
+        """For a captured step: lets the scheduler write the plan it made last straight into the
+        upload buffer (tokens, positions, slots, block tables) if that plan is one token for each
+        of exactly this step's number of requests and nothing else; uploads it then. False (and
+        nothing written) otherwise."""
+        self.wait_uploaded()
+        host = self._host
+        groups = len(host) - 8
+        rows = scheduler.fill_decode(self.num_rows, host[0], host[1], host[4], self._table_stride,
+                                     host[8] if groups else None, self.num_rows * self._table_stride)
+        if rows != self.num_rows:
+            if rows >= 0:
+                raise StepError(f"the plan has {rows} rows, the captured step {self.num_rows}")
+            return False
+        self.upload()
+        return True
 
     def position_tables(self, part):
         key = part.key()
@@ -298,6 +323,24 @@ class Stepper:
         captured = _CapturedDecode(ctx)
         self._graphs[batch] = captured
         return captured
+
+    def captured_step(self, batch: int) -> Optional["_CapturedDecode"]:
+        """The captured decode step of this batch size, if one has been recorded."""
+        captured = self._graphs.get(batch) if self.use_graphs else None
+        return captured if captured is not None and captured.graph is not None else None
+
+    def replay_planned(self, captured: "_CapturedDecode", scheduler) -> Optional[torch.Tensor]:
+        """A decode step straight from the scheduler's plan (see ``StepContext.fill_from``): the
+        pages are reserved by the plan and the lengths are committed when the scheduler completes
+        it, so the cache manager is not asked again. Logits of every row, or None if the plan is
+        not such a step (nothing has run then)."""
+        if not captured.ctx.fill_from(scheduler):
+            return None
+        captured.graph.replay()
+        self.graph_replays += 1
+        self.steps += 1
+        self.tokens_run += captured.ctx.num_rows
+        return captured.logits
 
     def _replay(self, captured: "_CapturedDecode", entries: Sequence[StepEntry], described=None) -> Optional[torch.Tensor]:
         cache = self.cache

@@ -10,6 +10,7 @@ from typing import Optional
 from .kernels.build import ensure_host_built
 
 ERROR, OUT_OF_PAGES, NO_PAGE = -1, -2, -1
+NOT_DECODE_ONLY = -3
 ABI_VERSION = 1
 
 _LIB: Optional[ctypes.CDLL] = None
@@ -57,6 +58,8 @@ _SIGNATURES = {
     "fwh_plan_segments": (c_int, [c_void_p, _IDS, _INTS, _INTS, _INTS]),
     "fwh_plan_list": (c_int, [c_void_p, c_int, _IDS]),
     "fwh_scheduler_complete": (c_int, [c_void_p, _IDS, _INTS, c_int, _IDS, _INTS, _INTS, c_int]),
+    "fwh_plan_fill_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int]),
+    "fwh_scheduler_complete_ordered": (c_int, [c_void_p, _INTS, c_int, _IDS, _INTS, _INTS, c_int]),
     "fwh_request_info": (c_int, [c_void_p, c_int64, _INTS]),
     "fwh_request_generated": (c_int, [c_void_p, c_int64, _INTS, c_int]),
     "fwh_request_error": (c_char_p, [c_void_p, c_int64]),

@@ -179,3 +179,46 @@ def test_cancel_frees_everything():
     events = scheduler.complete(plan, {})
     assert sorted(e[0] for e in events if e[2] == EVENT_FINISHED) == [a.id, b.id]
     assert not scheduler.has_work() and cache.stats()["pages_free"] == 8 and cache.slots.free_count == 4
+
+
+def test_a_plain_decode_step_goes_through_arrays_and_decides_the_same():
+    """plan_next / fill_decode / complete_ordered against schedule / complete: the same requests
+    driven both ways produce the same tokens, events and block tables at every step; a step that
+    is not one token per request (a prompt portion, an admission) is refused and read as objects."""
+    import numpy as np
+    prompts = [[3, 1, 4, 1, 5], [9, 2, 6], [5, 3, 5, 8, 9, 7, 9, 3, 2, 3, 8]]
+    results = []
+    for arrays in (False, True):
+        cache, scheduler = make(num_pages=8, max_requests=4, max_batch_tokens=64, chunk_size=8)
+        for prompt in prompts:
+            scheduler.submit(prompt, 20, GREEDY)
+        log = []
+        stride = 3
+        while scheduler.has_work():
+            counts = scheduler.plan_next()
+            rows = counts[0]
+            tokens, positions, slots = (np.full(rows, -7, dtype=np.int32) for _ in range(3))
+            tables = np.full((1, rows, stride), -7, dtype=np.int32)
+            filled = scheduler.fill_decode(rows, tokens, positions, slots, stride, tables, rows * stride) if arrays else -1
+            plain = rows and counts[0] == counts[1] and not any(counts[2:6])
+            if arrays:
+                assert (filled == rows) == bool(plain)
+            plan = scheduler.read_plan(counts)
+            if filled == rows:
+                # what the arrays hold is what the objects say
+                assert tokens.tolist() == [s.tokens[0] for s in plan.segments]
+                assert positions.tolist() == [s.request.computed for s in plan.segments]
+                assert slots.tolist() == [cache.slot_of(s.request.id) for s in plan.segments]
+                expected = cache.block_table_rows(0, [s.request.id for s in plan.segments], stride=stride)
+                assert tables[0].tolist() == expected.tolist()
+                drawn = np.asarray([oracle(s.request.tokens) for s in plan.segments], dtype=np.int32)
+                events = scheduler.complete_ordered(drawn)
+            else:
+                assert (tokens == -7).all() and (tables == -7).all(), "a refused plan writes nothing"
+                sampled = {s.request.id: oracle(s.request.tokens) for s in plan.segments if s.wants_logits}
+                events = scheduler.complete(plan, sampled)
+            log.append(events)
+            cache.check_invariants()
+        results.append((log, {r.id: r.generated for r in scheduler.requests.values()}))
+    assert results[0] == results[1]
+    assert any(len(events) >= 3 and all(kind == EVENT_TOKEN for _, _, kind in events) for events in results[1][0])
