@@ -81,33 +81,48 @@ def matmul_params(config) -> int:
     return config.num_hidden_layers * per_ffn + (config.num_hidden_layers - n_attn) * conv + n_attn * attn
 
 
+DECODE_STEPS_PER_TURN = 4      # decode steps the engine runs on the device before the host is asked again
+
+
+def steps_per_turn(steps: int, warmup: int) -> int:
+    """The engine's decode_steps_per_turn for a run: the timed steps and the warm-up are whole turns."""
+    return DECODE_STEPS_PER_TURN if steps % DECODE_STEPS_PER_TURN == 0 and warmup % DECODE_STEPS_PER_TURN == 0 else 1
+
+
 def decode_run(torch, model, config, batch: int, steps: int, warmup: int, seed: int = 0):
     """``batch`` requests with 2,048-token prompts; returns (seconds for ``steps`` decode steps, mean context)."""
     import numpy as np
     from flyweight_amd import Runtime
     # requests admitted earlier decode while later prompts are still running (continuous
     # batching), so they are up to ``batch`` tokens ahead when the timed steps begin
-    new_tokens = warmup + steps + batch + 2
+    new_tokens = warmup + steps + batch + 2 + DECODE_STEPS_PER_TURN
     pages_each = (PROMPT + new_tokens + 63) // 64
+    turn = steps_per_turn(steps, warmup)
     runtime = Runtime(model, context_limit=CONTEXT, parallel_sequences=batch, num_pages=pages_each * batch,
-                      max_batch_tokens=PROMPT + batch, prefill_rows=PROMPT).prepare()
+                      max_batch_tokens=PROMPT + batch, prefill_rows=PROMPT, decode_steps_per_turn=turn).prepare()
     rng = np.random.default_rng(seed)
     for _ in range(batch):
         runtime.task_submit(rng.integers(0, config.vocab_size, PROMPT).tolist(), new_tokens)
     # prompts: until every request has produced its first token
     while any(r.computed < len(r.prompt) for r in runtime.scheduler.requests.values()):
         runtime.engine_step()
-    for _ in range(warmup):
-        runtime.engine_step()
+
+    def decode(count: int) -> None:
+        """Exactly ``count`` decode steps of the whole batch (a turn of the engine may hold several)."""
+        tokens = 0
+        while tokens < count * batch:
+            runtime.decode_steps_per_turn = min(turn, count - tokens // batch)      # never past the steps asked for
+            tokens += sum(1 for event in runtime.engine_step() if event[2] == 0)
+        assert tokens == count * batch, "a step did not decode the whole batch"
+
+    decode(warmup)
     requests = list(runtime.scheduler.requests.values())
     before = sum(r.computed for r in requests) / batch
     torch.cuda.synchronize()
     began = time.perf_counter()
-    for _ in range(steps):
-        events = runtime.engine_step()
+    decode(steps)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - began
-    assert sum(1 for e in events if e[2] == 0) == batch, "a timed step did not decode the whole batch"
     mean_context = before + 1 + (steps - 1) / 2.0      # keys a row sees, averaged over requests and steps
     runtime.close()
     return elapsed, mean_context
@@ -258,7 +273,8 @@ def main() -> int:
                    "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim, "ff_dim": config.ff_dim,
                    "vocab": config.vocab_size, "attention_layers": len(config.full_attn_idxs),
                    "conv_L_cache": config.conv_L_cache, "global_batch": args.batch, "prompt_len": PROMPT,
-                   "seq_len": CONTEXT, "parallelism": "single GPU"},
+                   "seq_len": CONTEXT, "decode_steps_per_turn": steps_per_turn(args.steps, args.warmup),
+                   "parallelism": "single GPU"},
         "prefill": {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(prefill_flops / prefill_s / MFMA_BF16_PEAK, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

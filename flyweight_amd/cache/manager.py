@@ -272,9 +272,10 @@ class CacheManager:
             raise KeyError(next((r for r in requests if r not in self.requests), host.last_error()))
         return lengths[:count], slots[:count]
 
-    def reserve_all(self, requests: Sequence[Hashable], new_lengths: Sequence[int], natives=None) -> None:
-        """The reservations of a whole step: all of them, or OutOfPages and nothing changed."""
-        count = len(requests)
+    def reserve_all(self, requests: Sequence[Hashable], new_lengths: Sequence[int], natives=None, count=None) -> None:
+        """The reservations of a whole step: all of them, or OutOfPages and nothing changed.
+        (``natives`` with ``count``: the requests by the host library's ids alone.)"""
+        count = len(requests) if count is None else count
         natives = self.natives_of(requests) if natives is None else natives
         status = self._lib.fwh_cache_reserve_batch(self._native, natives, (ctypes.c_int * max(count, 1))(*new_lengths), count)
         if status == host.OUT_OF_PAGES:
@@ -303,13 +304,14 @@ class CacheManager:
 
     # ----- views for the step function ---------------------------------------------------
     def block_table_rows(self, group_index: int, requests: Sequence[Hashable], stride: Optional[int] = None,
-                         natives=None) -> np.ndarray:
+                         natives=None, count=None) -> np.ndarray:
         if natives is None:
             natives = self.natives_of(requests)
+        count = len(requests) if count is None else count
         if stride is None:
-            stride = max(self._lib.fwh_cache_longest_table(self._native, group_index, natives, len(requests)), 1)
-        rows = np.zeros((len(requests), stride), dtype=np.int32)
-        if self._lib.fwh_cache_fill_tables(self._native, group_index, natives, len(requests), stride, rows.ctypes.data) < 0:
+            stride = max(self._lib.fwh_cache_longest_table(self._native, group_index, natives, count), 1)
+        rows = np.zeros((count, stride), dtype=np.int32)
+        if self._lib.fwh_cache_fill_tables(self._native, group_index, natives, count, stride, rows.ctypes.data) < 0:
             for request in requests:
                 if request not in self.requests:
                     raise KeyError(f"request {request!r} is not live")

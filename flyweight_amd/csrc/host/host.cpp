@@ -270,6 +270,27 @@ int fwh_plan_fill_decode(void* scheduler, int capacity, int* tokens, int* positi
         return rows;
     });
 }
+int fwh_plan_steps_ahead(void* scheduler, int limit, int64_t* requests, int capacity) {
+    return guarded([&] {
+        fwh::Scheduler* s = scheduler_of(scheduler);
+        const fwh::Plan& plan = s->plan();
+        if (plan.segments.empty() || !plan.preempted.empty() || !plan.failed.empty() || !plan.admitted.empty() ||
+            !plan.cancelled.empty() || !s->waiting().empty())
+            return 0;
+        int ahead = limit;
+        for (const fwh::Segment& segment : plan.segments) {
+            const fwh::Request* request = segment.request;
+            if (segment.count != 1 || !segment.wants_logits || !request->stop_tokens.empty() || request->cancelled) return 0;
+            const int budget = request->max_new_tokens - (int)request->generated.size() - 1;
+            const int room = s->max_positions() - request->total() - 1;
+            ahead = std::min({ahead, budget, room});
+        }
+        if (ahead < 0) ahead = 0;
+        if (requests)
+            for (size_t i = 0; i < plan.segments.size() && (int)i < capacity; ++i) requests[i] = plan.segments[i].request->id;
+        return ahead;
+    });
+}
 int fwh_scheduler_complete_ordered(void* scheduler, const int* tokens, int count, int64_t* event_requests,
                                    int* event_values, int* event_kinds, int capacity) {
     return guarded([&] {

@@ -135,6 +135,7 @@ public:
     const std::vector<Request*>& running() const { return running_; }
     const Plan& plan() const { return plan_; }
     Cache& cache() { return *cache_; }
+    int max_positions() const { return max_positions_; }
 
     const Plan& schedule() {
         plan_.clear();

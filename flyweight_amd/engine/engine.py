@@ -15,7 +15,6 @@ from typing import Callable, Dict, Hashable, List, Optional, Sequence, Tuple
 import torch
 
 from ..cache import OutOfPages
-from ..kernels import ops
 from ..sampling import GREEDY, SamplingConfig, sample_rows
 from .model import CausalLM, load_model, parse_dtype
 from .scheduler import (EVENT_ERROR, EVENT_FINISHED, EVENT_PREFILL, EVENT_TOKEN, Request, Scheduler,
@@ -73,12 +72,17 @@ class Model:
 
 class Runtime:
     def __init__(self, model: Model, context_limit: Optional[int] = None, parallel_sequences: int = 16,
-                 num_pages: Optional[int] = None, max_batch_tokens: int = 2048, prefill_rows: int = 512):
+                 num_pages: Optional[int] = None, max_batch_tokens: int = 2048, prefill_rows: int = 512,
+                 decode_steps_per_turn: int = 1):
         """``context_limit``: most tokens (prompt + output) of one request, at most the
         model's ``max_position_embeddings``. ``parallel_sequences``: most requests live at
         once. ``num_pages``: cache pages (of 64 tokens) per page group; by default enough
         for every live request at the full context. ``prefill_rows``: most tokens of one
-        prompt portion; ``max_batch_tokens``: most tokens of one step."""
+        prompt portion; ``max_batch_tokens``: most tokens of one step. ``decode_steps_per_turn``:
+        when every running request decodes, takes the most likely token and can neither stop nor
+        be joined by another (no stop tokens, budget left, nobody waiting), up to this many decode
+        steps run back to back on the device before the host is asked again; ``engine_step`` then
+        returns the events of all of them. More throughput, tokens in bursts."""
         self.model = model
         spec = model.spec
         self.context_limit = min(context_limit or spec.max_positions, spec.max_positions)
@@ -87,6 +91,7 @@ class Runtime:
         self.num_pages = int(num_pages) if num_pages else per_request * self.parallel_sequences
         self.max_batch_tokens = int(max_batch_tokens)
         self.prefill_rows = int(prefill_rows)
+        self.decode_steps_per_turn = max(1, int(decode_steps_per_turn))
         self.stepper: Optional[Stepper] = None
         self.scheduler: Optional[Scheduler] = None
         self._errors: Dict[int, str] = {}
@@ -184,13 +189,19 @@ class Runtime:
             captured = self.stepper.captured_step(counts[0])
             if captured is not None:
                 began = time.perf_counter_ns()
-                logits = self.stepper.replay_planned(captured, scheduler)
-                if logits is not None:
-                    tokens = ops.argmax_rows(logits).cpu().numpy()
-                    self._counters["steps"] += 1
-                    self._counters["decode_calls"] += counts[0]
+                tokens = self.stepper.replay_planned(captured, scheduler, self.decode_steps_per_turn)
+                if tokens is not None:
+                    self._counters["steps"] += len(tokens)
+                    self._counters["decode_calls"] += counts[0] * len(tokens)
                     self._counters["decode_ns"] += time.perf_counter_ns() - began
-                    return scheduler.complete_ordered(tokens)
+                    events = scheduler.complete_ordered(tokens[0])
+                    for later in tokens[1:]:
+                        # the steps that ran ahead: the scheduler makes the plan they ran by, then takes their tokens
+                        again = scheduler.plan_next()
+                        if again[0] != counts[0] or again[1] != counts[0] or any(again[2:6]):
+                            raise EngineError("the scheduler's plan differs from the decode steps that ran ahead of it")
+                        events.extend(scheduler.complete_ordered(later))
+                    return events
         plan = scheduler.read_plan(counts)
         for request in plan.failed:
             self._errors[request.id] = request.error or "failed"

@@ -212,6 +212,16 @@ class Scheduler:
             raise SchedulerError(host.last_error())
         return rows
 
+    def steps_ahead(self, limit: int, rows: int):
+        """For a plain decode plan: how many further steps of exactly this batch are certain to
+        follow whatever tokens are drawn (nobody waits, no stop tokens, every request has the
+        budget), at most ``limit``; and the plan's requests (the host library's ids) in row order."""
+        requests = host.ids(rows)
+        ahead = self._lib.fwh_plan_steps_ahead(self._native, int(limit), requests, rows)
+        if ahead < 0:
+            raise SchedulerError(host.last_error())
+        return ahead, requests
+
     def complete_ordered(self, tokens) -> List[Tuple[int, int, int]]:
         """``complete`` for the plan made last, the tokens (int32 numpy array) in the order of
         its segments that wanted logits."""

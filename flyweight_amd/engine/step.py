@@ -329,18 +329,42 @@ class Stepper:
         captured = self._graphs.get(batch) if self.use_graphs else None
         return captured if captured is not None and captured.graph is not None else None
 
-    def replay_planned(self, captured: "_CapturedDecode", scheduler) -> Optional[torch.Tensor]:
-        """A decode step straight from the scheduler's plan (see ``StepContext.fill_from``): the
+    def replay_planned(self, captured: "_CapturedDecode", scheduler, steps: int = 1) -> Optional[np.ndarray]:
+        """Decode steps straight from the scheduler's plan (see ``StepContext.fill_from``): the
         pages are reserved by the plan and the lengths are committed when the scheduler completes
-        it, so the cache manager is not asked again. Logits of every row, or None if the plan is
-        not such a step (nothing has run then)."""
-        if not captured.ctx.fill_from(scheduler):
+        it, so the cache manager is not asked again. Every token is the most likely one. With
+        ``steps`` > 1 and a plan that is certain to repeat (``Scheduler.steps_ahead``), up to that
+        many steps run back to back on the device, each fed the tokens of the one before, and the
+        host reads all of them at once: it is then asked once per turn instead of once per step.
+        Returns the tokens, int32 [steps run, rows], or None if the plan is not a plain decode
+        step (nothing has run then)."""
+        ctx = captured.ctx
+        if not ctx.fill_from(scheduler):
             return None
+        rows = ctx.num_rows
+        ahead, natives = scheduler.steps_ahead(steps - 1, rows) if steps > 1 else (0, None)
         captured.graph.replay()
-        self.graph_replays += 1
-        self.steps += 1
-        self.tokens_run += captured.ctx.num_rows
-        return captured.logits
+        drawn = [ops.argmax_rows(captured.logits)]
+        cache = self.cache
+        for _ in range(ahead):
+            # the same requests one position on: pages for it, then positions and block tables anew
+            ctx.wait_uploaded()
+            positions = ctx._host[1]
+            try:
+                cache.reserve_all((), (positions[:rows] + 2).tolist(), natives=natives, count=rows)
+            except OutOfPages:
+                break                       # the scheduler will decide who gives way, one step at a time
+            positions[:rows] += 1
+            for g in range(len(cache.groups)):
+                ctx._host[8 + g][:] = cache.block_table_rows(g, (), stride=ctx._table_stride, natives=natives, count=rows).reshape(-1)
+            ctx.upload()
+            ctx.token_ids.copy_(drawn[-1])  # after the upload, which also carries the (stale) tokens
+            captured.graph.replay()
+            drawn.append(ops.argmax_rows(captured.logits))
+        self.graph_replays += len(drawn)
+        self.steps += len(drawn)
+        self.tokens_run += rows * len(drawn)
+        return torch.stack(drawn).cpu().numpy()
 
     def _replay(self, captured: "_CapturedDecode", entries: Sequence[StepEntry], described=None) -> Optional[torch.Tensor]:
         cache = self.cache

@@ -60,6 +60,7 @@ _SIGNATURES = {
     "fwh_scheduler_complete": (c_int, [c_void_p, _IDS, _INTS, c_int, _IDS, _INTS, _INTS, c_int]),
     "fwh_plan_fill_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int]),
     "fwh_scheduler_complete_ordered": (c_int, [c_void_p, _INTS, c_int, _IDS, _INTS, _INTS, c_int]),
+    "fwh_plan_steps_ahead": (c_int, [c_void_p, c_int, _IDS, c_int]),
     "fwh_request_info": (c_int, [c_void_p, c_int64, _INTS]),
     "fwh_request_generated": (c_int, [c_void_p, c_int64, _INTS, c_int]),
     "fwh_request_error": (c_char_p, [c_void_p, c_int64]),

@@ -193,6 +193,51 @@ def test_engine_tasks_equal_blocking_generation_and_survive_preemption(loaded):
     tight.stepper.cache.check_invariants()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decode_steps_that_run_ahead_of_the_host_give_the_same_tokens(loaded, dtype):
+    """With several decode steps per turn the device feeds each step's tokens to the next and
+    the host reads them in bursts: the same tokens in the same order as one step per turn (float32:
+    the plain model's), bursts cut short by the shortest budget, across page edges, and none for
+    a request that may stop on a token or while somebody still waits for a slot."""
+    m = loaded("B", dtype)
+    config, weights = m.plain_config, m.plain_weights
+    prompts = [random_tokens(m.config.vocab_size, n, seed=40 + n) for n in (3, 60, 9, 30)]
+    budgets = [70, 9, 23, 41]
+
+    def run(steps_per_turn, stop_tokens=(), parallel=4):
+        runtime = _runtime(m, parallel_sequences=parallel, prefill_rows=64, max_batch_tokens=128,
+                           decode_steps_per_turn=steps_per_turn)
+        ids = [runtime.task_submit(p, n, stop_tokens=stop_tokens if i == 0 else ()) for i, (p, n) in enumerate(zip(prompts, budgets))]
+        events, bursts = [], []
+        while runtime.scheduler.has_work():
+            got = runtime.engine_step()
+            bursts.append(max([sum(1 for e in got if e[0] == task and e[2] == 0) for task in ids] + [0]))
+            events += got
+        runtime.stepper.cache.check_invariants()
+        assert runtime.info["pages_free"] == runtime.num_pages and runtime.info["live_requests"] == 0
+        return [[e[1] for e in events if e[0] == task and e[2] == 0] for task in ids], max(bursts), events
+
+    single, burst, _ = run(1)
+    assert burst == 1
+    ahead, burst, events = run(4)
+    assert ahead == single and burst == 4
+    assert [len(tokens) for tokens in ahead] == budgets
+    for task_events in ([e for e in events if e[0] == task] for task in {e[0] for e in events}):
+        assert task_events[-1][2] == 1 and all(e[2] != 1 for e in task_events[:-1]), "finished is a request's last event"
+    if dtype == "float32":
+        assert ahead == [plain.greedy(config, weights, p, n) for p, n in zip(prompts, budgets)]
+    # a request with a stop token keeps the whole batch at one step per turn while it runs
+    stop = single[0][20]
+    stopped, burst, _ = run(4, stop_tokens=(stop,))
+    cut = single[0].index(stop) + 1
+    assert stopped[0] == single[0][:cut] and stopped[1:] == single[1:]
+    # two slots for four requests: somebody waits until the last two run, only then steps run ahead
+    queued, burst, _ = run(4, parallel=2)
+    assert burst == 4 and [len(tokens) for tokens in queued] == budgets
+    if dtype == "float32":          # (in bfloat16 a prompt that runs beside other rows may round to another of two near-equal tokens)
+        assert queued == single
+
+
 def test_seeded_sampling_does_not_depend_on_the_batch(loaded):
     """Temperature 0.8, seed 7, portions of 16 mixed with decode rows: a request draws the
     same tokens alone and among others, and they are the plain sampler's tokens given the
