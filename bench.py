@@ -163,13 +163,14 @@ def serving_run(torch, workload: str, requests: int, seed: int = 0) -> dict:
     pages = sum((p + o + 63) // 64 for p, o in zip(prompts, outputs))
     # a step holds 2,048 tokens: the decoded tokens of the running requests first, portions of prompts in the rest
     runtime = Runtime(model, context_limit=context, parallel_sequences=requests, num_pages=pages,
-                      max_batch_tokens=PROMPT, prefill_rows=PROMPT).prepare()
+                      max_batch_tokens=PROMPT, prefill_rows=PROMPT, decode_steps_per_turn=DECODE_STEPS_PER_TURN).prepare()
     # a short request first: every kernel and library is loaded before the clock starts
     runtime.generate(rng.integers(0, config.vocab_size, 100).tolist(), 4)
     for prompt, output in zip(prompts, outputs):
         runtime.task_submit(rng.integers(0, config.vocab_size, prompt).tolist(), output)
     log(f"{requests} requests, {sum(prompts)} prompt tokens, {sum(outputs)} tokens to generate")
     generated = finished = steps = 0
+    steps_before = runtime.info["steps"]
     torch.cuda.synchronize()
     began = last = time.perf_counter()
     while runtime.scheduler.has_work():
@@ -187,6 +188,7 @@ def serving_run(torch, workload: str, requests: int, seed: int = 0) -> dict:
     assert finished == requests and generated == sum(outputs), (finished, generated)
     info = runtime.info
     preemptions = info["preemptions"]
+    steps = info["steps"] - steps_before       # a turn of the engine may hold several decode steps
     runtime.close()
     return {
         "metric": f"tokens/s, prompt and generated ({workload} workload, {spec['name']})",
@@ -200,7 +202,8 @@ def serving_run(torch, workload: str, requests: int, seed: int = 0) -> dict:
                    "head_dim": config.head_dim, "ff_dim": config.ff_dim, "vocab": config.vocab_size,
                    "attention_layers": len(config.full_attn_idxs), "requests": requests,
                    "prompt_tokens": sum(prompts), "generated_tokens": generated, "longest_context": context,
-                   "portion": PROMPT, "cache_pages": pages, "preemptions": preemptions},
+                   "portion": PROMPT, "cache_pages": pages, "preemptions": preemptions,
+                   "decode_steps_per_turn": DECODE_STEPS_PER_TURN},
     }
 
 
