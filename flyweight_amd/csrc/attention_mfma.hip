@@ -69,7 +69,7 @@ struct Columns {
 // (all pages but those on the diagonal, at a window's edge, and a sequence's last) skips the
 // mask. The scale is folded into the exponent's argument: the maximum is taken over the raw
 // scores (the scale is positive) and kept scaled.
-template <int HD, int NH, bool CLEAN_V, bool K_PADDED>
+template <int HD, int NH, bool CLEAN_V, bool K_PADDED, bool EARLY_V = false>
 __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t* __restrict__ k_page,
                                             const uint16_t* __restrict__ v_page, int head_dim, float scale_log2,
                                             int lo, int hi, int last_written, int k_stride, int v_stride) {
@@ -89,6 +89,20 @@ __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t
                 if (dc * 32 + g * 8 < head_dim) kf[kt][dc] = *reinterpret_cast<const bf16x8*>(key + dc * 32);
             }
         }
+    }
+    // EARLY_V (pages read from global memory, one page per wave): the values are asked for
+    // together with the keys, so that they travel while the scores are formed, not after them.
+    u32x2 early_a[EARLY_V ? 2 : 1][EARLY_V ? HD / 16 : 1], early_b[EARLY_V ? 2 : 1][EARLY_V ? HD / 16 : 1];
+    if (EARLY_V) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int t = 0; t < HD / 16; ++t) {
+                const int channel = t * 16 + i16 < head_dim ? t * 16 + i16 : head_dim - 1;
+                const uint16_t* value = v_page + (size_t)channel * v_stride + kb * 32 + g * 4;
+                early_a[kb][t] = *reinterpret_cast<const u32x2*>(value);
+                early_b[kb][t] = *reinterpret_cast<const u32x2*>(value + 16);
+            }
     }
     // scores of all heads
     f32x4 s[NH][4];
@@ -186,8 +200,14 @@ __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t
         for (int t = 0; t < HD / 16; ++t) {
             const int channel = t * 16 + i16 < head_dim ? t * 16 + i16 : head_dim - 1;
             const uint16_t* value = v_page + (size_t)channel * v_stride;
-            u32x2 va = *reinterpret_cast<const u32x2*>(value + key_a);
-            u32x2 vb = *reinterpret_cast<const u32x2*>(value + key_b);
+            u32x2 va, vb;
+            if (EARLY_V) {
+                va = early_a[kb][t];
+                vb = early_b[kb][t];
+            } else {
+                va = *reinterpret_cast<const u32x2*>(value + key_a);
+                vb = *reinterpret_cast<const u32x2*>(value + key_b);
+            }
             u32x4 vw = {va[0], va[1], vb[0], vb[1]};
             if (CLEAN_V) vw = u32x4{va[0] & keep_a0, va[1] & keep_a1, vb[0] & keep_b0, vb[1] & keep_b1};
             const bf16x8 vf = __builtin_bit_cast(bf16x8, vw);
@@ -394,6 +414,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) void attention_decode_split_kerne
     const int kvh = blockIdx.y / head_tiles, head_tile = blockIdx.y % head_tiles;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, g = lane >> 4;
     const int pos = row_pos[row];
+    const int segment = row_seg[row];       // asked for together with the position, not behind the branch below
     const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
     // splits are counted from the first page that holds a visible key
     const int first_block = first / PAGE + split * SPLIT_PAGES;
@@ -408,11 +429,11 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) void attention_decode_split_kerne
     load_query<HD>(c, q + ((size_t)row * num_heads + head) * head_dim, head_dim, valid);
     const int block = first_block + wave;
     if (block <= last_block) {
-        const int page = block_table[(size_t)row_seg[row] * table_stride + block];
+        const int page = block_table[(size_t)segment * table_stride + block];
         const size_t at = ((size_t)page * num_kv_heads + kvh) * PAGE * head_dim;
         const int base = block * PAGE;
         // a lane without a head computes along (q = 0, nothing of it is stored)
-        attend_page<HD, 1, true, false>(columns_of_wave, k_pages + at, v_pages + at, head_dim, scale_log2, first - base, pos - base, pos - base,
+        attend_page<HD, 1, true, false, (HD <= 128)>(columns_of_wave, k_pages + at, v_pages + at, head_dim, scale_log2, first - base, pos - base, pos - base,
                         head_dim, PAGE);
     }
     const float l = fw_quad_sum(c.l);
@@ -476,32 +497,33 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) void attention_decode_split_kerne
     for (int item = threadIdx.x; item < columns * head_dim; item += 64 * SPLIT_PAGES) {
         const int merged_head = kvh * group + head_tile * 16 + item / head_dim, d = item % head_dim;
         const float* source = partial + ((size_t)row * num_heads + merged_head) * max_splits * stride;
-        // eight parts are requested at a time (past the last one: the last one again, not used)
+        // Sixteen parts are requested at a time (past the last one: the last one again, not used),
+        // maximum, weight and value together: one round trip for up to sixteen parts. The running
+        // sums are rescaled when a later batch of parts raises the maximum.
         auto part_at = [&](int sp, int offset) {
             const int clamped = sp < row_splits ? sp : row_splits - 1;
             return __hip_atomic_load(source + (size_t)clamped * stride + offset, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         };
-        float m = NEG_BIG;
-        for (int sp0 = 0; sp0 < row_splits; sp0 += 8) {
-            float ms[8];
+        constexpr int AT_ONCE = 16;
+        float m = NEG_BIG, total = 0.0f, acc = 0.0f;
+        for (int sp0 = 0; sp0 < row_splits; sp0 += AT_ONCE) {
+            float ms[AT_ONCE], ls[AT_ONCE], vs[AT_ONCE];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) ms[u] = part_at(sp0 + u, head_dim);
-#pragma unroll
-            for (int u = 0; u < 8; ++u) m = fmaxf(m, ms[u]);
-        }
-        float total = 0.0f, acc = 0.0f;
-        for (int sp0 = 0; sp0 < row_splits; sp0 += 8) {
-            float ms[8], ls[8], vs[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < AT_ONCE; ++u) {
                 ms[u] = part_at(sp0 + u, head_dim);
                 ls[u] = part_at(sp0 + u, head_dim + 1);
                 vs[u] = part_at(sp0 + u, d);
             }
+            float highest = m;
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                if (sp0 + u >= row_splits) break;
-                const float weight = exp2f(ms[u] - m);
+            for (int u = 0; u < AT_ONCE; ++u) highest = fmaxf(highest, ms[u]);
+            const float keep = exp2f(m - highest);      // 0 for the first batch, whose sums are 0 anyway
+            total *= keep;
+            acc *= keep;
+            m = highest;
+#pragma unroll
+            for (int u = 0; u < AT_ONCE; ++u) {
+                const float weight = sp0 + u < row_splits ? exp2f(ms[u] - m) : 0.0f;
                 total += weight * ls[u];
                 acc += weight * vs[u];
             }

@@ -87,21 +87,26 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
     const float* norm_w = p.norm_weight;
     const float one = p.one_centered ? 1.0f : 0.0f;
 
+    // Pre-normed rows: this lane's share of the partial sums of x^2 that the rows' producer left
+    // (the waves and the four lanes of a row split the tiles in a fixed order). The loads are
+    // issued here, in front of the stream of W, and their values are first used behind the
+    // product: a wave issues in order, so a sum formed here would hold W back by a round trip.
+    constexpr int SQ_HELD = 8;
+    float held[SQ_HELD];
     float prepared_square = 0.0f;
-    if (PRO == 2 && r16 < M) {
-        // This lane's share of the partial sums of x^2 that the rows' producer left: the waves
-        // and the four lanes of a row split the tiles in a fixed order, four loads in flight;
-        // the shares meet in the epilogue like the norm prologue's own.
-        const float* from = p.squares + r16;
-        float part[4] = {0.f, 0.f, 0.f, 0.f};
-        int t = wave * 4 + g;
-        const int step = WAVES * 4;
-        for (; t + 3 * step < p.squares_tiles; t += 4 * step)
+    bool prepared = false;
+    if (PRO == 2) {
+        const float* from = p.squares + r16;        // a row of 16 per tile: every lane's column exists
+        const int last = p.squares_tiles - 1;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) part[u] += from[(size_t)(t + u * step) * 16];
-        for (; t < p.squares_tiles; t += step) part[0] += from[(size_t)t * 16];
-        prepared_square = (part[0] + part[1]) + (part[2] + part[3]);
+        for (int u = 0; u < SQ_HELD; ++u) {
+            const int t = wave * 4 + g + u * WAVES * 4;
+            held[u] = from[(size_t)(t < last ? t : last) * 16];
+        }
     }
+    // The convolution's request slot, asked for before anything else needs waiting for.
+    int conv_slot = 0;
+    if (EPI == DG_CONV) conv_slot = p.seg_slot[r16 < M ? r16 : 0];
     for (int tile = blockIdx.x; tile < num_tiles; tile += gridDim.x) {
         const uint16_t* w_row[RT];
         bool w_ok[RT];
@@ -116,6 +121,20 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) acc[rt] = f32x4{0.f, 0.f, 0.f, 0.f};
         float square = 0.0f;
+        // What the accumulating epilogue reads (the residual stream's old values, the next norm's
+        // weight) is asked for here, so that it has arrived when the sums have: places that do
+        // not exist are read from element 0 and dropped. One tile kind (RT 1): wave 0 finishes.
+        float old_value[4] = {0.f, 0.f, 0.f, 0.f}, next_weight[4] = {0.f, 0.f, 0.f, 0.f};
+        if (EPI == DG_ACCUMULATE) {
+            const bool row_ok = r16 < M && !(ROWS == 8 && g >= 2);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int n = tile * ROWS + g * 4 + r;
+                const bool ok = row_ok && n < N;
+                old_value[r] = static_cast<const float*>(p.out)[ok ? (size_t)r16 * N + n : 0];
+                if (p.next_norm_weight) next_weight[r] = p.next_norm_weight[ok ? n : 0];
+            }
+        }
 #pragma unroll 2
         for (int k0 = wave * DG_CHUNK; k0 < K; k0 += WAVES * DG_CHUNK) {
             bf16x8 wf[RT][4], af[4];
@@ -163,11 +182,43 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
         }
         fw_mfma_drain();     // the loop is left by a branch; the accumulators are read next
 
+        // The convolution's state and taps of this lane's channels (kernels of up to four taps;
+        // longer ones read them in the epilogue): asked for in front of the barrier, so that they
+        // travel while the partial sums meet.
+        float early_state[4][3], early_taps[4][4];
+        const bool early = EPI == DG_CONV && p.kernel_size <= 4;
+        if (EPI == DG_CONV && early && wave == 0) {
+            const int history = p.kernel_size - 1;
+            const bool row_ok = r16 < M && !(ROWS == 8 && g >= 2);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int n = tile * ROWS + g * 4 + r;
+                const bool ok = row_ok && n < N;
+                const float* channel_state = p.state + (ok ? ((size_t)conv_slot * N + n) * history : 0);
+                const float* channel_taps = p.taps + (ok ? (size_t)n * p.kernel_size : 0);
+#pragma unroll
+                for (int k = 0; k < 3; ++k) early_state[r][k] = channel_state[k < history ? k : 0];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) early_taps[r][j] = channel_taps[j < p.kernel_size ? j : 0];
+            }
+        }
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) partial[wave][rt][lane][r] = acc[rt][r];
-        if (PRO == 2) square = prepared_square;
+        if (PRO == 2) {
+            if (!prepared) {
+                float part[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int u = 0; u < SQ_HELD; ++u)
+                    part[u & 3] += wave * 4 + g + u * WAVES * 4 < p.squares_tiles ? held[u] : 0.0f;
+                const float* from = p.squares + r16;
+                for (int t = wave * 4 + g + SQ_HELD * WAVES * 4; t < p.squares_tiles; t += WAVES * 4) part[0] += from[(size_t)t * 16];
+                prepared_square = (part[0] + part[1]) + (part[2] + part[3]);
+                prepared = true;
+            }
+            square = prepared_square;
+        }
         if (PRO != 0) {
             // this wave's share of sum x^2 of row r16: over the four k groups
             square += __shfl_xor(square, 16, 64);
@@ -202,10 +253,10 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
                     if (p.bias) value += p.bias[n];
                     TO* out = static_cast<TO*>(p.out);
                     const size_t at = (size_t)m * N + n;
-                    if (EPI == DG_ACCUMULATE) value += load_as_float(out, at);
+                    if (EPI == DG_ACCUMULATE) value += old_value[r];
                     store_from_float(out, at, value);
                     if (EPI == DG_ACCUMULATE && p.next_activations) {
-                        const float w = p.next_norm_weight[n] + (p.next_one_centered ? 1.0f : 0.0f);
+                        const float w = next_weight[r] + (p.next_one_centered ? 1.0f : 0.0f);
                         p.next_activations[at] = float_to_bf16_bits(value * w);
                         row_square += value * value;
                     }
@@ -241,15 +292,34 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
                     store_from_float(out, (size_t)m * N + n, dg_silu(total[0][r]) * total[RT > 1 ? 1 : 0][r]);
                 } else {        // DG_CONV: tiles are B, C, x of channel n; the row is a segment of one token
                     const int history = p.kernel_size - 1;
-                    float* channel_state = p.state + ((size_t)p.seg_slot[m] * N + n) * history;
-                    const float* channel_taps = p.taps + (size_t)n * p.kernel_size;
-                    float window[DG_MAX_TAPS];
-                    for (int k = 0; k < history; ++k) window[k] = channel_state[k];
-                    window[history] = total[0][r] * total[RT > 2 ? 2 : 0][r];
+                    float* channel_state = p.state + ((size_t)conv_slot * N + n) * history;
+                    const float newest = total[0][r] * total[RT > 2 ? 2 : 0][r];
                     float y = 0.0f;
-                    for (int j = 0; j < p.kernel_size; ++j) y = fmaf(channel_taps[j], window[j], y);
-                    if (p.conv_bias) y += p.conv_bias[n];
-                    for (int k = 0; k < history; ++k) channel_state[k] = window[k + 1];
+                    if (early) {
+                        // the same sum in the same order, over values that are already here
+                        float window[4];
+#pragma unroll
+                        for (int k = 0; k < 3; ++k) window[k] = k < history ? early_state[r][k] : 0.0f;
+                        window[3] = 0.0f;
+#pragma unroll
+                        for (int k = 0; k < 4; ++k)
+                            if (k == history) window[k] = newest;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (j < p.kernel_size) y = fmaf(early_taps[r][j], window[j], y);
+                        if (p.conv_bias) y += p.conv_bias[n];
+#pragma unroll
+                        for (int k = 0; k < 3; ++k)
+                            if (k < history) channel_state[k] = window[k + 1];
+                    } else {
+                        const float* channel_taps = p.taps + (size_t)n * p.kernel_size;
+                        float window[DG_MAX_TAPS];
+                        for (int k = 0; k < history; ++k) window[k] = channel_state[k];
+                        window[history] = newest;
+                        for (int j = 0; j < p.kernel_size; ++j) y = fmaf(channel_taps[j], window[j], y);
+                        if (p.conv_bias) y += p.conv_bias[n];
+                        for (int k = 0; k < history; ++k) channel_state[k] = window[k + 1];
+                    }
                     store_from_float(out, (size_t)m * N + n, total[RT > 1 ? 1 : 0][r] * y);
                 }
             }

@@ -85,20 +85,7 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r16 = lane & 15, g = lane >> 4;
     const int ft = wave % FW, kp = wave / FW;
     const int M = p.M, N = p.N, K = p.K;
-    // prepared activations: this thread's share of the sums of squares of one row, requested first
     const int square_stride = gm_square_stride(M);
-    float square_share = 0.0f;
-    if (p.squares) {
-        const int row = threadIdx.x % square_stride, part = threadIdx.x / square_stride, parts = GM_THREADS / square_stride;
-        const float* from = p.squares + row;
-        float share[4] = {0.f, 0.f, 0.f, 0.f};
-        int e = part;
-        for (; e + 3 * parts < p.squares_rows; e += 4 * parts)
-#pragma unroll
-            for (int u = 0; u < 4; ++u) share[u] += from[(size_t)(e + u * parts) * square_stride];
-        for (; e < p.squares_rows; e += parts) share[0] += from[(size_t)e * square_stride];
-        square_share = (share[0] + share[1]) + (share[2] + share[3]);
-    }
     const int tile = blockIdx.x, tiles = gridDim.x;
     const int n0 = tile * 16 * FW;
     const int k_begin = blockIdx.y * p.k_per_split;
@@ -173,6 +160,21 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
 
 #pragma unroll
     for (int d = 0; d < GM_DEPTH; ++d) load(d, d);
+    // prepared activations: this thread's share of the sums of squares of one row, asked for
+    // behind the first chunks of W (a wave issues in order: in front of them the sums would
+    // hold the stream of W back by a round trip)
+    float square_share = 0.0f;
+    if (p.squares) {
+        const int row = threadIdx.x % square_stride, part = threadIdx.x / square_stride, parts = GM_THREADS / square_stride;
+        const float* from = p.squares + row;
+        float share[4] = {0.f, 0.f, 0.f, 0.f};
+        int e = part;
+        for (; e + 3 * parts < p.squares_rows; e += 4 * parts)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) share[u] += from[(size_t)(e + u * parts) * square_stride];
+        for (; e < p.squares_rows; e += parts) share[0] += from[(size_t)e * square_stride];
+        square_share = (share[0] + share[1]) + (share[2] + share[3]);
+    }
     stage(0, 0, 0);
     if (p.squares) square_parts[threadIdx.x] = square_share;
     fw_lds_barrier();
@@ -220,6 +222,22 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
     // that workgroups on different dies do not share, so no cache has to be written back or
     // dropped as a whole (what a device-wide fence does): a wave waits for its own stores to be
     // acknowledged, the workgroup meets, then one thread takes the ticket.
+    // What the accumulating epilogue reads beside the sums (the residual stream's old values, the
+    // next norm's weight) is asked for before the slices of the other workgroups are, so that one
+    // round trip covers both.
+    const int early_first = n0 + 16 * ft + 4 * g;
+    const bool early_whole = early_first + 3 < N && (N & 3) == 0;
+    f32x4 early_old[MT], early_weight = {0.f, 0.f, 0.f, 0.f};
+    auto fetch_early = [&]() {
+        if (MODE != GM_ACCUMULATE || sizeof(TO) != 4 || !early_whole) return;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + r16;
+            early_old[mt] = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p.out) + (size_t)(m < M ? m : 0) * N + early_first);
+        }
+        if (p.next_activations) early_weight = *reinterpret_cast<const f32x4*>(p.next_norm_weight + early_first);
+    };
+    if (p.splits <= 1 && kp == 0) fetch_early();
     if (p.splits > 1) {
         float* mine = p.partials + ((((size_t)blockIdx.y * tiles + tile) * (KINDS * MT) * FW + ft) * 64 + lane) * 4;
         if (kp == 0)
@@ -238,6 +256,7 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
         __syncthreads();
         if (ticket_shared != p.splits - 1) return;
         if (kp == 0) {
+            fetch_early();
 #pragma unroll
             for (int kind = 0; kind < KINDS; ++kind)
 #pragma unroll
@@ -285,7 +304,7 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
                 if (whole) {
                     f32x4 packed = {v[0], v[1], v[2], v[3]};
                     if (MODE == GM_ACCUMULATE) {
-                        const f32x4 old = *reinterpret_cast<const f32x4*>(to);
+                        const f32x4 old = early_old[mt];
 #pragma unroll
                         for (int r = 0; r < 4; ++r) packed[r] = v[r] = v[r] + old[r];
                     }
@@ -319,7 +338,7 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
             if (mine) {
                 const float one = p.next_one_centered ? 1.0f : 0.0f;
                 if (whole) {
-                    const f32x4 w = *reinterpret_cast<const f32x4*>(p.next_norm_weight + n_first);
+                    const f32x4 w = early_weight;
                     uint2 packed;
                     packed.x = (uint32_t)float_to_bf16_bits(v[0] * (w[0] + one)) | ((uint32_t)float_to_bf16_bits(v[1] * (w[1] + one)) << 16);
                     packed.y = (uint32_t)float_to_bf16_bits(v[2] * (w[2] + one)) | ((uint32_t)float_to_bf16_bits(v[3] * (w[3] + one)) << 16);

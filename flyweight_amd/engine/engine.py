@@ -243,7 +243,9 @@ class Runtime:
                 if kind == EVENT_TOKEN:
                     produced.append(value)
                     if callback is not None and callback(value) is False:
+                        # Tokens of the same turn that lie behind this one are dropped.
                         self.task_cancel(task)
+                        return produced
                 elif kind == EVENT_ERROR:
                     raise EngineError(self.task_error(task) or "generation failed")
                 elif kind == EVENT_FINISHED:
