@@ -29,63 +29,44 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
     const int lane = threadIdx.x;
     const int width = (num_heads + 2 * num_kv_heads) * head_dim;
     const TI* source = qkv + (size_t)row * width + (size_t)vec * head_dim;
-    // Everything the wave reads is asked for at once: the page of the row's position is two
-    // dependent loads away, and the head's channels, the norm weight and the rotation's table
-    // travel meanwhile. A lane holds channels lane, lane + 64, ... (head_dim is at most 256);
-    // places past head_dim are read from channel 0 and dropped.
-    constexpr int PER_LANE = ATTN_MAX_HEAD_DIM / 64;
-    const bool is_value = vec >= num_heads + num_kv_heads;
-    const bool is_query = vec < num_heads;
-    const float* weight = is_value ? nullptr : (is_query ? q_norm_weight : k_norm_weight);
-    const int half = rotary_dim / 2;
     const int pos = row_pos[row];
-    const int segment = row_seg[row];
-    float v[PER_LANE], w[PER_LANE], c[PER_LANE], sn[PER_LANE];
-#pragma unroll
-    for (int i = 0; i < PER_LANE; ++i) {
-        const int d = lane + 64 * i;
-        const bool ok = d < head_dim;
-        v[i] = load_as_float(source, ok ? d : 0);
-        w[i] = weight ? weight[ok ? d : 0] : 1.0f;
-        const bool turned = ok && !is_value && d < rotary_dim;
-        const int pair = d < half ? d : d - half;
-        c[i] = turned ? cos_table[(size_t)row * half + pair] : 1.0f;
-        sn[i] = turned ? sin_table[(size_t)row * half + pair] : 0.0f;
-    }
-    const int page = block_table[(size_t)segment * table_stride + pos / ATTN_PAGE];
+    const int page = block_table[(size_t)row_seg[row] * table_stride + pos / ATTN_PAGE];
     const int slot = pos % ATTN_PAGE;
 
-    if (is_value) {      // value head: transposed store
+    if (vec >= num_heads + num_kv_heads) {      // value head: transposed store
         const int kvh = vec - num_heads - num_kv_heads;
         T* dest = v_pages + ((size_t)page * num_kv_heads + kvh) * head_dim * ATTN_PAGE;
-#pragma unroll
-        for (int i = 0; i < PER_LANE; ++i)
-            if (lane + 64 * i < head_dim) store_from_float(dest, (size_t)(lane + 64 * i) * ATTN_PAGE + slot, v[i]);
+        for (int d = lane; d < head_dim; d += 64) store_from_float(dest, (size_t)d * ATTN_PAGE + slot, load_as_float(source, d));
         return;
     }
+    const bool is_query = vec < num_heads;
+    const float* weight = is_query ? q_norm_weight : k_norm_weight;
     float inv = 1.0f;
     if (weight) {
         float sum = 0.0f;
-#pragma unroll
-        for (int i = 0; i < PER_LANE; ++i)
-            if (lane + 64 * i < head_dim) sum += v[i] * v[i];
+        for (int d = lane; d < head_dim; d += 64) {
+            const float v = load_as_float(source, d);
+            sum += v * v;
+        }
         sum = wave_sum(sum);
         inv = rsqrtf(sum / (float)head_dim + eps);
     }
-#pragma unroll
-    for (int i = 0; i < PER_LANE; ++i)
-        if (lane + 64 * i < head_dim) normed[lane + 64 * i] = weight ? v[i] * inv * w[i] : v[i];
+    for (int d = lane; d < head_dim; d += 64) {
+        const float v = load_as_float(source, d);
+        normed[d] = weight ? v * inv * weight[d] : v;
+    }
     __syncthreads();
+    const int half = rotary_dim / 2;
     T* dest = is_query ? q_out + ((size_t)row * num_heads + vec) * head_dim
                        : k_pages + (((size_t)page * num_kv_heads + (vec - num_heads)) * ATTN_PAGE + slot) * head_dim;
-#pragma unroll
-    for (int i = 0; i < PER_LANE; ++i) {
-        const int d = lane + 64 * i;
-        if (d >= head_dim) continue;
+    for (int d = lane; d < head_dim; d += 64) {
         float value = normed[d];
         if (d < rotary_dim) {
+            const int pair = d < half ? d : d - half;
             const float other = normed[d < half ? d + half : d - half];
-            value = d < half ? value * c[i] - other * sn[i] : value * c[i] + other * sn[i];
+            const float c = cos_table[(size_t)row * half + pair];
+            const float s = sin_table[(size_t)row * half + pair];
+            value = d < half ? value * c - other * s : value * c + other * s;
         }
         store_from_float(dest, d, value);
     }

@@ -158,21 +158,33 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
                     acc[kind][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[d][kind][ks], af[ks][mt], acc[kind][mt], 0, 0, 0);
     };
 
-#pragma unroll
-    for (int d = 0; d < GM_DEPTH; ++d) load(d, d);
-    // prepared activations: this thread's share of the sums of squares of one row, asked for
-    // behind the first chunks of W (a wave issues in order: in front of them the sums would
-    // hold the stream of W back by a round trip)
-    float square_share = 0.0f;
+    // prepared activations: this thread's share of the sums of squares of one row is asked for
+    // first and added up behind the first chunks of W (a wave issues in order: a sum formed here
+    // would hold the stream of W back by a round trip)
+    constexpr int SQ_HELD = 32;
+    float held[SQ_HELD];
     if (p.squares) {
         const int row = threadIdx.x % square_stride, part = threadIdx.x / square_stride, parts = GM_THREADS / square_stride;
         const float* from = p.squares + row;
-        float share[4] = {0.f, 0.f, 0.f, 0.f};
-        int e = part;
-        for (; e + 3 * parts < p.squares_rows; e += 4 * parts)
+        const int last = p.squares_rows - 1;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) share[u] += from[(size_t)(e + u * parts) * square_stride];
-        for (; e < p.squares_rows; e += parts) share[0] += from[(size_t)e * square_stride];
+        for (int u = 0; u < SQ_HELD; ++u) {
+            const int e = part + u * parts;
+            held[u] = from[(size_t)(e < last ? e : last) * square_stride];
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < GM_DEPTH; ++d) load(d, d);
+    // the shares of the sums of squares have been on their way since before W: they are the
+    // oldest loads, so adding them up here waits for nothing that was asked for after them
+    float square_share = 0.0f;
+    if (p.squares) {
+        const int row = threadIdx.x % square_stride, part = threadIdx.x / square_stride, parts = GM_THREADS / square_stride;
+        float share[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < SQ_HELD; ++u) share[u & 3] += part + u * parts < p.squares_rows ? held[u] : 0.0f;
+        const float* from = p.squares + row;
+        for (int e = part + SQ_HELD * parts; e < p.squares_rows; e += parts) share[0] += from[(size_t)e * square_stride];
         square_share = (share[0] + share[1]) + (share[2] + share[3]);
     }
     stage(0, 0, 0);
