@@ -238,6 +238,30 @@ def test_decode_steps_that_run_ahead_of_the_host_give_the_same_tokens(loaded, dt
         assert queued == single
 
 
+def test_generate_stops_at_the_token_its_callback_refuses_even_inside_a_burst(loaded):
+    """With several decode steps per turn a turn brings several tokens of a request: the callback
+    that returns False ends the generation at its token; the tokens of the same turn behind it are
+    dropped, the request's pages and slot are given back."""
+    m = loaded("A", "float32")
+    prompt = random_tokens(m.config.vocab_size, 11, seed=5)
+    whole = _runtime(m, parallel_sequences=2, prefill_rows=64, max_batch_tokens=128).generate(prompt, 24)
+    assert len(whole) == 24
+    for stop_after in (1, 6, 7, 10):
+        runtime = _runtime(m, parallel_sequences=2, prefill_rows=64, max_batch_tokens=128, decode_steps_per_turn=4)
+        seen = []
+
+        def callback(token):
+            seen.append(token)
+            return len(seen) < stop_after
+
+        got = runtime.generate(prompt, 24, callback)
+        assert got == whole[:stop_after] and seen == got
+        while runtime.scheduler.has_work():
+            runtime.engine_step()
+        runtime.stepper.cache.check_invariants()
+        assert runtime.info["pages_free"] == runtime.num_pages and runtime.info["live_requests"] == 0
+
+
 def test_seeded_sampling_does_not_depend_on_the_batch(loaded):
     """Temperature 0.8, seed 7, portions of 16 mixed with decode rows: a request draws the
     same tokens alone and among others, and they are the plain sampler's tokens given the
