@@ -41,6 +41,9 @@ def _add_runtime(parser: argparse.ArgumentParser, context_default: int) -> None:
     group.add_argument("--parallel", type=int, default=1, metavar="N", help="requests that may be live at once")
     group.add_argument("--prefill-rows", type=int, default=512, metavar="N", help="most tokens of one prompt portion")
     group.add_argument("--max-batch-tokens", type=int, default=2048, metavar="N", help="most tokens of one step")
+    group.add_argument("--decode-steps-per-turn", type=int, default=1, metavar="N",
+                       help="decode steps that may run back to back on the device before the host reads their tokens "
+                            "(greedy requests without stop tokens; tokens then arrive in bursts)")
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -100,7 +103,8 @@ def _runtime(args, context: Optional[int] = None):
     model = Model(args.model, dtype=args.dtype)
     limit = min(context or args.context_window, model.spec.max_positions)
     return model, Runtime(model, context_limit=limit, parallel_sequences=args.parallel,
-                          prefill_rows=args.prefill_rows, max_batch_tokens=args.max_batch_tokens).prepare()
+                          prefill_rows=args.prefill_rows, max_batch_tokens=args.max_batch_tokens,
+                          decode_steps_per_turn=args.decode_steps_per_turn).prepare()
 
 
 def _generate(args) -> int:
