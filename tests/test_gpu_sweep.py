@@ -1,0 +1,90 @@
+"""Random tiny configurations against the plain implementation: head sizes in steps of 16 up to
+256, any number of heads and groups, widths and vocabularies that are no power of two, two to five
+layers in any arrangement of the two mixers, two to six taps with and without biases, tied and
+untied heads. Each is stepped whole, in portions with single tokens between them, and as two
+requests of which one decodes beside portions of the other, in float32 and in bfloat16."""
+
+import tempfile
+
+import numpy as np
+import pytest
+
+import plain_lfm2 as plain
+from gpu_common import feed
+from helpers import assert_close, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+
+def random_config(rng) -> dict:
+    head_dim = int(rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 256]))
+    kv_heads = int(rng.choice([1, 2, 3]))
+    heads = kv_heads * int(rng.choice([1, 2, 3, 4, 5, 8]))
+    if heads * head_dim > 1536:         # keeps the plain implementation quick
+        heads = max(kv_heads, (1536 // head_dim) // kv_heads * kv_heads)
+    layers = int(rng.integers(2, 6))
+    types = [str(rng.choice(["conv", "full_attention"])) for _ in range(layers)]
+    for kind in ("conv", "full_attention"):
+        if kind not in types:
+            types[int(rng.integers(0, layers))] = kind
+    return dict(
+        architectures=["Lfm2ForCausalLM"], model_type="lfm2", vocab_size=int(rng.choice([130, 257, 500, 1001])),
+        hidden_size=heads * head_dim, num_hidden_layers=layers, num_attention_heads=heads, num_key_value_heads=kv_heads,
+        intermediate_size=int(rng.choice([72, 160, 200, 384])), block_auto_adjust_ff_dim=bool(rng.integers(0, 2)),
+        block_ffn_dim_multiplier=float(rng.choice([1.0, 1.5])), block_multiple_of=int(rng.choice([8, 24, 64])),
+        norm_eps=float(rng.choice([1e-5, 1e-6])), rope_theta=float(rng.choice([1e4, 1e6])),
+        conv_L_cache=int(rng.integers(2, 7)), conv_bias=bool(rng.integers(0, 2)),
+        tie_word_embeddings=bool(rng.integers(0, 2)), max_position_embeddings=512, layer_types=types)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_a_random_configuration_matches_the_plain_model(seed):
+    from flyweight_amd.config import config_from_dict
+    from flyweight_amd.engine import StepEntry, Stepper, load_model
+    from flyweight_amd.weights import write_random_model
+    rng = np.random.default_rng(1000 + seed)
+    config = random_config(rng)
+    what = (f"head_dim {config['hidden_size'] // config['num_attention_heads']} heads {config['num_attention_heads']}/"
+            f"{config['num_key_value_heads']} layers {config['layer_types']} taps {config['conv_L_cache']}")
+    with tempfile.TemporaryDirectory() as folder:
+        write_random_model(folder, config_from_dict(config), seed=seed, scale="fan_in")
+        plain_config, plain_weights = plain.read_folder(folder)
+        tokens = random_tokens(config["vocab_size"], 140, seed=seed)
+        other = random_tokens(config["vocab_size"], 75, seed=seed + 100)
+        want, want_other = plain.forward(plain_config, plain_weights, tokens), plain.forward(plain_config, plain_weights, other)
+        for dtype in ("float32", "bfloat16"):
+            _, model = load_model(folder, dtype=dtype)
+            stepper = Stepper(model, num_pages=6, max_requests=3)
+            stepper.admit("r")
+            assert_close(feed(stepper, "r", tokens, [140]), want, dtype, f"{what}: {dtype} whole")
+            stepper.release("r")
+            stepper.admit("r")
+            cuts = [63, 2, 1, 1, 30, 1, 1, 1, 1, 1, 1, 1, 1, 20] + [1] * 20
+            assert_close(feed(stepper, "r", tokens, cuts), want, dtype, f"{what}: {dtype} in portions")
+            stepper.release("r")
+            # two requests: "a" decodes token by token beside portions of one to eight tokens of "b"
+            stepper.admit("a")
+            stepper.admit("b")
+            got_a = [stepper.step([StepEntry("a", tokens[:100], list(range(100)))]).cpu().numpy()]
+            got_b, at_a, at_b = [], 100, 0
+            while at_a < len(tokens) or at_b < len(other):
+                entries, rows_a = [], 0
+                if at_a < len(tokens):
+                    entries.append(StepEntry("a", tokens[at_a:at_a + 1], [0]))
+                    rows_a = 1
+                portion = min(int(rng.integers(1, 9)), len(other) - at_b)
+                if portion > 0:
+                    entries.append(StepEntry("b", other[at_b:at_b + portion], list(range(portion))))
+                out = stepper.step(entries).cpu().numpy()
+                if rows_a:
+                    got_a.append(out[:1])
+                    at_a += 1
+                if portion > 0:
+                    got_b.append(out[rows_a:])
+                    at_b += portion
+            assert_close(np.concatenate(got_a), want, dtype, f"{what}: {dtype} decoding beside another's portions")
+            assert_close(np.concatenate(got_b), want_other, dtype, f"{what}: {dtype} portions beside another's decoding")
+            stepper.release("a")
+            stepper.release("b")
+            stepper.cache.check_invariants()
+            assert stepper.cache.groups[0].pool.in_use == 0
