@@ -318,6 +318,8 @@ def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out
         entry = library().fw_gemm_skinny
     elif M > BIG_MIN_ROWS and library().fw_gemm_mfma_big_tiles(mode, M, N, K) >= BIG_TILES_MIN:
         entry = library().fw_gemm_mfma_big      # enough 256 x 256 tiles to fill the chip
+    elif K >= DEEP_MIN_K and DEEP_TILES_MIN <= library().fw_gemm_mfma_deep_tiles(mode, M, N, K) <= DEEP_TILES_MAX:
+        entry = library().fw_gemm_mfma_deep     # one 128 x 128 tile per compute unit over a long K: the waves split K
     else:
         need_bytes, need_counters = ctypes.c_size_t(0), ctypes.c_int(0)
         _check(library().fw_gemm_mfma_split_plan(mode, M, N, K, ctypes.byref(need_bytes), ctypes.byref(need_counters)))
@@ -334,6 +336,8 @@ def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out
 SKINNY_MAX_ROWS = 16
 MEDIUM_MAX_ROWS = 64
 BIG_TILES_MIN = 192      # 256 x 256 tiles from which the large-tile prompt product is used (256 compute units)
+DEEP_MIN_K = 4096         # below, the exchange between the waves at the end of a tile costs more than the main loop gains
+DEEP_TILES_MIN, DEEP_TILES_MAX = 200, 256   # one round of tiles over 256 compute units (2,048 x 2,048 x 8,192: 99 vs 124 us)
 BIG_MIN_ROWS = 128       # up to here a 256-row tile would be at least half empty (the head at 128 rows: 110 vs 78 us)
 _MEDIUM_COUNTERS = {}
 
@@ -420,6 +424,28 @@ def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
     gemm_medium_into(a, w, bias, out, _code(out_dtype), epilogue, N, squares=squares, eps=eps)
     return out
+
+
+def gemm_deep(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+              out_dtype: Optional[torch.dtype] = None, accumulate_into: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """a [M, K] . w [N, K]^T (+ bias) on 128 x 128 tiles whose waves split K (fw_gemm_mfma_deep),
+    whatever the dispatch of ``gemm`` would choose: bfloat16 operands, K a multiple of 64."""
+    _dev(a, w, bias, accumulate_into)
+    _want(a, torch.bfloat16, "a")
+    _want(w, torch.bfloat16, "w")
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or (bias is not None and (bias.dtype != torch.float32 or bias.shape != (N,))):
+        raise KernelError(f"gemm_deep: a is {tuple(a.shape)}, w is {tuple(w.shape)}; bias is float32 [N]")
+    if accumulate_into is not None:
+        _want(accumulate_into, torch.float32, "accumulate_into")
+        if accumulate_into.shape != (M, N):
+            raise KernelError(f"gemm_deep: destination is {tuple(accumulate_into.shape)}, expected {(M, N)}")
+        target, mode = accumulate_into, 1
+    else:
+        target, mode = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device), 0
+    _check(library().fw_gemm_mfma_deep(_p(a), _p(w), _p(bias), _p(target), _code(target.dtype), mode, M, N, K, _stream()))
+    return target
 
 
 def _fast_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
