@@ -13,7 +13,9 @@
 //  * slabs of 128 rows x 64 k of both operands travel from global memory straight into LDS
 //    (global_load_lds_dwordx4), three slabs ahead of the one being multiplied, four stages of
 //    32 KB; a row is 128 bytes, its eight 16-byte chunks stored permuted (chunk c of row r in slot
-//    c ^ (r % 8)) so that the operand reads of eight consecutive rows cover all banks;
+//    c ^ ((r / 2) % 8)) so that the operand reads of sixteen consecutive rows, two rows to 256
+//    bytes, cover all 64 banks once (with c ^ (r % 8) rows r and r + 8 met in the same banks:
+//    two conflict cycles per MFMA on the counters);
 //  * one wave per SIMD: the operands of the next slab are read between the MFMAs of this one, and
 //    the loads of the slab three ahead are issued there too; one barrier per slab;
 //  * workgroups are numbered so that each XCD works on a compact group of tiles.
@@ -56,14 +58,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
     // The copy: a wave-wide load writes 1,024 contiguous bytes of LDS, lane l its 16 bytes at
-    // l * 16: 8 rows of 128 bytes. Lane l asks for chunk (l % 8) ^ (r % 8) of row r = l / 8 of its
-    // 8 rows (rows past the end of a or w are read from the last row and never stored).
+    // l * 16: 8 rows of 128 bytes. Lane l asks for chunk (l % 8) ^ ((r / 2) % 8) of row r = l / 8 of
+    // its 8 rows (rows past the end of a or w are read from the last row and never stored).
     const uint16_t* a_src[D_LOADS];
     const uint16_t* w_src[D_LOADS];
 #pragma unroll
     for (int i = 0; i < D_LOADS; ++i) {
         const int row = (wave * D_LOADS + i) * 8 + (lane >> 3);
-        const int chunk = (lane & 7) ^ (row & 7);
+        const int chunk = (lane & 7) ^ ((row >> 1) & 7);
         int am = m0 + row;
         am = am < M ? am : M - 1;
         a_src[i] = a + (size_t)am * K + chunk * 8;
@@ -93,7 +95,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // This wave's k16 step of every slab: chunks 2 * wave and 2 * wave + 1 of a row, the lower for
     // lanes 0..31, the upper for lanes 32..63. Every row a lane reads is (lane % 32) plus a
     // multiple of 32, so one permutation serves all of them.
-    const int slot = ((2 * wave + (lane >> 5)) ^ (lane & 7)) * 16;
+    const int slot = ((2 * wave + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
     const int row_offset = (lane & 31) * (DK * 2) + slot;
     struct Operands {
         bf16x8 fa[4], fb[4];
