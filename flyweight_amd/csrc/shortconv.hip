@@ -47,6 +47,68 @@ __global__ void shortconv_rows_kernel(const T* __restrict__ bcx, TO* __restrict_
     store_from_float(out, (size_t)row * hidden + channel, gate * y);
 }
 
+// The same for kernels of up to four taps, eight consecutive rows of a channel per thread: the
+// products B * x of the rows and of the three before them are formed once and slide through
+// the taps in registers (a row's product is otherwise read by as many threads as there are taps),
+// and the chain of dependent loads in front (segment of the row, its first row, its slot) is paid
+// once for eight rows: with a thread per (row, channel) a prompt's 16 thousand workgroups were
+// bound by that chain. The taps are aligned to the end of a window of four: tap j of a kernel of L
+// taps sits at place j + 4 - L; the places in front are skipped. Sums in the order of the taps, as above.
+#define CONV_TILE_ROWS 8
+#define CONV_TILE_HISTORY 3
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void shortconv_rows8_kernel(const T* __restrict__ bcx, TO* __restrict__ out,
+                                                              const float* __restrict__ taps, const float* __restrict__ conv_bias,
+                                                              const float* __restrict__ state, const int32_t* __restrict__ row_seg,
+                                                              const int32_t* __restrict__ seg_row0, const int32_t* __restrict__ seg_slot,
+                                                              int rows, int hidden, int kernel_size) {
+    constexpr int R = CONV_TILE_ROWS, H = CONV_TILE_HISTORY;
+    const int r0 = blockIdx.y * R;
+    const int channel = blockIdx.x * blockDim.x + threadIdx.x;
+    if (channel >= hidden) return;
+    const int history = kernel_size - 1, unused = H - history;      // places of the window in front of tap 0
+    // every row's segment and place in it, asked for together and first (two dependent loads each)
+    int seg_of[R], offset_of[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) seg_of[i] = row_seg[r0 + i < rows ? r0 + i : rows - 1];
+#pragma unroll
+    for (int i = 0; i < R; ++i) offset_of[i] = r0 + i - seg_row0[seg_of[i]];
+    // the products of rows r0 - 3 .. r0 + 7 (0 where that is no row of this step)
+    float product[R + H];
+#pragma unroll
+    for (int p = 0; p < R + H; ++p) {
+        const int row = r0 - H + p;
+        const bool valid = row >= 0 && row < rows;
+        const T* source = bcx + (size_t)(valid ? row : 0) * 3 * hidden;
+        const float value = load_as_float(source, channel) * load_as_float(source, 2 * (size_t)hidden + channel);
+        product[p] = valid ? value : 0.0f;
+    }
+    float tap[H + 1];
+#pragma unroll
+    for (int place = 0; place <= H; ++place)
+        tap[place] = place >= unused ? taps[(size_t)channel * kernel_size + (place - unused)] : 0.0f;
+    const float bias = conv_bias ? conv_bias[channel] : 0.0f;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        const int row = r0 + i;
+        if (row >= rows) break;
+        const int seg = seg_of[i], offset_in_segment = offset_of[i];
+        float y = 0.0f;
+#pragma unroll
+        for (int place = 0; place <= H; ++place) {
+            if (place < unused) continue;       // in front of tap 0: not this kernel's (and never multiplied, not even by 0)
+            float value = product[i + place];
+            const int offset = offset_in_segment - H + place;       // where in the segment this place lies
+            if (offset < 0)                                         // in front of the segment: the request's state
+                value = state[((size_t)seg_slot[seg] * hidden + channel) * history + history + offset];
+            y = fmaf(tap[place], value, y);
+        }
+        y += bias;
+        const float gate = load_as_float(bcx, (size_t)row * 3 * hidden + hidden + channel);
+        store_from_float(out, (size_t)row * hidden + channel, gate * y);
+    }
+}
+
 template <typename T>
 __global__ void shortconv_state_kernel(const T* __restrict__ bcx, float* __restrict__ state,
                                        const int32_t* __restrict__ seg_row0, const int32_t* __restrict__ seg_slot,
@@ -99,8 +161,12 @@ static void launch(const void* bcx, void* out, const float* taps, const float* c
             (const T*)bcx, (TO*)out, taps, conv_bias, state, seg_slot, hidden, kernel_size);
         return;
     }
-    shortconv_rows_kernel<T, TO><<<dim3(bx, rows), 256, 0, stream>>>(
-        (const T*)bcx, (TO*)out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, hidden, kernel_size);
+    if (kernel_size <= CONV_TILE_HISTORY + 1 && rows >= 4 * CONV_TILE_ROWS)
+        shortconv_rows8_kernel<T, TO><<<dim3(bx, fw_ceil_div(rows, CONV_TILE_ROWS)), 256, 0, stream>>>(
+            (const T*)bcx, (TO*)out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, rows, hidden, kernel_size);
+    else
+        shortconv_rows_kernel<T, TO><<<dim3(bx, rows), 256, 0, stream>>>(
+            (const T*)bcx, (TO*)out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, hidden, kernel_size);
     shortconv_state_kernel<T><<<dim3(bx, segments), 256, 0, stream>>>(
         (const T*)bcx, state, seg_row0, seg_slot, hidden, kernel_size);
 }
