@@ -72,6 +72,71 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
     }
 }
 
+// The same for heads of up to 64 channels (a channel per lane), eight rows of one head-vector per
+// wave: what the wave reads for its eight rows is asked for together, so the chain of dependent
+// loads in front (position and segment of the row, its page) is paid once for eight rows. A prompt
+// of 2,048 rows has a hundred thousand (row, head-vector) pairs; as waves of one pair each they
+// were bound by that chain. The rotation's partner channel comes from the partner lane. The same
+// arithmetic in the same order as above.
+#define QK_ROWS 8
+template <typename TI, typename T>
+__global__ __launch_bounds__(64) void qk_norm_rope_kv_write_rows_kernel(
+    const TI* __restrict__ qkv, T* __restrict__ q_out, const float* __restrict__ q_norm_weight,
+    const float* __restrict__ k_norm_weight, float eps, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, int rotary_dim, T* __restrict__ k_pages, T* __restrict__ v_pages,
+    const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int rows) {
+    const int r0 = blockIdx.x * QK_ROWS;
+    const int vec = blockIdx.y;
+    const int lane = threadIdx.x;
+    const int width = (num_heads + 2 * num_kv_heads) * head_dim;
+    const bool active = lane < head_dim;
+    const bool is_value = vec >= num_heads + num_kv_heads, is_query = vec < num_heads;
+    const float* weight = is_value ? nullptr : (is_query ? q_norm_weight : k_norm_weight);
+    const int half = rotary_dim / 2;
+    const bool turned = !is_value && lane < rotary_dim;
+    const int pair = lane < half ? lane : lane - half;
+    int row_of[QK_ROWS], pos[QK_ROWS], page[QK_ROWS];
+    float v[QK_ROWS], c[QK_ROWS], sn[QK_ROWS];
+#pragma unroll
+    for (int i = 0; i < QK_ROWS; ++i) {
+        row_of[i] = r0 + i < rows ? r0 + i : rows - 1;
+        pos[i] = row_pos[row_of[i]];
+        page[i] = row_seg[row_of[i]];
+    }
+#pragma unroll
+    for (int i = 0; i < QK_ROWS; ++i) {
+        v[i] = load_as_float(qkv + (size_t)row_of[i] * width + (size_t)vec * head_dim, active ? lane : 0);
+        c[i] = turned ? cos_table[(size_t)row_of[i] * half + pair] : 1.0f;
+        sn[i] = turned ? sin_table[(size_t)row_of[i] * half + pair] : 0.0f;
+    }
+    const float w = (weight && active) ? weight[lane] : 1.0f;
+#pragma unroll
+    for (int i = 0; i < QK_ROWS; ++i) page[i] = block_table[(size_t)page[i] * table_stride + pos[i] / ATTN_PAGE];
+#pragma unroll
+    for (int i = 0; i < QK_ROWS; ++i) {
+        if (r0 + i >= rows) break;
+        const int slot = pos[i] % ATTN_PAGE;
+        if (is_value) {      // value head: transposed store
+            const int kvh = vec - num_heads - num_kv_heads;
+            T* dest = v_pages + ((size_t)page[i] * num_kv_heads + kvh) * head_dim * ATTN_PAGE;
+            if (active) store_from_float(dest, (size_t)lane * ATTN_PAGE + slot, v[i]);
+            continue;
+        }
+        float value = active ? v[i] : 0.0f;
+        if (weight) {
+            const float sum = wave_sum(value * value);
+            const float inv = rsqrtf(sum / (float)head_dim + eps);
+            value = value * inv * w;
+        }
+        const float other = __shfl(value, lane < half ? lane + half : lane - half, 64);
+        if (lane < rotary_dim) value = lane < half ? value * c[i] - other * sn[i] : value * c[i] + other * sn[i];
+        T* dest = is_query ? q_out + ((size_t)row_of[i] * num_heads + vec) * head_dim
+                           : k_pages + (((size_t)page[i] * num_kv_heads + (vec - num_heads)) * ATTN_PAGE + slot) * head_dim;
+        if (active) store_from_float(dest, lane, value);
+    }
+}
+
 extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int dtype, const float* q_norm_weight,
                                         const float* k_norm_weight, float eps, const float* cos_table,
                                         const float* sin_table, int rotary_dim, void* k_pages, void* v_pages,
@@ -91,6 +156,20 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
     FW_REQUIRE(vectors <= 65535, "qk_norm_rope: too many heads (%d)", vectors);
     dim3 grid(rows, vectors);
     hipStream_t s = (hipStream_t)stream;
+    if (head_dim <= 64 && rows >= 8 * QK_ROWS) {    // a prompt's rows, eight to a wave
+        dim3 by_rows((rows + QK_ROWS - 1) / QK_ROWS, vectors);
+#define FW_QK_ROWS_LAUNCH(TI, T)                                                                                     \
+    qk_norm_rope_kv_write_rows_kernel<TI, T><<<by_rows, 64, 0, s>>>(                                                 \
+        (const TI*)qkv, (T*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim, (T*)k_pages, \
+        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, rows)
+        if (in_dtype == FW_F32 && dtype == FW_F32) FW_QK_ROWS_LAUNCH(float, float);
+        else if (in_dtype == FW_F32 && dtype == FW_BF16) FW_QK_ROWS_LAUNCH(float, bf16_t);
+        else if (in_dtype == FW_BF16 && dtype == FW_BF16) FW_QK_ROWS_LAUNCH(bf16_t, bf16_t);
+        else FW_REQUIRE(false, "qk_norm_rope: unsupported dtypes in=%d out=%d", in_dtype, dtype);
+#undef FW_QK_ROWS_LAUNCH
+        FW_LAUNCH_CHECK("qk_norm_rope_kv_write");
+        return 0;
+    }
 #define FW_QK_LAUNCH(TI, T)                                                                                          \
     qk_norm_rope_kv_write_kernel<TI, T><<<grid, 64, 0, s>>>(                                                         \
         (const TI*)qkv, (T*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim, (T*)k_pages, \
