@@ -55,8 +55,17 @@ __device__ __forceinline__ float from_neighbour(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
 }
 
+template <int TN>
+struct BigTile {
+    static constexpr int WIDE = 2 * TN * 32;               // columns of a tile
+    static constexpr int W_LOADS = WIDE / 64;              // wave-wide loads per wave for a slab of w (16 rows each)
+    static constexpr int SLAB_LOADS = B_LOADS + W_LOADS;   // and for a slab of both operands
+};
+
 // K must be a multiple of BK (the loads go straight to LDS: nothing can be zeroed on the way).
-template <int MODE, typename TO>
+// TN: 32-column product tiles per wave, 4 (a 256 x 256 tile) or 3 (256 x 192: a width of 6,144
+// features gives 192 tiles of 256 columns for 256 compute units, but exactly 256 tiles of 192).
+template <int MODE, typename TO, int TN>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mfma_big_kernel(
     const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, const float* __restrict__ bias,
     TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n, int per_xcd, int up_offset) {
@@ -70,7 +79,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int group_size = tiles_m - first_m < BGROUP_M ? tiles_m - first_m : BGROUP_M;
     const int pid_m = first_m + (logical % width) % group_size;
     const int pid_n = (logical % width) / group_size;
-    const int features = MODE == MB_SWIGLU ? BT / 2 : BT;
+    static_assert(TN == 4 || (TN == 3 && MODE != MB_SWIGLU), "three column tiles per wave: store and accumulate only");
+    constexpr int WIDE = BigTile<TN>::WIDE, W_LOADS = BigTile<TN>::W_LOADS, SLAB_LOADS = BigTile<TN>::SLAB_LOADS;
+    const int features = MODE == MB_SWIGLU ? BT / 2 : WIDE;
     const int m0 = pid_m * BT, n0 = pid_n * features;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -83,7 +94,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // otherwise share theirs). Lane l therefore ASKS for chunk (l % 4) ^ ((r / 4) % 4) of row
     // r = l / 4 of its 16 rows.
     const uint16_t* a_src[B_LOADS];
-    const uint16_t* w_src[B_LOADS];
+    const uint16_t* w_src[B_LOADS];     // W_LOADS of them are used (with w_src[W_LOADS] the host pass emitted no launch stub)
 #pragma unroll
     for (int i = 0; i < B_LOADS; ++i) {
         const int row = (wave * B_LOADS + i) * 16 + (lane >> 2);
@@ -91,6 +102,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         int am = m0 + row;
         am = am < M ? am : M - 1;                       // rows past the end are computed and dropped
         a_src[i] = a + (size_t)am * K + chunk * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+        const int row = (wave * W_LOADS + i) * 16 + (lane >> 2);
+        const int chunk = (lane & 3) ^ ((row >> 2) & 3);
         int wr;
         if (MODE == MB_SWIGLU) wr = row < BT / 2 ? n0 + row : up_offset + n0 + row - BT / 2;
         else wr = n0 + row;
@@ -99,31 +115,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         w_src[i] = w + (size_t)wr * K + chunk * 8;
     }
     auto request = [&](int slab) {
-        unsigned char* stage = lds + (slab % BSTAGES) * 2 * BSLAB + wave * B_LOADS * 1024;
+        unsigned char* stage = lds + (slab % BSTAGES) * 2 * BSLAB;
         const int k0 = slab * BK;
 #pragma unroll
         for (int i = 0; i < B_LOADS; ++i)
-            __builtin_amdgcn_global_load_lds(a_src[i] + k0, reinterpret_cast<uint32_t*>(stage + i * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(a_src[i] + k0, reinterpret_cast<uint32_t*>(stage + (wave * B_LOADS + i) * 1024), 16, 0, 0);
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i)
-            __builtin_amdgcn_global_load_lds(w_src[i] + k0, reinterpret_cast<uint32_t*>(stage + BSLAB + i * 1024), 16, 0, 0);
+        for (int i = 0; i < W_LOADS; ++i)
+            __builtin_amdgcn_global_load_lds(w_src[i] + k0, reinterpret_cast<uint32_t*>(stage + BSLAB + (wave * W_LOADS + i) * 1024), 16, 0, 0);
     };
 
-    f32x16 acc[4][4];
+    f32x16 acc[4][TN];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
     // this wave's rows of the a slab, and its rows of the w slab: for SwiGLU the columns of a wave
     // are 64 gate features (tiles 0, 1) and the 64 up features of the same columns (tiles 2, 3)
     const int a_row0 = wm * 128 + (lane & 31);
-    int b_row[4];
+    int b_row[TN];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-        b_row[j] = MODE == MB_SWIGLU ? (j >> 1) * (BT / 2) + wn * 64 + (j & 1) * 32 + (lane & 31) : wn * 128 + j * 32 + (lane & 31);
+    for (int j = 0; j < TN; ++j)
+        b_row[j] = MODE == MB_SWIGLU ? (j >> 1) * (BT / 2) + wn * 64 + (j & 1) * 32 + (lane & 31) : wn * (TN * 32) + j * 32 + (lane & 31);
     // every row this lane reads is (lane % 32) plus a multiple of 32: one permutation for all
     const int swizzle = ((lane & 31) >> 2) & 3;
     int slot[BK / 16];
@@ -132,7 +148,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
     // operand registers of one k16 step: four row tiles of a, four column tiles of w
     struct Operands {
-        bf16x8 fa[4], fb[4];
+        bf16x8 fa[4], fb[TN];
     };
     auto read = [&](Operands& f, int slab, int t) {
         const unsigned char* sa = lds + (slab % BSTAGES) * 2 * BSLAB;
@@ -141,14 +157,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         for (int i = 0; i < 4; ++i)
             f.fa[i] = *reinterpret_cast<const bf16x8*>(sa + (a_row0 + 32 * i) * (BK * 2) + slot[t]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
             f.fb[j] = *reinterpret_cast<const bf16x8*>(sb + b_row[j] * (BK * 2) + slot[t]);
     };
     auto multiply = [&](const Operands& f, int first_row_tile, int row_tiles) {
 #pragma unroll
         for (int i = first_row_tile; i < first_row_tile + row_tiles; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < TN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.fa[i], f.fb[j], acc[i][j], 0, 0, 0);
     };
     // Asks the scheduler to issue `count` times: `mfmas` MFMAs, then one instruction of `kind`
@@ -162,13 +178,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // Tells the compiler that these operands are needed HERE, so that it waits for their LDS reads
     // before the next reads are issued and not, for all reads together, in front of the MFMAs.
     auto arrived = [&](const Operands& f) {
-        asm volatile("" ::"v"(f.fa[0]), "v"(f.fa[1]), "v"(f.fa[2]), "v"(f.fa[3]), "v"(f.fb[0]), "v"(f.fb[1]), "v"(f.fb[2]), "v"(f.fb[3]));
+        asm volatile("" ::"v"(f.fa[0]), "v"(f.fa[1]), "v"(f.fa[2]), "v"(f.fa[3]), "v"(f.fb[0]), "v"(f.fb[1]), "v"(f.fb[2]), "v"(f.fb[TN - 1]));
     };
-    // waits until at most `slabs` of this wave's requested slabs are still on their way (8 loads each)
+    // waits until at most `slabs` of this wave's requested slabs are still on their way (SLAB_LOADS loads each)
     auto wait_for_all_but = [&](int slabs) {
-        if (slabs >= 3) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
-        else if (slabs == 2) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-        else if (slabs == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        if (slabs >= 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * SLAB_LOADS) : "memory");
+        else if (slabs == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SLAB_LOADS) : "memory");
+        else if (slabs == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(1 * SLAB_LOADS) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     };
 
@@ -192,20 +208,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         arrived(f0);
         read(f1, s, 1);
         multiply(f0, 0, 2);
-        FW_INTERLEAVE(8, 1, 0x100)
+        FW_INTERLEAVE(2 * TN, 1, 0x100)         // (with three column tiles one read of seven is left to the scheduler)
         __builtin_amdgcn_sched_barrier(0);
         arrived(f1);                                        // slab s has been read
-        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");   // slab s + 1 has landed; s + 2 and s + 3 may still fly
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SLAB_LOADS) : "memory");   // slab s + 1 has landed; s + 2 and s + 3 may still fly
         __builtin_amdgcn_s_barrier();
         // second half, with the requests for slab s + 4 between its MFMAs
         request(s + BSTAGES);
         multiply(f0, 2, 2);
-        FW_INTERLEAVE(8, 1, 0x020)
+        FW_INTERLEAVE(2 * TN, 1, 0x020)
         __builtin_amdgcn_sched_barrier(0);
         // step 1, with the reads of step 0 of slab s + 1 between its MFMAs
         read(f0, s + 1, 0);
         multiply(f1, 0, 4);
-        FW_INTERLEAVE(8, 2, 0x100)
+        FW_INTERLEAVE(2 * TN, 2, 0x100)
         __builtin_amdgcn_sched_barrier(0);
     }
     // the last slabs: nothing more to request
@@ -235,7 +251,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // With one workgroup per compute unit nothing runs beside the epilogue, so its length counts.
     const bool inside = m0 + BT <= M && n0 + features <= N && (sizeof(TO) == 4 || (N & 1) == 0);
     const bool odd = lane & 1;
-    if (MODE == MB_SWIGLU) {
+    if constexpr (MODE == MB_SWIGLU) {
         if (inside) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
@@ -274,8 +290,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
     if (inside) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int n = n0 + wn * 128 + j * 32 + col;
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + wn * (TN * 32) + j * 32 + col;
             const float b = bias ? bias[n] : 0.0f;
             if constexpr (sizeof(TO) == 4) {
                 float* column = reinterpret_cast<float*>(out) + (size_t)(m0 + wm * 128 + row_base) * N + n;
@@ -307,8 +323,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         return;
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int n = n0 + wn * 128 + j * 32 + col;
+    for (int j = 0; j < TN; ++j) {
+        const int n = n0 + wn * (TN * 32) + j * 32 + col;
         if (n >= N) continue;
         const float b = bias ? bias[n] : 0.0f;
 #pragma unroll
@@ -325,15 +341,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
 }
 
-template <int MODE, typename TO>
+template <int MODE, typename TO, int TN = 4>
 static int launch_big(const void* a, const void* w, const float* bias, void* out, int M, int N, int K, hipStream_t stream) {
-    const int features = MODE == MB_SWIGLU ? BT / 2 : BT;
+    const int features = MODE == MB_SWIGLU ? BT / 2 : 2 * TN * 32;
     const int tiles_m = fw_ceil_div(M, BT), tiles_n = fw_ceil_div(N, features);
     const int per_xcd = fw_ceil_div((long long)tiles_m * tiles_n, 8);
     const int lds_bytes = BSTAGES * 2 * BSLAB;
     static bool configured = false;     // per instantiation
     if (!configured) {
-        hipError_t status = hipFuncSetAttribute((const void*)gemm_mfma_big_kernel<MODE, TO>,
+        hipError_t status = hipFuncSetAttribute((const void*)gemm_mfma_big_kernel<MODE, TO, TN>,
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (status != hipSuccess) {
             fw_set_error("gemm_mfma_big: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(status));
@@ -341,9 +357,16 @@ static int launch_big(const void* a, const void* w, const float* bias, void* out
         }
         configured = true;
     }
-    gemm_mfma_big_kernel<MODE, TO><<<per_xcd * 8, 256, lds_bytes, stream>>>(
+    gemm_mfma_big_kernel<MODE, TO, TN><<<per_xcd * 8, 256, lds_bytes, stream>>>(
         (const uint16_t*)a, (const uint16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n, per_xcd, N);
     return 0;
+}
+
+// Whether tiles of 192 columns serve a storing or accumulating product better than tiles of 256:
+// rounds of tiles over the chip's 256 compute units, a narrow tile counting three quarters.
+static bool narrow_tiles_pay(int M, int N) {
+    const long long wide = (long long)fw_ceil_div(M, BT) * fw_ceil_div(N, BT), narrow = (long long)fw_ceil_div(M, BT) * fw_ceil_div(N, 192);
+    return 3 * fw_ceil_div(narrow, 256) < 4 * fw_ceil_div(wide, 256);
 }
 
 // How many 256 x 256 tiles a shape gives (the caller decides whether that fills the chip); 0 if
@@ -365,10 +388,14 @@ extern "C" int fw_gemm_mfma_big(const void* a, const void* w, const float* bias,
     FW_REQUIRE((long long)fw_ceil_div(M, BT) * fw_ceil_div(N, BT / 2) < (1ll << 30), "gemm_mfma_big: too many tiles");
     hipStream_t s = (hipStream_t)stream;
     int status;
+    const bool narrow = mode != MB_SWIGLU && narrow_tiles_pay(M, N);
     if (mode == MB_SWIGLU) status = launch_big<MB_SWIGLU, bf16_t>(a, w, nullptr, out, M, N, K, s);
-    else if (mode == MB_ACCUMULATE) status = launch_big<MB_ACCUMULATE, float>(a, w, bias, out, M, N, K, s);
-    else if (out_dtype == FW_F32) status = launch_big<MB_STORE, float>(a, w, bias, out, M, N, K, s);
-    else status = launch_big<MB_STORE, bf16_t>(a, w, bias, out, M, N, K, s);
+    else if (mode == MB_ACCUMULATE) status = narrow ? launch_big<MB_ACCUMULATE, float, 3>(a, w, bias, out, M, N, K, s)
+                                                    : launch_big<MB_ACCUMULATE, float>(a, w, bias, out, M, N, K, s);
+    else if (out_dtype == FW_F32) status = narrow ? launch_big<MB_STORE, float, 3>(a, w, bias, out, M, N, K, s)
+                                                  : launch_big<MB_STORE, float>(a, w, bias, out, M, N, K, s);
+    else status = narrow ? launch_big<MB_STORE, bf16_t, 3>(a, w, bias, out, M, N, K, s)
+                         : launch_big<MB_STORE, bf16_t>(a, w, bias, out, M, N, K, s);
     if (status != 0) return status;
     FW_LAUNCH_CHECK("gemm_mfma_big");
     return 0;

@@ -357,10 +357,12 @@ def test_fast_gemm_every_epilogue(ops, M, N, K):
         close(ops.gemm_swiglu(a, w), act, torch.bfloat16, 0.4)
 
 
-@pytest.mark.parametrize("M,N,K", [(2048, 6144, 96), (1500, 8200, 160), (4000, 3100, 64)])
+@pytest.mark.parametrize("M,N,K", [(2048, 6144, 96), (1500, 8200, 160), (4000, 3100, 64), (1800, 6000, 2080)])
 def test_large_tile_prompt_product(ops, M, N, K):
     """Shapes with at least 192 tiles of 256 x 256 go to the large-tile kernel: every epilogue,
-    edges in both directions, few and many slabs."""
+    edges in both directions, few and many slabs. The first and the last shape give exactly one
+    round of tiles over the chip with tiles of 192 columns, which storing and accumulating
+    products then take; the gated product keeps the 256 x 256 tiles."""
     assert ops.library().fw_gemm_mfma_big_tiles(0, M, N, K) >= ops.BIG_TILES_MIN and not ops.library().fw_gemm_mfma_big_tiles(0, M, N, K + 8)
     a = as_dev(gen(M, K), torch.bfloat16)
     w = as_dev(gen(N, K, seed=1, scale=K ** -0.5), torch.bfloat16)
