@@ -196,6 +196,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // D layout of the 32x32 product: lane holds column lane % 32; register r is row
     // 8 * (r / 4) + 4 * (lane / 32) + r % 4
     const int col = lane & 31, row_base = (lane >> 5) * 4;
+    // the accumulating epilogue's old values of the four product tiles this wave will finish are
+    // asked for now: they travel while the parts are exchanged
+    float old_value[2][2][16];
+    if (MODE == MD_ACCUMULATE) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int tile = wave * 2 + u, i = half * 2 + (tile >> 2), j = tile & 3;
+                const int n = n0 + j * 32 + col;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + i * 32 + 8 * (r >> 2) + row_base + (r & 3);
+                    old_value[half][u][r] = load_as_float(out, (m < M && n < N) ? (size_t)m * N + n : 0);
+                }
+            }
+    }
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
         __syncthreads();        // the operands (first half) or the parts of the first half have been read
@@ -228,7 +245,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     if (m >= M || n >= N) continue;
                     const size_t at = (size_t)m * N + n;
                     float value = sum[e] + b;
-                    if (MODE == MD_ACCUMULATE) value += load_as_float(out, at);
+                    if (MODE == MD_ACCUMULATE) value += old_value[half][u][4 * q + e];
                     store_from_float(out, at, value);
                 }
             }

@@ -318,8 +318,8 @@ def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out
         entry = library().fw_gemm_skinny
     elif M > BIG_MIN_ROWS and library().fw_gemm_mfma_big_tiles(mode, M, N, K) >= BIG_TILES_MIN:
         entry = library().fw_gemm_mfma_big      # enough 256 x 256 tiles to fill the chip
-    elif K >= DEEP_MIN_K and DEEP_TILES_MIN <= library().fw_gemm_mfma_deep_tiles(mode, M, N, K) <= DEEP_TILES_MAX:
-        entry = library().fw_gemm_mfma_deep     # one 128 x 128 tile per compute unit over a long K: the waves split K
+    elif K >= (DEEP_MIN_K if mode == 1 else DEEP_MIN_K_STORE) and _fills_rounds(library().fw_gemm_mfma_deep_tiles(mode, M, N, K)):
+        entry = library().fw_gemm_mfma_deep     # whole rounds of one 128 x 128 tile per compute unit: the waves split K
     else:
         need_bytes, need_counters = ctypes.c_size_t(0), ctypes.c_int(0)
         _check(library().fw_gemm_mfma_split_plan(mode, M, N, K, ctypes.byref(need_bytes), ctypes.byref(need_counters)))
@@ -336,8 +336,17 @@ def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out
 SKINNY_MAX_ROWS = 16
 MEDIUM_MAX_ROWS = 64
 BIG_TILES_MIN = 192      # 256 x 256 tiles from which the large-tile prompt product is used (256 compute units)
-DEEP_MIN_K = 4096         # below, the exchange between the waves at the end of a tile costs more than the main loop gains
-DEEP_TILES_MIN, DEEP_TILES_MAX = 200, 256   # one round of tiles over 256 compute units (2,048 x 2,048 x 8,192: 99 vs 124 us)
+DEEP_MIN_K = 2048         # adding into the residual (2,048 x 2,048 x 2,048: 31 vs 39 us; x 8,192: 87 vs 124 us)
+DEEP_MIN_K_STORE = 4096   # storing: no old values travel during the exchange at a tile's end, a short K gains nothing
+DEEP_ROUND = 256          # tiles of a round: one per compute unit
+DEEP_FILL = 0.78          # least share of the rounds' places that the tiles must fill (320 tiles, 0.63: 198 vs 191 us)
+
+
+def _fills_rounds(tiles: int) -> bool:
+    rounds = -(-tiles // DEEP_ROUND)
+    return tiles > 0 and tiles >= DEEP_FILL * rounds * DEEP_ROUND
+
+
 BIG_MIN_ROWS = 128       # up to here a 256-row tile would be at least half empty (the head at 128 rows: 110 vs 78 us)
 _MEDIUM_COUNTERS = {}
 
