@@ -43,12 +43,13 @@ int fw_gemm_mfma(const void* a, const void* w, const float* bias, void* out, int
 int fw_gemm_mfma_big(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                      int M, int N, int K, void* stream);
 int fw_gemm_mfma_big_tiles(int mode, int M, int N, int K);     // 0: the kernel does not take the shape
-// The prompt product with 128 x 128 tiles whose four waves split K (half the LDS traffic per flop
-// of fw_gemm_mfma's tiles), for outputs too narrow for the 256 x 256 tiles to fill the chip.
-// Modes 0 and 1; K a multiple of 64 (fw_gemm_mfma_deep_tiles says 0 for shapes it does not take).
+// The prompt product with tiles of 128 rows and `columns` (128 or 64) columns whose four waves split
+// K (half the LDS traffic per flop of fw_gemm_mfma's tiles), for outputs too narrow for the
+// 256 x 256 tiles to fill the chip. Modes 0 and 1; K a multiple of 64 (fw_gemm_mfma_deep_tiles says
+// 0 for shapes it does not take, else the number of tiles).
 int fw_gemm_mfma_deep(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
-                      int M, int N, int K, void* stream);
-int fw_gemm_mfma_deep_tiles(int mode, int M, int N, int K);
+                      int M, int N, int K, int columns, void* stream);
+int fw_gemm_mfma_deep_tiles(int mode, int M, int N, int K, int columns);
 // fw_gemm_mfma with K cut into slices for products with fewer tiles than compute units (a few
 // hundred rows, a narrow output). fw_gemm_mfma_split_plan says what a shape needs: bytes of
 // workspace and int32 counters that are zero before the first call and are left zero (both 0: the

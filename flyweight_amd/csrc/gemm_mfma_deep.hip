@@ -39,7 +39,10 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 enum { MD_STORE = 0, MD_ACCUMULATE = 1 };
 
-template <int MODE, typename TO>
+// TN: 32-column product tiles of a tile, 4 (128 x 128) or 2 (128 x 64: an output of 1,024 features
+// gives 128 tiles of 128 columns for 256 compute units, but 256 of 64; six operand reads for eight
+// MFMAs then).
+template <int MODE, typename TO, int TN>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mfma_deep_kernel(
     const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, const float* __restrict__ bias,
     TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n, int per_xcd) {
@@ -53,7 +56,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int group_size = tiles_m - first_m < DGROUP_M ? tiles_m - first_m : DGROUP_M;
     const int pid_m = first_m + (logical % width) % group_size;
     const int pid_n = (logical % width) / group_size;
-    const int m0 = pid_m * DT, n0 = pid_n * DT;
+    static_assert(TN == 4 || TN == 2, "128 or 64 columns");
+    constexpr int W_LOADS = TN;             // wave-wide loads per wave for a slab of w: 32 * TN rows, 8 rows a load, 4 waves
+    constexpr int SLAB_LOADS = D_LOADS + W_LOADS;
+    const int m0 = pid_m * DT, n0 = pid_n * (32 * TN);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
@@ -61,7 +67,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // l * 16: 8 rows of 128 bytes. Lane l asks for chunk (l % 8) ^ ((r / 2) % 8) of row r = l / 8 of
     // its 8 rows (rows past the end of a or w are read from the last row and never stored).
     const uint16_t* a_src[D_LOADS];
-    const uint16_t* w_src[D_LOADS];
+    const uint16_t* w_src[D_LOADS];         // W_LOADS of them are used
 #pragma unroll
     for (int i = 0; i < D_LOADS; ++i) {
         const int row = (wave * D_LOADS + i) * 8 + (lane >> 3);
@@ -69,26 +75,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         int am = m0 + row;
         am = am < M ? am : M - 1;
         a_src[i] = a + (size_t)am * K + chunk * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+        const int row = (wave * W_LOADS + i) * 8 + (lane >> 3);
+        const int chunk = (lane & 7) ^ ((row >> 1) & 7);
         int wr = n0 + row;
         wr = wr < N ? wr : N - 1;
         w_src[i] = w + (size_t)wr * K + chunk * 8;
     }
     auto request = [&](int slab) {
-        unsigned char* stage = lds + (slab % DSTAGES) * 2 * DSLAB + wave * D_LOADS * 1024;
+        unsigned char* stage = lds + (slab % DSTAGES) * 2 * DSLAB;
         const int k0 = slab * DK;
 #pragma unroll
         for (int i = 0; i < D_LOADS; ++i)
-            __builtin_amdgcn_global_load_lds(a_src[i] + k0, reinterpret_cast<uint32_t*>(stage + i * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(a_src[i] + k0, reinterpret_cast<uint32_t*>(stage + (wave * D_LOADS + i) * 1024), 16, 0, 0);
 #pragma unroll
-        for (int i = 0; i < D_LOADS; ++i)
-            __builtin_amdgcn_global_load_lds(w_src[i] + k0, reinterpret_cast<uint32_t*>(stage + DSLAB + i * 1024), 16, 0, 0);
+        for (int i = 0; i < W_LOADS; ++i)
+            __builtin_amdgcn_global_load_lds(w_src[i] + k0, reinterpret_cast<uint32_t*>(stage + DSLAB + (wave * W_LOADS + i) * 1024), 16, 0, 0);
     };
 
-    f32x16 acc[4][4];
+    f32x16 acc[4][TN];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
@@ -98,7 +109,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int slot = ((2 * wave + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
     const int row_offset = (lane & 31) * (DK * 2) + slot;
     struct Operands {
-        bf16x8 fa[4], fb[4];
+        bf16x8 fa[4], fb[TN];
     };
     auto read = [&](Operands& f, int slab) {
         const unsigned char* sa = lds + (slab % DSTAGES) * 2 * DSLAB + row_offset;
@@ -106,13 +117,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
         for (int i = 0; i < 4; ++i) f.fa[i] = *reinterpret_cast<const bf16x8*>(sa + 32 * i * (DK * 2));
 #pragma unroll
-        for (int j = 0; j < 4; ++j) f.fb[j] = *reinterpret_cast<const bf16x8*>(sb + 32 * j * (DK * 2));
+        for (int j = 0; j < TN; ++j) f.fb[j] = *reinterpret_cast<const bf16x8*>(sb + 32 * j * (DK * 2));
     };
     auto multiply = [&](const Operands& f) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < TN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.fa[i], f.fb[j], acc[i][j], 0, 0, 0);
     };
     // Asks the scheduler to issue `count` times: `mfmas` MFMAs, then one instruction of `kind`
@@ -123,13 +134,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         __builtin_amdgcn_sched_group_barrier((kind), 1, 0);        \
     }
     auto arrived = [&](const Operands& f) {
-        asm volatile("" ::"v"(f.fa[0]), "v"(f.fa[1]), "v"(f.fa[2]), "v"(f.fa[3]), "v"(f.fb[0]), "v"(f.fb[1]), "v"(f.fb[2]), "v"(f.fb[3]));
+        asm volatile("" ::"v"(f.fa[0]), "v"(f.fa[1]), "v"(f.fa[2]), "v"(f.fa[3]), "v"(f.fb[0]), "v"(f.fb[1]), "v"(f.fb[TN - 2]), "v"(f.fb[TN - 1]));
     };
-    // waits until at most `slabs` of this wave's requested slabs are still on their way (8 loads each)
+    // waits until at most `slabs` of this wave's requested slabs are still on their way (SLAB_LOADS loads each)
     auto wait_for_all_but = [&](int slabs) {
-        if (slabs >= 3) asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
-        else if (slabs == 2) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-        else if (slabs == 1) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        if (slabs >= 3) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(3 * SLAB_LOADS) : "memory");
+        else if (slabs == 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SLAB_LOADS) : "memory");
+        else if (slabs == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(1 * SLAB_LOADS) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     };
 
@@ -148,22 +159,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // steady state, two slabs per turn so that the operand sets keep their names
     for (; s + DSTAGES + 1 < steps; s += 2) {
         arrived(f0);                                        // slab s has been read
-        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");   // slab s + 1 has landed; s + 2 and s + 3 may still fly
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SLAB_LOADS) : "memory");   // slab s + 1 has landed; s + 2 and s + 3 may still fly
         __builtin_amdgcn_s_barrier();
         read(f1, s + 1);
         request(s + DSTAGES);
         multiply(f0);
-        FW_INTERLEAVE(8, 1, 0x100)
-        FW_INTERLEAVE(8, 1, 0x020)
+        FW_INTERLEAVE(2 * TN, 1, 0x100)     // (with two column tiles: eight MFMAs for six reads and six loads,
+        FW_INTERLEAVE(2 * TN, 1, 0x020)     //  four of each placed here, the rest left to the scheduler)
         __builtin_amdgcn_sched_barrier(0);
         arrived(f1);
-        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SLAB_LOADS) : "memory");
         __builtin_amdgcn_s_barrier();
         read(f0, s + 2);
         request(s + 1 + DSTAGES);
         multiply(f1);
-        FW_INTERLEAVE(8, 1, 0x100)
-        FW_INTERLEAVE(8, 1, 0x020)
+        FW_INTERLEAVE(2 * TN, 1, 0x100)     // (with two column tiles: eight MFMAs for six reads and six loads,
+        FW_INTERLEAVE(2 * TN, 1, 0x020)     //  four of each placed here, the rest left to the scheduler)
         __builtin_amdgcn_sched_barrier(0);
     }
     // the last slabs: one at a time, asking for what is left to ask for
@@ -187,50 +198,53 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #undef FW_INTERLEAVE
     fw_mfma_drain();     // branches follow that lead to code reading the accumulators
 
-    // The four partial tiles meet in LDS (free now: 128 KB), the upper eight product tiles (row
-    // tiles 0 and 1) first, then the lower eight: every wave leaves its parts of the eight (4 KB
-    // each), then finishes two of them: the four parts added in the order of the waves, whatever
-    // the timing, and sent through the epilogue. Which accumulators a wave reads does not depend
-    // on the wave (only where it reads the parts from does), so they stay where they are.
-    f32x4* exchange = reinterpret_cast<f32x4*>(lds);       // [wave][tile of the half][four rows][lane]
+    // The four partial tiles meet in LDS (free now: 128 KB), eight product tiles at a time (with
+    // four column tiles: row tiles 0 and 1, then 2 and 3; with two: all at once): every wave leaves
+    // its parts of the eight (4 KB each), then finishes two of them: the four parts added in the
+    // order of the waves, whatever the timing, and sent through the epilogue. Which accumulators a
+    // wave reads does not depend on the wave (only where it reads the parts from does), so they
+    // stay where they are.
+    constexpr int PASSES = TN / 2, PASS_ROWS = 8 / TN;     // passes of eight product tiles; row tiles in a pass
+    f32x4* exchange = reinterpret_cast<f32x4*>(lds);       // [wave][tile of the pass][four rows][lane]
     // D layout of the 32x32 product: lane holds column lane % 32; register r is row
     // 8 * (r / 4) + 4 * (lane / 32) + r % 4
     const int col = lane & 31, row_base = (lane >> 5) * 4;
-    // the accumulating epilogue's old values of the four product tiles this wave will finish are
-    // asked for now: they travel while the parts are exchanged
-    float old_value[2][2][16];
+    // the accumulating epilogue's old values of the product tiles this wave will finish are asked
+    // for now: they travel while the parts are exchanged (with one workgroup per compute unit
+    // nothing else would hide that read)
+    float old_value[PASSES][2][16];
     if (MODE == MD_ACCUMULATE) {
 #pragma unroll
-        for (int half = 0; half < 2; ++half)
+        for (int pass = 0; pass < PASSES; ++pass)
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
-                const int tile = wave * 2 + u, i = half * 2 + (tile >> 2), j = tile & 3;
+                const int tile = wave * 2 + u, i = pass * PASS_ROWS + tile / TN, j = tile % TN;
                 const int n = n0 + j * 32 + col;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int m = m0 + i * 32 + 8 * (r >> 2) + row_base + (r & 3);
-                    old_value[half][u][r] = load_as_float(out, (m < M && n < N) ? (size_t)m * N + n : 0);
+                    old_value[pass][u][r] = load_as_float(out, (m < M && n < N) ? (size_t)m * N + n : 0);
                 }
             }
     }
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-        __syncthreads();        // the operands (first half) or the parts of the first half have been read
+    for (int pass = 0; pass < PASSES; ++pass) {
+        __syncthreads();        // the operands (first pass) or the parts of the pass before have been read
 #pragma unroll
-        for (int i2 = 0; i2 < 2; ++i2)
+        for (int i2 = 0; i2 < PASS_ROWS; ++i2)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                f32x4* to = exchange + (size_t)((wave * 8 + i2 * 4 + j) * 4) * 64 + lane;
+            for (int j = 0; j < TN; ++j) {
+                f32x4* to = exchange + (size_t)((wave * 8 + i2 * TN + j) * 4) * 64 + lane;
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const f32x16& t = acc[half * 2 + i2][j];
+                    const f32x16& t = acc[pass * PASS_ROWS + i2][j];
                     to[q * 64] = f32x4{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
                 }
             }
         __syncthreads();
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const int tile = wave * 2 + u, i = half * 2 + (tile >> 2), j = tile & 3;
+            const int tile = wave * 2 + u, i = pass * PASS_ROWS + tile / TN, j = tile % TN;
             const int n = n0 + j * 32 + col;
             const float b = (bias && n < N) ? bias[n] : 0.0f;
             const f32x4* from = exchange + (size_t)(tile * 4) * 64 + lane;
@@ -245,7 +259,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                     if (m >= M || n >= N) continue;
                     const size_t at = (size_t)m * N + n;
                     float value = sum[e] + b;
-                    if (MODE == MD_ACCUMULATE) value += old_value[half][u][4 * q + e];
+                    if (MODE == MD_ACCUMULATE) value += old_value[pass][u][4 * q + e];
                     store_from_float(out, at, value);
                 }
             }
@@ -253,14 +267,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
 }
 
-template <int MODE, typename TO>
+template <int MODE, typename TO, int TN>
 static int launch_deep(const void* a, const void* w, const float* bias, void* out, int M, int N, int K, hipStream_t stream) {
-    const int tiles_m = fw_ceil_div(M, DT), tiles_n = fw_ceil_div(N, DT);
+    const int tiles_m = fw_ceil_div(M, DT), tiles_n = fw_ceil_div(N, 32 * TN);
     const int per_xcd = fw_ceil_div((long long)tiles_m * tiles_n, 8);
     const int lds_bytes = DSTAGES * 2 * DSLAB;
     static bool configured = false;     // per instantiation
     if (!configured) {
-        hipError_t status = hipFuncSetAttribute((const void*)gemm_mfma_deep_kernel<MODE, TO>,
+        hipError_t status = hipFuncSetAttribute((const void*)gemm_mfma_deep_kernel<MODE, TO, TN>,
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (status != hipSuccess) {
             fw_set_error("gemm_mfma_deep: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(status));
@@ -268,32 +282,39 @@ static int launch_deep(const void* a, const void* w, const float* bias, void* ou
         }
         configured = true;
     }
-    gemm_mfma_deep_kernel<MODE, TO><<<per_xcd * 8, 256, lds_bytes, stream>>>(
+    gemm_mfma_deep_kernel<MODE, TO, TN><<<per_xcd * 8, 256, lds_bytes, stream>>>(
         (const uint16_t*)a, (const uint16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n, per_xcd);
     return 0;
 }
 
-// How many 128 x 128 tiles a shape gives; 0 if the kernel does not take the shape (K must be a
-// multiple of 64; SwiGLU is not served).
-extern "C" int fw_gemm_mfma_deep_tiles(int mode, int M, int N, int K) {
-    if (K <= 0 || K % DK || mode < 0 || mode > 1) return 0;
-    return fw_ceil_div(M, DT) * fw_ceil_div(N, DT);
+// How many tiles a shape gives with tiles of `columns` (128 or 64) columns; 0 if the kernel does
+// not take the shape (K must be a multiple of 64; SwiGLU is not served).
+extern "C" int fw_gemm_mfma_deep_tiles(int mode, int M, int N, int K, int columns) {
+    if (K <= 0 || K % DK || mode < 0 || mode > 1 || (columns != 128 && columns != 64)) return 0;
+    return fw_ceil_div(M, DT) * fw_ceil_div(N, columns);
 }
 
-// fw_gemm_mfma's contract for modes 0 and 1.
+// fw_gemm_mfma's contract for modes 0 and 1, on tiles of 128 rows and `columns` (128 or 64) columns.
 extern "C" int fw_gemm_mfma_deep(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
-                                 int M, int N, int K, void* stream) {
+                                 int M, int N, int K, int columns, void* stream) {
     FW_REQUIRE(M >= 1 && N > 0 && K > 0 && K % DK == 0, "gemm_mfma_deep: K (%d) must be a positive multiple of %d; M=%d N=%d", K, DK, M, N);
     FW_REQUIRE(mode == MD_STORE || mode == MD_ACCUMULATE, "gemm_mfma_deep: mode %d is not served", mode);
+    FW_REQUIRE(columns == 128 || columns == 64, "gemm_mfma_deep: tiles have 128 or 64 columns, not %d", columns);
     FW_REQUIRE(mode != MD_ACCUMULATE || out_dtype == FW_F32, "gemm_mfma_deep: accumulation needs a float32 destination");
     FW_REQUIRE(out_dtype == FW_F32 || out_dtype == FW_BF16, "gemm_mfma_deep: unknown out dtype %d", out_dtype);
     FW_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_mfma_deep: operands must be 16-byte aligned");
-    FW_REQUIRE((long long)fw_ceil_div(M, DT) * fw_ceil_div(N, DT) < (1ll << 30), "gemm_mfma_deep: too many tiles");
+    FW_REQUIRE((long long)fw_ceil_div(M, DT) * fw_ceil_div(N, 64) < (1ll << 30), "gemm_mfma_deep: too many tiles");
     hipStream_t s = (hipStream_t)stream;
     int status;
-    if (mode == MD_ACCUMULATE) status = launch_deep<MD_ACCUMULATE, float>(a, w, bias, out, M, N, K, s);
-    else if (out_dtype == FW_F32) status = launch_deep<MD_STORE, float>(a, w, bias, out, M, N, K, s);
-    else status = launch_deep<MD_STORE, bf16_t>(a, w, bias, out, M, N, K, s);
+    if (columns == 128) {
+        if (mode == MD_ACCUMULATE) status = launch_deep<MD_ACCUMULATE, float, 4>(a, w, bias, out, M, N, K, s);
+        else if (out_dtype == FW_F32) status = launch_deep<MD_STORE, float, 4>(a, w, bias, out, M, N, K, s);
+        else status = launch_deep<MD_STORE, bf16_t, 4>(a, w, bias, out, M, N, K, s);
+    } else {
+        if (mode == MD_ACCUMULATE) status = launch_deep<MD_ACCUMULATE, float, 2>(a, w, bias, out, M, N, K, s);
+        else if (out_dtype == FW_F32) status = launch_deep<MD_STORE, float, 2>(a, w, bias, out, M, N, K, s);
+        else status = launch_deep<MD_STORE, bf16_t, 2>(a, w, bias, out, M, N, K, s);
+    }
     if (status != 0) return status;
     FW_LAUNCH_CHECK("gemm_mfma_deep");
     return 0;

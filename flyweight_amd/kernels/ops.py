@@ -318,8 +318,11 @@ def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out
         entry = library().fw_gemm_skinny
     elif M > BIG_MIN_ROWS and library().fw_gemm_mfma_big_tiles(mode, M, N, K) >= BIG_TILES_MIN:
         entry = library().fw_gemm_mfma_big      # enough 256 x 256 tiles to fill the chip
-    elif K >= (DEEP_MIN_K if mode == 1 else DEEP_MIN_K_STORE) and _fills_rounds(library().fw_gemm_mfma_deep_tiles(mode, M, N, K)):
-        entry = library().fw_gemm_mfma_deep     # whole rounds of one 128 x 128 tile per compute unit: the waves split K
+    elif K >= (DEEP_MIN_K if mode == 1 else DEEP_MIN_K_STORE) and _deep_columns(mode, M, N, K):
+        # whole rounds of one tile per compute unit: the waves split K
+        _check(library().fw_gemm_mfma_deep(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K,
+                                           _deep_columns(mode, M, N, K), _stream()))
+        return
     else:
         need_bytes, need_counters = ctypes.c_size_t(0), ctypes.c_int(0)
         _check(library().fw_gemm_mfma_split_plan(mode, M, N, K, ctypes.byref(need_bytes), ctypes.byref(need_counters)))
@@ -336,15 +339,24 @@ def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out
 SKINNY_MAX_ROWS = 16
 MEDIUM_MAX_ROWS = 64
 BIG_TILES_MIN = 192      # 256 x 256 tiles from which the large-tile prompt product is used (256 compute units)
-DEEP_MIN_K = 2048         # adding into the residual (2,048 x 2,048 x 2,048: 31 vs 39 us; x 8,192: 87 vs 124 us)
+DEEP_MIN_K = 1024         # adding into the residual (2,048 x 2,048 x 2,048: 31 vs 39 us; x 8,192: 83 vs 118 us; 2,048 x 1,024 x 1,024: 13 vs 15 us)
 DEEP_MIN_K_STORE = 4096   # storing: no old values travel during the exchange at a tile's end, a short K gains nothing
 DEEP_ROUND = 256          # tiles of a round: one per compute unit
-DEEP_FILL = 0.78          # least share of the rounds' places that the tiles must fill (320 tiles, 0.63: 198 vs 191 us)
+DEEP_FILL = 0.85          # least share of the rounds' places that the tiles must fill (640 narrow tiles, 0.83: 193 vs 189 us)
 
 
 def _fills_rounds(tiles: int) -> bool:
     rounds = -(-tiles // DEEP_ROUND)
     return tiles > 0 and tiles >= DEEP_FILL * rounds * DEEP_ROUND
+
+
+def _deep_columns(mode: int, M: int, N: int, K: int) -> int:
+    """The width of the tiles whose waves split K that serves this shape: 128 columns if they fill
+    whole rounds over the chip, else 64 if those do (an output of 1,024 features), else 0."""
+    for columns in (128, 64):
+        if _fills_rounds(library().fw_gemm_mfma_deep_tiles(mode, M, N, K, columns)):
+            return columns
+    return 0
 
 
 BIG_MIN_ROWS = 128       # up to here a 256-row tile would be at least half empty (the head at 128 rows: 110 vs 78 us)
@@ -436,7 +448,8 @@ def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
 
 
 def gemm_deep(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
-              out_dtype: Optional[torch.dtype] = None, accumulate_into: Optional[torch.Tensor] = None) -> torch.Tensor:
+              out_dtype: Optional[torch.dtype] = None, accumulate_into: Optional[torch.Tensor] = None,
+              columns: int = 128) -> torch.Tensor:
     """a [M, K] . w [N, K]^T (+ bias) on 128 x 128 tiles whose waves split K (fw_gemm_mfma_deep),
     whatever the dispatch of ``gemm`` would choose: bfloat16 operands, K a multiple of 64."""
     _dev(a, w, bias, accumulate_into)
@@ -453,7 +466,7 @@ def gemm_deep(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = N
         target, mode = accumulate_into, 1
     else:
         target, mode = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device), 0
-    _check(library().fw_gemm_mfma_deep(_p(a), _p(w), _p(bias), _p(target), _code(target.dtype), mode, M, N, K, _stream()))
+    _check(library().fw_gemm_mfma_deep(_p(a), _p(w), _p(bias), _p(target), _code(target.dtype), mode, M, N, K, int(columns), _stream()))
     return target
 
 

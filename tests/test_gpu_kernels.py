@@ -408,8 +408,9 @@ def test_tiled_product_cuts_k_into_slices(ops, M, N, K):
         close(ops.gemm_swiglu(a, w), F.silu(want[:, :half]) * want[:, half:], torch.bfloat16, 0.4)
 
 
+@pytest.mark.parametrize("columns", [128, 64])
 @pytest.mark.parametrize("M,N,K", [(1, 1, 64), (128, 128, 64), (130, 70, 192), (300, 200, 448), (129, 257, 2112), (1000, 520, 8192)])
-def test_tiles_whose_waves_split_k(ops, M, N, K):
+def test_tiles_whose_waves_split_k(ops, M, N, K, columns):
     """128 x 128 tiles of which every wave multiplies a quarter of each slab of K and the four
     partial tiles meet in LDS: one slab, fewer slabs than stages, many; edges in rows and
     features; store (float32, bfloat16) and accumulate; bitwise the same every time."""
@@ -417,23 +418,24 @@ def test_tiles_whose_waves_split_k(ops, M, N, K):
     w = as_dev(gen(N, K, seed=1, scale=K ** -0.5), torch.bfloat16)
     bias = gen(N, seed=2).float().to(DEV)
     want = back(a) @ back(w).T
-    first = ops.gemm_deep(a, w, bias, out_dtype=torch.float32)
+    first = ops.gemm_deep(a, w, bias, out_dtype=torch.float32, columns=columns)
     close(first, want + bias.cpu().double(), torch.float32, 2.0)
-    assert torch.equal(ops.gemm_deep(a, w, bias, out_dtype=torch.float32), first)
-    close(ops.gemm_deep(a, w), want, torch.bfloat16, 0.4)
+    assert torch.equal(ops.gemm_deep(a, w, bias, out_dtype=torch.float32, columns=columns), first)
+    close(ops.gemm_deep(a, w, columns=columns), want, torch.bfloat16, 0.4)
     residual = gen(M, N, seed=3).float().to(DEV)
     before = residual.cpu().double()
-    ops.gemm_deep(a, w, accumulate_into=residual)
+    ops.gemm_deep(a, w, accumulate_into=residual, columns=columns)
     close(residual, before + want, torch.float32, 2.0)
     with pytest.raises(ops.KernelError, match="multiple of 64"):
         ops.gemm_deep(a[:, :K - 8].contiguous(), w[:, :K - 8].contiguous())
 
 
-@pytest.mark.parametrize("M,N,K", [(2048, 2048, 4096), (1800, 1990, 4160)])
+@pytest.mark.parametrize("M,N,K", [(2048, 2048, 4096), (1800, 1990, 4160), (2048, 1024, 2048)])
 def test_the_prompt_product_of_one_round_of_tiles_over_a_long_k(ops, M, N, K):
     """What the dispatch sends to those tiles: about one 128 x 128 tile per compute unit and a
     long K (the w2 product of a 2,048-token prompt)."""
-    assert ops._fills_rounds(ops.library().fw_gemm_mfma_deep_tiles(1, M, N, K)) and K >= ops.DEEP_MIN_K
+    columns = ops._deep_columns(1, M, N, K)
+    assert columns == (64 if N == 1024 else 128) and K >= ops.DEEP_MIN_K
     a = as_dev(gen(M, K), torch.bfloat16)
     w = as_dev(gen(N, K, seed=1, scale=K ** -0.5), torch.bfloat16)
     want = back(a) @ back(w).T
@@ -442,7 +444,7 @@ def test_the_prompt_product_of_one_round_of_tiles_over_a_long_k(ops, M, N, K):
     ops.gemm(a, w, accumulate_into=residual)
     close(residual, before + want, torch.float32, 2.0)
     direct = before.float().to(DEV)
-    ops.gemm_deep(a, w, accumulate_into=direct)
+    ops.gemm_deep(a, w, accumulate_into=direct, columns=columns)
     assert torch.equal(direct, residual)
     close(ops.gemm(a, w, out_dtype=torch.float32), want, torch.float32, 2.0)
 
