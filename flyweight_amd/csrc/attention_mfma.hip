@@ -246,8 +246,13 @@ __device__ __forceinline__ void load_query(Columns<HD>& c, const uint16_t* __res
 // softmax arithmetic. tile_seg / tile_row0: the segment of each tile and its first row (a tile never
 // spans two segments). LDS rows are padded by 16 bytes against bank conflicts.
 #define KV_PAD 8
+// Where the kernel needs no more than 256 registers a wave it says so (two waves per SIMD at
+// least): the compiler then keeps the MFMA results in ordinary registers. Left with all 512 it puts
+// them into the accumulation registers, and the softmax's rescaling of the output and the masks on
+// the scores then cost a move out and a move back per value and page (112 + 80 of the ~560 vector
+// instructions of two pages).
 template <int HD, int NH>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 && NH == 1) ? 2 : 1))) void attention_prefill_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ tile_seg, const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ seg_row0,
@@ -399,7 +404,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(
 // no ticket. The last workgroup of a (row, kv head, head tile) to arrive merges what the others
 // left; the only workgroup of a short row writes the result at once.
 template <int HD>
-__global__ __launch_bounds__(64 * SPLIT_PAGES) void attention_decode_split_kernel(
+__global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_eu(HD <= 128 ? 2 : 1))) void attention_decode_split_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* partial, int* tickets,
     const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
