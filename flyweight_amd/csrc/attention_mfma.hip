@@ -151,7 +151,13 @@ __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t
         // A column without any key so far (maximum NEG_BIG) subtracts nothing, so that the same holds.
         shift[h] = new_max > 0.5f * NEG_BIG ? -new_max : 0.0f;
     }
-    if (__any(rose)) {          // the maximum of some column rose (seldom after the first pages)
+    // One head of up to 64 channels whose output lies in ordinary registers: rescaling it always
+    // (sixteen multiplications by a factor that is 1 after the first pages) costs less than the
+    // register moves that joining two paths, of which one writes the output, costs per page.
+    if (NH == 1 && HD <= 64) {
+#pragma unroll
+        for (int t = 0; t < HD / 16; ++t) c[0].o[t] *= alpha[0];
+    } else if (__any(rose)) {   // the maximum of some column rose (seldom after the first pages)
 #pragma unroll
         for (int h = 0; h < NH; ++h)
 #pragma unroll
