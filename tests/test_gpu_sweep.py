@@ -90,18 +90,19 @@ def test_a_random_configuration_matches_the_plain_model(seed):
             assert stepper.cache.groups[0].pool.in_use == 0
 
 
-def test_a_wide_model_on_the_prompt_kernels():
+@pytest.mark.parametrize("hidden,heads,intermediate", [(2048, 32, 12288), (1024, 16, 6656)])
+def test_a_wide_model_on_the_prompt_kernels(hidden, heads, intermediate):
     """The tiny models never reach the kernels that a real width selects for a prompt of 2,048
-    tokens (256 x 256 and 256 x 192 tiles, the tiles whose waves split K, eight rows per thread in
-    the row-wise kernels). Three layers of the 1.2B shape's width with a small vocabulary do, and
-    the plain model still takes seconds: one step of 2,048 rows and 40 decoded tokens, then the
-    same in portions that end inside pages, in bfloat16."""
+    tokens (256 x 256 and 256 x 192 tiles, the tiles of 128 or 64 columns whose waves split K,
+    eight rows per thread in the row-wise kernels). Three layers of the 1.2B or the 350M shape's
+    width with a small vocabulary do, and the plain model still takes seconds: one step of 2,048
+    rows and 40 decoded tokens, then the same in portions that end inside pages, in bfloat16."""
     from flyweight_amd.config import config_from_dict
     from flyweight_amd.engine import Stepper, load_model
     from flyweight_amd.weights import write_random_model
     config = dict(
-        architectures=["Lfm2ForCausalLM"], model_type="lfm2", vocab_size=4096, hidden_size=2048, num_hidden_layers=3,
-        num_attention_heads=32, num_key_value_heads=8, intermediate_size=12288, block_auto_adjust_ff_dim=True,
+        architectures=["Lfm2ForCausalLM"], model_type="lfm2", vocab_size=4096, hidden_size=hidden, num_hidden_layers=3,
+        num_attention_heads=heads, num_key_value_heads=8, intermediate_size=intermediate, block_auto_adjust_ff_dim=True,
         block_ffn_dim_multiplier=1.0, block_multiple_of=256, norm_eps=1e-5, rope_theta=1000000.0, conv_L_cache=3,
         conv_bias=False, tie_word_embeddings=True, max_position_embeddings=4096,
         layer_types=["conv", "full_attention", "conv"])
