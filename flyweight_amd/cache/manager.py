@@ -142,15 +142,19 @@ class CacheManager:
         self.k_pages: Dict[int, torch.Tensor] = {}
         self.v_pages: Dict[int, torch.Tensor] = {}
         self.state: Dict[int, torch.Tensor] = {}
+        # One page and one slot lie behind those the pools hand out: rows that only fill a step up to
+        # a size it was recorded for (see Stepper.planned_decode) write there, and nobody reads it.
+        self.spare_page = num_pages
+        self.spare_slot = max_requests
         if device is not None:
             for group in self.groups:
                 n = group.need
                 for entry in group.entries:
                     # K keeps a key's channels together, V a channel's tokens (see the attention kernels)
-                    self.k_pages[entry] = torch.zeros((num_pages, n.num_kv_heads, page_size, n.head_dim), dtype=dtype, device=device)
-                    self.v_pages[entry] = torch.zeros((num_pages, n.num_kv_heads, n.head_dim, page_size), dtype=dtype, device=device)
+                    self.k_pages[entry] = torch.zeros((num_pages + 1, n.num_kv_heads, page_size, n.head_dim), dtype=dtype, device=device)
+                    self.v_pages[entry] = torch.zeros((num_pages + 1, n.num_kv_heads, n.head_dim, page_size), dtype=dtype, device=device)
             for entry, need in self.state_entries.items():
-                self.state[entry] = torch.zeros((max_requests, *need.shape), dtype=need.dtype, device=device)
+                self.state[entry] = torch.zeros((max_requests + 1, *need.shape), dtype=need.dtype, device=device)
 
     def __del__(self):
         if getattr(self, "_native", None):

@@ -186,7 +186,7 @@ class Runtime:
         # one, nothing else happened) that a captured step serves goes from the scheduler's plan to
         # the upload buffer and back without an object per request.
         if counts[0] and counts[0] == counts[1] and not any(counts[2:6]) and scheduler.all_greedy:
-            captured = self.stepper.captured_step(counts[0])
+            captured = self.stepper.planned_decode(counts[0])
             if captured is not None:
                 began = time.perf_counter_ns()
                 tokens = self.stepper.replay_planned(captured, scheduler, self.decode_steps_per_turn)

@@ -219,22 +219,33 @@ class StepContext:
             self._uploaded = torch.cuda.Event()
         self._uploaded.record()
 
-    def fill_from(self, scheduler) -> bool:
+    def fill_from(self, scheduler, cache: CacheManager) -> int:
         """For a captured step: lets the scheduler write the plan it made last straight into the
         upload buffer (tokens, positions, slots, block tables) if that plan is one token for each
-        of exactly this step's number of requests and nothing else; uploads it then. False (and
-        nothing written) otherwise."""
+        of at most this step's number of requests and nothing else; fills the rows behind them up
+        and uploads it then, returning the plan's number of rows. -1 (and nothing written) otherwise."""
         self.wait_uploaded()
         host = self._host
         groups = len(host) - 8
         rows = scheduler.fill_decode(self.num_rows, host[0], host[1], host[4], self._table_stride,
                                      host[8] if groups else None, self.num_rows * self._table_stride)
-        if rows != self.num_rows:
-            if rows >= 0:
-                raise StepError(f"the plan has {rows} rows, the captured step {self.num_rows}")
-            return False
+        if rows < 0:
+            return -1
+        self.fill_up(rows, cache)
         self.upload()
-        return True
+        return rows
+
+    def fill_up(self, rows: int, cache: CacheManager) -> None:
+        """Rows behind the plan's (a step recorded for more requests than the plan has): token 0
+        at position 0 of nobody's sequence, in the cache's spare page and slot."""
+        if rows == self.num_rows:
+            return
+        host = self._host
+        host[0][rows:] = 0
+        host[1][rows:] = 0
+        host[4][rows:] = cache.spare_slot
+        for g in range(len(host) - 8):
+            host[8 + g][rows * self._table_stride:] = cache.spare_page
 
     def position_tables(self, part):
         key = part.key()
@@ -272,7 +283,6 @@ class Stepper:
         # replayed, if every part of the model allows it
         self.use_graphs = all(block.graph_safe for block in model.layers) and model.final_norm.graph_safe
         self._graphs: Dict[int, "_CapturedDecode"] = {}
-        self._eager_decodes: Dict[int, int] = {}
         self.graph_replays = 0
 
     def admit(self, request: Hashable) -> None:
@@ -296,9 +306,7 @@ class Stepper:
         # reserve everything first so that a failure leaves no request half-served
         cache.reserve_all(requests, new_lengths, described[2])
         if self.use_graphs and all(len(entry.tokens) == 1 for entry in entries):
-            captured = self._captured_decode(len(entries))
-            if captured is not None:
-                return self._replay(captured, entries, described)
+            return self._replay(self._decode_step(len(entries)), entries, described)
         ctx = StepContext(entries, cache, self.device, spec.vocab_size, spec.max_positions, described=described)
         logits = self.model.forward(ctx, cache)
         cache.commit_all(ctx.requests, ctx.new_lengths, described[2])
@@ -307,27 +315,56 @@ class Stepper:
         return logits
 
     # ----- captured decode steps ----------------------------------------------------------
-    def _captured_decode(self, batch: int) -> Optional["_CapturedDecode"]:
-        """The graph for this batch size; the first decode step of a size runs eagerly (it
-        also sets the kernels' attributes), the second is captured."""
+    def _decode_step(self, batch: int) -> "_CapturedDecode":
+        """The decode step of this many rows with its persistent index arrays."""
         captured = self._graphs.get(batch)
-        if captured is not None:
-            return captured
-        seen = self._eager_decodes.get(batch, 0)
-        self._eager_decodes[batch] = seen + 1
-        if seen < 1:
-            return None
-        cache = self.cache
-        ctx = StepContext.for_decode_graph(batch, cache, self.device, max_context=self.model.spec.max_positions,
-                                           table_stride=cache.max_pages_per_request)
-        captured = _CapturedDecode(ctx)
-        self._graphs[batch] = captured
+        if captured is None:
+            cache = self.cache
+            ctx = StepContext.for_decode_graph(batch, cache, self.device, max_context=self.model.spec.max_positions,
+                                               table_stride=cache.max_pages_per_request)
+            captured = self._graphs[batch] = _CapturedDecode(ctx)
         return captured
 
-    def captured_step(self, batch: int) -> Optional["_CapturedDecode"]:
-        """The captured decode step of this batch size, if one has been recorded."""
-        captured = self._graphs.get(batch) if self.use_graphs else None
-        return captured if captured is not None and captured.graph is not None else None
+    @staticmethod
+    def kept_batch(rows: int) -> int:
+        """The size of the step that serves a scheduler's plan of ``rows`` decoded tokens: every
+        size below 8 has a step of its own, beyond that multiples of 8 up to 64 and of 16 above
+        (the sizes at which the products change kernels, 16 and 64, are among them). A serving
+        run whose requests end one by one sees every batch size for a few steps only; recording
+        a step for each would cost more than the rows that fill a step up."""
+        if rows < 8:
+            return rows
+        multiple = 8 if rows <= 64 else 16
+        return (rows + multiple - 1) // multiple * multiple
+
+    def planned_decode(self, rows: int) -> Optional["_CapturedDecode"]:
+        """The decode step that serves a scheduler's plan of ``rows`` single tokens, or None
+        where decode steps are not recorded."""
+        return self._decode_step(self.kept_batch(rows)) if self.use_graphs else None
+
+    def _run(self, captured: "_CapturedDecode") -> None:
+        """Runs the step whose index arrays have been uploaded; its logits are ``captured.logits``
+        afterwards. The first time eagerly (kernels set their attributes and workspaces are
+        allocated then, which a recording must not hold), the second time it is recorded (that
+        runs nothing) and replayed, from then on replayed."""
+        ctx = captured.ctx
+        if captured.graph is None and not captured.ran:
+            captured.ran = True
+            ctx._position_tables = {}
+            captured.logits = self.model.forward(ctx, self.cache)
+            return
+        if captured.graph is None:
+            ctx._position_tables = {}           # the recording must hold the kernels that make them
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                with torch.cuda.graph(graph, stream=side):
+                    captured.logits = self.model.forward(ctx, self.cache)
+            torch.cuda.current_stream().wait_stream(side)
+            captured.graph = graph
+        captured.graph.replay()
+        self.graph_replays += 1
 
     def replay_planned(self, captured: "_CapturedDecode", scheduler, steps: int = 1) -> Optional[np.ndarray]:
         """Decode steps straight from the scheduler's plan (see ``StepContext.fill_from``): the
@@ -339,13 +376,14 @@ class Stepper:
         Returns the tokens, int32 [steps run, rows], or None if the plan is not a plain decode
         step (nothing has run then)."""
         ctx = captured.ctx
-        if not ctx.fill_from(scheduler):
-            return None
-        rows = ctx.num_rows
-        ahead, natives = scheduler.steps_ahead(steps - 1, rows) if steps > 1 else (0, None)
-        captured.graph.replay()
-        drawn = [ops.argmax_rows(captured.logits)]
         cache = self.cache
+        rows = ctx.fill_from(scheduler, cache)
+        if rows < 0:
+            return None
+        ahead, natives = scheduler.steps_ahead(steps - 1, rows) if steps > 1 else (0, None)
+        self._run(captured)
+        drawn = [ops.argmax_rows(captured.logits)]
+        stride = ctx._table_stride
         for _ in range(ahead):
             # the same requests one position on: pages for it, then positions and block tables anew
             ctx.wait_uploaded()
@@ -356,32 +394,20 @@ class Stepper:
                 break                       # the scheduler will decide who gives way, one step at a time
             positions[:rows] += 1
             for g in range(len(cache.groups)):
-                ctx._host[8 + g][:] = cache.block_table_rows(g, (), stride=ctx._table_stride, natives=natives, count=rows).reshape(-1)
+                ctx._host[8 + g][:rows * stride] = cache.block_table_rows(g, (), stride=stride, natives=natives, count=rows).reshape(-1)
             ctx.upload()
-            ctx.token_ids.copy_(drawn[-1])  # after the upload, which also carries the (stale) tokens
-            captured.graph.replay()
+            ctx.token_ids[:rows].copy_(drawn[-1][:rows])    # after the upload, which also carries the (stale) tokens
+            self._run(captured)
             drawn.append(ops.argmax_rows(captured.logits))
-        self.graph_replays += len(drawn)
         self.steps += len(drawn)
         self.tokens_run += rows * len(drawn)
-        return torch.stack(drawn).cpu().numpy()
+        return torch.stack(drawn)[:, :rows].cpu().numpy()
 
     def _replay(self, captured: "_CapturedDecode", entries: Sequence[StepEntry], described=None) -> Optional[torch.Tensor]:
         cache = self.cache
         ctx = captured.ctx
         ctx.refresh(entries, cache, described)
-        if captured.graph is None:
-            # record the step once; recording runs nothing, the replay below does
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.stream(side):
-                with torch.cuda.graph(graph, stream=side):
-                    captured.logits = self.model.forward(ctx, cache)
-            torch.cuda.current_stream().wait_stream(side)
-            captured.graph = graph
-        captured.graph.replay()
-        self.graph_replays += 1
+        self._run(captured)
         cache.commit_all(ctx.requests, ctx.new_lengths, None if described is None else described[2])
         self.steps += 1
         self.tokens_run += ctx.num_rows
@@ -398,3 +424,4 @@ class _CapturedDecode:
         self.ctx = ctx
         self.graph = None
         self.logits = None
+        self.ran = False            # whether the step has run eagerly once

@@ -54,8 +54,8 @@ def test_groups_share_pages_across_their_layers_and_slots_across_states():
     cache = CacheManager(NEEDS, num_pages=6, max_requests=3, device=torch.device("cpu"))
     assert len(cache.groups) == 1 and cache.groups[0].entries == [1, 3]
     assert cache.entry_group == {1: 0, 3: 0}
-    assert set(cache.state) == {0, 2} and cache.state[0].shape == (3, 8, 2)
-    assert cache.k_pages[1].shape == (6, 2, 64, 16) and cache.v_pages[3].shape == (6, 2, 16, 64)
+    assert set(cache.state) == {0, 2} and cache.state[0].shape == (3 + 1, 8, 2)      # one spare slot behind the pool's
+    assert cache.k_pages[1].shape == (6 + 1, 2, 64, 16) and cache.v_pages[3].shape == (6 + 1, 2, 16, 64)
     other = CacheManager({0: KV, 1: PagedKV(2, 16, window=100), 2: PagedKV(4, 16)}, num_pages=4, max_requests=1)
     assert len(other.groups) == 3       # a window or another head count is a group of its own
 

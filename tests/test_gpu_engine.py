@@ -238,6 +238,34 @@ def test_decode_steps_that_run_ahead_of_the_host_give_the_same_tokens(loaded, dt
         assert queued == single
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_decode_steps_are_filled_up_to_the_sizes_that_are_kept(loaded, dtype):
+    """Eleven requests that end one by one: the engine's decode steps run at the kept sizes (16,
+    then 8, then every size below), the rows behind the plan's filled up with a token of nobody's
+    in the cache's spare page and slot. Every request gets the tokens it gets alone."""
+    from flyweight_amd.engine.step import Stepper
+    assert [Stepper.kept_batch(n) for n in (1, 7, 8, 9, 16, 17, 64, 65, 81, 128)] == [1, 7, 8, 16, 16, 24, 64, 80, 96, 128]
+    m = loaded("A", dtype)
+    config, weights = m.plain_config, m.plain_weights
+    prompts = [random_tokens(m.config.vocab_size, 2 + 5 * i, seed=70 + i) for i in range(11)]
+    budgets = [6 + 3 * i for i in range(11)]
+    for steps_per_turn in (1, 4):
+        runtime = _runtime(m, parallel_sequences=11, prefill_rows=64, max_batch_tokens=128, decode_steps_per_turn=steps_per_turn)
+        ids = [runtime.task_submit(p, n) for p, n in zip(prompts, budgets)]
+        tokens = runtime.run()
+        sizes = set(runtime.stepper._graphs)
+        assert {16, 8} <= sizes and not sizes & {9, 10, 11, 12, 13, 14, 15}, sizes
+        runtime.stepper.cache.check_invariants()
+        assert runtime.info["pages_free"] == runtime.num_pages and runtime.info["live_requests"] == 0
+        alone = _runtime(m, parallel_sequences=1)
+        for task, prompt, budget in zip(ids, prompts, budgets):
+            assert len(tokens[task]) == budget
+            if dtype == "float32":
+                assert tokens[task] == plain.greedy(config, weights, prompt, budget)
+            else:
+                assert tokens[task][0] == alone.generate(prompt, 1)[0]
+
+
 def test_generate_stops_at_the_token_its_callback_refuses_even_inside_a_burst(loaded):
     """With several decode steps per turn a turn brings several tokens of a request: the callback
     that returns False ends the generation at its token; the tokens of the same turn behind it are
