@@ -148,8 +148,9 @@ int fw_attention_decode(const void* q, void* out, float* partial, int max_splits
                         const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
                         int head_dim, float scale, int window, int page_size, int num_pages, void* stream);
 
-// ids[r] = argmax(logits[r]) with ties to the lowest id; workspace: rows * 64 64-bit words
-int fw_argmax_rows(const float* logits, int32_t* ids, void* workspace, int rows, int vocab, void* stream);
+// ids[r] = argmax(logits[r]) with ties to the lowest id, also written to also[r] if that is not null;
+// workspace: rows * 64 64-bit words
+int fw_argmax_rows(const float* logits, int32_t* ids, int32_t* also, void* workspace, int rows, int vocab, void* stream);
 
 // the k largest logits of every row, sorted by (value descending, id ascending)
 int fw_topk_rows(const float* logits, float* values, int32_t* ids, int rows, int vocab, int k,

@@ -213,8 +213,10 @@ class StepContext:
         if uploaded is not None:
             uploaded.synchronize()
 
-    def upload(self) -> None:
-        self.device_buffer.copy_(self.host_buffer, non_blocking=True)
+    def upload(self, keep_tokens: bool = False) -> None:
+        """``keep_tokens``: the token ids on the device stay (the step before has written them)."""
+        first = self.num_rows if keep_tokens else 0       # the token ids lead the buffer
+        self.device_buffer[first:].copy_(self.host_buffer[first:], non_blocking=True)
         if getattr(self, "_uploaded", None) is None:
             self._uploaded = torch.cuda.Event()
         self._uploaded.record()
@@ -381,10 +383,13 @@ class Stepper:
         if rows < 0:
             return None
         ahead, natives = scheduler.steps_ahead(steps - 1, rows) if steps > 1 else (0, None)
+        # a step's most likely tokens go to the turn's record and, while a step follows, to that step's token ids
+        drawn = torch.empty((ahead + 1, ctx.num_rows), dtype=torch.int32, device=self.device)
         self._run(captured)
-        drawn = [ops.argmax_rows(captured.logits)]
+        ops.argmax_rows(captured.logits, out=drawn[0], also=ctx.token_ids if ahead else None)
+        ran = 1
         stride = ctx._table_stride
-        for _ in range(ahead):
+        while ran <= ahead:
             # the same requests one position on: pages for it, then positions and block tables anew
             ctx.wait_uploaded()
             positions = ctx._host[1]
@@ -395,13 +400,13 @@ class Stepper:
             positions[:rows] += 1
             for g in range(len(cache.groups)):
                 ctx._host[8 + g][:rows * stride] = cache.block_table_rows(g, (), stride=stride, natives=natives, count=rows).reshape(-1)
-            ctx.upload()
-            ctx.token_ids[:rows].copy_(drawn[-1][:rows])    # after the upload, which also carries the (stale) tokens
+            ctx.upload(keep_tokens=True)
             self._run(captured)
-            drawn.append(ops.argmax_rows(captured.logits))
-        self.steps += len(drawn)
-        self.tokens_run += rows * len(drawn)
-        return torch.stack(drawn)[:, :rows].cpu().numpy()
+            ops.argmax_rows(captured.logits, out=drawn[ran], also=ctx.token_ids if ran < ahead else None)
+            ran += 1
+        self.steps += ran
+        self.tokens_run += rows * ran
+        return drawn[:ran, :rows].cpu().numpy()
 
     def _replay(self, captured: "_CapturedDecode", entries: Sequence[StepEntry], described=None) -> Optional[torch.Tensor]:
         cache = self.cache

@@ -307,6 +307,11 @@ def test_argmax_and_topk(ops):
     logits[3, 5] = float("nan"); logits[3, 6] = 40.0    # NaN sorts last
     ids = ops.argmax_rows(logits.to(DEV)).cpu().tolist()
     assert ids[:4] == [17, 999, 0, 6] and ids[4] == int(logits[4].argmax())
+    # into a row of a record and into a second place (the next step's token ids; longer than the rows)
+    record = torch.full((2, 5), -1, dtype=torch.int32, device=DEV)
+    second = torch.full((8,), -1, dtype=torch.int32, device=DEV)
+    assert ops.argmax_rows(logits.to(DEV), out=record[1], also=second).data_ptr() == record[1].data_ptr()
+    assert record.cpu().tolist() == [[-1] * 5, ids] and second.cpu().tolist() == ids + [-1] * 3
     values, top = ops.topk_rows(logits.to(DEV), 7)
     assert top[0, :2].cpu().tolist() == [17, 900] and top[2].cpu().tolist() == list(range(7))
     order = sorted(range(1000), key=lambda i: (-float(logits[4, i]), i))[:7]
