@@ -213,10 +213,12 @@ class StepContext:
         if uploaded is not None:
             uploaded.synchronize()
 
-    def upload(self, keep_tokens: bool = False) -> None:
-        """``keep_tokens``: the token ids on the device stay (the step before has written them)."""
-        first = self.num_rows if keep_tokens else 0       # the token ids lead the buffer
-        self.device_buffer[first:].copy_(self.host_buffer[first:], non_blocking=True)
+    def upload(self, keep_tokens: bool = False, positions_only: bool = False) -> None:
+        """``keep_tokens``: the token ids on the device stay (the step before has written them).
+        ``positions_only``: nothing but the positions has changed since the last upload."""
+        first = self.num_rows if keep_tokens or positions_only else 0       # the token ids lead the buffer, the positions follow
+        last = 2 * self.num_rows if positions_only else self.host_buffer.numel()
+        self.device_buffer[first:last].copy_(self.host_buffer[first:last], non_blocking=True)
         if getattr(self, "_uploaded", None) is None:
             self._uploaded = torch.cuda.Event()
         self._uploaded.record()
@@ -398,9 +400,13 @@ class Stepper:
             except OutOfPages:
                 break                       # the scheduler will decide who gives way, one step at a time
             positions[:rows] += 1
-            for g in range(len(cache.groups)):
-                ctx._host[8 + g][:rows * stride] = cache.block_table_rows(g, (), stride=stride, natives=natives, count=rows).reshape(-1)
-            ctx.upload(keep_tokens=True)
+            # a block table gets a page only where a token is the first of its page (entries that a
+            # window has passed are never read, so their going needs no upload)
+            new_pages = bool((positions[:rows] % cache.page_size == 0).any())
+            if new_pages:
+                for g in range(len(cache.groups)):
+                    ctx._host[8 + g][:rows * stride] = cache.block_table_rows(g, (), stride=stride, natives=natives, count=rows).reshape(-1)
+            ctx.upload(keep_tokens=True, positions_only=not new_pages)
             self._run(captured)
             ops.argmax_rows(captured.logits, out=drawn[ran], also=ctx.token_ids if ran < ahead else None)
             ran += 1
