@@ -16,7 +16,7 @@ void fw_set_error(const char* format, ...) {
     va_end(args);
 }
 extern "C" const char* fw_last_error(void) { return fw_error_text; }
-extern "C" int fw_abi_version(void) { return 2; }
+extern "C" int fw_abi_version(void) { return 3; }
 
 // ---- embedding -------------------------------------------------------------------------
 // The reference gathers one row per token and widens it to float32
@@ -285,7 +285,8 @@ __global__ __launch_bounds__(256) void argmax_parts_kernel(const float* __restri
 }
 
 __global__ __launch_bounds__(64) void argmax_finish_kernel(const unsigned long long* __restrict__ best_of_part,
-                                                           int32_t* __restrict__ ids, int32_t* __restrict__ also) {
+                                                           int32_t* __restrict__ ids, int32_t* __restrict__ also,
+                                                           int32_t* __restrict__ advance) {
     const int row = blockIdx.x;
     unsigned long long best = best_of_part[(size_t)row * ARGMAX_PARTS + threadIdx.x];     // 64 parts, 64 lanes
     best = wave_max_u64(best);
@@ -293,19 +294,21 @@ __global__ __launch_bounds__(64) void argmax_finish_kernel(const unsigned long l
         const int id = (int)(0xffffffffu - (uint32_t)(best & 0xffffffffull));
         ids[row] = id;
         if (also) also[row] = id;
+        if (advance) advance[row] += 1;
     }
 }
 
 // workspace: rows * 64 64-bit words (the best key of each part of each row). also: null, or a second
-// place for the ids (the next decode step's token ids, which saves the copy between two steps)
-extern "C" int fw_argmax_rows(const float* logits, int32_t* ids, int32_t* also, void* workspace, int rows, int vocab,
-                              void* stream) {
+// place for the ids; advance: null, or a counter per row that goes up by one. (A decode step that
+// follows at once takes its token ids and positions from these: nothing crosses to the host between.)
+extern "C" int fw_argmax_rows(const float* logits, int32_t* ids, int32_t* also, int32_t* advance, void* workspace,
+                              int rows, int vocab, void* stream) {
     FW_REQUIRE(rows >= 0 && rows <= 65535 && vocab > 0, "argmax_rows: bad sizes rows=%d vocab=%d", rows, vocab);
     if (rows == 0) return 0;
     FW_REQUIRE(workspace != nullptr && (uintptr_t)workspace % 8 == 0, "argmax_rows: needs an 8-byte aligned workspace");
     argmax_parts_kernel<<<dim3(ARGMAX_PARTS, rows), 256, 0, (hipStream_t)stream>>>(logits, (unsigned long long*)workspace, vocab);
     FW_LAUNCH_CHECK("argmax_rows (parts)");
-    argmax_finish_kernel<<<rows, 64, 0, (hipStream_t)stream>>>((const unsigned long long*)workspace, ids, also);
+    argmax_finish_kernel<<<rows, 64, 0, (hipStream_t)stream>>>((const unsigned long long*)workspace, ids, also, advance);
     FW_LAUNCH_CHECK("argmax_rows");
     return 0;
 }

@@ -149,8 +149,9 @@ int fw_attention_decode(const void* q, void* out, float* partial, int max_splits
                         int head_dim, float scale, int window, int page_size, int num_pages, void* stream);
 
 // ids[r] = argmax(logits[r]) with ties to the lowest id, also written to also[r] if that is not null;
-// workspace: rows * 64 64-bit words
-int fw_argmax_rows(const float* logits, int32_t* ids, int32_t* also, void* workspace, int rows, int vocab, void* stream);
+// advance[r] += 1 if that is not null; workspace: rows * 64 64-bit words
+int fw_argmax_rows(const float* logits, int32_t* ids, int32_t* also, int32_t* advance, void* workspace, int rows, int vocab,
+                   void* stream);
 
 // the k largest logits of every row, sorted by (value descending, id ascending)
 int fw_topk_rows(const float* logits, float* values, int32_t* ids, int rows, int vocab, int k,

@@ -213,12 +213,8 @@ class StepContext:
         if uploaded is not None:
             uploaded.synchronize()
 
-    def upload(self, keep_tokens: bool = False, positions_only: bool = False) -> None:
-        """``keep_tokens``: the token ids on the device stay (the step before has written them).
-        ``positions_only``: nothing but the positions has changed since the last upload."""
-        first = self.num_rows if keep_tokens or positions_only else 0       # the token ids lead the buffer, the positions follow
-        last = 2 * self.num_rows if positions_only else self.host_buffer.numel()
-        self.device_buffer[first:last].copy_(self.host_buffer[first:last], non_blocking=True)
+    def upload(self) -> None:
+        self.device_buffer.copy_(self.host_buffer, non_blocking=True)
         if getattr(self, "_uploaded", None) is None:
             self._uploaded = torch.cuda.Event()
         self._uploaded.record()
@@ -226,8 +222,8 @@ class StepContext:
     def fill_from(self, scheduler, cache: CacheManager) -> int:
         """For a captured step: lets the scheduler write the plan it made last straight into the
         upload buffer (tokens, positions, slots, block tables) if that plan is one token for each
-        of at most this step's number of requests and nothing else; fills the rows behind them up
-        and uploads it then, returning the plan's number of rows. -1 (and nothing written) otherwise."""
+        of at most this step's number of requests and nothing else, and fills the rows behind them
+        up; returns the plan's number of rows (the caller uploads). -1 (and nothing written) otherwise."""
         self.wait_uploaded()
         host = self._host
         groups = len(host) - 8
@@ -236,7 +232,6 @@ class StepContext:
         if rows < 0:
             return -1
         self.fill_up(rows, cache)
-        self.upload()
         return rows
 
     def fill_up(self, rows: int, cache: CacheManager) -> None:
@@ -385,31 +380,29 @@ class Stepper:
         if rows < 0:
             return None
         ahead, natives = scheduler.steps_ahead(steps - 1, rows) if steps > 1 else (0, None)
-        # a step's most likely tokens go to the turn's record and, while a step follows, to that step's token ids
-        drawn = torch.empty((ahead + 1, ctx.num_rows), dtype=torch.int32, device=self.device)
-        self._run(captured)
-        ops.argmax_rows(captured.logits, out=drawn[0], also=ctx.token_ids if ahead else None)
-        ran = 1
-        stride = ctx._table_stride
-        while ran <= ahead:
-            # the same requests one position on: pages for it, then positions and block tables anew
-            ctx.wait_uploaded()
+        if ahead:
+            # Pages for all the steps of the turn now, and the block tables with them: a table that
+            # already holds the page a later step will write to reads the same for the steps before.
             positions = ctx._host[1]
+            stride = ctx._table_stride
             try:
-                cache.reserve_all((), (positions[:rows] + 2).tolist(), natives=natives, count=rows)
+                cache.reserve_all((), (positions[:rows] + 1 + ahead).tolist(), natives=natives, count=rows)
             except OutOfPages:
-                break                       # the scheduler will decide who gives way, one step at a time
-            positions[:rows] += 1
-            # a block table gets a page only where a token is the first of its page (entries that a
-            # window has passed are never read, so their going needs no upload)
-            new_pages = bool((positions[:rows] % cache.page_size == 0).any())
-            if new_pages:
+                ahead = 0                   # one step; the scheduler will decide who gives way
+            else:
                 for g in range(len(cache.groups)):
                     ctx._host[8 + g][:rows * stride] = cache.block_table_rows(g, (), stride=stride, natives=natives, count=rows).reshape(-1)
-            ctx.upload(keep_tokens=True, positions_only=not new_pages)
+        ctx.upload()
+        # Nothing crosses to the host between the steps of a turn: the kernel that finds a step's most
+        # likely tokens writes them to the turn's record and to the next step's token ids, and moves
+        # every row's position on by one.
+        drawn = torch.empty((ahead + 1, ctx.num_rows), dtype=torch.int32, device=self.device)
+        for step in range(ahead):
             self._run(captured)
-            ops.argmax_rows(captured.logits, out=drawn[ran], also=ctx.token_ids if ran < ahead else None)
-            ran += 1
+            ops.argmax_rows(captured.logits, out=drawn[step], also=ctx.token_ids, advance=ctx.row_pos)
+        self._run(captured)
+        ops.argmax_rows(captured.logits, out=drawn[ahead])
+        ran = ahead + 1
         self.steps += ran
         self.tokens_run += rows * ran
         return drawn[:ran, :rows].cpu().numpy()

@@ -33,8 +33,8 @@ def library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
         lib.fw_last_error.restype = ctypes.c_char_p
         lib.fw_abi_version.restype = ctypes.c_int
-        if lib.fw_abi_version() != 2:
-            raise KernelError(f"{path}: kernel library ABI {lib.fw_abi_version()} != 2; rebuild it")
+        if lib.fw_abi_version() != 3:
+            raise KernelError(f"{path}: kernel library ABI {lib.fw_abi_version()} != 3; rebuild it")
         _lib = lib
     return _lib
 
@@ -281,21 +281,23 @@ def attention_generic(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     return out
 
 
-def argmax_rows(logits: torch.Tensor, out: Optional[torch.Tensor] = None, also: Optional[torch.Tensor] = None) -> torch.Tensor:
+def argmax_rows(logits: torch.Tensor, out: Optional[torch.Tensor] = None, also: Optional[torch.Tensor] = None,
+                advance: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The id of each row's largest logit (ties: the lowest id), int32 [rows], into ``out`` if
-    given and into ``also`` as well (both contiguous int32 of at least ``rows`` elements)."""
+    given and into ``also`` as well; ``advance[r]`` goes up by one (all contiguous int32 of at
+    least ``rows`` elements)."""
     _dev(logits)
     _want(logits, torch.float32, "logits")
     rows, vocab = logits.shape
     ids = out if out is not None else torch.empty((rows,), dtype=torch.int32, device=logits.device)
-    for name, target in (("out", out), ("also", also)):
+    for name, target in (("out", out), ("also", also), ("advance", advance)):
         if target is not None:
             _dev(target)
             _want(target, torch.int32, name)
             if target.numel() < rows or not target.is_contiguous():
                 raise KernelError(f"argmax_rows: {name} must be contiguous and hold {rows} ids")
     workspace = torch.empty((max(rows, 1), 64), dtype=torch.int64, device=logits.device)       # best key of each part
-    _check(library().fw_argmax_rows(_p(logits), _p(ids), _p(also), _p(workspace), rows, vocab, _stream()))
+    _check(library().fw_argmax_rows(_p(logits), _p(ids), _p(also), _p(advance), _p(workspace), rows, vocab, _stream()))
     return ids
 
 

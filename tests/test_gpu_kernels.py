@@ -310,8 +310,10 @@ def test_argmax_and_topk(ops):
     # into a row of a record and into a second place (the next step's token ids; longer than the rows)
     record = torch.full((2, 5), -1, dtype=torch.int32, device=DEV)
     second = torch.full((8,), -1, dtype=torch.int32, device=DEV)
-    assert ops.argmax_rows(logits.to(DEV), out=record[1], also=second).data_ptr() == record[1].data_ptr()
+    counters = torch.arange(10, 18, dtype=torch.int32, device=DEV)       # a counter per row goes up by one
+    assert ops.argmax_rows(logits.to(DEV), out=record[1], also=second, advance=counters).data_ptr() == record[1].data_ptr()
     assert record.cpu().tolist() == [[-1] * 5, ids] and second.cpu().tolist() == ids + [-1] * 3
+    assert counters.cpu().tolist() == [11, 12, 13, 14, 15, 15, 16, 17]
     values, top = ops.topk_rows(logits.to(DEV), 7)
     assert top[0, :2].cpu().tolist() == [17, 900] and top[2].cpu().tolist() == list(range(7))
     order = sorted(range(1000), key=lambda i: (-float(logits[4, i]), i))[:7]
