@@ -370,8 +370,9 @@ class Stepper:
         pages are reserved by the plan and the lengths are committed when the scheduler completes
         it, so the cache manager is not asked again. Every token is the most likely one. With
         ``steps`` > 1 and a plan that is certain to repeat (``Scheduler.steps_ahead``), up to that
-        many steps run back to back on the device, each fed the tokens of the one before, and the
-        host reads all of them at once: it is then asked once per turn instead of once per step.
+        many steps run back to back on the device (their pages reserved and their block tables
+        uploaded before the first), each fed the tokens of the one before, and the host reads all
+        of them at once: it is then asked once per turn instead of once per step.
         Returns the tokens, int32 [steps run, rows], or None if the plan is not a plain decode
         step (nothing has run then)."""
         ctx = captured.ctx
