@@ -1,0 +1,73 @@
+"""The command line in-process on the GPU: generate, benchmark and inspect on tiny model
+folders, against the plain implementation where tokens are decided."""
+
+import json
+
+import pytest
+
+import plain_lfm2 as plain
+from helpers import make_model, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    root = tmp_path_factory.mktemp("models")
+    return {name: make_model(str(root / name), name, seed=33) for name in ("A", "B")}
+
+
+def run(capsys, *argv):
+    from flyweight_amd.cli import main
+    status = main(list(argv))
+    captured = capsys.readouterr()
+    return status, captured.out, captured.err
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_generate_prints_the_plain_models_greedy_tokens(folders, name, capsys, tmp_path):
+    config, weights = plain.read_folder(folders[name])
+    prompt = random_tokens(config["vocab_size"], 11, seed=4)
+    expected = plain.greedy(config, weights, prompt, 6)
+    ids = ",".join(str(t) for t in prompt)
+    # a stop token that the model cannot produce, so that its eos does not end the generation early
+    common = ("--max-tokens", "6", "--temperature", "0", "--dtype", "float32", "--stop-token", str(config["vocab_size"] + 7))
+    status, out, _ = run(capsys, "generate", folders[name], "--tokens", ids, *common)
+    assert status == 0 and [int(t) for t in out.split()] == expected
+    # the same from a file, in turns of several decode steps; a stop token ends it behind that token
+    listed = tmp_path / "prompt.txt"
+    listed.write_text(" ".join(str(t) for t in prompt))
+    status, out, _ = run(capsys, "generate", folders[name], "--tokens-file", str(listed), "--max-new-tokens", "6",
+                         "--temperature", "0", "--dtype", "float32", "--decode-steps-per-turn", "4",
+                         "--stop-token", str(expected[3]))
+    assert status == 0 and [int(t) for t in out.split()] == expected[:expected.index(expected[3]) + 1]
+
+
+def test_generate_with_a_seed_reproduces_and_refuses_what_it_cannot_do(folders, capsys):
+    folder = folders["B"]
+    sampled = ("generate", folder, "--tokens", "3,1,4,1,5", "--max-tokens", "12", "--temperature", "0.8", "--top-k", "40",
+               "--seed", "7", "--stop-token", "100000")
+    first = run(capsys, *sampled)
+    second = run(capsys, *sampled)
+    assert first[0] == 0 and first[1] == second[1] and len(first[1].split()) == 12
+    status, out, err = run(capsys, "generate", folder, "--max-tokens", "3")
+    assert status == 2 and "--tokens" in err and out == ""
+    status, out, err = run(capsys, "generate", folder, "--tokens", "1,2", "--temperature", "-1")
+    assert status == 1 and "temperature" in err
+    status, out, err = run(capsys, "generate", folder + "-missing", "--tokens", "1,2")
+    assert status == 1 and err.startswith("flyweight-amd:")
+
+
+def test_benchmark_and_inspect_print_json(folders, capsys):
+    status, out, _ = run(capsys, "benchmark", folders["A"], "--tokens", "5,6,7", "--warmup", "2", "--iterations", "9")
+    report = json.loads(out)
+    assert status == 0 and report["prompt_tokens"] == 3 and report["iterations"] == 9
+    assert report["decode_tokens_per_second"] > 0 and 0 < report["median_seconds"] <= report["p99_seconds"]
+    assert report["prompt_and_first_token_seconds"] > 0 and report["prepare_seconds"] > 0
+    status, out, _ = run(capsys, "inspect", folders["B"])
+    shown = json.loads(out)
+    config, weights = plain.read_folder(folders["B"])
+    assert status == 0 and shown["architecture"] == "Lfm2ForCausalLM"
+    assert shown["config"]["hidden_size"] == config["hidden_size"] and shown["derived"]["layers"] == config["num_hidden_layers"]
+    assert set(shown["tensors"]) == set(weights)
+    assert shown["derived"]["parameters"] == sum(int(w.size) for w in weights.values())
