@@ -299,6 +299,28 @@ class CacheManager:
         if self._lib.fwh_cache_commit(self._native, self._id(request), int(new_length)) < 0:
             raise ValueError(host.last_error())
 
+    def truncate(self, request: Hashable, token_count: int) -> None:
+        """Gives back the pages behind the first ``token_count`` tokens in every group (the
+        reference's truncate_tokens, native/src/paged_kv.h:180-187): reservations a step did not
+        use after all, or a sequence cut back. Fixed-size state cannot be rewound, so a model that
+        keeps any can only drop reservations, never tokens it has run."""
+        if request not in self.requests:
+            raise KeyError(f"request {request!r} is not live")
+        if self.state_entries and token_count < self.length_of(request):
+            raise CacheAccountingError(f"request {request!r} holds fixed-size state of {self.length_of(request)} tokens, "
+                                       f"which cannot be cut back to {token_count}")
+        if self._lib.fwh_cache_truncate(self._native, self._id(request), int(token_count)) < 0:
+            raise CacheAccountingError(host.last_error())
+
+    def drop_reservations(self, requests: Sequence[Hashable], natives=None) -> None:
+        """After a step that did not run: the pages reserved for it beyond each request's
+        length go back to the pools."""
+        count = len(requests)
+        natives = self.natives_of(requests) if natives is None else natives
+        lengths, _ = self.describe(requests, natives)
+        if self._lib.fwh_cache_truncate_batch(self._native, natives, (ctypes.c_int * max(count, 1))(*lengths), count) < 0:
+            raise CacheAccountingError(host.last_error())
+
     def release(self, request: Hashable) -> None:
         if request not in self.requests:
             raise CacheAccountingError(f"request {request!r} is released but not live")

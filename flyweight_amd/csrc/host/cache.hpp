@@ -176,6 +176,31 @@ public:
                 }
         }
     }
+    // Gives back the pages behind the first token_count tokens in every group, as the reference's
+    // truncate_tokens (native/src/paged_kv.h:180-187): reservations that were not used after all, or
+    // a sequence cut back. The length becomes token_count if it was longer. A windowed group cannot
+    // be cut back to where its window has passed pages already: those keys are gone.
+    void truncate(int64_t request, int token_count) {
+        Live& state = live_.at(request);
+        if (token_count < 0) throw std::invalid_argument("a sequence has no negative length");
+        const int keep = pages_for(token_count);
+        if (token_count < state.length)
+            for (const Group& group : groups_) {
+                const std::vector<int>& table = group.tables.at(request);
+                for (int block = first_needed_block(group, token_count); block < keep && block < (int)table.size(); ++block)
+                    if (table[block] == NO_PAGE)
+                        throw std::invalid_argument("request " + std::to_string(request) + " cannot be cut back to " +
+                                                    std::to_string(token_count) + " tokens: its window has passed keys it would need");
+            }
+        for (Group& group : groups_) {
+            std::vector<int>& table = group.tables[request];
+            while ((int)table.size() > keep) {
+                if (table.back() != NO_PAGE) group.pool.free(table.back());
+                table.pop_back();
+            }
+        }
+        if (token_count < state.length) state.length = token_count;
+    }
     void release(int64_t request) {
         auto it = live_.find(request);
         if (it == live_.end()) throw AccountingError("request " + std::to_string(request) + " is released but not live");

@@ -39,6 +39,10 @@ void* fwh_cache_slot_pool(void* cache);
 int fwh_cache_admit(void* cache, int64_t request);      // the slot; FWH_OUT_OF_PAGES when no slot is free
 int fwh_cache_reserve(void* cache, int64_t request, int new_length);    // all groups or nothing
 int fwh_cache_commit(void* cache, int64_t request, int new_length);     // windowed groups give pages back
+// pages behind the first token_count tokens go back to the pools (unused reservations, or a
+// sequence cut back: the length becomes token_count if it was longer)
+int fwh_cache_truncate(void* cache, int64_t request, int token_count);
+int fwh_cache_truncate_batch(void* cache, const int64_t* requests, const int* token_counts, int count);
 int fwh_cache_release(void* cache, int64_t request);
 int fwh_cache_is_live(void* cache, int64_t request);
 int fwh_cache_slot_of(void* cache, int64_t request);
@@ -63,18 +67,24 @@ int fwh_cache_check(void* cache);                       // no page lost, held tw
 #define FWH_EVENT_ERROR 2
 #define FWH_EVENT_PREFILL 3
 
+// vocab_size: token ids of prompts and stop tokens are checked against it at submit (0: not known, not checked).
 void* fwh_scheduler_create(void* cache, int max_positions, int max_batch_tokens, int chunk_size, int max_live,
-                           int max_queued);
+                           int max_queued, int vocab_size);
 void fwh_scheduler_destroy(void* scheduler);
 int64_t fwh_scheduler_submit(void* scheduler, const int* prompt, int prompt_len, int max_new_tokens,
                              const int* stop_tokens, int num_stop);    // the request's id (>= 1)
 int fwh_scheduler_cancel(void* scheduler, int64_t request);            // 1 if it was still going
+// Ends one request with an error (text kept for fwh_request_error): it leaves the queue or gives
+// back its pages and slot, and leaves the plan made last, whose other segments and reservations
+// stand; its error event comes out of the next completion. 1 if it was still going.
+int fwh_scheduler_fail(void* scheduler, int64_t request, const char* message);
 int fwh_scheduler_has_work(void* scheduler);
 int fwh_scheduler_preemptions(void* scheduler);
 int fwh_scheduler_queue(void* scheduler, int which, int64_t* requests, int capacity);   // 0 waiting, 1 running
 // Plans the next step (reserving its pages) and keeps the plan until the next call.
-// counts: segments, tokens, preempted, failed, admitted, cancelled.
-int fwh_scheduler_schedule(void* scheduler, int counts[6]);
+// counts: segments, tokens, preempted, failed, admitted, cancelled, and the most tokens that a
+// sequence of the plan reaches or that its block tables cover (what a step's tables must hold).
+int fwh_scheduler_schedule(void* scheduler, int counts[7]);
 int fwh_plan_segments(void* scheduler, int64_t* requests, int* num_tokens, int* wants_logits, int* tokens);
 int fwh_plan_list(void* scheduler, int which, int64_t* requests);      // 0 preempted, 1 failed, 2 admitted, 3 cancelled
 // After the step: the token drawn for every segment that wanted logits. Events (request, token or

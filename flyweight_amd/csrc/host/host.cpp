@@ -38,7 +38,7 @@ int copy_ids(const std::vector<fwh::Request*>& from, int64_t* to) {
 extern "C" {
 
 const char* fwh_last_error(void) { return last_error.c_str(); }
-int fwh_abi_version(void) { return 1; }
+int fwh_abi_version(void) { return 2; }
 
 // ---- pools ---------------------------------------------------------------------------------
 void* fwh_pool_create(int size) {
@@ -77,6 +77,15 @@ int fwh_cache_reserve(void* cache, int64_t request, int new_length) {
 }
 int fwh_cache_commit(void* cache, int64_t request, int new_length) {
     return guarded([&] { cache_of(cache)->commit(request, new_length); return 0; });
+}
+int fwh_cache_truncate(void* cache, int64_t request, int token_count) {
+    return guarded([&] { cache_of(cache)->truncate(request, token_count); return 0; });
+}
+int fwh_cache_truncate_batch(void* cache, const int64_t* requests, const int* token_counts, int count) {
+    return guarded([&] {
+        for (int i = 0; i < count; ++i) cache_of(cache)->truncate(requests[i], token_counts[i]);
+        return 0;
+    });
 }
 int fwh_cache_release(void* cache, int64_t request) { return guarded([&] { cache_of(cache)->release(request); return 0; }); }
 int fwh_cache_is_live(void* cache, int64_t request) { return cache_of(cache)->is_live(request) ? 1 : 0; }
@@ -160,10 +169,11 @@ int fwh_cache_live(void* cache, int64_t* requests, int capacity) {
 int fwh_cache_check(void* cache) { return guarded([&] { cache_of(cache)->check(); return 0; }); }
 
 // ---- scheduler -----------------------------------------------------------------------------
-void* fwh_scheduler_create(void* cache, int max_positions, int max_batch_tokens, int chunk_size, int max_live, int max_queued) {
+void* fwh_scheduler_create(void* cache, int max_positions, int max_batch_tokens, int chunk_size, int max_live, int max_queued,
+                           int vocab_size) {
     void* made = nullptr;
     guarded([&] {
-        made = new fwh::Scheduler(cache_of(cache), max_positions, max_batch_tokens, chunk_size, max_live, max_queued);
+        made = new fwh::Scheduler(cache_of(cache), max_positions, max_batch_tokens, chunk_size, max_live, max_queued, vocab_size);
         return 0;
     });
     return made;
@@ -176,6 +186,9 @@ int64_t fwh_scheduler_submit(void* scheduler, const int* prompt, int prompt_len,
     return id;
 }
 int fwh_scheduler_cancel(void* scheduler, int64_t request) { return scheduler_of(scheduler)->cancel(request) ? 1 : 0; }
+int fwh_scheduler_fail(void* scheduler, int64_t request, const char* message) {
+    return guarded([&] { return scheduler_of(scheduler)->fail_request(request, message ? message : "failed") ? 1 : 0; });
+}
 int fwh_scheduler_has_work(void* scheduler) { return scheduler_of(scheduler)->has_work() ? 1 : 0; }
 int fwh_scheduler_preemptions(void* scheduler) { return scheduler_of(scheduler)->preemptions(); }
 int fwh_scheduler_queue(void* scheduler, int which, int64_t* requests, int capacity) {
@@ -189,9 +202,18 @@ int fwh_scheduler_queue(void* scheduler, int which, int64_t* requests, int capac
     else for (const fwh::Request* request : s->running()) put(request);
     return n;
 }
-int fwh_scheduler_schedule(void* scheduler, int counts[6]) {
+int fwh_scheduler_schedule(void* scheduler, int counts[7]) {
     return guarded([&] {
-        const fwh::Plan& plan = scheduler_of(scheduler)->schedule();
+        fwh::Scheduler* s = scheduler_of(scheduler);
+        const fwh::Plan& plan = s->schedule();
+        fwh::Cache& cache = s->cache();
+        int covered = 0;
+        for (const fwh::Segment& segment : plan.segments) {
+            covered = std::max(covered, segment.first + segment.count);
+            for (int g = 0; g < cache.num_groups(); ++g)
+                covered = std::max(covered, (int)cache.group(g).tables.at(segment.request->id).size() * cache.page_size());
+        }
+        counts[6] = covered;
         counts[0] = (int)plan.segments.size();
         counts[1] = plan.num_tokens;
         counts[2] = (int)plan.preempted.size();

@@ -85,18 +85,32 @@ struct Plan {
 
 class Scheduler {
 public:
-    Scheduler(Cache* cache, int max_positions, int max_batch_tokens, int chunk_size, int max_live, int max_queued)
+    // vocab_size 0: the vocabulary is not known and token ids are not looked at.
+    Scheduler(Cache* cache, int max_positions, int max_batch_tokens, int chunk_size, int max_live, int max_queued,
+              int vocab_size = 0)
         : cache_(cache), max_positions_(max_positions), max_batch_tokens_(max_batch_tokens), chunk_size_(chunk_size),
-          max_queued_(max_queued) {
+          max_queued_(max_queued), vocab_size_(vocab_size) {
         if (max_batch_tokens < 1 || chunk_size < 1) throw SchedulerError("max_batch_tokens and chunk_size must be positive");
         max_live_ = max_live > 0 && max_live < cache->max_requests() ? max_live : cache->max_requests();
     }
 
     // Validation as the reference's task submit: a prompt, room for prompt + output in the
-    // context, a bounded queue.
+    // context, a bounded queue; and what its decode refuses token by token
+    // (native/src/v2_runtime.cpp:27529-27530), here before the request takes a place: every token
+    // id inside the vocabulary, so that no step ever meets one that is not.
     Request* submit(const int* prompt, int prompt_len, int max_new_tokens, const int* stop, int num_stop) {
         if (prompt_len < 1) throw SchedulerError("the prompt is empty");
         if (max_new_tokens < 1) throw SchedulerError("max_tokens must be at least 1");
+        if (vocab_size_ > 0) {
+            for (int i = 0; i < prompt_len; ++i)
+                if (prompt[i] < 0 || prompt[i] >= vocab_size_)
+                    throw SchedulerError("token id " + std::to_string(prompt[i]) + " at place " + std::to_string(i) +
+                                         " of the prompt is outside the vocabulary (0.." + std::to_string(vocab_size_ - 1) + ")");
+            for (int i = 0; i < num_stop; ++i)
+                if (stop[i] < 0 || stop[i] >= vocab_size_)
+                    throw SchedulerError("stop token " + std::to_string(stop[i]) + " is outside the vocabulary (0.." +
+                                         std::to_string(vocab_size_ - 1) + ")");
+        }
         if (prompt_len + max_new_tokens > max_positions_)
             throw SchedulerError("prompt (" + std::to_string(prompt_len) + ") + max_tokens (" + std::to_string(max_new_tokens) +
                                  ") exceeds the context of " + std::to_string(max_positions_));
@@ -118,6 +132,25 @@ public:
         request->cancelled = true;
         return true;
     }
+    // A request that cannot go on (the step refused its tokens, or failed while it ran them, so
+    // that what the cache holds of it cannot be trusted): it ends with an error, whatever it holds
+    // is given back, and it leaves the plan made last, whose other segments stand as they are;
+    // its error event comes with that plan's completion. The reference isolates a task's failure
+    // the same way (native/src/v2_runtime.cpp:33788-33797). False if it has ended already.
+    bool fail_request(int64_t id, const std::string& message) {
+        Request* request = find(id);
+        if (!request || request->finished) return false;
+        plan_.drop(request);
+        auto queued = std::find(waiting_.begin(), waiting_.end(), request);
+        if (queued != waiting_.end()) waiting_.erase(queued);
+        auto listed = [&](std::vector<Request*>& list) {
+            list.erase(std::remove(list.begin(), list.end(), request), list.end());
+        };
+        listed(plan_.preempted);
+        listed(plan_.admitted);
+        fail(request, message, plan_);
+        return true;
+    }
     bool has_work() const { return !waiting_.empty() || !running_.empty(); }
     int preemptions() const { return preemptions_; }
     Request* find(int64_t id) {
@@ -127,7 +160,9 @@ public:
     bool forget(int64_t id) {
         Request* request = find(id);
         if (!request || !request->finished) return false;
-        plan_.clear();              // it may still name the request
+        plan_.drop(request);        // the plan made last may still name it
+        for (std::vector<Request*>* list : {&plan_.preempted, &plan_.failed, &plan_.admitted, &plan_.cancelled})
+            list->erase(std::remove(list->begin(), list->end(), request), list->end());
         requests_.erase(id);
         return true;
     }
@@ -138,8 +173,12 @@ public:
     int max_positions() const { return max_positions_; }
 
     const Plan& schedule() {
+        // endings whose events no completion has handed out yet (a request failed between two plans)
+        std::vector<Request*> failed_before = plan_.failed, cancelled_before = plan_.cancelled;
         plan_.clear();
         Plan& plan = plan_;
+        plan.failed = failed_before;
+        plan.cancelled = cancelled_before;
         // cancelled requests leave first
         for (Request* request : std::vector<Request*>(running_))
             if (request->cancelled) {
@@ -280,7 +319,7 @@ private:
     }
 
     Cache* cache_;
-    int max_positions_, max_batch_tokens_, chunk_size_, max_live_, max_queued_;
+    int max_positions_, max_batch_tokens_, chunk_size_, max_live_, max_queued_, vocab_size_;
     std::deque<Request*> waiting_;
     std::vector<Request*> running_;         // in admission order, oldest first
     std::unordered_map<int64_t, std::unique_ptr<Request>> requests_;

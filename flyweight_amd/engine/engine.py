@@ -19,9 +19,10 @@ from ..sampling import GREEDY, SamplingConfig, sample_rows
 from .model import CausalLM, load_model, parse_dtype
 from .scheduler import (EVENT_ERROR, EVENT_FINISHED, EVENT_PREFILL, EVENT_TOKEN, Request, Scheduler,
                         SchedulerError)
-from .step import StepEntry, Stepper
+from .step import StepEntry, StepError, Stepper
 
 PAGE_SIZE = 64
+MAX_KEPT_ERRORS = 1024
 
 
 class EngineError(RuntimeError):
@@ -94,7 +95,10 @@ class Runtime:
         self.decode_steps_per_turn = max(1, int(decode_steps_per_turn))
         self.stepper: Optional[Stepper] = None
         self.scheduler: Optional[Scheduler] = None
-        self._errors: Dict[int, str] = {}
+        self._errors: Dict[int, str] = {}           # task -> text, the last MAX_KEPT_ERRORS of them
+        self._outputs: Dict[int, List[int]] = {}    # live task -> tokens so far
+        self._collecting: Optional[Dict[int, List[int]]] = None
+        self._held_events: List[Tuple[int, int, int]] = []
         self._decode_request: Optional[Hashable] = None
         self._counters = {"decode_calls": 0, "decode_ns": 0, "prefill_calls": 0, "prefill_tokens": 0, "prefill_ns": 0,
                           "steps": 0}
@@ -103,10 +107,10 @@ class Runtime:
     def prepare(self) -> "Runtime":
         if self.stepper is None:
             self.stepper = Stepper(self.model.model, num_pages=self.num_pages, max_requests=self.parallel_sequences,
-                                   page_size=PAGE_SIZE)
+                                   page_size=PAGE_SIZE, context_limit=self.context_limit)
             self.scheduler = Scheduler(self.stepper.cache, max_positions=self.context_limit,
                                        max_batch_tokens=self.max_batch_tokens, chunk_size=self.prefill_rows,
-                                       max_live=self.parallel_sequences)
+                                       max_live=self.parallel_sequences, vocab_size=self.model.spec.vocab_size)
         return self
 
     def reset(self) -> None:
@@ -117,9 +121,11 @@ class Runtime:
             self.stepper.cache.release(request)
         self.scheduler = Scheduler(self.stepper.cache, max_positions=self.context_limit,
                                    max_batch_tokens=self.max_batch_tokens, chunk_size=self.prefill_rows,
-                                   max_live=self.parallel_sequences)
+                                   max_live=self.parallel_sequences, vocab_size=self.model.spec.vocab_size)
         self._decode_request = None
         self._errors.clear()
+        self._outputs.clear()
+        self._held_events = []
 
     def close(self) -> None:
         self.stepper = None
@@ -161,6 +167,9 @@ class Runtime:
     def task_submit(self, prompt: Sequence[int], max_tokens: int, stop_tokens: Sequence[int] = (),
                     temperature: float = 0.0, top_k: int = 20, top_p: float = 0.95, min_p: float = 0.0,
                     seed: Optional[int] = None) -> int:
+        """Queues a request and returns its task id. Refused here, before it takes a place: an
+        empty prompt, ``max_tokens`` < 1, prompt + ``max_tokens`` beyond the context, a token id
+        or stop token outside the vocabulary, sampling settings out of range, a full queue."""
         self.prepare()
         sampling = SamplingConfig(temperature=temperature, top_k=top_k, top_p=top_p, min_p=min_p, seed=seed)
         try:
@@ -176,20 +185,32 @@ class Runtime:
 
     def engine_step(self) -> List[Tuple[int, int, int]]:
         """One step of everything that can move: returns (task id, token or progress, kind)
-        with kind 0 token, 1 finished, 2 error, 3 prefill progress."""
+        with kind 0 token, 1 finished, 2 error, 3 prefill progress. A request that the step
+        refuses, or that took part in a step that failed while it ran, ends with an error event
+        (its text in ``task_error``) and gives back what it held; the others go on, as the
+        reference isolates a task's failure (native/src/v2_runtime.cpp:33788-33797)."""
         self.prepare()
+        held, self._held_events = self._held_events, []
+        if not self.scheduler.has_work():
+            return held
+        events = self._advance()
+        self._note(events)
+        return held + events if held else events
+
+    def _advance(self) -> List[Tuple[int, int, int]]:
         scheduler = self.scheduler
-        if not scheduler.has_work():
-            return []
         counts = scheduler.plan_next()
         # A plain decode step (one token for every request of the plan, every token the most likely
         # one, nothing else happened) that a captured step serves goes from the scheduler's plan to
         # the upload buffer and back without an object per request.
         if counts[0] and counts[0] == counts[1] and not any(counts[2:6]) and scheduler.all_greedy:
-            captured = self.stepper.planned_decode(counts[0])
+            captured = self.stepper.planned_decode(counts[0], counts[6] + self.decode_steps_per_turn - 1)
             if captured is not None:
                 began = time.perf_counter_ns()
-                tokens = self.stepper.replay_planned(captured, scheduler, self.decode_steps_per_turn)
+                try:
+                    tokens = self.stepper.replay_planned(captured, scheduler, self.decode_steps_per_turn)
+                except Exception as error:
+                    return self._fail_step(scheduler.read_plan(counts), error)
                 if tokens is not None:
                     self._counters["steps"] += len(tokens)
                     self._counters["decode_calls"] += counts[0] * len(tokens)
@@ -203,18 +224,29 @@ class Runtime:
                         events.extend(scheduler.complete_ordered(later))
                     return events
         plan = scheduler.read_plan(counts)
-        for request in plan.failed:
-            self._errors[request.id] = request.error or "failed"
         sampled: Dict[int, int] = {}
-        if plan.segments:
+        while plan.segments:
             entries = [StepEntry(s.request.id, s.tokens, [len(s.tokens) - 1] if s.wants_logits else [])
                        for s in plan.segments]
             began = time.perf_counter_ns()
-            logits = self.stepper.step(entries)
-            wanting = [s.request for s in plan.segments if s.wants_logits]
-            if wanting:
-                tokens = sample_rows(logits, [r.sampling for r in wanting], [r.rng for r in wanting])
-                sampled = {r.id: t for r, t in zip(wanting, tokens)}
+            try:
+                logits = self.stepper.step(entries)
+                wanting = [s.request for s in plan.segments if s.wants_logits]
+                if wanting:
+                    tokens = sample_rows(logits, [r.sampling for r in wanting], [r.rng for r in wanting])
+                    sampled = {r.id: t for r, t in zip(wanting, tokens)}
+            except StepError as error:
+                # Found before anything ran or changed: the request at fault leaves, the rest of the
+                # plan stands (its pages stay reserved) and runs without it.
+                at_fault = [s for s in plan.segments if s.request.id == error.request]
+                if not at_fault:
+                    return self._fail_step(plan, error)
+                scheduler.fail(error.request, str(error))
+                plan.failed.append(at_fault[0].request)
+                plan.segments = [s for s in plan.segments if s.request.id != error.request]
+                continue
+            except Exception as error:
+                return self._fail_step(plan, error)
             elapsed = time.perf_counter_ns() - began
             self._counters["steps"] += 1
             prompt_tokens = sum(len(s.tokens) for s in plan.segments if len(s.tokens) > 1)
@@ -225,18 +257,54 @@ class Runtime:
             else:
                 self._counters["decode_calls"] += len(plan.segments)
                 self._counters["decode_ns"] += elapsed
+            break
         return scheduler.complete(plan, sampled)
+
+    def _fail_step(self, plan, error: Exception) -> List[Tuple[int, int, int]]:
+        """A step failed while it ran (or for a reason that names no request): what the cache
+        holds of the requests that took part cannot be trusted any more (fixed-size state is
+        updated in place), so each of them ends with an error and gives back its pages and slot.
+        Requests that were not in the step are untouched and go on with the next one."""
+        text = f"the step failed: {type(error).__name__}: {error}"
+        for segment in plan.segments:
+            self.scheduler.fail(segment.request.id, text)
+            plan.failed.append(segment.request)
+        plan.segments = []
+        self._counters["failed_steps"] = self._counters.get("failed_steps", 0) + 1
+        return self.scheduler.complete(plan, {})
+
+    def _note(self, events: List[Tuple[int, int, int]]) -> None:
+        """Keeps what the runtime itself needs of new events: the output so far of live tasks
+        (for ``run``), the error text of tasks that failed; and lets the scheduler forget a task
+        once its last event is on its way to the caller, so that a long-lived runtime does not
+        grow with every task it has served."""
+        scheduler = self.scheduler
+        for task, value, kind in events:
+            if kind == EVENT_TOKEN:
+                self._outputs.setdefault(task, []).append(value)
+            elif kind in (EVENT_FINISHED, EVENT_ERROR):
+                tokens = self._outputs.pop(task, [])
+                if self._collecting is not None:
+                    self._collecting[task] = tokens
+                if kind == EVENT_ERROR:
+                    request = scheduler.requests.get(task)
+                    self._errors[task] = (request.error if request is not None else None) or "failed"
+                    while len(self._errors) > MAX_KEPT_ERRORS:
+                        self._errors.pop(next(iter(self._errors)))
+                scheduler.forget(task)
 
     # ----- blocking generation ------------------------------------------------------------
     def generate(self, prompt: Sequence[int], max_tokens: int,
                  callback: Optional[Callable[[int], Optional[bool]]] = None, **sampling) -> List[int]:
         """Generates up to ``max_tokens`` tokens after ``prompt``; ``callback(token)`` is
         called for each and stops the generation by returning False (as the reference's
-        generate, src/flyweight/v2.py:3837-3876). Greedy unless sampling settings are given."""
+        generate, src/flyweight/v2.py:3837-3876). Greedy unless sampling settings are given.
+        Events of other tasks that move meanwhile are kept for the next ``engine_step``."""
         task = self.task_submit(prompt, max_tokens, **sampling)
         produced: List[int] = []
         while True:
             events = self.engine_step()
+            self._held_events.extend(event for event in events if event[0] != task)
             for task_id, value, kind in events:
                 if task_id != task:
                     continue
@@ -254,10 +322,18 @@ class Runtime:
                 return produced
 
     def run(self) -> Dict[int, List[int]]:
-        """Steps until every submitted task has ended; returns task id -> generated tokens."""
-        while self.scheduler.has_work():
-            self.engine_step()
-        return {task: list(request.generated) for task, request in self.scheduler.requests.items()}
+        """Steps until every submitted task has ended; returns task id -> generated tokens for
+        the tasks that ended meanwhile (a failed task: what it had generated; its text is in
+        ``task_error``). Events are not handed out."""
+        self.prepare()
+        self._collecting = {}
+        try:
+            while self.scheduler.has_work():
+                self.engine_step()
+            return self._collecting
+        finally:
+            self._collecting = None
+            self._held_events = []
 
     # ----- counters ---------------------------------------------------------------------
     @property

@@ -116,7 +116,9 @@ class StepPlan:
 
 class Scheduler:
     def __init__(self, cache: CacheManager, max_positions: int, max_batch_tokens: int = 2048,
-                 chunk_size: int = 512, max_live: Optional[int] = None):
+                 chunk_size: int = 512, max_live: Optional[int] = None, vocab_size: Optional[int] = None):
+        """``vocab_size``: token ids of prompts and stop tokens are checked against it when a
+        request is submitted (None: the vocabulary is not known here and nothing is checked)."""
         if max_batch_tokens < 1 or chunk_size < 1:
             raise SchedulerError("max_batch_tokens and chunk_size must be positive")
         self.cache = cache
@@ -127,7 +129,7 @@ class Scheduler:
         self.requests: Dict[int, Request] = {}
         self._lib = host.library()
         self._native = self._lib.fwh_scheduler_create(cache.native_handle, max_positions, max_batch_tokens, chunk_size,
-                                                      self.max_live, MAX_QUEUED)
+                                                      self.max_live, MAX_QUEUED, int(vocab_size or 0))
         if not self._native:
             raise SchedulerError(host.last_error())
         self._serial = 0
@@ -160,6 +162,26 @@ class Scheduler:
             return False
         return bool(self._lib.fwh_scheduler_cancel(self._native, int(request_id)))
 
+    def fail(self, request_id: int, message: str) -> bool:
+        """Ends one request with an error: it gives back what it holds and leaves the plan made
+        last (whose other segments stand); its error event comes out of that plan's completion.
+        False if it has ended already."""
+        if request_id not in self.requests:
+            return False
+        status = self._lib.fwh_scheduler_fail(self._native, int(request_id), str(message).encode("utf-8", "replace"))
+        if status < 0:
+            raise SchedulerError(host.last_error())
+        return bool(status)
+
+    def forget(self, request_id: int) -> bool:
+        """Drops the record of a request that has ended (its prompt, its output, its error text)."""
+        request = self.requests.get(request_id)
+        if request is None or not self._lib.fwh_scheduler_forget(self._native, int(request_id)):
+            return False
+        del self.requests[request_id]
+        self._drawing.discard(request_id)
+        return True
+
     def has_work(self) -> bool:
         return bool(self._lib.fwh_scheduler_has_work(self._native))
 
@@ -188,8 +210,8 @@ class Scheduler:
     # buffer and ``complete_ordered`` finishes it; ``read_plan`` gives any plan as objects.
     def plan_next(self):
         """Plans the next step (pages reserved); returns its counts: segments, tokens,
-        preempted, failed, admitted, cancelled."""
-        counts = host.ints(6)
+        preempted, failed, admitted, cancelled, and the most tokens its block tables cover."""
+        counts = host.ints(7)
         if self._lib.fwh_scheduler_schedule(self._native, counts) < 0:
             raise SchedulerError(host.last_error())
         self._serial += 1

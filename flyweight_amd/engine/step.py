@@ -22,7 +22,12 @@ from .model import CacheView, CausalLM
 
 
 class StepError(ValueError):
-    pass
+    """What a step refuses, found before anything ran or changed. ``request`` names the entry
+    at fault where there is one, so that a caller can leave that request out and run the rest."""
+
+    def __init__(self, message: str, request: Hashable = None):
+        super().__init__(message)
+        self.request = request
 
 
 @dataclass
@@ -44,40 +49,40 @@ def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size:
         seen = set()
         for request in requests:
             if request in seen:
-                raise StepError(f"request {request!r} appears twice in one step")
+                raise StepError(f"request {request!r} appears twice in one step", request)
             seen.add(request)
     natives = cache.natives_of(requests)
     try:
         lengths, slots = cache.describe(requests, natives)
     except KeyError as error:
-        raise StepError(f"request {error.args[0]!r} was not admitted") from None
+        raise StepError(f"request {error.args[0]!r} was not admitted", error.args[0]) from None
     if all(len(entry.tokens) == 1 for entry in entries):
         # a decode step: the same checks without a loop over the entries' fields
         tokens = [entry.tokens[0] for entry in entries]
         if max(lengths) + 1 > max_positions:
             entry, start = next((e, s) for e, s in zip(entries, lengths) if s + 1 > max_positions)
-            raise StepError(f"request {entry.request!r} would reach {start + 1} tokens; the model's limit is {max_positions}")
+            raise StepError(f"request {entry.request!r} would reach {start + 1} tokens; the model's limit is {max_positions}", entry.request)
         if not (0 <= int(min(tokens)) and int(max(tokens)) < vocab_size):
             entry = next(e for e in entries if not 0 <= int(e.tokens[0]) < vocab_size)
-            raise StepError(f"token id {entry.tokens[0]} of request {entry.request!r} is outside the vocabulary (0..{vocab_size - 1})")
+            raise StepError(f"token id {entry.tokens[0]} of request {entry.request!r} is outside the vocabulary (0..{vocab_size - 1})", entry.request)
         for entry in entries:
             for place in entry.want:
                 if int(place) != 0:
-                    raise StepError(f"request {entry.request!r} wants logits at place {place} of 1 tokens")
+                    raise StepError(f"request {entry.request!r} wants logits at place {place} of 1 tokens", entry.request)
         return lengths, slots, natives
     for entry, start in zip(entries, lengths):
         n = len(entry.tokens)
         if n < 1:
-            raise StepError(f"request {entry.request!r} brings no tokens")
+            raise StepError(f"request {entry.request!r} brings no tokens", entry.request)
         if start + n > max_positions:
-            raise StepError(f"request {entry.request!r} would reach {start + n} tokens; the model's limit is {max_positions}")
+            raise StepError(f"request {entry.request!r} would reach {start + n} tokens; the model's limit is {max_positions}", entry.request)
         low, high = (min(entry.tokens), max(entry.tokens)) if n > 1 else (entry.tokens[0], entry.tokens[0])
         if not (0 <= int(low) and int(high) < vocab_size):
             bad = next(t for t in entry.tokens if not 0 <= int(t) < vocab_size)
-            raise StepError(f"token id {bad} of request {entry.request!r} is outside the vocabulary (0..{vocab_size - 1})")
+            raise StepError(f"token id {bad} of request {entry.request!r} is outside the vocabulary (0..{vocab_size - 1})", entry.request)
         for place in entry.want:
             if not 0 <= int(place) < n:
-                raise StepError(f"request {entry.request!r} wants logits at place {place} of {n} tokens")
+                raise StepError(f"request {entry.request!r} wants logits at place {place} of {n} tokens", entry.request)
     return lengths, slots, natives
 
 
@@ -267,21 +272,29 @@ class Stepper:
     """Owns the model's cache and runs steps. ``admit`` a request before its first step,
     ``release`` it when it ends."""
 
-    def __init__(self, model: CausalLM, num_pages: int, max_requests: int, page_size: int = 64):
+    def __init__(self, model: CausalLM, num_pages: int, max_requests: int, page_size: int = 64,
+                 context_limit: Optional[int] = None):
+        """``context_limit``: the most tokens one request may reach here, at most the model's
+        own limit (the default). Block tables and everything sized by a sequence's length follow
+        this number, not the model's: a model that allows 128,000 positions costs a run of 4,096
+        no more than one that allows 4,096."""
         if not model.bound:
             raise StepError("the model has no weights yet")
         self.model = model
         self.device = model.device
-        max_pages = (model.spec.max_positions + page_size - 1) // page_size
+        self.context_limit = min(int(context_limit or model.spec.max_positions), model.spec.max_positions)
+        if self.context_limit < 1:
+            raise StepError("the context limit must be positive")
+        max_pages = (self.context_limit + page_size - 1) // page_size
         self.cache = CacheManager(model.cache_needs(), num_pages=num_pages, max_requests=max_requests,
                                   page_size=page_size, max_pages_per_request=max_pages, dtype=model.dtype,
                                   device=model.device)
         self.steps = 0
         self.tokens_run = 0
         # decode steps (every segment one token) are captured in a HIP graph per batch size and
-        # replayed, if every part of the model allows it
+        # context bucket and replayed, if every part of the model allows it
         self.use_graphs = all(block.graph_safe for block in model.layers) and model.final_norm.graph_safe
-        self._graphs: Dict[int, "_CapturedDecode"] = {}
+        self._graphs: Dict[tuple, "_CapturedDecode"] = {}
         self.graph_replays = 0
 
     def admit(self, request: Hashable) -> None:
@@ -295,33 +308,54 @@ class Stepper:
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Returns float32 logits [wanted, vocab] on the device, rows in the order of the
-        entries and of each entry's ``want`` (None if nothing is wanted). Raises
-        OutOfPages, having changed nothing, when the cache cannot hold the new tokens."""
+        entries and of each entry's ``want`` (None if nothing is wanted). Raises StepError
+        (naming the request at fault) or OutOfPages, having changed nothing, when an entry is
+        refused or the cache cannot hold the new tokens."""
         cache = self.cache
         spec = self.model.spec
-        described = check_entries(entries, cache, spec.vocab_size, spec.max_positions)
+        described = check_entries(entries, cache, spec.vocab_size, self.context_limit)
         requests = [entry.request for entry in entries]
         new_lengths = [start + len(entry.tokens) for entry, start in zip(entries, described[0])]
         # reserve everything first so that a failure leaves no request half-served
         cache.reserve_all(requests, new_lengths, described[2])
-        if self.use_graphs and all(len(entry.tokens) == 1 for entry in entries):
-            return self._replay(self._decode_step(len(entries)), entries, described)
-        ctx = StepContext(entries, cache, self.device, spec.vocab_size, spec.max_positions, described=described)
-        logits = self.model.forward(ctx, cache)
+        try:
+            if self.use_graphs and all(len(entry.tokens) == 1 for entry in entries):
+                return self._replay(self._decode_step(len(entries), max(new_lengths)), entries, described)
+            ctx = StepContext(entries, cache, self.device, spec.vocab_size, self.context_limit, described=described)
+            logits = self.model.forward(ctx, cache)
+        except BaseException:
+            # The lengths stay where they were and the pages reserved for this step go back. What
+            # the kernels that did run have written past those lengths is never read; fixed-size
+            # state of the step's requests may have moved on, though: the caller has to release them.
+            cache.drop_reservations(requests, described[2])
+            raise
         cache.commit_all(ctx.requests, ctx.new_lengths, described[2])
         self.steps += 1
         self.tokens_run += ctx.num_rows
         return logits
 
     # ----- captured decode steps ----------------------------------------------------------
-    def _decode_step(self, batch: int) -> "_CapturedDecode":
-        """The decode step of this many rows with its persistent index arrays."""
-        captured = self._graphs.get(batch)
+    def kept_pages(self, context: int) -> int:
+        """The block-table width (pages) of the captured step that serves sequences of up to
+        ``context`` tokens: the next power of two, at least one run of the split-key decode
+        kernel, at most what the context limit needs. The split-key grid, the workspace of partial
+        results and the uploaded block-table rows are sized by this, so a step costs what the live
+        sequences need, and a request that grows past a bucket moves on to the next step recorded."""
+        cache = self.cache
+        pages = max(cache.pages_for(context), ops.DECODE_SPLIT_PAGES)
+        bucket = 1 << (pages - 1).bit_length()
+        return max(1, min(bucket, cache.max_pages_per_request))
+
+    def _decode_step(self, batch: int, context: int) -> "_CapturedDecode":
+        """The decode step of this many rows for sequences of up to ``context`` tokens (after the
+        step), with its persistent index arrays."""
+        pages = self.kept_pages(context)
+        captured = self._graphs.get((batch, pages))
         if captured is None:
             cache = self.cache
-            ctx = StepContext.for_decode_graph(batch, cache, self.device, max_context=self.model.spec.max_positions,
-                                               table_stride=cache.max_pages_per_request)
-            captured = self._graphs[batch] = _CapturedDecode(ctx)
+            ctx = StepContext.for_decode_graph(batch, cache, self.device, max_context=pages * cache.page_size,
+                                               table_stride=pages)
+            captured = self._graphs[(batch, pages)] = _CapturedDecode(ctx)
         return captured
 
     @staticmethod
@@ -336,10 +370,10 @@ class Stepper:
         multiple = 8 if rows <= 64 else 16
         return (rows + multiple - 1) // multiple * multiple
 
-    def planned_decode(self, rows: int) -> Optional["_CapturedDecode"]:
-        """The decode step that serves a scheduler's plan of ``rows`` single tokens, or None
-        where decode steps are not recorded."""
-        return self._decode_step(self.kept_batch(rows)) if self.use_graphs else None
+    def planned_decode(self, rows: int, context: int) -> Optional["_CapturedDecode"]:
+        """The decode step that serves a scheduler's plan of ``rows`` single tokens whose
+        sequences reach at most ``context`` tokens, or None where decode steps are not recorded."""
+        return self._decode_step(self.kept_batch(rows), context) if self.use_graphs else None
 
     def _run(self, captured: "_CapturedDecode") -> None:
         """Runs the step whose index arrays have been uploaded; its logits are ``captured.logits``
@@ -416,10 +450,12 @@ class Stepper:
         cache.commit_all(ctx.requests, ctx.new_lengths, None if described is None else described[2])
         self.steps += 1
         self.tokens_run += ctx.num_rows
-        wanted = [i for i, entry in enumerate(entries) if len(entry.want)]
+        # one row of logits for every wanted place, as the eager path gives them (an entry of one
+        # token may name its place more than once)
+        wanted = [i for i, entry in enumerate(entries) for _ in entry.want]
         if not wanted:
             return None
-        if len(wanted) == len(entries):
+        if wanted == list(range(len(entries))):
             return captured.logits          # overwritten by the next replay of this batch size
         return captured.logits[wanted]
 

@@ -14,7 +14,7 @@ import sys
 from typing import IO, List, Optional
 
 PAGE_SIZE = 64
-MAX_LIVE = 8
+MAX_LIVE_SLOTS = 64     # state slots are memory per request: bounded even when the pool is large
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -28,7 +28,8 @@ def build_parser() -> argparse.ArgumentParser:
     parser.add_argument("--out", required=True, metavar="DIR", help="where the logits files go")
     parser.add_argument("--max-tokens", required=True, type=int, metavar="N",
                         help="the most tokens live requests hold at any time, each request rounded up to a multiple "
-                             f"of {PAGE_SIZE}; the cache pool is made for this many")
+                             f"of {PAGE_SIZE}; the cache pool is made for this many. As many requests may be live "
+                             f"as the pool has pages (a request holds at least one), at most {MAX_LIVE_SLOTS}")
     parser.add_argument("--device", default="cuda:0", help=argparse.SUPPRESS)
     return parser
 
@@ -46,7 +47,7 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[
     os.makedirs(out_dir, exist_ok=True)
     _, model = load_model(model_dir, dtype=dtype, device=device)
     num_pages = (max_tokens + PAGE_SIZE - 1) // PAGE_SIZE
-    stepper = Stepper(model, num_pages=num_pages, max_requests=MAX_LIVE, page_size=PAGE_SIZE)
+    stepper = Stepper(model, num_pages=num_pages, max_requests=min(num_pages, MAX_LIVE_SLOTS), page_size=PAGE_SIZE)
     for number, line in enumerate(lines):
         line = line.strip()
         if not line:

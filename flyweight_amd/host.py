@@ -11,7 +11,7 @@ from .kernels.build import ensure_host_built
 
 ERROR, OUT_OF_PAGES, NO_PAGE = -1, -2, -1
 NOT_DECODE_ONLY = -3
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _LIB: Optional[ctypes.CDLL] = None
 _INTS, _IDS = POINTER(c_int), POINTER(c_int64)
@@ -34,6 +34,8 @@ _SIGNATURES = {
     "fwh_cache_admit": (c_int, [c_void_p, c_int64]),
     "fwh_cache_reserve": (c_int, [c_void_p, c_int64, c_int]),
     "fwh_cache_commit": (c_int, [c_void_p, c_int64, c_int]),
+    "fwh_cache_truncate": (c_int, [c_void_p, c_int64, c_int]),
+    "fwh_cache_truncate_batch": (c_int, [c_void_p, _IDS, _INTS, c_int]),
     "fwh_cache_release": (c_int, [c_void_p, c_int64]),
     "fwh_cache_is_live": (c_int, [c_void_p, c_int64]),
     "fwh_cache_slot_of": (c_int, [c_void_p, c_int64]),
@@ -47,10 +49,11 @@ _SIGNATURES = {
     "fwh_cache_commit_batch": (c_int, [c_void_p, _IDS, _INTS, c_int]),
     "fwh_cache_live": (c_int, [c_void_p, _IDS, c_int]),
     "fwh_cache_check": (c_int, [c_void_p]),
-    "fwh_scheduler_create": (c_void_p, [c_void_p, c_int, c_int, c_int, c_int, c_int]),
+    "fwh_scheduler_create": (c_void_p, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int]),
     "fwh_scheduler_destroy": (None, [c_void_p]),
     "fwh_scheduler_submit": (c_int64, [c_void_p, _INTS, c_int, c_int, _INTS, c_int]),
     "fwh_scheduler_cancel": (c_int, [c_void_p, c_int64]),
+    "fwh_scheduler_fail": (c_int, [c_void_p, c_int64, c_char_p]),
     "fwh_scheduler_has_work": (c_int, [c_void_p]),
     "fwh_scheduler_preemptions": (c_int, [c_void_p]),
     "fwh_scheduler_queue": (c_int, [c_void_p, c_int, _IDS, c_int]),

@@ -373,17 +373,22 @@ BIG_MIN_ROWS = 128       # up to here a 256-row tile would be at least half empt
 _MEDIUM_COUNTERS = {}
 
 
+TICKET_COUNTERS = 1 << 20      # 4 MB per device
+
+
 def _medium_counters(device: torch.device, count: int) -> torch.Tensor:
     """Zeroed int32 counters for the tickets of the kernels whose last workgroup finishes the
     work of the others (the medium product, decode attention), one set per device: each kernel
     leaves them at zero, and calls on one device follow each other in stream order (work on
-    several streams of one device at once would need a set per stream)."""
+    several streams of one device at once would need a set per stream). The set is allocated
+    once and never replaced: recorded graphs hold its address."""
     have = _MEDIUM_COUNTERS.get(device.index)
-    if have is None or have.numel() < count:
+    if have is None:
         if torch.cuda.is_current_stream_capturing():
-            raise KernelError("gemm_medium: its counters must exist before a graph is captured (prepare_device)")
-        have = torch.zeros(max(count, 65536), dtype=torch.int32, device=device)
-        _MEDIUM_COUNTERS[device.index] = have
+            raise KernelError("the ticket counters must exist before a graph is captured (prepare_device)")
+        have = _MEDIUM_COUNTERS[device.index] = torch.zeros(TICKET_COUNTERS, dtype=torch.int32, device=device)
+    if count > have.numel():
+        raise KernelError(f"a kernel asks for {count} ticket counters; the device's set holds {have.numel()}")
     return have
 
 

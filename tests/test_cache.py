@@ -50,6 +50,57 @@ def test_lifecycle_of_the_reference_contract():
     cache.check_invariants()
 
 
+def test_truncate_of_the_reference_contract():
+    # native/tests/paged_kv_contract.cpp:244-296: 64 pages; one sequence of 100 tokens (2 pages), one
+    # of 200 (4); the second cut back to 128 tokens keeps exactly 2 pages; releases leave none out
+    cache = CacheManager({0: KV}, num_pages=64, max_requests=2)
+    pool = cache.groups[0].pool
+    cache.admit("one")
+    cache.admit("two")
+    cache.reserve("one", 100)
+    assert len(cache.groups[0].tables["one"]) == 2 and pool.free_count == 62
+    cache.reserve("two", 200)
+    cache.commit("two", 200)
+    assert len(cache.groups[0].tables["two"]) == 4 and pool.free_count == 58
+    kept = cache.groups[0].tables["two"][:2]
+    cache.truncate("two", 128)
+    assert cache.groups[0].tables["two"] == kept and pool.free_count == 60 and cache.length_of("two") == 128
+    cache.check_invariants()
+    cache.truncate("two", 129)          # one token more would need a third page: nothing to give back
+    assert len(cache.groups[0].tables["two"]) == 2
+    cache.release("one")
+    assert pool.free_count == 62
+    cache.release("two")
+    assert pool.free_count == 64
+    cache.check_invariants()
+
+
+def test_truncate_drops_reservations_but_never_rewinds_state_or_a_window():
+    cache = CacheManager(NEEDS, num_pages=6, max_requests=3)
+    cache.admit("r")
+    cache.reserve("r", 70)
+    cache.commit("r", 70)
+    cache.reserve("r", 200)             # a step that will not run after all
+    assert cache.groups[0].pool.in_use == 4
+    cache.drop_reservations(["r"])
+    assert cache.groups[0].pool.in_use == 2 and cache.length_of("r") == 70
+    with pytest.raises(CacheAccountingError, match="fixed-size state"):
+        cache.truncate("r", 10)         # the state slot has seen 70 tokens and cannot go back
+    cache.check_invariants()
+    windowed = CacheManager({0: PagedKV(1, 16, window=70)}, num_pages=8, max_requests=1)
+    windowed.admit("w")
+    windowed.reserve("w", 300)
+    windowed.commit("w", 300)           # keys before 231 are gone: blocks 0..2 were given back
+    assert windowed.groups[0].tables["w"][:3] == [-1, -1, -1]
+    windowed.truncate("w", 280)         # needs keys from 211 on: block 3 onwards, all there
+    assert windowed.length_of("w") == 280
+    with pytest.raises(CacheAccountingError, match="window has passed"):
+        windowed.truncate("w", 200)     # would need keys from 131 on: block 2 is gone
+    windowed.check_invariants()
+    windowed.release("w")
+    assert windowed.groups[0].pool.free_count == 8
+
+
 def test_groups_share_pages_across_their_layers_and_slots_across_states():
     cache = CacheManager(NEEDS, num_pages=6, max_requests=3, device=torch.device("cpu"))
     assert len(cache.groups) == 1 and cache.groups[0].entries == [1, 3]

@@ -343,6 +343,105 @@ def test_errors_are_reported_not_hidden(loaded):
     assert stepper.step([StepEntry("a", [1] * 64, [63])]).shape == (1, m.config.vocab_size)
 
 
+def _run_to_the_end(runtime):
+    events = []
+    while runtime.scheduler.has_work():
+        events += runtime.engine_step()
+    return events
+
+
+@pytest.mark.parametrize("bad_place", [3, 21])
+def test_a_request_the_step_refuses_ends_alone_and_the_others_go_on(loaded, bad_place):
+    """Three tasks, the middle one with a token id outside the vocabulary in its first portion or
+    in its second (the scheduler here does not know the vocabulary, so only the step finds it):
+    it ends with an error event and its text, the other two generate the plain model's tokens,
+    and every page and slot is back."""
+    from flyweight_amd.engine import EVENT_ERROR, EVENT_FINISHED, EVENT_TOKEN, EngineError, Scheduler
+    m = loaded("A", "float32")
+    config, weights = m.plain_config, m.plain_weights
+    vocab = m.config.vocab_size
+    good = [random_tokens(vocab, 30, seed=5), random_tokens(vocab, 19, seed=6)]
+    bad = random_tokens(vocab, 40, seed=7)
+    bad[bad_place] = vocab
+    runtime = _runtime(m, parallel_sequences=4, prefill_rows=16, max_batch_tokens=40, num_pages=6)
+    with pytest.raises(EngineError, match=f"token id {vocab} at place {bad_place} of the prompt is outside the vocabulary"):
+        runtime.task_submit(bad, 5)
+    with pytest.raises(EngineError, match="stop token"):
+        runtime.task_submit(good[0], 5, stop_tokens=[vocab + 7])
+    assert not runtime.scheduler.has_work()
+    runtime.scheduler = Scheduler(runtime.stepper.cache, max_positions=runtime.context_limit, max_batch_tokens=40,
+                                  chunk_size=16, max_live=4)      # no vocabulary: nothing is checked at submit
+    first = runtime.task_submit(good[0], 8)
+    middle = runtime.task_submit(bad, 8)
+    last = runtime.task_submit(good[1], 8)
+    events = _run_to_the_end(runtime)
+    assert [e[2] for e in events if e[0] == middle and e[2] != 3] == [EVENT_ERROR]
+    assert any(e[0] == middle and e[2] == 3 for e in events) == (bad_place >= 16)      # its first portion ran
+    assert "outside the vocabulary" in runtime.task_error(middle) and runtime.task_error(first) is None
+    for task, prompt in ((first, good[0]), (last, good[1])):
+        assert [e[1] for e in events if e[0] == task and e[2] == EVENT_TOKEN] == plain.greedy(config, weights, prompt, 8)
+        assert [e[2] for e in events if e[0] == task][-1] == EVENT_FINISHED
+    assert runtime.info["pages_free"] == 6 and runtime.info["slots_free"] == 4 and runtime.info["live_requests"] == 0
+    runtime.stepper.cache.check_invariants()
+    assert not runtime.scheduler.requests, "finished tasks are forgotten once their last event is handed out"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_step_that_fails_while_it_runs_ends_its_requests_only(loaded, dtype, monkeypatch):
+    """A kernel refuses in the middle of a step (forced here from the host: the third forward pass
+    raises before it launches anything): the requests of that step end with an error, their pages
+    and slots come back, and the request that was still waiting runs to the plain model's tokens."""
+    from flyweight_amd.engine import EVENT_ERROR, EVENT_TOKEN
+    from flyweight_amd.kernels.ops import KernelError
+    m = loaded("B", dtype)
+    vocab = m.config.vocab_size
+    prompts = [random_tokens(vocab, n, seed=40 + n) for n in (20, 33, 25)]
+    runtime = _runtime(m, parallel_sequences=2, prefill_rows=16, max_batch_tokens=32, num_pages=5)
+    tasks = [runtime.task_submit(p, 6) for p in prompts]      # two slots: the third waits
+    calls = {"n": 0}
+    forward = m.model.forward
+
+    def failing(ctx, cache):
+        calls["n"] += 1
+        if calls["n"] == 3:
+            raise KernelError("forced: a kernel refused its operands")
+        return forward(ctx, cache)
+    monkeypatch.setattr(m.model, "forward", failing)
+    events = _run_to_the_end(runtime)
+    monkeypatch.undo()
+    for task in tasks[:2]:
+        assert [e[2] for e in events if e[0] == task][-1] == EVENT_ERROR
+        assert "KernelError" in runtime.task_error(task) and "forced" in runtime.task_error(task)
+    got = [e[1] for e in events if e[0] == tasks[2] and e[2] == EVENT_TOKEN]
+    if dtype == "float32":
+        assert got == plain.greedy(m.plain_config, m.plain_weights, prompts[2], 6)
+    assert len(got) == 6 and runtime.info["failed_steps"] == 1
+    assert runtime.info["pages_free"] == 5 and runtime.info["slots_free"] == 2
+    runtime.stepper.cache.check_invariants()
+    # the runtime is as good as new: the same prompts again, nothing forced
+    again = [runtime.task_submit(p, 6) for p in prompts]
+    result = runtime.run()
+    if dtype == "float32":
+        for task, prompt in zip(again, prompts):
+            assert result[task] == plain.greedy(m.plain_config, m.plain_weights, prompt, 6)
+    assert sorted(result) == sorted(again)
+
+
+def test_generate_beside_other_tasks_keeps_their_events(loaded):
+    from flyweight_amd.engine import EVENT_FINISHED, EVENT_TOKEN
+    m = loaded("A", "float32")
+    vocab = m.config.vocab_size
+    other_prompt, own_prompt = random_tokens(vocab, 12, seed=1), random_tokens(vocab, 7, seed=2)
+    runtime = _runtime(m, parallel_sequences=2)
+    other = runtime.task_submit(other_prompt, 9)
+    own = runtime.generate(own_prompt, 4)
+    assert own == plain.greedy(m.plain_config, m.plain_weights, own_prompt, 4)
+    events = _run_to_the_end(runtime) + runtime.engine_step()
+    assert [e[1] for e in events if e[0] == other and e[2] == EVENT_TOKEN] == plain.greedy(m.plain_config, m.plain_weights, other_prompt, 9)
+    assert [e[2] for e in events if e[0] == other][-1] == EVENT_FINISHED
+    assert not runtime.scheduler.requests
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_captured_decode_steps_replay_to_the_eager_result(loaded, dtype):
     """Decode steps are recorded in a HIP graph per batch size and replayed. Every replay,

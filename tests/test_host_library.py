@@ -57,19 +57,23 @@ def test_scheduler_through_the_c_entry_points():
     lib = host.library()
     windows = (ctypes.c_int * 1)(0)
     cache = lib.fwh_cache_create(1, windows, 8, 2, 64, 0)
-    scheduler = lib.fwh_scheduler_create(cache, 512, 96, 64, 0, 2)
+    scheduler = lib.fwh_scheduler_create(cache, 512, 96, 64, 0, 2, 100)
     try:
         prompt = (ctypes.c_int * 70)(*range(70))
         none = (ctypes.c_int * 1)()
         assert lib.fwh_scheduler_submit(scheduler, prompt, 0, 4, none, 0) == host.ERROR and "empty" in host.last_error()
         assert lib.fwh_scheduler_submit(scheduler, prompt, 70, 500, none, 0) == host.ERROR and "context" in host.last_error()
+        prompt[3] = 100     # the vocabulary given above has 100 entries
+        assert lib.fwh_scheduler_submit(scheduler, prompt, 70, 2, none, 0) == host.ERROR and "place 3" in host.last_error()
+        prompt[3] = 3
+        assert lib.fwh_scheduler_submit(scheduler, prompt, 70, 2, (ctypes.c_int * 1)(-1), 1) == host.ERROR and "stop token" in host.last_error()
         first = lib.fwh_scheduler_submit(scheduler, prompt, 70, 2, none, 0)
         second = lib.fwh_scheduler_submit(scheduler, prompt, 40, 2, (ctypes.c_int * 1)(5), 1)
         assert (first, second) == (1, 2)
         assert lib.fwh_scheduler_submit(scheduler, prompt, 3, 1, none, 0) == host.ERROR and "queue" in host.last_error()
-        counts = host.ints(6)
+        counts = host.ints(7)
         assert lib.fwh_scheduler_schedule(scheduler, counts) == 0
-        assert list(counts) == [2, 96, 0, 0, 2, 0]      # a portion of 64, then 32 of the second prompt: the budget
+        assert list(counts) == [2, 96, 0, 0, 2, 0, 64]  # a portion of 64, then 32 of the second prompt: the budget; a page each
         owners, lengths, wants, tokens = host.ids(2), host.ints(2), host.ints(2), host.ints(96)
         lib.fwh_plan_segments(scheduler, owners, lengths, wants, tokens)
         assert list(owners) == [1, 2] and list(lengths) == [64, 32] and list(wants) == [0, 0]

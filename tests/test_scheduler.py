@@ -72,6 +72,20 @@ def test_submit_validation():
         scheduler.submit([1], 1)
 
 
+def test_token_ids_are_checked_against_the_vocabulary_at_submit():
+    cache = CacheManager(NEEDS, num_pages=8, max_requests=4)
+    scheduler = Scheduler(cache, max_positions=4096, vocab_size=97)
+    with pytest.raises(SchedulerError, match=r"token id 97 at place 2 of the prompt is outside the vocabulary \(0\.\.96\)"):
+        scheduler.submit([1, 96, 97], 4)
+    with pytest.raises(SchedulerError, match="token id -1 at place 0"):
+        scheduler.submit([-1], 4)
+    with pytest.raises(SchedulerError, match="stop token 500"):
+        scheduler.submit([1], 4, stop_tokens=[500])
+    assert not scheduler.has_work() and not scheduler.requests
+    scheduler.submit([0, 96], 4, stop_tokens=[96])
+    assert scheduler.has_work()
+
+
 def test_prompt_is_cut_into_portions_under_the_budget_and_decodes_come_first():
     cache, scheduler = make(num_pages=16, max_batch_tokens=24, chunk_size=16)
     a = scheduler.submit(list(range(40)), 5)
@@ -222,3 +236,76 @@ def test_a_plain_decode_step_goes_through_arrays_and_decides_the_same():
         results.append((log, {r.id: r.generated for r in scheduler.requests.values()}))
     assert results[0] == results[1]
     assert any(len(events) >= 3 and all(kind == EVENT_TOKEN for _, _, kind in events) for events in results[1][0])
+
+
+def drive_with_failures(scheduler, cache, refuses, max_steps=1000):
+    """``drive`` with a step function that fails: ``refuses(segment)`` true means the step would
+    refuse that segment before anything ran, as a check of the entries does. The request at fault
+    is failed, the rest of the plan runs."""
+    seen = {}
+    steps = 0
+    while scheduler.has_work():
+        plan = scheduler.schedule()
+        for segment in list(plan.segments):
+            if refuses(segment):
+                assert scheduler.fail(segment.request.id, f"refused at {segment.request.computed}")
+                plan.segments.remove(segment)
+                plan.failed.append(segment.request)
+        for segment in plan.segments:       # the others' reservations stand
+            r = segment.request
+            assert r.live and cache.pages_missing(r.id, r.computed + len(segment.tokens)) == {0: 0}
+        sampled = {s.request.id: oracle(s.request.tokens) for s in plan.segments if s.wants_logits}
+        for event in scheduler.complete(plan, sampled):
+            seen.setdefault(event[0], []).append(event)
+        cache.check_invariants()
+        steps += 1
+        assert steps < max_steps
+    return seen
+
+
+@pytest.mark.parametrize("fails_at", [0, 16, 37])
+def test_one_request_that_fails_leaves_the_others_running(fails_at):
+    """Three requests, the middle one fails in its first portion, in its second, or while it decodes:
+    it ends with one error event and gives everything back, the other two produce what they
+    produce alone."""
+    cache, scheduler = make(num_pages=8, max_requests=4, max_batch_tokens=48, chunk_size=16)
+    first = scheduler.submit(list(range(30)), 6)
+    bad = scheduler.submit(list(range(5, 40)), 6)
+    last = scheduler.submit(list(range(7, 20)), 6)
+    seen = drive_with_failures(scheduler, cache, lambda s: s.request is bad and s.request.computed + len(s.tokens) > fails_at)
+    assert [kind for _, _, kind in seen[bad.id] if kind != EVENT_PREFILL] == [EVENT_TOKEN] * (3 if fails_at == 37 else 0) + [EVENT_ERROR]
+    assert bad.finished and not bad.live and "refused at" in bad.error
+    assert not scheduler.fail(bad.id, "again")          # it has ended already
+    assert first.generated == expected_tokens(list(range(30)), 6)
+    assert last.generated == expected_tokens(list(range(7, 20)), 6)
+    assert [kind for _, _, kind in seen[first.id]][-1] == EVENT_FINISHED
+    assert cache.stats()["pages_free"] == 8 and cache.stats()["slots_free"] == 4 and not cache.requests
+
+
+def test_a_whole_step_that_fails_ends_its_requests_and_the_queue_goes_on():
+    cache, scheduler = make(num_pages=8, max_requests=2, max_batch_tokens=64, chunk_size=32)
+    a, b = scheduler.submit([1] * 20, 3), scheduler.submit([2] * 20, 3)
+    waiting = scheduler.submit([3] * 20, 3)             # no slot for it yet
+    plan = scheduler.schedule()
+    assert [s.request for s in plan.segments] == [a, b]
+    for segment in plan.segments:                       # the step failed while it ran
+        scheduler.fail(segment.request.id, "the step failed")
+    plan.failed.extend(s.request for s in plan.segments)
+    plan.segments = []
+    events = scheduler.complete(plan, {})
+    assert sorted(events) == [(a.id, 0, EVENT_ERROR), (b.id, 0, EVENT_ERROR)]
+    cache.check_invariants()
+    seen = drive(scheduler, cache)
+    assert waiting.generated == expected_tokens([3] * 20, 3) and cache.stats()["pages_free"] == 8
+
+
+def test_a_failure_between_two_plans_is_not_lost():
+    cache, scheduler = make(num_pages=8, max_requests=2)
+    a, b = scheduler.submit([1] * 5, 3), scheduler.submit([2] * 5, 3)
+    plan = scheduler.schedule()
+    scheduler.complete(plan, {a.id: oracle(a.tokens), b.id: oracle(b.tokens)})
+    assert scheduler.fail(b.id, "gone")                 # no plan is outstanding
+    seen = drive(scheduler, cache)
+    assert [e for e in seen[b.id]] == [(b.id, 0, EVENT_ERROR)]
+    assert a.generated == expected_tokens([1] * 5, 3)
+    assert scheduler.forget(b.id) and b.id not in scheduler.requests and not scheduler.forget(b.id)
