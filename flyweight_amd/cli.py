@@ -50,31 +50,33 @@ def build_parser() -> argparse.ArgumentParser:
     parser = argparse.ArgumentParser(prog="flyweight-amd", description="LFM2 inference on the AMD Instinct MI355X")
     commands = parser.add_subparsers(dest="command", required=True)
 
-    generate = commands.add_parser("generate", help="print one continuation and exit")
+    generate = commands.add_parser("generate", help="generate the tokens that follow a prompt, print them, exit")
     _add_model(generate)
     request = generate.add_argument_group("request")
     request.add_argument("--tokens", "--prompt", dest="tokens", type=_token_list, metavar="IDS",
                          help="the prompt as token ids, e.g. 1,2,3")
     request.add_argument("--tokens-file", metavar="FILE", help="a file of token ids instead of --tokens")
     request.add_argument("--max-tokens", "--max-new-tokens", dest="max_new_tokens", type=int, default=64, metavar="N",
-                         help="maximum generated tokens")
+                         help="stop after this many new tokens")
     request.add_argument("--stop-token", dest="stop_tokens", type=int, action="append", default=[], metavar="ID",
-                         help="end the generation at this token (may be given several times; default: the model's eos)")
+                         help="a token id that ends the output when it is produced; repeat the option for several (without it: the eos id of the model's configuration)")
+    request.add_argument("--ignore-eos", action="store_true",
+                         help="do not end at the model's eos id either: only --stop-token ids and --max-tokens end the output")
     sampling = generate.add_argument_group("sampling")
-    sampling.add_argument("--temperature", type=float, default=0.8, metavar="X", help="sampling temperature; 0 is greedy")
-    sampling.add_argument("--top-k", type=int, default=40, metavar="N", help="how many candidates the sampler considers")
+    sampling.add_argument("--temperature", type=float, default=0.8, metavar="X", help="divides the logits before the draw; 0 always takes the most likely token")
+    sampling.add_argument("--top-k", type=int, default=40, metavar="N", help="draw among the N most likely tokens only (0: among all)")
     sampling.add_argument("--top-p", type=float, default=0.95, metavar="X",
-                          help="nucleus cut over those candidates, in (0, 1]")
+                          help="keep the most likely tokens until their probabilities add up to X, a number in (0, 1]")
     sampling.add_argument("--min-p", type=float, default=0.05, metavar="X",
-                          help="drop candidates below this fraction of the best one's probability, in [0, 1] (0 disables)")
-    sampling.add_argument("--seed", type=int, metavar="N", help="fixed RNG seed, for a sample that reproduces")
+                          help="leave out tokens less probable than X times the most probable one; X in [0, 1], 0 keeps all")
+    sampling.add_argument("--seed", type=int, metavar="N", help="start the request's random stream here, so that a run can be repeated")
     _add_runtime(generate, 32768)
 
-    benchmark = commands.add_parser("benchmark", help="measure prompt and decode speed")
+    benchmark = commands.add_parser("benchmark", help="time the prompt with its first token, then decode steps, and print the figures as JSON")
     _add_model(benchmark)
-    benchmark.add_argument("--tokens", type=_token_list, default=[0], metavar="IDS", help="the prompt as token ids")
-    benchmark.add_argument("--warmup", type=int, default=3, metavar="N", help="untimed decode steps")
-    benchmark.add_argument("--iterations", type=int, default=128, metavar="N", help="timed decode steps")
+    benchmark.add_argument("--tokens", type=_token_list, default=[0], metavar="IDS", help="token ids of the prompt, comma-separated")
+    benchmark.add_argument("--warmup", type=int, default=3, metavar="N", help="decode steps before the clock starts")
+    benchmark.add_argument("--iterations", type=int, default=128, metavar="N", help="decode steps under the clock")
     benchmark.add_argument("--temperature", type=float, default=0.0)
     benchmark.add_argument("--top-k", type=int, default=0)
     benchmark.add_argument("--top-p", type=float, default=0.0)
@@ -117,7 +119,7 @@ def _generate(args) -> int:
         return 2
     model, runtime = _runtime(args)
     stops = list(args.stop_tokens)
-    if not stops and model.spec.eos_token_id is not None:
+    if not stops and not args.ignore_eos and model.spec.eos_token_id is not None:
         stops = [model.spec.eos_token_id]
     produced = runtime.generate(tokens, args.max_new_tokens, stop_tokens=stops, temperature=args.temperature,
                                 top_k=args.top_k, top_p=args.top_p, min_p=args.min_p, seed=args.seed)

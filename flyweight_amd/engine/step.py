@@ -61,7 +61,7 @@ def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size:
         tokens = [entry.tokens[0] for entry in entries]
         if max(lengths) + 1 > max_positions:
             entry, start = next((e, s) for e, s in zip(entries, lengths) if s + 1 > max_positions)
-            raise StepError(f"request {entry.request!r} would reach {start + 1} tokens; the model's limit is {max_positions}", entry.request)
+            raise StepError(f"request {entry.request!r} would reach {start + 1} tokens; the context limit is {max_positions}", entry.request)
         if not (0 <= int(min(tokens)) and int(max(tokens)) < vocab_size):
             entry = next(e for e in entries if not 0 <= int(e.tokens[0]) < vocab_size)
             raise StepError(f"token id {entry.tokens[0]} of request {entry.request!r} is outside the vocabulary (0..{vocab_size - 1})", entry.request)
@@ -75,7 +75,7 @@ def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size:
         if n < 1:
             raise StepError(f"request {entry.request!r} brings no tokens", entry.request)
         if start + n > max_positions:
-            raise StepError(f"request {entry.request!r} would reach {start + n} tokens; the model's limit is {max_positions}", entry.request)
+            raise StepError(f"request {entry.request!r} would reach {start + n} tokens; the context limit is {max_positions}", entry.request)
         low, high = (min(entry.tokens), max(entry.tokens)) if n > 1 else (entry.tokens[0], entry.tokens[0])
         if not (0 <= int(low) and int(high) < vocab_size):
             bad = next(t for t in entry.tokens if not 0 <= int(t) < vocab_size)

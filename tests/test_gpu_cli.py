@@ -30,8 +30,8 @@ def test_generate_prints_the_plain_models_greedy_tokens(folders, name, capsys, t
     prompt = random_tokens(config["vocab_size"], 11, seed=4)
     expected = plain.greedy(config, weights, prompt, 6)
     ids = ",".join(str(t) for t in prompt)
-    # a stop token that the model cannot produce, so that its eos does not end the generation early
-    common = ("--max-tokens", "6", "--temperature", "0", "--dtype", "float32", "--stop-token", str(config["vocab_size"] + 7))
+    # the model's eos must not end the generation early
+    common = ("--max-tokens", "6", "--temperature", "0", "--dtype", "float32", "--ignore-eos")
     status, out, _ = run(capsys, "generate", folders[name], "--tokens", ids, *common)
     assert status == 0 and [int(t) for t in out.split()] == expected
     # the same from a file, in turns of several decode steps; a stop token ends it behind that token
@@ -46,7 +46,7 @@ def test_generate_prints_the_plain_models_greedy_tokens(folders, name, capsys, t
 def test_generate_with_a_seed_reproduces_and_refuses_what_it_cannot_do(folders, capsys):
     folder = folders["B"]
     sampled = ("generate", folder, "--tokens", "3,1,4,1,5", "--max-tokens", "12", "--temperature", "0.8", "--top-k", "40",
-               "--seed", "7", "--stop-token", "100000")
+               "--seed", "7", "--ignore-eos")
     first = run(capsys, *sampled)
     second = run(capsys, *sampled)
     assert first[0] == 0 and first[1] == second[1] and len(first[1].split()) == 12
@@ -54,6 +54,10 @@ def test_generate_with_a_seed_reproduces_and_refuses_what_it_cannot_do(folders, 
     assert status == 2 and "--tokens" in err and out == ""
     status, out, err = run(capsys, "generate", folder, "--tokens", "1,2", "--temperature", "-1")
     assert status == 1 and "temperature" in err
+    status, out, err = run(capsys, "generate", folder, "--tokens", "1,2", "--stop-token", "100000")
+    assert status == 1 and "stop token 100000 is outside the vocabulary" in err
+    status, out, err = run(capsys, "generate", folder, "--tokens", "1,100000")
+    assert status == 1 and "token id 100000 at place 1" in err
     status, out, err = run(capsys, "generate", folder + "-missing", "--tokens", "1,2")
     assert status == 1 and err.startswith("flyweight-amd:")
 

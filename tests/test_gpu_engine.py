@@ -253,17 +253,23 @@ def test_decode_steps_are_filled_up_to_the_sizes_that_are_kept(loaded, dtype):
         runtime = _runtime(m, parallel_sequences=11, prefill_rows=64, max_batch_tokens=128, decode_steps_per_turn=steps_per_turn)
         ids = [runtime.task_submit(p, n) for p, n in zip(prompts, budgets)]
         tokens = runtime.run()
-        sizes = set(runtime.stepper._graphs)
+        sizes = {batch for batch, _ in runtime.stepper._graphs}
         assert {16, 8} <= sizes and not sizes & {9, 10, 11, 12, 13, 14, 15}, sizes
         runtime.stepper.cache.check_invariants()
         assert runtime.info["pages_free"] == runtime.num_pages and runtime.info["live_requests"] == 0
-        alone = _runtime(m, parallel_sequences=1)
-        for task, prompt, budget in zip(ids, prompts, budgets):
+        # the same requests with every decode step at its exact size: rows are independent in every
+        # kernel, so a row that only fills a step up changes nothing of the others, in bfloat16 with
+        # its fused kernels as in float32
+        exact = _runtime(m, parallel_sequences=11, prefill_rows=64, max_batch_tokens=128, decode_steps_per_turn=steps_per_turn)
+        exact.stepper.kept_batch = lambda rows: rows
+        exact_ids = [exact.task_submit(p, n) for p, n in zip(prompts, budgets)]
+        exact_tokens = exact.run()
+        assert {batch for batch, _ in exact.stepper._graphs} >= {9, 10, 11}
+        for task, exact_task, prompt, budget in zip(ids, exact_ids, prompts, budgets):
             assert len(tokens[task]) == budget
+            assert tokens[task] == exact_tokens[exact_task]
             if dtype == "float32":
                 assert tokens[task] == plain.greedy(config, weights, prompt, budget)
-            else:
-                assert tokens[task][0] == alone.generate(prompt, 1)[0]
 
 
 def test_generate_stops_at_the_token_its_callback_refuses_even_inside_a_burst(loaded):
@@ -470,6 +476,47 @@ def test_captured_decode_steps_replay_to_the_eager_result(loaded, dtype):
             out.append(logits.cpu().numpy())
         runs.append(out)
         if use_graphs:
-            assert stepper.graph_replays >= 30 and set(stepper._graphs) == {2, 3}
+            assert stepper.graph_replays >= 30 and {batch for batch, _ in stepper._graphs} == {2, 3}
     for eager, replayed in zip(*runs):
         assert eager.shape == replayed.shape and np.array_equal(eager, replayed)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_captured_decode_steps_are_sized_by_the_run_not_by_the_model(folders, tmp_path, dtype):
+    """The same weights under ``max_position_embeddings`` 128,000 and 512: the captured decode
+    steps are sized by the contexts that are live (block-table rows and split-key grid of the
+    next power of two of their pages), so the large limit costs nothing, and a sequence that
+    grows past a bucket moves to the next recorded step; the logits are the same bit for bit."""
+    import json
+    import shutil
+    from flyweight_amd.engine import StepEntry, Stepper, load_model
+    wide = str(tmp_path / "wide")
+    shutil.copytree(folders["B"], wide)
+    with open(f"{wide}/config.json") as handle:
+        raw = json.load(handle)
+    raw["max_position_embeddings"] = 128000
+    with open(f"{wide}/config.json", "w") as handle:
+        json.dump(raw, handle)
+    vocab = raw["vocab_size"]
+    runs, keys = [], []
+    for folder, limit in ((folders["B"], None), (wide, None), (wide, 4096)):
+        _, model = load_model(folder, dtype=dtype)
+        stepper = Stepper(model, num_pages=16, max_requests=3, context_limit=limit)
+        rng = np.random.default_rng(11)
+        for request in ("a", "b"):
+            stepper.admit(request)
+        stepper.step([StepEntry("a", rng.integers(0, vocab, 250).tolist(), []), StepEntry("b", rng.integers(0, vocab, 40).tolist(), [])])
+        out = []
+        for step in range(12):      # "a" goes from 250 to 262 tokens: past the first bucket of 256
+            out.append(stepper.step([StepEntry("a", [int(rng.integers(0, vocab))], [0]),
+                                     StepEntry("b", [int(rng.integers(0, vocab))], [0, 0])]).cpu().numpy())
+        assert out[0].shape == (3, vocab)       # a place named twice gives two rows, recorded step or not
+        runs.append(out)
+        keys.append(sorted(stepper._graphs))
+        assert stepper.cache.max_pages_per_request == {None: raw["max_position_embeddings"] if folder == wide else 512, 4096: 4096}[limit] // 64
+    assert keys[0] == keys[1] == keys[2] == [(2, 4), (2, 8)]
+    for other in runs[1:]:
+        for small, large in zip(runs[0], other):
+            assert np.array_equal(small, large)
+    with pytest.raises(Exception, match="context limit is 4096"):
+        stepper.step([StepEntry("a", [1] * 4000, [])])
