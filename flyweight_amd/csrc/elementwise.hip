@@ -313,6 +313,49 @@ extern "C" int fw_argmax_rows(const float* logits, int32_t* ids, int32_t* also, 
     return 0;
 }
 
+// ---- argmax for callers that cannot allocate ----------------------------------------------
+// fw_argmax_rows without a workspace argument: the best keys of the parts live in a file-scope
+// device array, of which every GPU holds its own copy at its own address until the process ends
+// (FW_ARGMAX_STATIC_MAX_ROWS * 64 keys of 8 bytes = 512 KB). The array's name is only a stand-in
+// on the host: its address on the current device is looked up once per device and kept, and that
+// pointer is what the kernels get, as they get the workspace in fw_argmax_rows. Nothing has to
+// start at zero (the first kernel writes all 64 keys of every row before the second reads them), so
+// nothing is cleared; what the last call left is overwritten. Calls that overlap on one GPU (two
+// streams, two threads) share the array and race.
+#define FW_ARGMAX_STATIC_MAX_ROWS 1024
+#define FW_ARGMAX_STATIC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned long long fw_argmax_static_scratch[FW_ARGMAX_STATIC_MAX_ROWS * ARGMAX_PARTS];
+static unsigned long long* fw_argmax_static_address[FW_ARGMAX_STATIC_MAX_DEVICES];     // per device, null until looked up
+
+extern "C" int fw_argmax_rows_static_max_rows(void) { return FW_ARGMAX_STATIC_MAX_ROWS; }
+
+extern "C" int fw_argmax_rows_static(const float* logits, int32_t* ids, int32_t* also, int32_t* advance, int rows,
+                                     int vocab, void* stream) {
+    FW_REQUIRE(vocab > 0 && rows >= 0, "argmax_rows_static: bad sizes rows=%d vocab=%d", rows, vocab);
+    FW_REQUIRE(rows <= FW_ARGMAX_STATIC_MAX_ROWS,
+               "argmax_rows_static: %d rows, but the built-in scratch holds %d (use fw_argmax_rows with a workspace)", rows,
+               FW_ARGMAX_STATIC_MAX_ROWS);
+    if (rows == 0) return 0;
+    FW_REQUIRE(logits != nullptr && ids != nullptr, "argmax_rows_static: logits and ids must be given");
+    int device = -1;
+    hipError_t status = hipGetDevice(&device);
+    FW_REQUIRE(status == hipSuccess, "argmax_rows_static: hipGetDevice failed: %s", hipGetErrorString(status));
+    FW_REQUIRE(device >= 0 && device < FW_ARGMAX_STATIC_MAX_DEVICES, "argmax_rows_static: device %d is beyond the %d this entry point keeps an address for",
+               device, FW_ARGMAX_STATIC_MAX_DEVICES);
+    unsigned long long* scratch = __atomic_load_n(&fw_argmax_static_address[device], __ATOMIC_ACQUIRE);
+    if (scratch == nullptr) {       // first call on this device: two threads at once find the same address
+        status = hipGetSymbolAddress((void**)&scratch, HIP_SYMBOL(fw_argmax_static_scratch));
+        FW_REQUIRE(status == hipSuccess && scratch != nullptr, "argmax_rows_static: the scratch array's address on device %d: %s", device,
+                   hipGetErrorString(status));
+        __atomic_store_n(&fw_argmax_static_address[device], scratch, __ATOMIC_RELEASE);
+    }
+    argmax_parts_kernel<<<dim3(ARGMAX_PARTS, rows), 256, 0, (hipStream_t)stream>>>(logits, scratch, vocab);
+    FW_LAUNCH_CHECK("argmax_rows_static (parts)");
+    argmax_finish_kernel<<<rows, 64, 0, (hipStream_t)stream>>>(scratch, ids, also, advance);
+    FW_LAUNCH_CHECK("argmax_rows_static");
+    return 0;
+}
+
 // ---- fill ------------------------------------------------------------------------------
 __global__ void fill_zero_kernel(uint32_t* __restrict__ ptr, long long words) {
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < words;

@@ -153,6 +153,17 @@ int fw_attention_decode(const void* q, void* out, float* partial, int max_splits
 int fw_argmax_rows(const float* logits, int32_t* ids, int32_t* also, int32_t* advance, void* workspace, int rows, int vocab,
                    void* stream);
 
+// fw_argmax_rows for callers that cannot allocate device memory (code under HIP graph capture,
+// tight serving loops, harnesses that forbid hipMalloc) and so have no workspace to bring. It has no
+// counterpart in the reference. The keys of the parts go to an array built into the library, one
+// copy per GPU (512 KB, held until the process ends); at most fw_argmax_rows_static_max_rows() rows
+// (1,024), more is refused with an error. The call allocates and frees nothing. Every call on a GPU
+// uses that GPU's one array: calls that overlap there (several streams or threads) race; calls that
+// follow each other in one stream do not. Same results as fw_argmax_rows.
+int fw_argmax_rows_static(const float* logits, int32_t* ids, int32_t* also, int32_t* advance, int rows, int vocab,
+                          void* stream);
+int fw_argmax_rows_static_max_rows(void);
+
 // the k largest logits of every row, sorted by (value descending, id ascending)
 int fw_topk_rows(const float* logits, float* values, int32_t* ids, int rows, int vocab, int k,
                  void* stream);
