@@ -100,9 +100,12 @@ def causal_attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float,
     return out
 
 
-def attention_mixer(h: np.ndarray, w: Dict[str, np.ndarray], prefix: str, config: dict) -> np.ndarray:
-    """native/src/v2_runtime.cpp:28429-28478: q, k, v projections; per-head RMS norm of q
-    and k; rotation; causal softmax attention; output projection."""
+def attention_qkv(h: np.ndarray, w: Dict[str, np.ndarray], prefix: str, config: dict, positions: np.ndarray):
+    """Queries, keys and values as the attention reads them: projections; then, per head, the
+    RMS norm of q and of k over the head's channels, one weight of head_dim for all heads, with
+    the model's one eps (native/include/flyweight_v2_native_kernels.hpp:1015-1032); then the
+    rotation of the normed vectors (:1033-1047); v as projected. The head size is
+    hidden / heads (native/src/v2_runtime.cpp:4222)."""
     T = h.shape[0]
     nh, nkv = config["num_attention_heads"], config["num_key_value_heads"]
     hd = config["hidden_size"] // nh
@@ -112,10 +115,18 @@ def attention_mixer(h: np.ndarray, w: Dict[str, np.ndarray], prefix: str, config
     v = (h @ w[prefix + "v_proj.weight"].T).reshape(T, nkv, hd)
     q = rms_norm(q, w[prefix + "q_layernorm.weight"], eps)
     k = rms_norm(k, w[prefix + "k_layernorm.weight"], eps)
-    cos, sin = rope_angles(np.arange(T), hd, config["rope_theta"])
-    q, k = rope_half_split(q, cos, sin), rope_half_split(k, cos, sin)
-    out = causal_attention(q, k, v, 1.0 / math.sqrt(hd))
-    return out.reshape(T, nh * hd) @ w[prefix + "out_proj.weight"].T
+    cos, sin = rope_angles(positions, hd, config["rope_theta"])
+    return rope_half_split(q, cos, sin), rope_half_split(k, cos, sin), v
+
+
+def attention_mixer(h: np.ndarray, w: Dict[str, np.ndarray], prefix: str, config: dict) -> np.ndarray:
+    """native/src/v2_runtime.cpp:28429-28478: q, k, v projections; per-head RMS norm of q
+    and k; rotation; causal softmax attention with scores scaled by 1 / sqrt(head_dim);
+    output projection."""
+    T = h.shape[0]
+    q, k, v = attention_qkv(h, w, prefix, config, np.arange(T))
+    out = causal_attention(q, k, v, 1.0 / math.sqrt(q.shape[-1]))
+    return out.reshape(T, -1) @ w[prefix + "out_proj.weight"].T
 
 
 def causal_depthwise_conv(bx: np.ndarray, taps: np.ndarray) -> np.ndarray:
@@ -186,13 +197,24 @@ def forward(config: dict, w: Dict[str, np.ndarray], tokens: Sequence[int]) -> np
     return h @ head.T
 
 
+def most_likely(logits: np.ndarray) -> int:
+    """The largest logit's id; among equal ones the lowest id wins
+    (native/include/flyweight_v2_qwen_kernels.hpp:2391-2405: the key orders by value, then by
+    0xffffffff - id)."""
+    best = 0
+    for index in range(1, len(logits)):
+        if logits[index] > logits[best]:
+            best = index
+    return best
+
+
 def greedy(config: dict, w: Dict[str, np.ndarray], prompt: Sequence[int], count: int) -> List[int]:
-    """Greedy continuation, ties to the lowest id (native/include/flyweight_v2_qwen_kernels.hpp:2391-2405)."""
+    """Greedy continuation."""
     tokens = list(prompt)
     produced = []
     for _ in range(count):
         logits = forward(config, w, tokens)[-1]
-        token = int(np.argmax(logits))
+        token = most_likely(logits)
         produced.append(token)
         tokens.append(token)
     return produced

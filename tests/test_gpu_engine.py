@@ -520,3 +520,28 @@ def test_captured_decode_steps_are_sized_by_the_run_not_by_the_model(folders, tm
             assert np.array_equal(small, large)
     with pytest.raises(Exception, match="context limit is 4096"):
         stepper.step([StepEntry("a", [1] * 4000, [])])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_equal_logits_give_the_lowest_id_through_the_engine(folders, tmp_path, dtype):
+    """With a tied head a copy of an embedding row has that row's logit bit for bit, in either
+    precision: the engine must generate the lower of the two ids, as the plain model does."""
+    import shutil
+    from safetensors.torch import load_file, save_file
+    import flyweight_amd
+    config, weights = plain.read_folder(folders["A"])
+    prompt = random_tokens(config["vocab_size"], 9, seed=2)
+    with flyweight_amd.Runtime(flyweight_amd.Model(folders["A"], dtype=dtype)) as runtime:
+        winner = runtime.generate(prompt, 1)[0]
+    free = [t for t in range(config["vocab_size"]) if t not in prompt and t != winner]
+    for copy, expected in ((max(free), winner), (min(free), min(free))):
+        folder = str(tmp_path / f"copy{copy}")
+        shutil.copytree(folders["A"], folder)
+        tensors = load_file(f"{folder}/model.safetensors")
+        tensors["model.embed_tokens.weight"][copy] = tensors["model.embed_tokens.weight"][winner]
+        save_file(tensors, f"{folder}/model.safetensors")
+        with flyweight_amd.Runtime(flyweight_amd.Model(folder, dtype=dtype)) as runtime:
+            assert runtime.generate(prompt, 1) == [expected]
+        if dtype == "float32":
+            changed_config, changed = plain.read_folder(folder)
+            assert plain.greedy(changed_config, changed, prompt, 1) == [expected]

@@ -36,11 +36,6 @@ def bound(part, dtype, seed=0):
     return {n: t.double().numpy() for n, t in tensors.items()}
 
 
-def context(part_needs, segments, num_pages=8):
-    """segments: (request, start, count). Sequences are first advanced to ``start``."""
-    from flyweight_amd.cache import CacheManager
-    from flyweight_amd.engine.step import StepContext, StepEntry
-    return CacheManager, StepContext, StepEntry
 
 
 class Harness:

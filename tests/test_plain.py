@@ -191,9 +191,109 @@ def test_block_order_head_and_whole_model_invariants(tmp_path, name):
     for suffix in ("conv.conv.weight", "self_attn.v_proj.weight", "feed_forward.w3.weight"):
         cut = {k: (np.zeros_like(v) if k.endswith(suffix) else v) for k, v in w.items()}
         assert np.abs(plain.forward(config, cut, tokens) - logits).max() > 0.05 * np.abs(logits).max()
-    # greedy: lowest id among equals
-    assert plain.greedy(config, w, tokens[:5], 3) == plain.greedy(config, w, tokens[:5], 3)
 
 
-def test_greedy_ties_go_to_the_lowest_id():
-    assert int(np.argmax(np.array([1.0, 3.0, 3.0, 2.0]))) == 1
+def test_greedy_ties_go_to_the_lowest_id(tmp_path):
+    assert plain.most_likely(np.array([1.0, 3.0, 3.0, 2.0])) == 1
+    assert plain.most_likely(np.array([-np.inf, -np.inf])) == 0
+    # through the whole model: with a tied head a copy of the winner's embedding row has the
+    # winner's logit exactly; whichever of the two ids is lower must be generated
+    folder = make_model(str(tmp_path / "A"), "A", seed=3)
+    config, w = plain.read_folder(folder)
+    prompt = random_tokens(config["vocab_size"], 9, 2)
+    winner = plain.greedy(config, w, prompt, 1)[0]
+    free = [t for t in range(config["vocab_size"]) if t not in prompt and t != winner]
+    above, below = max(free), min(free)
+    assert below < winner < above
+    table = w["model.embed_tokens.weight"]
+    for copy, expected in ((above, winner), (below, below)):
+        changed = dict(w)
+        changed["model.embed_tokens.weight"] = table.copy()
+        changed["model.embed_tokens.weight"][copy] = table[winner]
+        logits = plain.forward(config, changed, prompt)[-1]
+        assert logits[copy] == logits[winner] == logits.max()
+        assert plain.greedy(config, changed, prompt, 1) == [expected]
+
+
+# ----- the attention mixer's own choices: what is normed, when, with which eps and scale ------
+def _attention_setup(nh=4, nkv=2, hd=8, T=6, eps=1e-5, theta=100.0):
+    H = nh * hd
+    config = {"hidden_size": H, "num_attention_heads": nh, "num_key_value_heads": nkv, "norm_eps": eps, "rope_theta": theta}
+    w = {"a.q_proj.weight": RNG.normal(size=(nh * hd, H)), "a.k_proj.weight": RNG.normal(size=(nkv * hd, H)),
+         "a.v_proj.weight": RNG.normal(size=(nkv * hd, H)), "a.out_proj.weight": np.eye(H),
+         "a.q_layernorm.weight": 1.0 + 0.3 * RNG.normal(size=hd), "a.k_layernorm.weight": 1.0 + 0.3 * RNG.normal(size=hd)}
+    return config, w, RNG.normal(size=(T, H))
+
+
+def test_qk_norm_comes_before_the_rotation():
+    """A norm weight that is one-hot on channel 0 leaves a vector along channel 0; the rotation
+    then spreads it over channels 0 and hd/2 at every position but the first. Rotating first and
+    norming after would leave channel 0 alone everywhere."""
+    config, w, h = _attention_setup()
+    hd = 8
+    for name in ("a.q_layernorm.weight", "a.k_layernorm.weight"):
+        w[name] = np.zeros(hd)
+        w[name][0] = 1.0
+    q, k, _ = plain.attention_qkv(h, w, "a.", config, np.arange(6))
+    raw = (h @ w["a.q_proj.weight"].T).reshape(6, 4, hd)
+    length = raw[..., 0] / np.sqrt((raw ** 2).mean(-1) + config["norm_eps"])      # channel 0 after the norm
+    for p in range(6):
+        others = [c for c in range(hd) if c not in (0, hd // 2)]
+        assert np.abs(q[p][:, others]).max() == 0.0 and np.abs(k[p][:, others]).max() == 0.0
+        # channel 0's pair turns by the angle p / theta^0 = p
+        np.testing.assert_allclose(q[p][:, 0], length[p] * math.cos(p), rtol=1e-12, atol=1e-15)
+        np.testing.assert_allclose(q[p][:, hd // 2], length[p] * math.sin(p), rtol=1e-12, atol=1e-15)
+    assert np.abs(q[0][:, hd // 2]).max() == 0.0 and np.abs(q[1][:, hd // 2]).min() > 0.0
+
+
+def test_qk_norm_is_per_head_with_one_weight_for_all_heads():
+    config, w, h = _attention_setup()
+    nh, nkv, hd, group = 4, 2, 8, 2
+    out = plain.attention_mixer(h, w, "a.", config).reshape(6, nh, hd)       # out_proj is the identity
+    # swapping the two query heads of kv group 0 swaps their outputs: one norm weight serves both
+    rows = w["a.q_proj.weight"].reshape(nh, hd, -1)
+    swapped = dict(w)
+    swapped["a.q_proj.weight"] = rows[[1, 0, 2, 3]].reshape(nh * hd, -1)
+    np.testing.assert_allclose(plain.attention_mixer(h, swapped, "a.", config).reshape(6, nh, hd), out[:, [1, 0, 2, 3]], rtol=1e-12)
+    # the norm is over a head's channels alone: making one head's projection 50 times larger leaves
+    # the other heads exactly alone, and that head itself nearly so (eps is all that notices)
+    louder = dict(w)
+    scaled = rows.copy()
+    scaled[2] *= 50.0
+    louder["a.q_proj.weight"] = scaled.reshape(nh * hd, -1)
+    loud = plain.attention_mixer(h, louder, "a.", config).reshape(6, nh, hd)
+    np.testing.assert_allclose(loud[:, [0, 1, 3]], out[:, [0, 1, 3]], rtol=1e-12)
+    np.testing.assert_allclose(loud[:, 2], out[:, 2], rtol=1e-4)
+    # v is not normed: doubling v_proj doubles the output
+    double = dict(w)
+    double["a.v_proj.weight"] = 2 * w["a.v_proj.weight"]
+    np.testing.assert_allclose(plain.attention_mixer(h, double, "a.", config).reshape(6, nh, hd), 2 * out, rtol=1e-12)
+
+
+def test_qk_norm_uses_the_models_eps_inside_the_root():
+    """mean(x^2) + eps under the root, per head: a huge eps shrinks q and k, the scores vanish and
+    every row attends evenly, so the output becomes the running mean of v."""
+    config, w, h = _attention_setup(eps=1e12)
+    nh, nkv, hd = 4, 2, 8
+    out = plain.attention_mixer(h, w, "a.", config).reshape(6, nh, hd)
+    v = (h @ w["a.v_proj.weight"].T).reshape(6, nkv, hd)
+    running = np.cumsum(v, axis=0) / np.arange(1, 7)[:, None, None]
+    np.testing.assert_allclose(out, np.repeat(running, nh // nkv, axis=1), rtol=1e-6, atol=1e-9)
+    config["norm_eps"] = 1e-5
+    assert np.abs(plain.attention_mixer(h, w, "a.", config).reshape(6, nh, hd) - np.repeat(running, 2, axis=1)).max() > 0.1
+    # and it is the norm's eps as rms_norm has it: q of the mixer is rms_norm of the projection
+    q, _, _ = plain.attention_qkv(h, w, "a.", config, np.zeros(6))            # position 0: no rotation
+    raw = (h @ w["a.q_proj.weight"].T).reshape(6, nh, hd)
+    np.testing.assert_allclose(q, raw / np.sqrt((raw ** 2).mean(-1, keepdims=True) + 1e-5) * w["a.q_layernorm.weight"], rtol=1e-12)
+
+
+@pytest.mark.parametrize("hd", [8, 32])
+def test_the_mixer_scales_scores_by_one_over_root_head_dim(hd):
+    """The library's attention divides by sqrt(head_dim) when no scale is given: fed the mixer's
+    own q, k and v it must give the mixer's output, for two head sizes."""
+    config, w, h = _attention_setup(nh=4, nkv=2, hd=hd, T=7)
+    q, k, v = plain.attention_qkv(h, w, "a.", config, np.arange(7))
+    tq, tk, tv = (torch.tensor(a).transpose(0, 1)[None] for a in (q, k, v))
+    lib = F.scaled_dot_product_attention(tq, tk.repeat_interleave(2, 1), tv.repeat_interleave(2, 1), is_causal=True)
+    np.testing.assert_allclose(plain.attention_mixer(h, w, "a.", config), lib[0].transpose(0, 1).reshape(7, 4 * hd).numpy(),
+                               rtol=1e-10, atol=1e-12)

@@ -62,6 +62,35 @@ def test_top_k_and_top_p_cuts():
     assert _support(SamplingConfig(temperature=0.0, top_k=0, top_p=1.0, min_p=0.0), draws=5) == {0}
 
 
+def _support_of(shares, draws=600, **settings):
+    logits = np.log(np.asarray(shares, dtype=np.float64)).astype(np.float32)
+    config = SamplingConfig(temperature=1.0, **settings)
+    values, ids = host_candidates(logits, config.top_k)
+    mine, plain = XorShift64Star(5), plain_lfm2.XorShift64Star(5)
+    found = set()
+    for _ in range(draws):
+        token = draw_from_candidates(values, ids, config, mine)
+        assert token == plain_lfm2.sample(logits, 1.0, config.top_k, config.top_p, config.min_p, plain)
+        found.add(token)
+    return found
+
+
+def test_top_p_counts_shares_of_all_candidates_and_min_p_cuts_after_it():
+    """native/src/v2_runtime.cpp:29714-29728: the nucleus is found on shares of the whole candidate
+    list, then min_p shortens what is left. With shares 0.4, 0.3, 0.2, 0.1, top_p 0.5 is reached by
+    the second candidate (0.7) and min_p 0.6 (floor 0.24) keeps the first two: {0, 1}. Cutting by
+    min_p first and taking the nucleus of what is left (0.4 / 0.7 = 0.57 >= 0.5) would keep {0}."""
+    shares = [0.4, 0.3, 0.2, 0.1]
+    assert _support_of(shares, top_k=0, top_p=0.5, min_p=0.6) == {0, 1}
+    assert _support_of(shares, top_k=0, top_p=0.5, min_p=0.0) == {0, 1}
+    assert _support_of(shares, top_k=0, top_p=1.0, min_p=0.6) == {0, 1}
+    assert _support_of(shares, top_k=0, top_p=0.35, min_p=0.6) == {0}
+    # the candidate list is cut to top_k before shares are formed (:29500-29566, then :29703-29710):
+    # of the best two, 0.4 / 0.7 = 0.57 reaches 0.55 alone; of all four, 0.4 would not
+    assert _support_of(shares, top_k=2, top_p=0.55, min_p=0.0) == {0}
+    assert _support_of(shares, top_k=0, top_p=0.55, min_p=0.0) == {0, 1}
+
+
 def test_candidates_order_ties_to_the_lowest_id_and_nan_last():
     logits = np.array([1.0, 5.0, float("nan"), 5.0, -2.0], dtype=np.float32)
     values, ids = host_candidates(logits, 0)
