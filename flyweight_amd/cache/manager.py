@@ -26,7 +26,7 @@ import numpy as np
 import torch
 
 from .. import host
-from .needs import FixedState, PagedKV
+from .needs import CacheNeed, CacheView
 from .pages import CacheAccountingError, OutOfPages, PagePool, SlotPool
 
 NO_PAGE = host.NO_PAGE
@@ -92,7 +92,7 @@ class _LiveRequests(Mapping):
 @dataclass
 class PageGroup:
     key: Tuple
-    need: PagedKV
+    need: CacheNeed
     entries: List[int]
     pool: PagePool
     tables: Mapping
@@ -102,8 +102,9 @@ class CacheManager:
     def __init__(self, needs: Mapping[int, object], num_pages: int, max_requests: int, page_size: int = 64,
                  max_pages_per_request: Optional[int] = None, dtype: torch.dtype = torch.float32,
                  device: Optional[torch.device] = None):
-        """``needs``: cache entry id -> PagedKV | FixedState. ``num_pages``: pages of every
-        page group. ``device`` None keeps the bookkeeping only (no storage)."""
+        """``needs``: cache entry id -> a :class:`CacheNeed` (``PagedKV``, ``FixedState`` or a
+        class of the mixer's own). ``num_pages``: pages of every page group. ``device`` None keeps
+        the bookkeeping only (no storage)."""
         self.page_size = page_size
         self.num_pages = num_pages
         self.max_requests = max_requests
@@ -112,17 +113,21 @@ class CacheManager:
         self.device = device
         self.groups: List[PageGroup] = []
         self.entry_group: Dict[int, int] = {}
-        self.state_entries: Dict[int, FixedState] = {}
-        grouped: Dict[Tuple, Tuple[PagedKV, List[int]]] = {}
+        self.state_entries: Dict[int, CacheNeed] = {}
+        self.needs: Dict[int, CacheNeed] = {}
+        grouped: Dict[Tuple, Tuple[CacheNeed, List[int]]] = {}
         for entry in sorted(needs):
             need = needs[entry]
-            if isinstance(need, PagedKV):
+            if need is None:
+                continue
+            if not isinstance(need, CacheNeed):
+                raise TypeError(f"cache entry {entry}: {need!r} is not a CacheNeed")
+            self.needs[entry] = need
+            if need.paged:
                 grouped.setdefault(need.group_key(), (need, []))[1].append(entry)
                 self.entry_group[entry] = list(grouped).index(need.group_key())
-            elif isinstance(need, FixedState):
+            else:
                 self.state_entries[entry] = need
-            elif need is not None:
-                raise TypeError(f"cache entry {entry}: unknown need {need!r}")
         # the bookkeeping lives in the host library
         self._lib = host.library()
         windows = (ctypes.c_int * max(len(grouped), 1))(*[int(need.window or 0) for need, _ in grouped.values()])
@@ -138,23 +143,33 @@ class CacheManager:
         self._ids: Dict[Hashable, int] = {}         # keys that are not small integers -> ids of the host library
         self._keys: Dict[int, Hashable] = {}
         self._next_named = _FIRST_NAMED_ID
-        # storage
-        self.k_pages: Dict[int, torch.Tensor] = {}
-        self.v_pages: Dict[int, torch.Tensor] = {}
-        self.state: Dict[int, torch.Tensor] = {}
         # One page and one slot lie behind those the pools hand out: rows that only fill a step up to
         # a size it was recorded for (see Stepper.planned_decode) write there, and nobody reads it.
         self.spare_page = num_pages
         self.spare_slot = max_requests
+        # storage: each need allocates its own
+        self.storage: Dict[int, object] = {}
         if device is not None:
-            for group in self.groups:
-                n = group.need
-                for entry in group.entries:
-                    # K keeps a key's channels together, V a channel's tokens (see the attention kernels)
-                    self.k_pages[entry] = torch.zeros((num_pages + 1, n.num_kv_heads, page_size, n.head_dim), dtype=dtype, device=device)
-                    self.v_pages[entry] = torch.zeros((num_pages + 1, n.num_kv_heads, n.head_dim, page_size), dtype=dtype, device=device)
-            for entry, need in self.state_entries.items():
-                self.state[entry] = torch.zeros((max_requests + 1, *need.shape), dtype=need.dtype, device=device)
+            for entry, need in self.needs.items():
+                units = (num_pages if need.paged else max_requests) + 1
+                self.storage[entry] = need.allocate(units, page_size, dtype, device)
+
+    def view(self, entry: int, block_table=None, writes: bool = True):
+        """What the mixer that uses cache entry ``entry`` sees of it."""
+        return self.needs[entry].view(self.storage[entry], block_table, writes)
+
+    # the tensors of the built-in needs, by entry
+    @property
+    def k_pages(self) -> Dict[int, torch.Tensor]:
+        return {entry: self.view(entry).k_pages for entry in self.entry_group if entry in self.storage}
+
+    @property
+    def v_pages(self) -> Dict[int, torch.Tensor]:
+        return {entry: self.view(entry).v_pages for entry in self.entry_group if entry in self.storage}
+
+    @property
+    def state(self) -> Dict[int, torch.Tensor]:
+        return {entry: self.view(entry).state for entry in self.state_entries if entry in self.storage}
 
     def __del__(self):
         if getattr(self, "_native", None):
@@ -216,13 +231,15 @@ class CacheManager:
             raise OutOfPages("out of request slots")
         if slot < 0:
             raise CacheAccountingError(host.last_error())
-        self.zero_slot(slot)
+        self.start_slot(slot)
         return slot
 
-    def zero_slot(self, slot: int) -> None:
-        """A slot's state starts at zero for the request that takes it."""
-        for tensor in self.state.values():
-            tensor[slot].zero_()
+    def start_slot(self, slot: int) -> None:
+        """A slot's state is what a request starts with (zero, unless the need says otherwise)
+        for the request that takes it."""
+        for entry, need in self.state_entries.items():
+            if entry in self.storage:
+                need.initial(self.storage[entry], slot)
 
     def slot_of(self, request: Hashable) -> int:
         slot = self._lib.fwh_cache_slot_of(self._native, self._live_id(request))

@@ -80,10 +80,17 @@ class ModelSpec:
     lm_head_name: Optional[str]     # None: the head is the embedding table (tied)
     bos_token_id: Optional[int] = None
     eos_token_id: Optional[int] = None
+    # What some architectures put around the layers: a factor on the embedding rows, a factor on
+    # the logits, a soft cap c on them (c * tanh(logits / c), after the factor; 0: none).
+    embedding_scale: float = 1.0
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0
 
     def validate(self) -> None:
         if self.hidden_size <= 0 or self.vocab_size <= 0:
             raise ConfigError("hidden_size and vocab_size must be positive")
+        if self.logit_softcap < 0:
+            raise ConfigError("logit_softcap must not be negative (0 switches it off)")
         if not self.layers or not self.schedule:
             raise ConfigError("a model needs at least one layer and one schedule entry")
         writers = {}

@@ -16,30 +16,31 @@ void fw_set_error(const char* format, ...) {
     va_end(args);
 }
 extern "C" const char* fw_last_error(void) { return fw_error_text; }
-extern "C" int fw_abi_version(void) { return 3; }
+extern "C" int fw_abi_version(void) { return 4; }
 
 // ---- embedding -------------------------------------------------------------------------
 // The reference gathers one row per token and widens it to float32
 // (native/include/flyweight_v2_native_kernels.hpp:98-151).
+// `scale` multiplies the row (architectures that scale their embeddings; 1 leaves it as stored).
 template <typename W>
 __global__ void embed_rows_kernel(const W* __restrict__ table, const int32_t* __restrict__ ids,
-                                  float* __restrict__ out, int hidden) {
+                                  float* __restrict__ out, int hidden, float scale) {
     const int row = blockIdx.y;
     const size_t base = (size_t)ids[row] * hidden;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < hidden; i += gridDim.x * blockDim.x)
-        out[(size_t)row * hidden + i] = load_as_float(table, base + i);
+        out[(size_t)row * hidden + i] = load_as_float(table, base + i) * scale;
 }
 
 extern "C" int fw_embed_rows(const void* table, int table_dtype, const int32_t* ids, float* out,
-                             int rows, int hidden, int vocab, void* stream) {
+                             int rows, int hidden, int vocab, float scale, void* stream) {
     FW_REQUIRE(rows >= 0 && hidden > 0 && vocab > 0, "embed_rows: bad sizes rows=%d hidden=%d vocab=%d", rows, hidden, vocab);
     FW_REQUIRE(rows <= 65535, "embed_rows: at most 65535 rows per call, got %d", rows);
     if (rows == 0) return 0;
     dim3 grid(fw_ceil_div(hidden, 256) > 64 ? 64 : fw_ceil_div(hidden, 256), rows);
     if (table_dtype == FW_F32)
-        embed_rows_kernel<float><<<grid, 256, 0, (hipStream_t)stream>>>((const float*)table, ids, out, hidden);
+        embed_rows_kernel<float><<<grid, 256, 0, (hipStream_t)stream>>>((const float*)table, ids, out, hidden, scale);
     else if (table_dtype == FW_BF16)
-        embed_rows_kernel<bf16_t><<<grid, 256, 0, (hipStream_t)stream>>>((const bf16_t*)table, ids, out, hidden);
+        embed_rows_kernel<bf16_t><<<grid, 256, 0, (hipStream_t)stream>>>((const bf16_t*)table, ids, out, hidden, scale);
     else
         FW_REQUIRE(false, "embed_rows: unknown table dtype %d", table_dtype);
     FW_LAUNCH_CHECK("embed_rows");
@@ -353,6 +354,27 @@ extern "C" int fw_argmax_rows_static(const float* logits, int32_t* ids, int32_t*
     FW_LAUNCH_CHECK("argmax_rows_static (parts)");
     argmax_finish_kernel<<<rows, 64, 0, (hipStream_t)stream>>>(scratch, ids, also, advance);
     FW_LAUNCH_CHECK("argmax_rows_static");
+    return 0;
+}
+
+// ---- logits: scale and soft cap ------------------------------------------------------------
+// x <- x * scale, then, with a cap c > 0, x <- c * tanh(x / c): for architectures whose head has a
+// logit scale or a soft cap. In place, float32.
+__global__ void scale_softcap_kernel(float* __restrict__ x, long long count, float scale, float cap) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (long long)gridDim.x * blockDim.x) {
+        float value = x[i] * scale;
+        if (cap > 0.0f) value = cap * tanhf(value / cap);
+        x[i] = value;
+    }
+}
+
+extern "C" int fw_scale_softcap(float* x, long long count, float scale, float cap, void* stream) {
+    FW_REQUIRE(count >= 0 && cap >= 0.0f, "scale_softcap: bad arguments count=%lld cap=%g", count, (double)cap);
+    if (count == 0) return 0;
+    long long blocks = (count + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    scale_softcap_kernel<<<(int)blocks, 256, 0, (hipStream_t)stream>>>(x, count, scale, cap);
+    FW_LAUNCH_CHECK("scale_softcap");
     return 0;
 }
 

@@ -14,9 +14,12 @@ extern "C" {
 const char* fw_last_error(void);
 int fw_abi_version(void);
 
-// out[r][:] = table[ids[r]][:]  (float32 out: the residual stream)
+// out[r][:] = table[ids[r]][:] * scale  (float32 out: the residual stream)
 int fw_embed_rows(const void* table, int table_dtype, const int32_t* ids, float* out,
-                  int rows, int hidden, int vocab, void* stream);
+                  int rows, int hidden, int vocab, float scale, void* stream);
+
+// x <- x * scale, then with cap > 0: x <- cap * tanh(x / cap); float32, in place
+int fw_scale_softcap(float* x, long long count, float scale, float cap, void* stream);
 
 // RMS norm of float32 rows: out[r] = x[src] * rsqrt(mean(x[src]^2) + eps) * w, where
 // src = row_index ? row_index[r] : r.  one_centered: multiply by (1 + w) instead of w.

@@ -9,6 +9,7 @@ from typing import Dict, List, Optional
 
 import torch
 
+from ..cache.needs import CacheView
 from ..config import ModelSpec, load_config
 from ..config.spec import ConfigError
 from ..kernels import ops
@@ -30,16 +31,6 @@ def parse_dtype(name) -> torch.dtype:
         return _DTYPES[str(name).lower()]
     except KeyError:
         raise ValueError(f"unknown dtype '{name}'; choose bfloat16 or float32") from None
-
-
-@dataclass
-class CacheView:
-    """What a mixer sees of the cache during one execution."""
-    k_pages: Optional[torch.Tensor] = None
-    v_pages: Optional[torch.Tensor] = None
-    block_table: Optional[torch.Tensor] = None     # [segments, stride] int32, rows in batch order
-    state: Optional[torch.Tensor] = None           # [slots, ...]
-    writes: bool = True
 
 
 class CausalLM:
@@ -93,11 +84,22 @@ class CausalLM:
             needs[entry.cache] = need
         return needs
 
+    def step_array_providers(self) -> List:
+        """The parts that ask for index arrays of their own in every step's upload
+        (``Part.step_arrays``), one for each distinct key."""
+        found: Dict = {}
+        for block in self.layers:
+            for part in getattr(block, "parts", tuple)():
+                key = part.step_arrays_key()
+                if key is not None:
+                    found.setdefault(key, part)
+        return list(found.values())
+
     # ----- forward ----------------------------------------------------------------------
     def forward(self, ctx, cache) -> Optional[torch.Tensor]:
         """Runs the rows of ``ctx`` through every scheduled layer; returns float32 logits
         [wanted, vocab] for ``ctx.want_rows`` (None when nothing is wanted)."""
-        x = ops.embed_rows(self.embedding, ctx.token_ids)
+        x = ops.embed_rows(self.embedding, ctx.token_ids, scale=self.spec.embedding_scale)
         schedule = self.spec.schedule
         ctx.prepared = None
         for at, entry in enumerate(schedule):
@@ -108,7 +110,10 @@ class CausalLM:
         ctx.prepared = ctx.norm_after_block = None
         if ctx.num_wanted == 0:
             return None
-        return self.head.forward(LazyNorm(self.final_norm, x, ctx, row_index=ctx.want_rows), out_dtype=torch.float32)
+        logits = self.head.forward(LazyNorm(self.final_norm, x, ctx, row_index=ctx.want_rows), out_dtype=torch.float32)
+        if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0.0:
+            ops.scale_softcap_(logits, self.spec.logit_scale, self.spec.logit_softcap)
+        return logits
 
 
 def declared_tensors(spec: ModelSpec) -> Dict[str, TensorDecl]:

@@ -284,7 +284,7 @@ class Scheduler:
         cache = self.cache
         for request in plan.admitted:
             if request.id in cache.requests:
-                cache.zero_slot(cache.slot_of(request.id))
+                cache.start_slot(cache.slot_of(request.id))
         return plan
 
     # ----- after the step ---------------------------------------------------------------

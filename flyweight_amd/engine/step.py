@@ -35,6 +35,10 @@ class StepEntry:
     request: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = ()       # places among ``tokens`` whose logits are asked for
+    # What the position encodings see for these tokens, if not their places in the sequence
+    # (the default): one non-negative number per token. Where a key lies in the cache and which
+    # keys a row may see follow the order of the tokens whatever is given here.
+    positions: Optional[Sequence[int]] = None
 
 
 def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int, max_positions: int):
@@ -56,7 +60,7 @@ def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size:
         lengths, slots = cache.describe(requests, natives)
     except KeyError as error:
         raise StepError(f"request {error.args[0]!r} was not admitted", error.args[0]) from None
-    if all(len(entry.tokens) == 1 for entry in entries):
+    if all(len(entry.tokens) == 1 and entry.positions is None for entry in entries):
         # a decode step: the same checks without a loop over the entries' fields
         tokens = [entry.tokens[0] for entry in entries]
         if max(lengths) + 1 > max_positions:
@@ -83,18 +87,25 @@ def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size:
         for place in entry.want:
             if not 0 <= int(place) < n:
                 raise StepError(f"request {entry.request!r} wants logits at place {place} of {n} tokens", entry.request)
+        if entry.positions is not None and (len(entry.positions) != n or min(entry.positions) < 0):
+            raise StepError(f"request {entry.request!r} gives {len(entry.positions)} positions for {n} tokens, or a negative one",
+                            entry.request)
     return lengths, slots, natives
 
 
 class StepContext:
     """The batch as the kernels see it: per-row and per-segment index arrays on the
-    device (one upload), block tables per page group, and per-step tables of the position
-    encodings."""
+    device (one upload), block tables per page group, per-step tables of the position
+    encodings, and whatever index arrays the model's parts ask for (``Part.step_arrays``: built
+    on the host from the batch, they travel in the same upload)."""
+
+    FIXED = 6       # tokens, positions, segment of each row, first row of each segment, slots, wanted rows
 
     def __init__(self, entries: Sequence[StepEntry], cache: CacheManager, device: torch.device, vocab_size: int,
-                 max_positions: int, described=None):
+                 max_positions: int, described=None, providers: Sequence = ()):
         """``described``: (lengths, slots) of the entries' requests if the caller has checked the
-        entries already (``check_entries``)."""
+        entries already (``check_entries``). ``providers``: the parts whose ``step_arrays`` this
+        step's upload carries."""
         starts, slots, natives = described if described is not None else check_entries(entries, cache, vocab_size, max_positions)
         # per-row arrays are put together from one numpy piece per entry: a prompt portion has
         # thousands of rows, and a Python loop over them would take longer than some kernels
@@ -104,11 +115,15 @@ class StepContext:
         want_rows: List[int] = []
         self.requests: List[Hashable] = [entry.request for entry in entries]
         self.new_lengths: List[int] = []
+        given_positions = any(entry.positions is not None for entry in entries)
+        encoding_parts = []
         for seg, (entry, start) in enumerate(zip(entries, starts)):
             n = len(entry.tokens)
             want_rows.extend(seg_row0[-1] + int(place) for place in entry.want)
             token_parts.append(np.asarray(entry.tokens, dtype=np.int32))
             pos_parts.append(np.arange(start, start + n, dtype=np.int32))
+            if given_positions:
+                encoding_parts.append(pos_parts[-1] if entry.positions is None else np.asarray(entry.positions, dtype=np.int32))
             seg_parts.append(np.full(n, seg, dtype=np.int32))
             seg_row0.append(seg_row0[-1] + n)
             self.new_lengths.append(start + n)
@@ -121,7 +136,7 @@ class StepContext:
         self.all_decode = self.num_rows == self.num_segments
         self.max_context = max(self.new_lengths)
         # segments of one token that a mixed step begins with (a scheduler puts the decoded tokens
-        # first): mixers may give them to their decode kernels. Their rows and query tiles are 0 .. n - 1.
+        # first): mixers may give them to their decode kernels. Their rows are 0 .. n - 1.
         self.decode_prefix = 0
         if not self.all_decode:
             while len(entries[self.decode_prefix].tokens) == 1:
@@ -132,64 +147,96 @@ class StepContext:
         self.host_seg_row0 = seg_row0
         self.host_seg_slot = seg_slot
 
-        tile_seg, tile_row0 = ops.query_tiles(seg_row0)        # tiles of up to 64 rows for the prompt attention kernel
-        # Workgroups start in the order of the tiles: those that see the most keys go first, the short
-        # ones fill in behind. The tiles of the leading single rows stay in front (mixers may hand
-        # those rows to their decode kernels and skip their tiles).
-        if len(tile_seg) - self.decode_prefix > 1:
-            tile_seg, tile_row0 = np.asarray(tile_seg, dtype=np.int32), np.asarray(tile_row0, dtype=np.int32)
-            tile_end = np.minimum(tile_row0 + ops.QUERY_TILE, np.asarray(seg_row0, dtype=np.int32)[tile_seg + 1])
-            keys_seen = row_pos[tile_end - 1].astype(np.int64)
-            keys_seen[:self.decode_prefix] = np.iinfo(np.int64).max
-            order = np.argsort(-keys_seen, kind="stable")
-            tile_seg, tile_row0 = tile_seg[order], tile_row0[order]
         tables = [cache.block_table_rows(g, self.requests, natives=natives) for g in range(len(cache.groups))]
-        pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows,
-                                                          tile_seg, tile_row0)]
+        pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows)]
         pieces += [t.reshape(-1) for t in tables]
+        if given_positions:
+            pieces.append(np.concatenate(encoding_parts))
+        extra = self._ask(providers)
+        pieces += [array for _, _, array in extra]
         packed = torch.from_numpy(np.concatenate(pieces)).to(device)
         views = []
         offset = 0
         for piece in pieces:
             views.append(packed[offset:offset + piece.size])
             offset += piece.size
-        (self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows, self.tile_seg,
-         self.tile_row0) = views[:8]
-        self.block_tables = [v.view(t.shape) for v, t in zip(views[8:], tables)]
+        self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows = views[:self.FIXED]
+        self.block_tables = [v.view(t.shape) for v, t in zip(views[self.FIXED:], tables)]
+        at = self.FIXED + len(tables)
+        # what the position encodings see: the places in the sequences, unless the entries say otherwise
+        self.encoding_pos = self.row_pos
+        if given_positions:
+            self.encoding_pos = views[at]
+            at += 1
+        self._arrays: Dict = {}
+        for (key, name, _), view in zip(extra, views[at:]):
+            self._arrays.setdefault(key, {})[name] = view
         self._position_tables: Dict = {}
+
+    def _ask(self, providers: Sequence):
+        """[(provider key, array name, int32 numpy array)] of every provider, in a fixed order."""
+        asked = []
+        for part in providers:
+            key = part.step_arrays_key()
+            for name, array in sorted(part.step_arrays(self).items()):
+                asked.append((key, name, np.ascontiguousarray(array, dtype=np.int32).reshape(-1)))
+        return asked
+
+    def step_arrays(self, part) -> Dict[str, torch.Tensor]:
+        """The device copies of what ``part.step_arrays`` built for this step. A part that was
+        not among the step's providers gets them made now, with an upload of their own."""
+        key = part.step_arrays_key()
+        if key not in self._arrays:
+            if self.host_seg_row0 is None:
+                raise StepError("a recorded step holds only the arrays of the parts it was built with")
+            self._arrays[key] = {name: torch.from_numpy(np.ascontiguousarray(array, dtype=np.int32)).to(self.device)
+                                 for name, array in part.step_arrays(self).items()}
+        return self._arrays[key]
 
     @classmethod
     def for_decode_graph(cls, batch: int, cache: CacheManager, device: torch.device, max_context: int,
-                         table_stride: int) -> "StepContext":
+                         table_stride: int, providers: Sequence = ()) -> "StepContext":
         """A context of ``batch`` single-token segments whose index arrays live in ONE
-        persistent device buffer, refreshed before every replay of the captured step."""
+        persistent device buffer, refreshed before every replay of the captured step. The parts'
+        own arrays are built once, for ``batch`` segments of one row each: a part whose arrays
+        depend on more than that (on positions, say) must not call itself ``graph_safe``."""
         self = cls.__new__(cls)
         self.num_rows = self.num_segments = self.num_wanted = batch
         self.all_decode = True
         self.decode_prefix = 0
         self.max_context = max_context          # bounds the split-key grid, not the result
         self.device = device
+        groups = len(cache.groups)
+        # what the parts' arrays are built from: ``batch`` segments of one row
+        self.host_row_pos = np.zeros(batch, dtype=np.int32)
+        self.host_seg_row0 = list(range(batch + 1))
+        self.host_seg_slot = [0] * batch
+        extra = self._ask(providers)
         self.host_row_pos = self.host_seg_row0 = self.host_seg_slot = None     # not for captured steps
-        sizes = [batch, batch, batch, batch + 1, batch, batch, batch, batch] + [batch * table_stride] * len(cache.groups)
-        self.host_buffer = torch.empty(sum(sizes), dtype=torch.int32, pin_memory=True)
-        self.device_buffer = torch.zeros(sum(sizes), dtype=torch.int32, device=device)
+        sizes = [batch, batch, batch, batch + 1, batch, batch] + [batch * table_stride] * groups
+        sizes += [array.size for _, _, array in extra]
+        self.host_buffer = torch.empty(max(sum(sizes), 1), dtype=torch.int32, pin_memory=True)
+        self.device_buffer = torch.zeros(max(sum(sizes), 1), dtype=torch.int32, device=device)
         views, host_views, offset = [], [], 0
         for size in sizes:
             views.append(self.device_buffer[offset:offset + size])
             host_views.append(self.host_buffer[offset:offset + size].numpy())
             offset += size
-        (self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows, self.tile_seg,
-         self.tile_row0) = views[:8]
-        self.block_tables = [v.view(batch, table_stride) for v in views[8:]]
+        self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows = views[:cls.FIXED]
+        self.encoding_pos = self.row_pos
+        self.block_tables = [v.view(batch, table_stride) for v in views[cls.FIXED:cls.FIXED + groups]]
         self._host = host_views
+        self._host_tables = host_views[cls.FIXED:cls.FIXED + groups]
         self._table_stride = table_stride
         # what never changes between replays
         rows = np.arange(batch, dtype=np.int32)
         host_views[2][:] = rows
         host_views[3][:] = np.arange(batch + 1, dtype=np.int32)
         host_views[5][:] = rows
-        host_views[6][:] = rows
-        host_views[7][:] = rows
+        self._arrays = {}
+        for (key, name, array), view, host_view in zip(extra, views[cls.FIXED + groups:], host_views[cls.FIXED + groups:]):
+            host_view[:] = array
+            self._arrays.setdefault(key, {})[name] = view
         self._position_tables = {}
         return self
 
@@ -207,8 +254,8 @@ class StepContext:
         host[0][:] = [int(e.tokens[0]) for e in entries]
         host[1][:] = starts
         host[4][:] = slots
-        for g in range(len(cache.groups)):
-            host[8 + g][:] = cache.block_table_rows(g, self.requests, stride=self._table_stride, natives=natives).reshape(-1)
+        for g, rows in enumerate(self._host_tables):
+            rows[:] = cache.block_table_rows(g, self.requests, stride=self._table_stride, natives=natives).reshape(-1)
         self.upload()
 
     def wait_uploaded(self) -> None:
@@ -231,9 +278,9 @@ class StepContext:
         up; returns the plan's number of rows (the caller uploads). -1 (and nothing written) otherwise."""
         self.wait_uploaded()
         host = self._host
-        groups = len(host) - 8
+        tables = self._host_tables
         rows = scheduler.fill_decode(self.num_rows, host[0], host[1], host[4], self._table_stride,
-                                     host[8] if groups else None, self.num_rows * self._table_stride)
+                                     tables[0] if tables else None, self.num_rows * self._table_stride)
         if rows < 0:
             return -1
         self.fill_up(rows, cache)
@@ -248,8 +295,8 @@ class StepContext:
         host[0][rows:] = 0
         host[1][rows:] = 0
         host[4][rows:] = cache.spare_slot
-        for g in range(len(host) - 8):
-            host[8 + g][rows * self._table_stride:] = cache.spare_page
+        for table in self._host_tables:
+            table[rows * self._table_stride:] = cache.spare_page
 
     def position_tables(self, part):
         key = part.key()
@@ -257,15 +304,14 @@ class StepContext:
             self._position_tables[key] = part.tables(self)
         return self._position_tables[key]
 
-    def cache_view(self, cache: CacheManager, entry) -> CacheView:
-        if entry.cache is None:
-            return CacheView(writes=False)
-        if entry.cache in cache.entry_group:
-            return CacheView(k_pages=cache.k_pages[entry.cache], v_pages=cache.v_pages[entry.cache],
-                             block_table=self.block_tables[cache.entry_group[entry.cache]], writes=entry.writes_cache)
-        if entry.cache in cache.state:
-            return CacheView(state=cache.state[entry.cache], writes=entry.writes_cache)
-        return CacheView(writes=entry.writes_cache)
+    def cache_view(self, cache: CacheManager, entry):
+        """What the mixer of schedule entry ``entry`` sees of the cache: the view its need class
+        gives of the entry's storage (with this step's block-table rows, for a paged one)."""
+        if entry.cache is None or entry.cache not in cache.needs:
+            return CacheView(writes=False if entry.cache is None else entry.writes_cache)
+        group = cache.entry_group.get(entry.cache)
+        table = None if group is None else self.block_tables[group]
+        return cache.view(entry.cache, table, entry.writes_cache)
 
 
 class Stepper:
@@ -291,6 +337,7 @@ class Stepper:
                                   device=model.device)
         self.steps = 0
         self.tokens_run = 0
+        self.providers = model.step_array_providers()      # parts whose index arrays travel with a step's upload
         # decode steps (every segment one token) are captured in a HIP graph per batch size and
         # context bucket and replayed, if every part of the model allows it
         self.use_graphs = all(block.graph_safe for block in model.layers) and model.final_norm.graph_safe
@@ -319,9 +366,10 @@ class Stepper:
         # reserve everything first so that a failure leaves no request half-served
         cache.reserve_all(requests, new_lengths, described[2])
         try:
-            if self.use_graphs and all(len(entry.tokens) == 1 for entry in entries):
+            if self.use_graphs and all(len(entry.tokens) == 1 and entry.positions is None for entry in entries):
                 return self._replay(self._decode_step(len(entries), max(new_lengths)), entries, described)
-            ctx = StepContext(entries, cache, self.device, spec.vocab_size, self.context_limit, described=described)
+            ctx = StepContext(entries, cache, self.device, spec.vocab_size, self.context_limit, described=described,
+                              providers=self.providers)
             logits = self.model.forward(ctx, cache)
         except BaseException:
             # The lengths stay where they were and the pages reserved for this step go back. What
@@ -354,7 +402,7 @@ class Stepper:
         if captured is None:
             cache = self.cache
             ctx = StepContext.for_decode_graph(batch, cache, self.device, max_context=pages * cache.page_size,
-                                               table_stride=pages)
+                                               table_stride=pages, providers=self.providers)
             captured = self._graphs[(batch, pages)] = _CapturedDecode(ctx)
         return captured
 
@@ -426,7 +474,7 @@ class Stepper:
                 ahead = 0                   # one step; the scheduler will decide who gives way
             else:
                 for g in range(len(cache.groups)):
-                    ctx._host[8 + g][:rows * stride] = cache.block_table_rows(g, (), stride=stride, natives=natives, count=rows).reshape(-1)
+                    ctx._host_tables[g][:rows * stride] = cache.block_table_rows(g, (), stride=stride, natives=natives, count=rows).reshape(-1)
         ctx.upload()
         # Nothing crosses to the host between the steps of a turn: the kernel that finds a step's most
         # likely tokens writes them to the turn's record and to the next step's token ids, and moves

@@ -17,6 +17,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256
+ABI_VERSION = 4
 
 _lib = None
 
@@ -33,8 +34,8 @@ def library() -> ctypes.CDLL:
         lib = ctypes.CDLL(path)
         lib.fw_last_error.restype = ctypes.c_char_p
         lib.fw_abi_version.restype = ctypes.c_int
-        if lib.fw_abi_version() != 3:
-            raise KernelError(f"{path}: kernel library ABI {lib.fw_abi_version()} != 3; rebuild it")
+        if lib.fw_abi_version() != ABI_VERSION:
+            raise KernelError(f"{path}: kernel library ABI {lib.fw_abi_version()} != {ABI_VERSION}; rebuild it")
         _lib = lib
     return _lib
 
@@ -88,7 +89,7 @@ def _want(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
 
 
 # ---------------------------------------------------------------------------------------
-def embed_rows(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+def embed_rows(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
     _dev(table, ids, out)
     _want(ids, torch.int32, "ids")
     vocab, hidden = table.shape
@@ -98,8 +99,19 @@ def embed_rows(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tenso
     _want(out, torch.float32, "out")
     if out.shape != (rows, hidden):
         raise KernelError(f"embed_rows: out is {tuple(out.shape)}, expected {(rows, hidden)}")
-    _check(library().fw_embed_rows(_p(table), _code(table.dtype), _p(ids), _p(out), rows, hidden, vocab, _stream()))
+    _check(library().fw_embed_rows(_p(table), _code(table.dtype), _p(ids), _p(out), rows, hidden, vocab,
+                                   ctypes.c_float(scale), _stream()))
     return out
+
+
+def scale_softcap_(x: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> torch.Tensor:
+    """In place on float32: x * scale, then with ``cap`` > 0 cap * tanh(x / cap)."""
+    _dev(x)
+    _want(x, torch.float32, "x")
+    if cap < 0:
+        raise KernelError("scale_softcap: the cap must not be negative")
+    _check(library().fw_scale_softcap(_p(x), ctypes.c_longlong(x.numel()), ctypes.c_float(scale), ctypes.c_float(cap), _stream()))
+    return x
 
 
 def rmsnorm_rows(x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
@@ -701,17 +713,28 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
     return out
 
 
+def attention_is_tiled(head_dim: int) -> bool:
+    """Whether bfloat16 attention with this head size runs on the matrix-core kernels (which
+    work on tiles of QUERY_TILE rows)."""
+    return head_dim % 16 == 0 and 16 <= head_dim <= MAX_HEAD_DIM
+
+
 def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
-              v_pages: torch.Tensor, block_table: torch.Tensor, ctx, scale: float, window: int = 0) -> torch.Tensor:
+              v_pages: torch.Tensor, block_table: torch.Tensor, ctx, scale: float, window: int = 0,
+              tile_seg: Optional[torch.Tensor] = None, tile_row0: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bfloat16 with a head size in steps of 16 runs on the matrix cores: the split-key decode
     kernel for segments of one row (all of them, or those a mixed step begins with: a single row
     would hold a 64-row tile of the prompt kernel and walk its whole context alone), the tiled
-    kernel for the rest; float32 and everything else on the generic kernel."""
-    fast = q.dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= MAX_HEAD_DIM
+    kernel for the rest (``tile_seg``, ``tile_row0``: the tiles of ``query_tiles`` in the order
+    workgroups take them, those of the leading single rows in front); float32 and everything
+    else on the generic kernel."""
+    fast = q.dtype == torch.bfloat16 and attention_is_tiled(head_dim)
     if fast and ctx.all_decode:
         return attention_decode(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                                 ctx.row_pos, scale, ctx.max_context, window)
     if fast:
+        if tile_seg is None or tile_row0 is None:
+            raise KernelError("attention: the tiled kernel needs the step's query tiles")
         single = getattr(ctx, "decode_prefix", 0)       # leading segments of one row: rows and tiles 0 .. single - 1
         # four query heads of a kv group per workgroup pay where the rows sit behind a long context
         # (a page is read once for the four); from the start of a prompt one head per workgroup
@@ -720,13 +743,13 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
         keys = min(window, ctx.max_context) if window else ctx.max_context      # the most keys a row can see
         together = 4 if head_dim <= 64 and num_heads // num_kv_heads >= 4 and keys >= 4 * rows else 0
         if single == 0:
-            return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.tile_seg,
-                                     ctx.tile_row0, ctx.seg_row0, ctx.row_pos, scale, window, heads_together=together)
+            return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, tile_seg,
+                                     tile_row0, ctx.seg_row0, ctx.row_pos, scale, window, heads_together=together)
         out = torch.empty_like(q)
         attention_decode(q[:single], num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                          ctx.row_pos, scale, ctx.max_context, window, out=out[:single])
         return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table,
-                                 ctx.tile_seg[single:], ctx.tile_row0[single:], ctx.seg_row0, ctx.row_pos, scale, window,
+                                 tile_seg[single:], tile_row0[single:], ctx.seg_row0, ctx.row_pos, scale, window,
                                  heads_together=together, out=out)
     return attention_generic(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                              ctx.row_pos, scale, window)

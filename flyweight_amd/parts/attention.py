@@ -12,6 +12,7 @@ from __future__ import annotations
 
 from typing import Dict
 
+import numpy as np
 import torch
 
 from ..cache.needs import PagedKV
@@ -86,6 +87,27 @@ class GQAttention(Mixer):
         self.q_norm_weight = tensors[self._name("q_norm")] if self.qk_norm else None
         self.k_norm_weight = tensors[self._name("k_norm")] if self.qk_norm else None
 
+    # The prompt kernel on the matrix cores works on tiles of up to 64 rows of one segment; which
+    # tiles there are, and in which order workgroups take them, is this part's business.
+    def step_arrays_key(self):
+        fast = getattr(self, "dtype", None) == torch.bfloat16 and ops.attention_is_tiled(self.head_dim)
+        return ("query_tiles", ops.QUERY_TILE) if fast else None
+
+    def step_arrays(self, batch):
+        seg_row0 = batch.host_seg_row0
+        tile_seg, tile_row0 = ops.query_tiles(seg_row0)
+        # Workgroups start in the order of the tiles: those that see the most keys go first, the short
+        # ones fill in behind. The tiles of the leading single rows stay in front (they go to the
+        # decode kernel and their tiles are skipped).
+        if len(tile_seg) - batch.decode_prefix > 1:
+            tile_seg, tile_row0 = np.asarray(tile_seg, dtype=np.int32), np.asarray(tile_row0, dtype=np.int32)
+            tile_end = np.minimum(tile_row0 + ops.QUERY_TILE, np.asarray(seg_row0, dtype=np.int32)[tile_seg + 1])
+            keys_seen = batch.host_row_pos[tile_end - 1].astype(np.int64)
+            keys_seen[:batch.decode_prefix] = np.iinfo(np.int64).max
+            order = np.argsort(-keys_seen, kind="stable")
+            tile_seg, tile_row0 = tile_seg[order], tile_row0[order]
+        return {"tile_seg": np.asarray(tile_seg, dtype=np.int32), "tile_row0": np.asarray(tile_row0, dtype=np.int32)}
+
     def forward(self, h, residual, ctx, cache):
         qkv = self.qkv.forward(h, out_dtype=torch.float32)      # normed, rotated and rounded once, below
         cos, sin = ctx.position_tables(self.position)
@@ -93,6 +115,8 @@ class GQAttention(Mixer):
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight,
             self.qk_norm_eps, cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table,
             ctx.row_seg, ctx.row_pos, write_kv=cache.writes)
+        tiles = ctx.step_arrays(self) if self.step_arrays_key() is not None else {}
         attended = ops.attention(q, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
-                                 cache.block_table, ctx, self.scale, int(self.window or 0))
+                                 cache.block_table, ctx, self.scale, int(self.window or 0),
+                                 tile_seg=tiles.get("tile_seg"), tile_row0=tiles.get("tile_row0"))
         return self.out.accumulate(attended, residual, then=getattr(ctx, "upcoming_norm", None))

@@ -47,6 +47,19 @@ class Part:
         self.dtype = dtype
         self.device = device
 
+    # Index arrays of a part's own that its kernels need for every step (the tiles a kernel cuts
+    # the rows into, the order it visits them in): built on the host from the batch, they travel
+    # to the device in the step's one upload and are found again with ``ctx.step_arrays(part)``.
+    def step_arrays_key(self):
+        """None: the part needs none (the default). Parts with equal keys share one set."""
+        return None
+
+    def step_arrays(self, batch) -> Dict[str, "numpy.ndarray"]:
+        """name -> int32 array, from ``batch.host_seg_row0`` (first row of each segment, and the
+        end), ``batch.host_row_pos``, ``batch.decode_prefix``, ``batch.num_rows``. For a recorded
+        decode step this is asked once, for segments of one row each."""
+        return {}
+
 
 class Norm(Part):
     def forward(self, x: torch.Tensor, ctx, row_index: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -35,7 +35,7 @@ class RotaryNeox(PositionEncoding):
     def tables(self, ctx):
         if self.rotary_dim == 0:
             return None, None
-        return ops.rope_table(ctx.row_pos, self._inv_freq)
+        return ops.rope_table(ctx.encoding_pos, self._inv_freq)
 
 
 @register_position_encoding("none")

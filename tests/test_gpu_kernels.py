@@ -566,13 +566,14 @@ def test_attention_gives_the_leading_single_rows_of_a_mixed_step_to_the_decode_k
     scale = 1 / math.sqrt(hd)
     d = lambda a: torch.tensor(np.asarray(a, dtype=np.int32), device=DEV)       # noqa: E731
     ctx = SimpleNamespace(all_decode=False, decode_prefix=2, max_context=max(lengths), row_seg=d(row_seg), row_pos=d(row_pos),
-                          tile_seg=d(tile_seg), tile_row0=d(tile_row0), seg_row0=d(seg_row0))
-    mixed = ops.attention(q, nh, nkv, hd, k_pages, v_pages, d(table), ctx, scale, window)
+                          seg_row0=d(seg_row0))
+    tiles = dict(tile_seg=d(tile_seg), tile_row0=d(tile_row0))
+    mixed = ops.attention(q, nh, nkv, hd, k_pages, v_pages, d(table), ctx, scale, window, **tiles)
     want = torch.stack([attention_reference(back(q)[r].reshape(nh, hd), keys[row_seg[r]], values[row_seg[r]], int(row_pos[r]),
                                             scale, window, nh // nkv).reshape(-1) for r in range(rows)])
     close(mixed, want, torch.bfloat16)
     ctx.decode_prefix = 0
-    tiled = ops.attention(q, nh, nkv, hd, k_pages, v_pages, d(table), ctx, scale, window)
+    tiled = ops.attention(q, nh, nkv, hd, k_pages, v_pages, d(table), ctx, scale, window, **tiles)
     assert torch.equal(mixed[2:], tiled[2:])        # the rows of the tiled kernel do not depend on who else it serves
 
 

@@ -1,6 +1,7 @@
 """Each part of a layer alone, built from its PartSpec with its own sizes, against the
-plain implementation's function for that part; and a toy mixer with state of its own,
-defined here, that is registered, built and stepped without touching the framework."""
+plain implementation's function for that part; and toy parts defined here (a mixer with state
+of its own kind that does not start at zero, a feed-forward with routing, another position
+encoding) that are registered, built and stepped without touching the framework."""
 
 import dataclasses
 import math
@@ -178,21 +179,50 @@ def test_attention_part_with_a_window_and_partial_rotation(dtype):
 
 
 # ----- a toy mixer with state of its own ----------------------------------------------------
+PRIOR_SUM, PRIOR_COUNT = 0.5, 2.0      # what the toy mixer's state starts with: not zero
+
+
 def register_toy():
-    from flyweight_amd.cache import FixedState
+    from flyweight_amd.cache import CacheNeed
     from flyweight_amd.parts import Linear, Mixer, register_mixer
     from flyweight_amd.weights import TensorDecl
 
+    class RunningSums(CacheNeed):
+        """A need class of the toy's own: per request a running sum and a count, which start as if
+        two tokens had been seen already. The cache manager stores it, hands out its slots and
+        starts them by asking this class alone."""
+        paged = False
+
+        def __init__(self, width):
+            self.width = width
+
+        def __eq__(self, other):
+            return isinstance(other, RunningSums) and other.width == self.width
+
+        def __hash__(self):
+            return hash(("running_sums", self.width))
+
+        def allocate(self, units, page_size, dtype, device):
+            return {"sums": torch.full((units, self.width), float("nan"), device=device),
+                    "counts": torch.full((units,), float("nan"), device=device)}
+
+        def initial(self, storage, slot):
+            storage["sums"][slot] = PRIOR_SUM
+            storage["counts"][slot] = PRIOR_COUNT
+
+        def view(self, storage, block_table, writes):
+            return storage
+
     @register_mixer("toy_running_mean")
     class RunningMean(Mixer):
-        """out_t = W . mean(h_0..h_t). State per request: the running sum and the count."""
+        """out_t = W . (prior + h_0 + .. + h_t) / (prior count + t + 1)."""
 
         def __init__(self, spec):
             super().__init__(spec)
             self.hidden = int(spec["hidden_size"])
 
         def cache_need(self):
-            return FixedState((self.hidden + 1,), torch.float32)
+            return RunningSums(self.hidden)
 
         def tensors(self):
             return {self.prefix + "mix.weight": TensorDecl((self.hidden, self.hidden))}
@@ -205,12 +235,11 @@ def register_toy():
             means = torch.empty_like(h)
             for seg in range(ctx.num_segments):
                 lo, hi, slot = ctx.host_seg_row0[seg], ctx.host_seg_row0[seg + 1], ctx.host_seg_slot[seg]
-                state = cache.state[slot]
-                sums = state[:self.hidden] + torch.cumsum(h[lo:hi].float(), dim=0)
-                counts = state[self.hidden] + torch.arange(1, hi - lo + 1, device=h.device, dtype=torch.float32)
+                sums = cache["sums"][slot] + torch.cumsum(h[lo:hi].float(), dim=0)
+                counts = cache["counts"][slot] + torch.arange(1, hi - lo + 1, device=h.device, dtype=torch.float32)
                 means[lo:hi] = (sums / counts[:, None]).to(h.dtype)
-                state[:self.hidden] = sums[-1]
-                state[self.hidden] = counts[-1]
+                cache["sums"][slot] = sums[-1]
+                cache["counts"][slot] = counts[-1]
             self.mix.accumulate(means, residual)
     return RunningMean
 
@@ -246,7 +275,7 @@ def test_a_toy_mixer_with_its_own_state_is_registered_built_and_stepped(tmp_path
         x = w["model.embed_tokens.weight"][tokens]
         def toy(x):
             h = plain.rms_norm(x, w["model.layers.0.operator_norm.weight"], eps)
-            means = np.cumsum(h, axis=0) / np.arange(1, len(h) + 1)[:, None]
+            means = (PRIOR_SUM + np.cumsum(h, axis=0)) / (PRIOR_COUNT + np.arange(1, len(h) + 1))[:, None]
             x = x + means @ w["model.layers.0.toy.mix.weight"].T
             return x + plain.swiglu(plain.rms_norm(x, w["model.layers.0.ffn_norm.weight"], eps), w, "model.layers.0.feed_forward.")
         def attention(x, i, reuse=None):
@@ -297,8 +326,168 @@ def test_a_toy_mixer_with_its_own_state_is_registered_built_and_stepped(tmp_path
         want = expected(tokens)
         found = np.concatenate(got[request])
         assert np.abs(found - want).max() <= tolerance * np.abs(want).max()
-    # the toy state slot is zeroed for the next request
+    # the toy state's slot is put back to its start for the next request
     stepper.release("a")
     stepper.admit("c")
     again = stepper.step([StepEntry("c", a[:20], list(range(20)))]).cpu().numpy()
     assert np.abs(again - expected(a[:20])).max() <= tolerance * np.abs(expected(a[:20])).max()
+
+
+# ----- a toy feed-forward with routing and a toy position encoding -----------------------------
+TOY_STRETCH = 4.0
+TOY_ROUTER_GAIN = 8.0       # router logits far apart: few rows sit near the border between the experts
+TOY_TOKENS_SEED = 11      # with these tokens no row comes closer than 0.67
+TOY_AMBIGUOUS = 0.5         # below this difference of router logits rounding may send a row the other way
+
+
+def register_toy_router_and_positions():
+    from flyweight_amd.kernels import ops
+    from flyweight_amd.parts import FeedForward, Linear, register_feed_forward
+    from flyweight_amd.parts.base import PositionEncoding, register_position_encoding
+    from flyweight_amd.weights import TensorDecl
+
+    @register_feed_forward("toy_top1_of_two")
+    class TopOneOfTwo(FeedForward):
+        """Two SwiGLU experts and a router: a row goes to the expert with the larger router logit
+        (float32; ties to the first) and its output is weighted by the softmax share of that logit."""
+
+        def __init__(self, spec):
+            super().__init__(spec)
+            self.hidden, self.width = int(spec["hidden_size"]), int(spec["intermediate_size"])
+
+        def tensors(self):
+            declared = {self.prefix + "router.weight": TensorDecl((2, self.hidden), "vector", "matrix")}
+            for e in range(2):
+                declared[f"{self.prefix}experts.{e}.gate_up.weight"] = TensorDecl((2 * self.width, self.hidden))
+                declared[f"{self.prefix}experts.{e}.down.weight"] = TensorDecl((self.hidden, self.width))
+            return declared
+
+        def bind(self, tensors, dtype, device):
+            super().bind(tensors, dtype, device)
+            self.router = tensors[self.prefix + "router.weight"].float()
+            self.experts = [(Linear(tensors[f"{self.prefix}experts.{e}.gate_up.weight"]),
+                             Linear(tensors[f"{self.prefix}experts.{e}.down.weight"])) for e in range(2)]
+
+        def forward(self, h, residual, ctx):
+            logits = TOY_ROUTER_GAIN * (h.float() @ self.router.T)
+            share = torch.softmax(logits, dim=-1)
+            chosen = (logits[:, 1] > logits[:, 0]).long()
+            for e, (gate_up, down) in enumerate(self.experts):
+                rows = torch.nonzero(chosen == e).flatten()
+                if rows.numel() == 0:
+                    continue
+                out = torch.zeros((rows.numel(), self.hidden), dtype=torch.float32, device=h.device)
+                down.accumulate(gate_up.swiglu(h[rows].contiguous()), out)
+                residual.index_add_(0, rows, out * share[rows, e, None])
+
+    @register_position_encoding("toy_stretched_rotary")
+    class StretchedRotary(PositionEncoding):
+        """Half-split rotation by the angle of position / stretch: the tables the attention part's
+        kernels take, made another way."""
+        graph_safe = True
+
+        def __init__(self, spec):
+            super().__init__(spec)
+            self.theta, self.rotary_dim, self.stretch = float(spec["theta"]), int(spec["head_dim"]), float(spec["stretch"])
+
+        def bind(self, tensors, dtype, device):
+            super().bind(tensors, dtype, device)
+            half = self.rotary_dim // 2
+            self.inv_freq = (self.theta ** (-(torch.arange(half, dtype=torch.float64) * 2.0 / self.rotary_dim)) / self.stretch).to(device)
+
+        def tables(self, ctx):
+            return ops.rope_table(ctx.encoding_pos, self.inv_freq)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_routing_feed_forward_and_position_encoding_need_no_change_to_the_framework(tmp_path, dtype):
+    """Layer 1 of tiny A gets a routed feed-forward and a stretched rotation, both defined in this
+    file; the model also scales its embeddings and caps its logits (``ModelSpec`` fields no LFM2
+    uses). Whole prompt against portions and decoded tokens, against a plain evaluation; and a
+    shift of the positions that the encoding sees leaves the logits where they were."""
+    from flyweight_amd.config import PartSpec, config_from_dict
+    from flyweight_amd.engine import CausalLM, StepEntry, Stepper
+    from flyweight_amd.engine.model import parse_dtype
+    from flyweight_amd.weights import load_tensors, random_tensors, write_file
+    from helpers import TINY_A
+    register_toy_router_and_positions()
+    base = config_from_dict(TINY_A).model_spec()
+    layer = base.layers[1]
+    position = PartSpec("toy_stretched_rotary", {"theta": 10000.0, "head_dim": 16, "stretch": TOY_STRETCH})
+    mixer = dataclasses.replace(layer.mixer, params={**layer.mixer.params, "position": position})
+    ffn = PartSpec("toy_top1_of_two", {"hidden_size": 64, "intermediate_size": 48}, prefix="model.layers.1.moe.")
+    spec = dataclasses.replace(base, layers=(base.layers[0], dataclasses.replace(layer, mixer=mixer, ffn=ffn)) + base.layers[2:],
+                               embedding_scale=1.5, logit_scale=0.5, logit_softcap=2.0)
+    model = CausalLM(spec)
+    folder = str(tmp_path / "toy2")
+    os.makedirs(folder)
+    write_file(os.path.join(folder, "model.safetensors"), random_tensors(model.tensors(), 9, scale="fan_in"))
+    torch_dtype = parse_dtype(dtype)
+    tensors = load_tensors(folder, model.tensors(), torch_dtype, DEV)
+    model.bind(tensors, torch_dtype, DEV)
+    w = {n: t.double().cpu().numpy() for n, t in tensors.items()}
+    config = dict(TINY_A)
+    eps = config["norm_eps"]
+
+    def expected(tokens, shift=0):
+        """Logits, and the first row whose routing is a close call (rows from there on may differ
+        in bfloat16: top-1 routing is not continuous)."""
+        x = 1.5 * w["model.embed_tokens.weight"][tokens]
+        T = len(tokens)
+        close_call = T
+        for i, is_attention in enumerate(plain.attention_layers(config)):
+            p = f"model.layers.{i}."
+            h = plain.rms_norm(x, w[p + "operator_norm.weight"], eps)
+            if is_attention:
+                positions = (np.arange(T) + shift) / (TOY_STRETCH if i == 1 else 1.0)
+                q, k, v = plain.attention_qkv(h, w, p + "self_attn.", config, positions)
+                x = x + plain.causal_attention(q, k, v, 0.25).reshape(T, -1) @ w[p + "self_attn.out_proj.weight"].T
+            else:
+                x = x + plain.short_conv_mixer(h, w, p + "conv.", config)
+            h = plain.rms_norm(x, w[p + "ffn_norm.weight"], eps)
+            if i == 1:
+                logits = TOY_ROUTER_GAIN * (h @ w[p + "moe.router.weight"].T)
+                share = np.exp(logits - logits.max(-1, keepdims=True))
+                share /= share.sum(-1, keepdims=True)
+                near = np.nonzero(np.abs(logits[:, 1] - logits[:, 0]) < TOY_AMBIGUOUS)[0]
+                close_call = int(near[0]) if len(near) else T
+                x = x.copy()
+                for t in range(T):
+                    e = int(logits[t, 1] > logits[t, 0])
+                    both = h[t] @ w[f"{p}moe.experts.{e}.gate_up.weight"].T
+                    x[t] = x[t] + share[t, e] * ((plain.silu(both[:48]) * both[48:]) @ w[f"{p}moe.experts.{e}.down.weight"].T)
+                assert 0.2 < (logits[:, 1] > logits[:, 0]).mean() < 0.8       # both experts work
+            else:
+                x = x + plain.swiglu(h, w, p + "feed_forward.")
+        logits = 0.5 * (plain.rms_norm(x, w["model.embedding_norm.weight"], eps) @ w["model.embed_tokens.weight"].T)
+        return 2.0 * np.tanh(logits / 2.0), close_call
+
+    tokens = np.random.default_rng(TOY_TOKENS_SEED).integers(0, 256, 100).tolist()
+    want, sure = expected(tokens)
+    assert sure >= 60                                           # chosen so: most rows are compared in bfloat16 too
+    compared = 100 if dtype == "float32" else sure
+    assert 0.3 < np.abs(want).max() < 2.0                      # the cap bends the logits but does not flatten them
+    stepper = Stepper(model, num_pages=6, max_requests=3)
+    tolerance = {"float32": 2e-5, "bfloat16": 3e-2}[dtype]
+    for request, cuts in (("whole", [100]), ("cut", [7, 2, 30, 1, 1, 1, 58])):
+        stepper.admit(request)
+        found, at = [], 0
+        for n in cuts:
+            found.append(stepper.step([StepEntry(request, tokens[at:at + n], list(range(n)))]).cpu().numpy())
+            at += n
+        assert np.abs(np.concatenate(found) - want)[:compared].max() <= tolerance * np.abs(want).max(), request
+    # positions are the encoding's business: shifted by a constant, only distances count, and the
+    # cache and the mask still follow the order of the tokens
+    stepper.admit("shifted")
+    found, at = [], 0
+    for n in (40, 1, 59):
+        entry = StepEntry("shifted", tokens[at:at + n], list(range(n)), positions=list(range(1000 + at, 1000 + at + n)))
+        found.append(stepper.step([entry]).cpu().numpy())
+        at += n
+    shifted = np.concatenate(found)
+    want_shifted, sure_shifted = expected(tokens, shift=1000)
+    compared = 100 if dtype == "float32" else min(sure, sure_shifted)
+    assert np.abs(shifted - want_shifted)[:compared].max() <= tolerance * np.abs(want).max()
+    assert np.abs(shifted - want)[:compared].max() <= 2 * tolerance * np.abs(want).max()
+    with pytest.raises(Exception, match="positions"):
+        stepper.step([StepEntry("shifted", [1, 2], [], positions=[5])])
