@@ -25,7 +25,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK = 2.5e15
 
-# BASELINE.json configs[2]: the LFM2-1.2B shape
+# The LFM2-1.2B shape, the headline configuration
 SHAPE = dict(
     architectures=["Lfm2ForCausalLM"], model_type="lfm2", vocab_size=65536, hidden_size=2048, num_hidden_layers=16,
     num_attention_heads=32, num_key_value_heads=8, intermediate_size=12288, block_auto_adjust_ff_dim=True,
@@ -34,9 +34,9 @@ SHAPE = dict(
 PROMPT = 2048
 CONTEXT = 4096
 
-# The two serving workloads BASELINE.json names beside the headline (configs[3] and configs[4]);
-# run with --workload, they print one JSON line of their own.
-SHAPE_350M = dict(SHAPE, hidden_size=1024, num_attention_heads=16, intermediate_size=6656, max_position_embeddings=33280)
+# The two serving workloads beside the headline (the LFM2-350M shape under long contexts, the
+# LFM2-2.6B shape under mixed traffic); run with --workload, they print one JSON line of their own.
+SHAPE_350M = dict(SHAPE, hidden_size=1024, num_attention_heads=16, intermediate_size=6656, max_position_embeddings=34816)
 SHAPE_2P6B = dict(SHAPE, num_hidden_layers=30, intermediate_size=10752, max_position_embeddings=9216,
                   full_attn_idxs=[2, 6, 10, 14, 18, 21, 24, 27])
 WORKLOADS = {
@@ -51,38 +51,6 @@ def log(text: str) -> None:
     print(f"[bench] {text}", file=sys.stderr, flush=True)
 
 
-def model_bytes(model) -> int:
-    """Bytes of every weight a decode step reads once (the tied table is read as the head)."""
-    seen, total = set(), 0
-    def add(t):
-        nonlocal total
-        if t is not None and t.data_ptr() not in seen:
-            seen.add(t.data_ptr())
-            total += t.numel() * t.element_size()
-    lm = model.model
-    add(lm.head.weight)
-    add(lm.final_norm.weight)
-    for block in lm.layers:
-        add(block.mixer_norm.weight), add(block.ffn_norm.weight)
-        add(block.ffn.gate_up.weight), add(block.ffn.down.weight)
-        mixer = block.mixer
-        for name in ("qkv", "out", "in_proj", "out_proj"):
-            if hasattr(mixer, name):
-                add(getattr(mixer, name).weight), add(getattr(mixer, name).bias)
-        for name in ("q_norm_weight", "k_norm_weight", "taps", "conv_bias"):
-            add(getattr(mixer, name, None))
-    return total
-
-
-def matmul_params(config) -> int:
-    h, ff = config.hidden_size, config.ff_dim
-    per_ffn = 3 * h * ff
-    conv = 3 * h * h + h * h
-    attn = (config.num_attention_heads + 2 * config.num_key_value_heads) * config.head_dim * h + h * config.num_attention_heads * config.head_dim
-    n_attn = len(config.full_attn_idxs)
-    return config.num_hidden_layers * per_ffn + (config.num_hidden_layers - n_attn) * conv + n_attn * attn
-
-
 DECODE_STEPS_PER_TURN = 4      # decode steps the engine runs on the device before the host is asked again
 
 
@@ -91,20 +59,27 @@ def steps_per_turn(steps: int, warmup: int) -> int:
     return DECODE_STEPS_PER_TURN if steps % DECODE_STEPS_PER_TURN == 0 and warmup % DECODE_STEPS_PER_TURN == 0 else 1
 
 
-def decode_run(torch, model, config, batch: int, steps: int, warmup: int, seed: int = 0):
-    """``batch`` requests with 2,048-token prompts; returns (seconds for ``steps`` decode steps, mean context)."""
+def decode_run(torch, model, config, batch: int, steps: int, warmup: int, seed: int = 0, prompt: int = PROMPT,
+               context: int = CONTEXT):
+    """``batch`` requests with prompts of ``prompt`` tokens; returns (seconds for ``steps`` decode steps, mean
+    context, bytes the step must read)."""
     import numpy as np
     from flyweight_amd import Runtime
+    from flyweight_amd.engine import accounting
     # requests admitted earlier decode while later prompts are still running (continuous
-    # batching), so they are up to ``batch`` tokens ahead when the timed steps begin
-    new_tokens = warmup + steps + batch + 2 + DECODE_STEPS_PER_TURN
-    pages_each = (PROMPT + new_tokens + 63) // 64
+    # batching), so they are up to one token for every portion of the later prompts ahead when the
+    # timed steps begin
+    portion = min(prompt, PROMPT)
+    new_tokens = warmup + steps + batch * -(-prompt // portion) + 2 + DECODE_STEPS_PER_TURN
+    if prompt + new_tokens > context:
+        raise ValueError(f"a context of {context} does not hold a prompt of {prompt} and {new_tokens} new tokens")
+    pages_each = (prompt + new_tokens + 63) // 64
     turn = steps_per_turn(steps, warmup)
-    runtime = Runtime(model, context_limit=CONTEXT, parallel_sequences=batch, num_pages=pages_each * batch,
-                      max_batch_tokens=PROMPT + batch, prefill_rows=PROMPT, decode_steps_per_turn=turn).prepare()
+    runtime = Runtime(model, context_limit=context, parallel_sequences=batch, num_pages=pages_each * batch,
+                      max_batch_tokens=portion + batch, prefill_rows=portion, decode_steps_per_turn=turn).prepare()
     rng = np.random.default_rng(seed)
     for _ in range(batch):
-        runtime.task_submit(rng.integers(0, config.vocab_size, PROMPT).tolist(), new_tokens)
+        runtime.task_submit(rng.integers(0, config.vocab_size, prompt).tolist(), new_tokens)
     # prompts: until every request has produced its first token
     while any(r.computed < len(r.prompt) for r in runtime.scheduler.requests.values()):
         runtime.engine_step()
@@ -126,27 +101,41 @@ def decode_run(torch, model, config, batch: int, steps: int, warmup: int, seed: 
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - began
     mean_context = before + 1 + (steps - 1) / 2.0      # keys a row sees, averaged over requests and steps
+    cache = runtime.stepper.cache
+    step_bytes = accounting.step_weight_bytes(model.model) + batch * (
+        mean_context * accounting.cache_bytes_per_token(cache) + accounting.state_bytes_per_request(cache))
     runtime.close()
-    return elapsed, mean_context
+    return elapsed, mean_context, step_bytes
 
 
-def prefill_run(torch, model, config, repeats: int = 3):
+def prefill_run(torch, model, config, repeats: int = 5, behind: int = 0, context: int = CONTEXT):
+    """The median time of one step of 2,048 prompt tokens (logits at the last) behind ``behind`` cached tokens
+    of the same request, and the flops of that step."""
+    import statistics
     import numpy as np
     from flyweight_amd import Runtime, StepEntry
-    runtime = Runtime(model, context_limit=CONTEXT, parallel_sequences=1, num_pages=PROMPT // 64 + 1).prepare()
-    tokens = np.random.default_rng(1).integers(0, config.vocab_size, PROMPT).tolist()
-    best = None
+    from flyweight_amd.engine import accounting
+    runtime = Runtime(model, context_limit=context, parallel_sequences=1, num_pages=(behind + PROMPT) // 64 + 1).prepare()
+    rng = np.random.default_rng(1)
+    times = []
     for i in range(repeats + 1):
         runtime.admit(i)
+        for _ in range(behind // PROMPT):
+            runtime.step([StepEntry(i, rng.integers(0, config.vocab_size, PROMPT).tolist(), [])])
+        tokens = rng.integers(0, config.vocab_size, PROMPT).tolist()
         torch.cuda.synchronize()
         began = time.perf_counter()
         runtime.step([StepEntry(i, tokens, [PROMPT - 1])])
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - began
         runtime.release(i)
-        if i > 0:
-            best = elapsed if best is None else min(best, elapsed)
-    return best
+        if i > 0:       # the first run loads kernels
+            times.append(elapsed)
+    lm = model.model
+    flops = (accounting.product_flops_per_token(lm) * PROMPT + accounting.head_flops_per_row(lm)
+             + accounting.attention_flops(lm, PROMPT, behind))
+    runtime.close()
+    return statistics.median(times), flops
 
 
 def attainable_run(torch):
@@ -224,14 +213,51 @@ def serving_run(torch, workload: str, requests: int, seed: int = 0) -> dict:
         "steps_with_prompt_tokens": {"count": info["prefill_calls"], "seconds": round(info["prefill_ns"] * 1e-9, 3)},
         "decode_only_steps": {"count": steps - info["prefill_calls"], "seconds": round(info["decode_ns"] * 1e-9, 3)},
         "higher_is_better": True, "dtype": "bf16", "data": "synthetic: seeded uniform token ids and lengths, random-init weights",
-        "config": {"model": spec["name"], "layers": config.num_hidden_layers, "hidden": config.hidden_size,
-                   "heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
-                   "head_dim": config.head_dim, "ff_dim": config.ff_dim, "vocab": config.vocab_size,
-                   "attention_layers": len(config.full_attn_idxs), "requests": requests,
-                   "prompt_tokens": sum(prompts), "generated_tokens": generated, "longest_context": context,
-                   "portion": PROMPT, "cache_pages": pages, "preemptions": preemptions,
-                   "decode_steps_per_turn": DECODE_STEPS_PER_TURN},
+        "config": config_record(config, spec["name"], requests=requests, prompt_tokens=sum(prompts),
+                                generated_tokens=generated, longest_context=context, portion=PROMPT, cache_pages=pages,
+                                preemptions=preemptions, decode_steps_per_turn=DECODE_STEPS_PER_TURN),
     }
+
+
+def config_record(config, name: str, **more) -> dict:
+    """Every size of the run, flat."""
+    record = {"model": name, "layers": config.num_hidden_layers, "layers_of_named_config": config.num_hidden_layers,
+              "hidden": config.hidden_size, "heads": config.num_attention_heads, "kv_heads": config.num_key_value_heads,
+              "head_dim": config.head_dim, "ff_dim": config.ff_dim, "vocab": config.vocab_size,
+              "attention_layers": len(config.full_attn_idxs), "conv_L_cache": config.conv_L_cache}
+    record.update(more)
+    return record
+
+
+def further_points(torch, args, points: dict) -> None:
+    """Decode and prefill at further sizes: more requests, a model that allows 128,000 positions run at a
+    4,096-token context, and the LFM2-350M shape behind 32,768-token contexts. Tokens a second, and for each
+    the fraction of the published peak that bounds it (``*_frac``)."""
+    from flyweight_amd import Model
+    from flyweight_amd.config import config_from_dict
+    config = config_from_dict(dict(SHAPE, max_position_embeddings=128000))
+    model = Model.random(config, seed=0, dtype="bfloat16")
+    for batch, steps in ((8, min(args.steps, 64)), (64, min(args.steps, 32)), (128, min(args.steps, 32)), (256, min(args.steps, 32))):
+        name = f"decode_b{batch}" + ("_maxpos128k" if batch <= 64 else "")
+        log(f"decode at batch {batch}, max_position_embeddings 128,000, context {CONTEXT}")
+        seconds, _, step_bytes = decode_run(torch, model, config, batch, steps, min(args.warmup, 8))
+        points[name] = round(batch * steps / seconds, 1)
+        points[name + "_frac"] = round(step_bytes / (seconds / steps) / 1e9 / HBM_PEAK_GBS, 4)
+    del model
+    torch.cuda.empty_cache()
+    long_context = 32768
+    config = config_from_dict(SHAPE_350M)
+    model = Model.random(config, seed=0, dtype="bfloat16")
+    log("LFM2-350M shape: a 2,048-token portion behind 30,720 cached tokens")
+    seconds, flops = prefill_run(torch, model, config, repeats=3, behind=long_context - PROMPT, context=long_context + 2048)
+    points["prefill_2048_behind_30720_350m"] = round(PROMPT / seconds, 1)
+    points["prefill_2048_behind_30720_350m_frac"] = round(flops / seconds / MFMA_BF16_PEAK, 4)
+    log("LFM2-350M shape: decode at batch 64 behind 32,768-token prompts")
+    steps = min(args.steps, 32)
+    seconds, _, step_bytes = decode_run(torch, model, config, 64, steps, min(args.warmup, 4), prompt=long_context,
+                                        context=long_context + 2048)
+    points["decode_b64_ctx32k_350m"] = round(64 * steps / seconds, 1)
+    points["decode_b64_ctx32k_350m_frac"] = round(step_bytes / (seconds / steps) / 1e9 / HBM_PEAK_GBS, 4)
 
 
 def main() -> int:
@@ -241,6 +267,7 @@ def main() -> int:
     parser.add_argument("--warmup", type=int, default=16)
     parser.add_argument("--batch", type=int, default=8)
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
+    parser.add_argument("--skip-further", action="store_true", help="without the points at further sizes")
     parser.add_argument("--only", choices=("decode", "prefill"), help="run one phase and print no JSON (for profiling)")
     parser.add_argument("--workload", choices=("headline",) + tuple(WORKLOADS), default="headline",
                         help="headline: the LFM2-1.2B decode and prefill figures; the others: a whole serving run")
@@ -249,7 +276,7 @@ def main() -> int:
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py measures one GPU: this engine has no multi-GPU path (asked for {args.gpus})", flush=True)
         return 2
-    if PROMPT + args.warmup + args.steps + 64 + 2 > CONTEXT:
+    if PROMPT + args.warmup + args.steps + 256 + 2 + DECODE_STEPS_PER_TURN > CONTEXT:
         print("bench.py: warmup + steps must leave the 4,096-token context room", flush=True)
         return 2
 
@@ -263,51 +290,44 @@ def main() -> int:
     config = config_from_dict(SHAPE)
     log("building the LFM2-1.2B shape with random bfloat16 weights")
     model = Model.random(config, seed=0, dtype="bfloat16")
-    weights = model_bytes(model)
-    kv_per_token = len(config.full_attn_idxs) * 2 * config.num_key_value_heads * config.head_dim * 2
-    state_per_request = (config.num_hidden_layers - len(config.full_attn_idxs)) * config.hidden_size * (config.conv_L_cache - 1) * 4
 
     if args.only == "decode":
-        elapsed, _ = decode_run(torch, model, config, args.batch, args.steps, args.warmup)
+        elapsed, _, _ = decode_run(torch, model, config, args.batch, args.steps, args.warmup)
         log(f"{args.batch * args.steps / elapsed:.1f} tokens/s")
         return 0
     log("prefill of 2,048 tokens")
-    prefill_s = prefill_run(torch, model, config)
+    prefill_s, prefill_flops = prefill_run(torch, model, config)
     if args.only == "prefill":
         log(f"{PROMPT / prefill_s:.1f} tokens/s")
         return 0
-    head_flops = 2 * config.vocab_size * config.hidden_size
-    attention_flops = len(config.full_attn_idxs) * 2 * config.num_attention_heads * config.head_dim * PROMPT * PROMPT
-    prefill_flops = 2 * matmul_params(config) * PROMPT + head_flops + attention_flops
 
     log(f"decode at batch {args.batch}: {args.warmup} warm-up and {args.steps} timed steps")
-    elapsed, mean_context = decode_run(torch, model, config, args.batch, args.steps, args.warmup)
+    elapsed, mean_context, step_bytes = decode_run(torch, model, config, args.batch, args.steps, args.warmup)
     value = args.batch * args.steps / elapsed
-    step_bytes = weights + args.batch * (mean_context * kv_per_token + state_per_request)
     achieved = step_bytes / (elapsed / args.steps) / 1e9
 
     points = {}
     if not args.skip_points:
         for batch, steps in ((1, min(args.steps, 128)), (64, min(args.steps, 64))):
             log(f"decode at batch {batch}")
-            seconds, _ = decode_run(torch, model, config, batch, steps, min(args.warmup, 8))
+            seconds, _, point_bytes = decode_run(torch, model, config, batch, steps, min(args.warmup, 8))
             points[f"decode_b{batch}"] = round(batch * steps / seconds, 1)
+            points[f"decode_b{batch}_frac"] = round(point_bytes / (seconds / steps) / 1e9 / HBM_PEAK_GBS, 4)
 
     log("a large copy and a large library product, for what the GPU gives a plain program")
     copy_gbs, product_tflops = attainable_run(torch)
+    if not args.skip_points and not args.skip_further:
+        del model
+        torch.cuda.empty_cache()
+        further_points(torch, args, points)
 
     print(json.dumps({
         "metric": "decode tok/s @ batch 8 (LFM2-1.2B shape, 2,048-token prompts, context 4,096)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic: seeded uniform token ids, random-init weights",
-        "config": {"model": "LFM2-1.2B shape", "layers": config.num_hidden_layers, "layers_of_named_config": 16,
-                   "hidden": config.hidden_size, "heads": config.num_attention_heads,
-                   "kv_heads": config.num_key_value_heads, "head_dim": config.head_dim, "ff_dim": config.ff_dim,
-                   "vocab": config.vocab_size, "attention_layers": len(config.full_attn_idxs),
-                   "conv_L_cache": config.conv_L_cache, "global_batch": args.batch, "prompt_len": PROMPT,
-                   "seq_len": CONTEXT, "decode_steps_per_turn": steps_per_turn(args.steps, args.warmup),
-                   "parallelism": "single GPU"},
+        "config": config_record(config, "LFM2-1.2B shape", global_batch=args.batch, prompt_len=PROMPT, seq_len=CONTEXT,
+                                decode_steps_per_turn=steps_per_turn(args.steps, args.warmup), parallelism="single GPU"),
         "prefill": {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(prefill_flops / prefill_s / MFMA_BF16_PEAK, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
