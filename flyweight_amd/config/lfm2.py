@@ -16,6 +16,7 @@ import os
 from dataclasses import dataclass, asdict
 from typing import Any, Dict, List, Mapping, Optional, Tuple
 
+from . import json_reader
 from .spec import (ConfigError, LayerSpec, ModelSpec, PartSpec, ScheduleEntry,
                    default_schedule)
 
@@ -24,9 +25,13 @@ _CONV_NAMES = ("conv", "short_conv", "shortconv")
 
 _REQUIRED = (
     "vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
-    "num_key_value_heads", "intermediate_size", "norm_eps", "rope_theta",
-    "conv_L_cache", "max_position_embeddings",
+    "num_key_value_heads", "max_position_embeddings",
 )
+# Keys that may be absent, and what stands for them then. rope_theta: the reference's default
+# (native/src/v2_runtime.cpp:4235); norm_eps: what its LFM2 fixture writes
+# (tests/lfm2_gguf_fixture.py:243); conv_L_cache: the width every LFM2 shape named here has.
+# Further: conv_bias false, tie_word_embeddings true, block_auto_adjust_ff_dim false.
+DEFAULTS = {"norm_eps": 1e-5, "rope_theta": 1000000.0, "conv_L_cache": 3}
 
 
 def _need(data: Mapping[str, Any], key: str) -> Any:
@@ -42,6 +47,23 @@ def _as_int(data: Mapping[str, Any], key: str) -> int:
             return int(value)
         raise ConfigError(f"config.json key '{key}' must be an integer, found {value!r}")
     return value
+
+
+def _with_defaults(data: Mapping[str, Any]) -> Dict[str, Any]:
+    """The keys with their documented defaults filled in, and the feed-forward width under its
+    one name: ``block_ff_dim`` is the architecture's original spelling of ``intermediate_size``."""
+    filled = dict(data)
+    for key, value in DEFAULTS.items():
+        if filled.get(key) is None:
+            filled[key] = value
+    width, original = filled.get("intermediate_size"), filled.get("block_ff_dim")
+    if width is not None and original is not None and width != original:
+        raise ConfigError(f"'intermediate_size' ({width}) and 'block_ff_dim' ({original}) disagree")
+    if width is None:
+        if original is None:
+            raise ConfigError("config.json is missing 'intermediate_size' (or 'block_ff_dim')")
+        filled["intermediate_size"] = original
+    return filled
 
 
 def _as_float(data: Mapping[str, Any], key: str) -> float:
@@ -154,6 +176,7 @@ class Lfm2Config:
             raise ConfigError("config.json must hold a JSON object")
         for key in _REQUIRED:
             _need(data, key)
+        data = _with_defaults(data)
         layers = _as_int(data, "num_hidden_layers")
         layer_types = _layer_types(data, layers)
         tie = _tie(data)
@@ -188,11 +211,10 @@ class Lfm2Config:
 
     @classmethod
     def from_json_file(cls, path: str) -> "Lfm2Config":
-        with open(path, "r", encoding="utf-8") as handle:
-            try:
-                data = json.load(handle)
-            except json.JSONDecodeError as error:
-                raise ConfigError(f"{path}: not valid JSON ({error})") from None
+        try:
+            data = json_reader.parse_file(path)
+        except json_reader.JsonError as error:
+            raise ConfigError(f"{path}: {error}") from None
         return cls.from_dict(data)
 
     def to_dict(self) -> Dict[str, Any]:

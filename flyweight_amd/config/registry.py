@@ -9,10 +9,10 @@ plan builder with a chain of string compares and refuses unknown names
 
 from __future__ import annotations
 
-import json
 import os
 from typing import Any, Dict, Mapping, Type
 
+from . import json_reader
 from .spec import ConfigError
 
 _ARCHITECTURES: Dict[str, Type] = {}
@@ -59,9 +59,8 @@ def load_config(model_dir: str):
     path = os.path.join(model_dir, "config.json")
     if not os.path.isfile(path):
         raise ConfigError(f"{model_dir}: no config.json")
-    with open(path, "r", encoding="utf-8") as handle:
-        try:
-            data = json.load(handle)
-        except json.JSONDecodeError as error:
-            raise ConfigError(f"{path}: not valid JSON ({error})") from None
+    try:
+        data = json_reader.parse_file(path)
+    except json_reader.JsonError as error:
+        raise ConfigError(f"{path}: {error}") from None
     return config_from_dict(data)

@@ -22,6 +22,8 @@ from typing import Dict, Iterable, List, Mapping, Tuple
 import numpy as np
 import torch
 
+from ..config import json_reader
+
 
 class SafetensorsError(ValueError):
     pass
@@ -67,8 +69,8 @@ def read_header(path: str) -> Dict[str, TensorEntry]:
                 f"{path}: header length {header_len} exceeds the file ({size} bytes); truncated?")
         raw = handle.read(header_len)
     try:
-        header = json.loads(raw.decode("utf-8"))
-    except (UnicodeDecodeError, json.JSONDecodeError) as error:
+        header = json_reader.parse(raw)
+    except json_reader.JsonError as error:
         raise SafetensorsError(f"{path}: header is not valid JSON ({error})") from None
     if not isinstance(header, dict):
         raise SafetensorsError(f"{path}: header must be a JSON object")
@@ -181,11 +183,10 @@ def checkpoint_files(model_dir: str) -> List[str]:
     native/src/v2_runtime.cpp:9961-9993)."""
     index = os.path.join(model_dir, "model.safetensors.index.json")
     if os.path.isfile(index):
-        with open(index, "r", encoding="utf-8") as handle:
-            try:
-                weight_map = json.load(handle)["weight_map"]
-            except (json.JSONDecodeError, KeyError, TypeError) as error:
-                raise SafetensorsError(f"{index}: malformed index ({error})") from None
+        try:
+            weight_map = json_reader.parse_file(index)["weight_map"]
+        except (json_reader.JsonError, KeyError, TypeError) as error:
+            raise SafetensorsError(f"{index}: malformed index ({error})") from None
         files = sorted(set(weight_map.values()))
     else:
         files = sorted(f for f in os.listdir(model_dir) if f.endswith(".safetensors"))

@@ -30,13 +30,33 @@ def test_feed_forward_width_rule(inter, auto, mult, multiple, expected):
 
 
 @pytest.mark.parametrize("key", ["vocab_size", "hidden_size", "num_hidden_layers", "num_attention_heads",
-                                 "num_key_value_heads", "intermediate_size", "norm_eps", "rope_theta",
-                                 "conv_L_cache", "max_position_embeddings"])
+                                 "num_key_value_heads", "intermediate_size", "max_position_embeddings"])
 def test_missing_key_is_named(key):
     data = dict(TINY_A)
     del data[key]
     with pytest.raises(ConfigError, match=key):
         config_from_dict(data)
+
+
+def test_documented_defaults_and_the_original_key_spellings():
+    """Keys that may be absent get their documented defaults; the architecture's original
+    spellings (block_ff_dim for the width, tie_embedding) are read as the generic ones are."""
+    from flyweight_amd.config.lfm2 import DEFAULTS
+    assert DEFAULTS == {"norm_eps": 1e-5, "rope_theta": 1000000.0, "conv_L_cache": 3}
+    data = {k: v for k, v in TINY_B.items() if k not in ("norm_eps", "rope_theta", "conv_L_cache", "conv_bias",
+                                                         "tie_word_embeddings", "block_auto_adjust_ff_dim")}
+    config = config_from_dict(data)
+    assert (config.norm_eps, config.rope_theta, config.conv_L_cache) == (1e-5, 1000000.0, 3)
+    assert (config.conv_bias, config.tie_word_embeddings, config.block_auto_adjust_ff_dim) == (False, True, False)
+    assert config.ff_dim == TINY_B["intermediate_size"]         # no adjustment unless asked for
+    original = dict(TINY_B, block_ff_dim=TINY_B["intermediate_size"], tie_embedding=False)
+    del original["intermediate_size"], original["tie_word_embeddings"]
+    assert config_from_dict(original) == config_from_dict(TINY_B)
+    assert config_from_dict(dict(TINY_B, block_ff_dim=TINY_B["intermediate_size"])) == config_from_dict(TINY_B)
+    with pytest.raises(ConfigError, match="disagree"):
+        config_from_dict(dict(TINY_B, block_ff_dim=TINY_B["intermediate_size"] + 64))
+    with pytest.raises(ConfigError, match="block_ff_dim"):
+        config_from_dict({k: v for k, v in TINY_B.items() if k != "intermediate_size"})
 
 
 def test_layer_kinds_from_either_key_and_their_agreement():
@@ -126,3 +146,38 @@ def test_round_trip_through_config_json(tmp_path):
     assert load_config(str(tmp_path)) == config
     with pytest.raises(ConfigError, match="no config.json"):
         load_config(str(tmp_path / "nothing"))
+
+
+# ----- the engine's own JSON reader -------------------------------------------------------------
+def test_json_reader_values_and_what_it_refuses():
+    import json
+    from flyweight_amd.config import json_reader
+    text = r'{"a": [1, -2, 3.5e2, true, false, null], "b": {"c": "x\n\u00e9\ud83d\ude00 \" \/"}, "n": 18446744073709551615, "f": 0.1}'
+    assert json.loads(text)["b"]["c"] == 'x\n\u00e9\U0001f600 " /'
+    value = json_reader.parse(text)
+    assert value == json.loads(text)
+    assert value["n"] == 2 ** 64 - 1 and isinstance(value["n"], int)       # offsets beyond 2^53 survive
+    assert value["f"].literal == "0.1" and value["a"][2].literal == "3.5e2" and isinstance(value["a"][0], int)
+    assert json_reader.parse(b"  [ ]  ") == [] and json_reader.parse("{}") == {}
+    for bad, offset, what in (('{"a": 1} x', 9, "follows"), ('{"a": 1,}', 8, "key"), ("[1 2]", 3, "','"), ('{"a" 1}', 5, "':'"),
+                              ('"abc', 0, "not closed"), ("01", 0, "leading zero"), ("[1.]", 1, "behind its point"),
+                              ('{"a": 1, "a": 2}', 9, "twice"), ("tru", 0, "expected a value"), ("", 0, "ends here"),
+                              ('"\\x"', 1, "escape")):
+        with pytest.raises(json_reader.JsonError, match=what) as caught:
+            json_reader.parse(bad)
+        assert caught.value.offset == offset, (bad, caught.value.offset)
+    deep = "[" * 64 + "]" * 64
+    assert json_reader.parse(deep) is not None
+    with pytest.raises(json_reader.JsonError, match="deeper than 64"):
+        json_reader.parse("[" * 65 + "]" * 65)
+    with pytest.raises(json_reader.JsonError, match="deeper"):
+        json_reader.parse("[" * 100000)            # no recursion error, whatever the depth
+
+
+def test_config_errors_carry_the_byte_offset(tmp_path):
+    from flyweight_amd.config import load_config
+    folder = tmp_path / "m"
+    folder.mkdir()
+    (folder / "config.json").write_text('{"architectures": ["Lfm2ForCausalLM"], "vocab_size": 12,, }')
+    with pytest.raises(ConfigError, match="byte 56: expected a key"):
+        load_config(str(folder))
