@@ -148,6 +148,10 @@ def ensure_built() -> str:
 HOST_DIR = os.path.join(CSRC, "host")
 HOST_LIB_NAME = "libflyweight_host.so"
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+HOST_SELFTEST = "selftest.cpp"      # a program of its own (see build_host_selftest), not part of the library
+# address and undefined-behaviour sanitizers, their runtimes linked into the program itself
+SANITIZE_FLAGS = ["-O1", "-g", "-std=c++17", "-Wall", "-fno-omit-frame-pointer", "-fsanitize=address,undefined",
+                  "-fno-sanitize-recover=undefined", "-static-libasan", "-static-libubsan"]
 
 
 def _host_fingerprint() -> str:
@@ -188,7 +192,7 @@ def find_host_library(require_current: bool = True) -> Optional[str]:
 def build_host(verbose: bool = True) -> str:
     folder = _writable_dir()
     started = time.time()
-    units = sorted(os.path.join(HOST_DIR, f) for f in os.listdir(HOST_DIR) if f.endswith(".cpp"))
+    units = sorted(os.path.join(HOST_DIR, f) for f in os.listdir(HOST_DIR) if f.endswith(".cpp") and f != HOST_SELFTEST)
     lib = os.path.join(folder, HOST_LIB_NAME)
     partial = lib + f".{os.getpid()}.tmp"
     result = subprocess.run([_host_compiler(), *HOST_FLAGS, "-o", partial, *units], capture_output=True, text=True)
@@ -200,6 +204,20 @@ def build_host(verbose: bool = True) -> str:
     if verbose:
         _say(f"built {lib} in {time.time() - started:.0f} s")
     return lib
+
+
+def build_host_selftest(folder: Optional[str] = None) -> str:
+    """Builds the host library's sources together with ``selftest.cpp`` into one program under
+    the address and undefined-behaviour sanitizers and returns its path. The program drives the
+    C entry points through random request lifetimes and scheduler runs and exits with 0 when
+    every check held and the sanitizers found nothing."""
+    folder = folder or _writable_dir()
+    program = os.path.join(folder, "host_selftest_sanitized")
+    units = sorted(os.path.join(HOST_DIR, f) for f in os.listdir(HOST_DIR) if f.endswith(".cpp"))
+    result = subprocess.run([_host_compiler(), *SANITIZE_FLAGS, "-o", program, *units], capture_output=True, text=True)
+    if result.returncode != 0:
+        raise RuntimeError(f"building the sanitized host self-test failed:\n{result.stderr}")
+    return program
 
 
 def ensure_host_built() -> str:
