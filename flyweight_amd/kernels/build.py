@@ -234,6 +234,51 @@ def ensure_host_built() -> str:
         raise
 
 
+# ----- the plain C++ references of the kernels: host code, for tests ------------------------------
+REFERENCE_DIR = os.path.join(CSRC, "reference")
+REFERENCE_LIB_NAME = "libflyweight_reference.so"
+
+
+def _reference_fingerprint() -> str:
+    digest = hashlib.sha256()
+    for name in sorted(os.listdir(REFERENCE_DIR)):
+        if name.endswith((".cpp", ".h")):
+            digest.update(name.encode())
+            with open(os.path.join(REFERENCE_DIR, name), "rb") as handle:
+                digest.update(handle.read())
+    digest.update(" ".join(HOST_FLAGS).encode())
+    return digest.hexdigest()
+
+
+def build_reference(verbose: bool = True) -> str:
+    folder = _writable_dir()
+    started = time.time()
+    units = sorted(os.path.join(REFERENCE_DIR, f) for f in os.listdir(REFERENCE_DIR) if f.endswith(".cpp"))
+    lib = os.path.join(folder, REFERENCE_LIB_NAME)
+    partial = lib + f".{os.getpid()}.tmp"
+    result = subprocess.run([_host_compiler(), *HOST_FLAGS, "-o", partial, *units], capture_output=True, text=True)
+    if result.returncode != 0:
+        raise RuntimeError(f"building {REFERENCE_LIB_NAME} failed:\n{result.stderr}")
+    os.replace(partial, lib)
+    with open(os.path.join(folder, "reference.stamp"), "w", encoding="utf-8") as handle:
+        handle.write(_reference_fingerprint())
+    if verbose:
+        _say(f"built {lib} in {time.time() - started:.0f} s")
+    return lib
+
+
+def ensure_reference_built() -> str:
+    wanted = _reference_fingerprint()
+    for folder in build_dirs():
+        lib, stamp = os.path.join(folder, REFERENCE_LIB_NAME), os.path.join(folder, "reference.stamp")
+        if os.path.isfile(lib) and os.path.isfile(stamp):
+            with open(stamp, "r", encoding="utf-8") as handle:
+                if handle.read().strip() == wanted:
+                    return lib
+    return build_reference()
+
+
 if __name__ == "__main__":
     build()
     build_host()
+    build_reference()
