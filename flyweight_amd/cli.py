@@ -80,6 +80,9 @@ def build_parser() -> argparse.ArgumentParser:
     benchmark.add_argument("--temperature", type=float, default=0.0)
     benchmark.add_argument("--top-k", type=int, default=0)
     benchmark.add_argument("--top-p", type=float, default=0.0)
+    benchmark.add_argument("--kernel-profile", action="store_true",
+                           help="bracket every kernel call with events and add GPU time per kernel to the report "
+                                "(steps then run launch by launch, not from recorded graphs; also FLYWEIGHT_KERNEL_PROFILE=1)")
     _add_runtime(benchmark, 2048)
 
     inspect = commands.add_parser("inspect", help="print the configuration, derived sizes and tensor table as JSON")
@@ -131,6 +134,9 @@ def _benchmark(args) -> int:
     """The reference's protocol (src/flyweight/runtime_benchmark.py:129-216, cli.py:1749-1794):
     prompt + first token as one latency, then warm-up decodes, then timed decodes."""
     import torch
+    from .kernels import ops
+    if args.kernel_profile:
+        ops.kernel_profile(True)
     began = time.perf_counter()
     model, runtime = _runtime(args)
     torch.cuda.synchronize()
@@ -151,7 +157,7 @@ def _benchmark(args) -> int:
     measured = sum(gaps)
     ordered = sorted(gaps)
     pick = lambda q: ordered[min(len(ordered) - 1, int(q * len(ordered)))] if ordered else 0.0   # noqa: E731
-    print(json.dumps({
+    report = {
         "prepare_seconds": prepare_seconds,
         "prompt_tokens": len(args.tokens),
         "prompt_and_first_token_seconds": first,
@@ -160,7 +166,10 @@ def _benchmark(args) -> int:
         "median_seconds": statistics.median(gaps) if gaps else 0.0,
         "p90_seconds": pick(0.90),
         "p99_seconds": pick(0.99),
-    }))
+    }
+    if ops.kernel_profile_active():
+        report["kernels"] = ops.kernel_profile_report()
+    print(json.dumps(report))
     return 0
 
 

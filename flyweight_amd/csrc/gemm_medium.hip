@@ -54,6 +54,7 @@ struct MediumArgs {
     const float* squares;           // [squares_rows][row stride]
     int squares_rows;
     float eps;
+    int rotate;                     // workgroups start their walk over K at different chunks
 };
 
 // rows of the sums of squares are 16 wide for up to 16 rows of a (the fused decode product's
@@ -117,8 +118,18 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
     // Nothing is done to a loaded value before the chunk is used (a select right behind a load
     // would wait for it at once): W comes from a clamped address as it is, and the rows of a are
     // zeroed outside the slice when they move to LDS, three chunks after their load.
+    // Workgroups walk their slice of K from different chunks on (and around): all of them read the
+    // same rows of a, and in step they would ask one cache line of it at a time from every compute
+    // unit at once. Where a workgroup starts depends on its tile alone, so the order of its sum
+    // over K does not depend on the batch or on timing.
+    const int rotate = p.rotate ? (int)((tile * 5u + blockIdx.y * 3u) % (unsigned)(chunks > 0 ? chunks : 1)) : 0;
+    auto chunk_start = [&](const int c) {
+        if (c >= chunks) return k_end;                  // past the slice: nothing of it is inside
+        const int turned = c + rotate;
+        return k_begin + (turned < chunks ? turned : turned - chunks) * CHUNK;
+    };
     auto load = [&](const int d, const int c) {
-        const int k0 = k_begin + c * CHUNK;
+        const int k0 = chunk_start(c);
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             const int k = k0 + kp * 64 + ks * 32 + g * 8;
@@ -138,7 +149,7 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
         for (int i = 0; i < AP; ++i)
             if (PIECES % GM_THREADS == 0 || piece_row[i] < MT * 16) {
                 // K and the slices are multiples of 8: a run of 8 is inside or outside as a whole
-                const bool inside = k_begin + c * CHUNK + piece_k[i] < k_end;
+                const bool inside = chunk_start(c) + piece_k[i] < k_end;
                 *reinterpret_cast<bf16x8*>(&a_lds[buffer][piece_row[i]][piece_k[i]]) = inside ? areg[d][i] : none;
             }
     };
@@ -374,6 +385,9 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
 }
 
 // ----- host side ---------------------------------------------------------------------------
+static int medium_rotate = 1;
+extern "C" void fw_gemm_medium_set_rotate(int on) { medium_rotate = on; }
+
 struct MediumPlan {
     int mt, fw, tiles, splits, k_per_split;
     size_t workspace_bytes;
@@ -458,6 +472,7 @@ extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, v
     args.next_norm_weight = next_norm_weight; args.next_one_centered = next_one_centered;
     args.next_activations = (uint16_t*)next_activations; args.next_squares = next_squares;
     args.squares = squares; args.squares_rows = squares_rows; args.eps = eps;
+    args.rotate = medium_rotate;
     const dim3 grid(plan.tiles, plan.splits);
     hipStream_t s = (hipStream_t)stream;
     if (plan.fw == 4) {

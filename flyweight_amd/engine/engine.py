@@ -342,4 +342,8 @@ class Runtime:
         if self.stepper is not None:
             data.update(self.stepper.cache.stats())
             data["preemptions"] = self.scheduler.preemptions
+        from ..kernels import ops
+        if ops.kernel_profile_active():
+            # per kernel entry point: calls, GPU and host-launch milliseconds (FLYWEIGHT_KERNEL_PROFILE=1)
+            data["kernels"] = ops.kernel_profile_report()
         return data

@@ -366,7 +366,7 @@ class Stepper:
         # reserve everything first so that a failure leaves no request half-served
         cache.reserve_all(requests, new_lengths, described[2])
         try:
-            if self.use_graphs and all(len(entry.tokens) == 1 and entry.positions is None for entry in entries):
+            if self.use_graphs and not ops.kernel_profile_active() and all(len(entry.tokens) == 1 and entry.positions is None for entry in entries):
                 return self._replay(self._decode_step(len(entries), max(new_lengths)), entries, described)
             ctx = StepContext(entries, cache, self.device, spec.vocab_size, self.context_limit, described=described,
                               providers=self.providers)
@@ -421,7 +421,7 @@ class Stepper:
     def planned_decode(self, rows: int, context: int) -> Optional["_CapturedDecode"]:
         """The decode step that serves a scheduler's plan of ``rows`` single tokens whose
         sequences reach at most ``context`` tokens, or None where decode steps are not recorded."""
-        return self._decode_step(self.kept_batch(rows), context) if self.use_graphs else None
+        return self._decode_step(self.kept_batch(rows), context) if self.use_graphs and not ops.kernel_profile_active() else None
 
     def _run(self, captured: "_CapturedDecode") -> None:
         """Runs the step whose index arrays have been uploaded; its logits are ``captured.logits``

@@ -8,7 +8,9 @@ or without a GPU these functions raise.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+import os
+import time
+from typing import Dict, Optional
 
 import torch
 
@@ -26,9 +28,80 @@ class KernelError(RuntimeError):
     pass
 
 
-def library() -> ctypes.CDLL:
+class _ProfiledLibrary:
+    """The kernel library with every call bracketed by two events on the current stream.
+    Nothing is waited for at a launch (a host that waits lets the GPU's clock drop, which would
+    rescale every figure): the events are read when the report is asked for, as the reference's
+    per-kernel profile does (native/src/v2_runtime.cpp:27590-27728)."""
+    CAPACITY = 1 << 16
+
+    def __init__(self, lib):
+        self._library = lib
+        self._pending = []          # (name, first event, second event)
+        self._totals: Dict[str, Dict[str, float]] = {}
+        self.overflow = 0
+
+    def __getattr__(self, name):
+        entry = getattr(self._library, name)
+        if not name.startswith("fw_") or name in ("fw_last_error", "fw_abi_version") or name.endswith(("_plan", "_fits", "_tiles")):
+            return entry
+
+        def timed(*args):
+            if len(self._pending) >= self.CAPACITY or torch.cuda.is_current_stream_capturing():
+                self.overflow += 1
+                return entry(*args)
+            first, second = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            first.record()
+            began = time.perf_counter()
+            status = entry(*args)
+            host_ms = (time.perf_counter() - began) * 1e3
+            second.record()
+            self._pending.append((name, first, second))
+            total = self._totals.setdefault(name, {"calls": 0, "gpu_ms": 0.0, "host_launch_ms": 0.0, "max_us": 0.0})
+            total["calls"] += 1
+            total["host_launch_ms"] += host_ms
+            return status
+        return timed
+
+    def report(self) -> Dict[str, Dict[str, float]]:
+        torch.cuda.synchronize()
+        for name, first, second in self._pending:
+            ms = first.elapsed_time(second)
+            total = self._totals[name]
+            total["gpu_ms"] += ms
+            total["max_us"] = max(total["max_us"], ms * 1e3)
+        self._pending = []
+        return {name: dict(total) for name, total in sorted(self._totals.items(), key=lambda item: -item[1]["gpu_ms"])}
+
+
+_profiled: Optional[_ProfiledLibrary] = None
+
+
+def kernel_profile(enable: bool = True) -> None:
+    """Switches the per-kernel profile on or off (also switched on by FLYWEIGHT_KERNEL_PROFILE=1
+    in the environment, as in the reference). While it is on, steps are not recorded into graphs."""
+    global _profiled
+    if enable and _profiled is None:
+        _profiled = _ProfiledLibrary(library())
+    elif not enable:
+        _profiled = None
+
+
+def kernel_profile_active() -> bool:
+    return _profiled is not None
+
+
+def kernel_profile_report() -> Dict[str, Dict[str, float]]:
+    """Entry point -> calls, GPU milliseconds between its two events, host milliseconds inside
+    the launching call, the longest single call in microseconds; sorted by GPU time."""
+    return _profiled.report() if _profiled is not None else {}
+
+
+def library():
     """Loads (building first if nothing is built) the kernel library."""
     global _lib
+    if _profiled is not None:
+        return _profiled
     if _lib is None:
         path = _build.ensure_built()
         lib = ctypes.CDLL(path)
@@ -37,6 +110,9 @@ def library() -> ctypes.CDLL:
         if lib.fw_abi_version() != ABI_VERSION:
             raise KernelError(f"{path}: kernel library ABI {lib.fw_abi_version()} != {ABI_VERSION}; rebuild it")
         _lib = lib
+        if os.environ.get("FLYWEIGHT_KERNEL_PROFILE", "")[:1] == "1":
+            kernel_profile(True)
+            return _profiled
     return _lib
 
 
@@ -333,7 +409,8 @@ def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out
     (K split over workgroups) for up to 64, the tiled ones beyond (large tiles where they fill the
     chip, K cut into slices where even the small tiles are too few)."""
     M, K = a.shape
-    if SKINNY_MAX_ROWS < M <= MEDIUM_MAX_ROWS:
+    if SKINNY_MAX_ROWS < M <= MEDIUM_MAX_ROWS or (M <= SKINNY_MAX_ROWS and w.numel() >= MEDIUM_LARGE and K % 8 == 0):
+        # also a few rows of a large W (a vocabulary's head: 65,536 x 2,048 at 8 rows 52 against 61 us)
         gemm_medium_into(a, w, bias, target, out_code, mode, N)
         return
     if M <= SKINNY_MAX_ROWS:
@@ -360,6 +437,7 @@ def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out
 
 SKINNY_MAX_ROWS = 16
 MEDIUM_MAX_ROWS = 64
+MEDIUM_LARGE = 1 << 25    # weights from which the medium product beats the skinny one at any number of rows
 BIG_TILES_MIN = 192      # 256 x 256 tiles from which the large-tile prompt product is used (256 compute units)
 DEEP_MIN_K = 1024         # adding into the residual (2,048 x 2,048 x 2,048: 31 vs 39 us; x 8,192: 83 vs 118 us; 2,048 x 1,024 x 1,024: 13 vs 15 us)
 DEEP_MIN_K_STORE = 4096   # storing: no old values travel during the exchange at a tile's end, a short K gains nothing

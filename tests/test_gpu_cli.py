@@ -68,6 +68,15 @@ def test_benchmark_and_inspect_print_json(folders, capsys):
     assert status == 0 and report["prompt_tokens"] == 3 and report["iterations"] == 9
     assert report["decode_tokens_per_second"] > 0 and 0 < report["median_seconds"] <= report["p99_seconds"]
     assert report["prompt_and_first_token_seconds"] > 0 and report["prepare_seconds"] > 0
+    # the same with the per-kernel profile: GPU time per kernel entry point, and steps without graphs
+    from flyweight_amd.kernels import ops
+    try:
+        status, out, _ = run(capsys, "benchmark", folders["A"], "--tokens", "5,6,7", "--warmup", "1", "--iterations", "4", "--kernel-profile")
+    finally:
+        ops.kernel_profile(False)
+    kernels = json.loads(out)["kernels"]
+    assert status == 0 and kernels["fw_embed_rows"]["calls"] >= 6 and kernels["fw_gemm_decode"]["gpu_ms"] > 0
+    assert all(entry["host_launch_ms"] > 0 and entry["max_us"] > 0 for entry in kernels.values())
     status, out, _ = run(capsys, "inspect", folders["B"])
     shown = json.loads(out)
     config, weights = plain.read_folder(folders["B"])
