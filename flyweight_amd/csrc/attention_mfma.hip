@@ -409,16 +409,73 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
 // unnormalised output, then maximum and sum; a split with nothing to do writes nothing and takes
 // no ticket. The last workgroup of a (row, kv head, head tile) to arrive merges what the others
 // left; the only workgroup of a short row writes the result at once.
-template <int HD>
+// What the fused variant does in front of the attention: the step's raw projections (float32
+// [rows][(heads + 2 kv heads) * head_dim]: queries, keys, values) get their per-head RMS norm and
+// rotation here, as qk_norm_rope_kv_write does in a kernel of its own (the same arithmetic in the
+// same order), so that a decode step needs no such kernel. Every workgroup norms and rotates the
+// query heads it works on; the workgroup whose pages include the row's own position also norms and
+// rotates the new key, stores it and the new value in their page, and reads them back from there
+// with the rest of the page (its own stores, ordered by a workgroup barrier).
+struct FusedProjections {
+    const float* qkv;               // null: q holds finished bfloat16 queries and the cache is up to date
+    const float* q_norm_weight;     // [head_dim] or null
+    const float* k_norm_weight;
+    float eps;
+    const float* cos_table;         // [rows][rotary_dim / 2]
+    const float* sin_table;
+    int rotary_dim;
+    int write_kv;                   // 0: another execution of the layer has stored this step's keys and values already
+};
+
+// One head-vector of head_dim channels by one wave: optional RMS norm, then the half-split rotation
+// of the first rotary_dim channels; `store(d, value)` takes the results. scratch: head_dim floats of
+// LDS of the wave's own. (native/include/flyweight_v2_native_kernels.hpp:1015-1050)
+template <typename Store>
+__device__ __forceinline__ void norm_rotate_vector(const float* __restrict__ source, const float* __restrict__ weight, float eps,
+                                                   const float* __restrict__ cos_row, const float* __restrict__ sin_row,
+                                                   int rotary_dim, int head_dim, float* scratch, Store store) {
+    const int lane = threadIdx.x & 63;
+    float inv = 1.0f;
+    if (weight) {
+        float sum = 0.0f;
+        for (int d = lane; d < head_dim; d += 64) {
+            const float v = source[d];
+            sum += v * v;
+        }
+        sum = wave_sum(sum);
+        inv = rsqrtf(sum / (float)head_dim + eps);
+    }
+    for (int d = lane; d < head_dim; d += 64) {
+        const float v = source[d];
+        scratch[d] = weight ? v * inv * weight[d] : v;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int half = rotary_dim / 2;
+    for (int d = lane; d < head_dim; d += 64) {
+        float value = scratch[d];
+        if (d < rotary_dim) {
+            const int pair = d < half ? d : d - half;
+            const float other = scratch[d < half ? d + half : d - half];
+            const float c = cos_row[pair], s = sin_row[pair];
+            value = d < half ? value * c - other * s : value * c + other * s;
+        }
+        store(d, value);
+    }
+}
+
+template <int HD, bool FUSED>
 __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_eu(HD <= 128 ? 2 : 1))) void attention_decode_split_kernel(
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* partial, int* tickets,
-    const uint16_t* __restrict__ k_pages,
-    const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
+    uint16_t* k_pages, uint16_t* v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ row_seg, const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads,
-    int head_dim, float scale_log2, int window, int max_splits) {
+    int head_dim, float scale_log2, int window, int max_splits, const FusedProjections fused) {
     __shared__ f32x4 shared_o[SPLIT_PAGES][HD / 16][64];
     __shared__ float shared_m[SPLIT_PAGES][16], shared_l[SPLIT_PAGES][16];
     __shared__ int ticket_shared;
+    __shared__ __attribute__((aligned(16))) uint16_t fused_q[FUSED ? 16 : 1][FUSED ? HD : 8];
+    __shared__ float fused_scratch[FUSED ? SPLIT_PAGES : 1][FUSED ? HD : 1];
     const int row = blockIdx.x, split = blockIdx.z;
     const int group = num_heads / num_kv_heads;
     const int head_tiles = (group + 15) / 16;
@@ -437,7 +494,43 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
 
     Columns<HD> columns_of_wave[1];
     Columns<HD>& c = columns_of_wave[0];
-    load_query<HD>(c, q + ((size_t)row * num_heads + head) * head_dim, head_dim, valid);
+    if (FUSED) {
+        const int width = (num_heads + 2 * num_kv_heads) * head_dim;
+        const float* projections = fused.qkv + (size_t)row * width;
+        const int half = fused.rotary_dim / 2;
+        const float* cos_row = fused.cos_table + (size_t)row * half;
+        const float* sin_row = fused.sin_table + (size_t)row * half;
+        const int columns = group - head_tile * 16 < 16 ? group - head_tile * 16 : 16;
+        // the vectors of this workgroup: its query heads, then (where the row's own position lies
+        // in its pages) the new key and the new value; a wave takes every fourth
+        const bool stores = fused.write_kv && last_block < first_block + SPLIT_PAGES;
+        const int vectors = columns + (stores ? 2 : 0);
+        const int slot = pos % PAGE;
+        const int own_page = stores ? block_table[(size_t)segment * table_stride + last_block] : 0;
+        for (int v = wave; v < vectors; v += SPLIT_PAGES) {
+            if (v < columns) {
+                uint16_t* dest = fused_q[v];
+                norm_rotate_vector(projections + (size_t)(kvh * group + head_tile * 16 + v) * head_dim, fused.q_norm_weight, fused.eps,
+                                   cos_row, sin_row, fused.rotary_dim, head_dim, fused_scratch[wave],
+                                   [&](int d, float value) { dest[d] = float_to_bf16_bits(value); });
+            } else if (v == columns) {
+                uint16_t* dest = k_pages + (((size_t)own_page * num_kv_heads + kvh) * PAGE + slot) * head_dim;
+                norm_rotate_vector(projections + (size_t)(num_heads + kvh) * head_dim, fused.k_norm_weight, fused.eps, cos_row, sin_row,
+                                   fused.rotary_dim, head_dim, fused_scratch[wave],
+                                   [&](int d, float value) { dest[d] = float_to_bf16_bits(value); });
+            } else {
+                const float* value = projections + (size_t)(num_heads + num_kv_heads + kvh) * head_dim;
+                uint16_t* dest = v_pages + ((size_t)own_page * num_kv_heads + kvh) * head_dim * PAGE + slot;
+                for (int d = lane; d < head_dim; d += 64) dest[(size_t)d * PAGE] = float_to_bf16_bits(value[d]);
+            }
+        }
+        // the page is read below by this workgroup's own waves: its stores have to be done first
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        load_query<HD>(c, fused_q[valid ? col : 0], head_dim, valid);
+    } else {
+        load_query<HD>(c, q + ((size_t)row * num_heads + head) * head_dim, head_dim, valid);
+    }
     const int block = first_block + wave;
     if (block <= last_block) {
         const int page = block_table[(size_t)segment * table_stride + block];
@@ -619,6 +712,46 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
     return 0;
 }
 
+static int decode_check(int max_splits, int max_context, int* tickets, int tickets_len, int table_stride, int rows, int num_heads,
+                        int num_kv_heads, int head_dim, int window, int page_size, int num_pages) {
+    if (check_common("attention_decode", rows, num_heads, num_kv_heads, head_dim, page_size, window, num_pages, table_stride)) return -1;
+    FW_REQUIRE(max_splits >= 1 && max_splits <= 65535, "attention_decode: max_splits %d outside 1..65535", max_splits);
+    FW_REQUIRE(max_context >= 1, "attention_decode: max_context must be positive");
+    int blocks = (max_context + PAGE - 1) / PAGE;
+    if (window > 0 && (window + PAGE - 2) / PAGE + 1 < blocks) blocks = (window + PAGE - 2) / PAGE + 1;
+    FW_REQUIRE(max_splits * SPLIT_PAGES >= blocks, "attention_decode: %d splits of %d pages do not cover %d pages of context",
+               max_splits, SPLIT_PAGES, blocks);
+    FW_REQUIRE((max_context + PAGE - 1) / PAGE <= table_stride, "attention_decode: a context of %d tokens exceeds the block table (%d pages)",
+               max_context, table_stride);
+    const int head_tiles = (num_heads / num_kv_heads + 15) / 16;
+    FW_REQUIRE(rows <= 1 << 20 && num_kv_heads * head_tiles <= 65535 && num_heads <= 65535, "attention_decode: grid too large");
+    FW_REQUIRE(rows == 0 || max_splits == 1 || (tickets != nullptr && (long long)tickets_len >= (long long)rows * num_kv_heads * head_tiles),
+               "attention_decode: %d rows need %d ticket counters", rows, rows * num_kv_heads * head_tiles);
+    return 0;
+}
+
+static int decode_launch(const void* q, void* out, float* partial, int max_splits, int* tickets, void* k_pages, void* v_pages,
+                         const int32_t* block_table, int table_stride, const int32_t* row_seg, const int32_t* row_pos, int rows,
+                         int num_heads, int num_kv_heads, int head_dim, float scale, int window, const FusedProjections& fused,
+                         void* stream) {
+    if (rows == 0) return 0;
+    const int head_tiles = (num_heads / num_kv_heads + 15) / 16;
+    dim3 grid(rows, num_kv_heads * head_tiles, max_splits);
+#define CALL(HD)                                                                                                              \
+    if (fused.qkv)                                                                                                            \
+        attention_decode_split_kernel<HD, true><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                          \
+            (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits, fused);     \
+    else                                                                                                                      \
+        attention_decode_split_kernel<HD, false><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                         \
+            (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits, fused)
+    FW_BY_HEAD_DIM(head_dim, CALL);
+#undef CALL
+    FW_LAUNCH_CHECK("attention_decode");
+    return 0;
+}
+
 // One row per request. partial: float32 workspace of rows * heads * max_splits * (head_dim + 4).
 // max_context: no row's position reaches it (the caller knows; the kernel cannot check);
 // max_splits must cover the keys such a row sees, in runs of 4 pages. tickets: rows * kv heads *
@@ -630,30 +763,34 @@ extern "C" int fw_attention_decode(const void* q, void* out, float* partial, int
                                    const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                                    int num_kv_heads, int head_dim, float scale, int window, int page_size,
                                    int num_pages, void* stream) {
-    if (check_common("attention_decode", rows, num_heads, num_kv_heads, head_dim, page_size, window, num_pages, table_stride)) return -1;
-    FW_REQUIRE(max_splits >= 1 && max_splits <= 65535, "attention_decode: max_splits %d outside 1..65535", max_splits);
-    FW_REQUIRE(max_context >= 1, "attention_decode: max_context must be positive");
-    {
-        int blocks = (max_context + PAGE - 1) / PAGE;
-        if (window > 0 && (window + PAGE - 2) / PAGE + 1 < blocks) blocks = (window + PAGE - 2) / PAGE + 1;
-        FW_REQUIRE(max_splits * SPLIT_PAGES >= blocks, "attention_decode: %d splits of %d pages do not cover %d pages of context",
-                   max_splits, SPLIT_PAGES, blocks);
-        FW_REQUIRE((max_context + PAGE - 1) / PAGE <= table_stride, "attention_decode: a context of %d tokens exceeds the block table (%d pages)",
-                   max_context, table_stride);
-    }
-    if (rows == 0) return 0;
-    const int group = num_heads / num_kv_heads;
-    const int head_tiles = (group + 15) / 16;
-    FW_REQUIRE(rows <= 1 << 20 && num_kv_heads * head_tiles <= 65535 && num_heads <= 65535, "attention_decode: grid too large");
-    FW_REQUIRE(max_splits == 1 || (tickets != nullptr && (long long)tickets_len >= (long long)rows * num_kv_heads * head_tiles),
-               "attention_decode: %d rows need %d ticket counters", rows, rows * num_kv_heads * head_tiles);
-    dim3 grid(rows, num_kv_heads * head_tiles, max_splits);
-#define CALL(HD)                                                                                                   \
-    attention_decode_split_kernel<HD><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                                        \
-        (const uint16_t*)q, (uint16_t*)out, partial, tickets, (const uint16_t*)k_pages, (const uint16_t*)v_pages, \
-        block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits)
-    FW_BY_HEAD_DIM(head_dim, CALL);
-#undef CALL
-    FW_LAUNCH_CHECK("attention_decode");
-    return 0;
+    if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, window,
+                     page_size, num_pages)) return -1;
+    return decode_launch(q, out, partial, max_splits, tickets, const_cast<void*>(k_pages), const_cast<void*>(v_pages), block_table,
+                         table_stride, row_seg, row_pos, rows, num_heads, num_kv_heads, head_dim, scale, window, FusedProjections{}, stream);
+}
+
+// fw_attention_decode with the work of fw_qk_norm_rope_kv_write in front of it, in the same kernel:
+// qkv float32 [rows][(heads + 2 kv heads) * head_dim] are the step's raw projections; the new keys and
+// values are stored in their pages (write_kv 0: they are there already and only the queries are
+// formed). Norm weights float32 [head_dim] or null, rotation tables float32 [rows][rotary_dim / 2]
+// (null with rotary_dim 0). Results as the two kernels one after the other give them.
+extern "C" int fw_attention_decode_fused(const float* qkv, const float* q_norm_weight, const float* k_norm_weight, float eps,
+                                         const float* cos_table, const float* sin_table, int rotary_dim, int write_kv, void* out,
+                                         float* partial, int max_splits, int max_context, int* tickets, int tickets_len,
+                                         void* k_pages, void* v_pages, const int32_t* block_table, int table_stride,
+                                         const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
+                                         int num_kv_heads, int head_dim, float scale, int window, int page_size, int num_pages,
+                                         void* stream) {
+    if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, window,
+                     page_size, num_pages)) return -1;
+    FW_REQUIRE(qkv != nullptr, "attention_decode_fused: the projections are missing");
+    FW_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0, "attention_decode_fused: rotary_dim %d with head_dim %d",
+               rotary_dim, head_dim);
+    FW_REQUIRE(rotary_dim == 0 || (cos_table != nullptr && sin_table != nullptr), "attention_decode_fused: the rotation tables are missing");
+    FW_REQUIRE((q_norm_weight == nullptr) == (k_norm_weight == nullptr), "attention_decode_fused: q and k are normed together or not at all");
+    FusedProjections fused;
+    fused.qkv = qkv; fused.q_norm_weight = q_norm_weight; fused.k_norm_weight = k_norm_weight; fused.eps = eps;
+    fused.cos_table = cos_table; fused.sin_table = sin_table; fused.rotary_dim = rotary_dim; fused.write_kv = write_kv;
+    return decode_launch(nullptr, out, partial, max_splits, tickets, k_pages, v_pages, block_table, table_stride, row_seg, row_pos,
+                         rows, num_heads, num_kv_heads, head_dim, scale, window, fused, stream);
 }

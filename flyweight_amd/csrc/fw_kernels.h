@@ -151,6 +151,17 @@ int fw_attention_decode(const void* q, void* out, float* partial, int max_splits
                         const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
                         int head_dim, float scale, int window, int page_size, int num_pages, void* stream);
 
+// The same with the work of fw_qk_norm_rope_kv_write in front of it, in one kernel: qkv float32
+// [rows][(heads + 2 kv_heads) * head_dim] are the step's raw projections; every workgroup norms and
+// rotates the query heads it works on, and the one whose pages hold the row's own position stores
+// the new key (normed, rotated) and value (write_kv 0: they are in the cache already).
+int fw_attention_decode_fused(const float* qkv, const float* q_norm_weight, const float* k_norm_weight, float eps,
+                              const float* cos_table, const float* sin_table, int rotary_dim, int write_kv, void* out,
+                              float* partial, int max_splits, int max_context, int* tickets, int tickets_len, void* k_pages,
+                              void* v_pages, const int32_t* block_table, int table_stride, const int32_t* row_seg,
+                              const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim, float scale,
+                              int window, int page_size, int num_pages, void* stream);
+
 // ids[r] = argmax(logits[r]) with ties to the lowest id, also written to also[r] if that is not null;
 // advance[r] += 1 if that is not null; workspace: rows * 64 64-bit words
 int fw_argmax_rows(const float* logits, int32_t* ids, int32_t* also, int32_t* advance, void* workspace, int rows, int vocab,

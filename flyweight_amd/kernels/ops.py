@@ -791,6 +791,48 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
     return out
 
 
+def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                           q_norm_weight: Optional[torch.Tensor], k_norm_weight: Optional[torch.Tensor], eps: float,
+                           cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rotary_dim: int, k_pages: torch.Tensor,
+                           v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
+                           scale: float, max_context: int, window: int = 0, write_kv: bool = True) -> torch.Tensor:
+    """One row per request, from the step's raw projections ``qkv`` (float32 [rows, (heads + 2 kv
+    heads) * head_dim]): per-head norm and rotation of queries and keys, the new keys and values
+    into their pages, and the split-key attention, in one kernel. Returns bfloat16 [rows, heads *
+    head_dim]; the same numbers as ``qk_norm_rope_kv_write`` followed by ``attention_decode``."""
+    _dev(qkv, q_norm_weight, k_norm_weight, cos, sin, k_pages, v_pages, block_table, row_seg, row_pos)
+    _want(qkv, torch.float32, "qkv")
+    rows, width = qkv.shape
+    if width != (num_heads + 2 * num_kv_heads) * head_dim:
+        raise KernelError(f"attention_decode_fused: qkv width {width} != ({num_heads} + 2 x {num_kv_heads}) x {head_dim}")
+    pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, torch.bfloat16)
+    for w in (q_norm_weight, k_norm_weight):
+        if w is not None:
+            _want(w, torch.float32, "norm weight")
+            if w.shape != (head_dim,):
+                raise KernelError("attention_decode_fused: a head norm weight must be [head_dim]")
+    if rotary_dim:
+        for t in (cos, sin):
+            _want(t, torch.float32, "rotation table")
+            if t.shape != (rows, rotary_dim // 2):
+                raise KernelError(f"attention_decode_fused: rotation table is {tuple(t.shape)}, expected {(rows, rotary_dim // 2)}")
+    for name, t in (("block_table", block_table), ("row_seg", row_seg), ("row_pos", row_pos)):
+        _want(t, torch.int32, name)
+    if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
+        raise KernelError("attention: batch index arrays are too short")
+    splits = decode_splits(max_context, window)
+    partial = torch.empty((rows, num_heads, splits, head_dim + 4), dtype=torch.float32, device=qkv.device)
+    out = torch.empty((rows, num_heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    group = num_heads // num_kv_heads
+    tickets = _medium_counters(qkv.device, rows * num_kv_heads * ((group + 15) // 16))
+    _check(library().fw_attention_decode_fused(
+        _p(qkv), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin), int(rotary_dim), int(write_kv), _p(out),
+        _p(partial), splits, int(max_context), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages), _p(block_table),
+        block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale), int(window),
+        PAGE_SIZE, pages, _stream()))
+    return out
+
+
 def attention_is_tiled(head_dim: int) -> bool:
     """Whether bfloat16 attention with this head size runs on the matrix-core kernels (which
     work on tiles of QUERY_TILE rows)."""

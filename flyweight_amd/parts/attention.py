@@ -111,6 +111,13 @@ class GQAttention(Mixer):
     def forward(self, h, residual, ctx, cache):
         qkv = self.qkv.forward(h, out_dtype=torch.float32)      # normed, rotated and rounded once, below
         cos, sin = ctx.position_tables(self.position)
+        if ctx.all_decode and qkv.dtype == torch.float32 and self.step_arrays_key() is not None:
+            # single-token segments on the matrix cores: norm, rotation, cache write and attention in one kernel
+            attended = ops.attention_decode_fused(
+                qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight, self.qk_norm_eps,
+                cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table, ctx.row_seg, ctx.row_pos,
+                self.scale, ctx.max_context, int(self.window or 0), write_kv=cache.writes)
+            return self.out.accumulate(attended, residual, then=getattr(ctx, "upcoming_norm", None))
         q = ops.qk_norm_rope_kv_write(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight,
             self.qk_norm_eps, cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table,

@@ -173,3 +173,47 @@ def test_norm_rotation_cache_write_and_attention_over_mixed_segments(ops, ref, d
         decoded = ops.attention_decode(q_d[last].contiguous(), nh, nkv, hd, k_d, v_d, ints(table), ints([0, 1, 2]), ints(row_pos[last]),
                                        scale, max(lengths), window)
         close(decoded, want[last], dtype)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,rotary,window,normed", [(32, 8, 64, 64, 0, True), (6, 2, 48, 48, 0, True), (5, 5, 16, 8, 0, True),
+                                                            (8, 1, 64, 64, 90, True), (3, 1, 112, 0, 0, False), (40, 2, 32, 32, 0, True)])
+def test_decode_attention_with_norm_rotation_and_cache_write_in_front(ops, ref, nh, nkv, hd, rotary, window, normed):
+    """One new token for each of five requests behind contexts that end at different places of a
+    page (its first key, its last, a page of its own): the fused kernel against the two kernels it
+    replaces, bit for bit (outputs and pages), and against the C++ reference."""
+    contexts = [0, 63, 64, 200, 449]
+    rows = len(contexts)
+    table = scattered_cache([c + 1 for c in contexts], nkv, hd, 16, seed=hd + nh)
+    k_h = np.zeros((16, nkv, 64, hd), dtype=np.float32)
+    v_h = np.zeros((16, nkv, hd, 64), dtype=np.float32)
+    for seg, length in enumerate(contexts):
+        for t in range(length):
+            page = table[seg, t // 64]
+            k_h[page, :, t % 64, :] = RNG.normal(size=(nkv, hd))
+            v_h[page, :, :, t % 64] = RNG.normal(size=(nkv, hd))
+    k_two, k_h = rounded(k_h, torch.bfloat16)
+    v_two, v_h = rounded(v_h, torch.bfloat16)
+    k_one, v_one = k_two.clone(), v_two.clone()
+    qkv = RNG.normal(size=(rows, (nh + 2 * nkv) * hd)).astype(np.float32)
+    qw = (1 + 0.3 * RNG.normal(size=hd)).astype(np.float32) if normed else None
+    kw = (1 + 0.3 * RNG.normal(size=hd)).astype(np.float32) if normed else None
+    dev = lambda a: None if a is None else torch.tensor(a, device=DEV)       # noqa: E731
+    inv_freq = 1000.0 ** (-(np.arange(rotary // 2, dtype=np.float64) * 2.0 / max(rotary, 1)))
+    positions, segments = ints(contexts), ints(range(rows))
+    cos, sin = ops.rope_table(positions, torch.tensor(inv_freq, device=DEV)) if rotary else (None, None)
+    scale = 1 / math.sqrt(hd)
+    q = ops.qk_norm_rope_kv_write(dev(qkv), nh, nkv, hd, dev(qw), dev(kw), 1e-5, cos, sin, rotary, k_two, v_two, ints(table), segments, positions)
+    two = ops.attention_decode(q, nh, nkv, hd, k_two, v_two, ints(table), segments, positions, scale, 512, window)
+    one = ops.attention_decode_fused(dev(qkv), nh, nkv, hd, dev(qw), dev(kw), 1e-5, cos, sin, rotary, k_one, v_one, ints(table), segments,
+                                     positions, scale, 512, window)
+    assert torch.equal(one, two) and torch.equal(k_one, k_two) and torch.equal(v_one, v_two)
+    # a layer that reads another's cache forms its queries and leaves the cache alone
+    k_other, v_other = k_one.clone(), v_one.clone()
+    again = ops.attention_decode_fused(dev(qkv * 1.0), nh, nkv, hd, dev(qw), dev(kw), 1e-5, cos, sin, rotary, k_other, v_other, ints(table),
+                                       segments, positions, scale, 512, window, write_kv=False)
+    assert torch.equal(again, two) and torch.equal(k_other, k_one) and torch.equal(v_other, v_one)
+    # and the C++ reference of the whole
+    cos_h, sin_h = ref.rope_table(contexts, inv_freq) if rotary else (None, None)
+    q_h = ref.qk_norm_rope_kv_write(qkv, nh, nkv, hd, qw, kw, 1e-5, cos_h, sin_h, rotary, k_h, v_h, table, range(rows), contexts)
+    want = ref.attention(q_h, nh, nkv, hd, k_h, v_h, table, range(rows), contexts, scale, window)
+    close(one, want, torch.bfloat16, 2.0)
