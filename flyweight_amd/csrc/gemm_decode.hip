@@ -63,7 +63,6 @@ struct DecodeGemmArgs {
     // pre-normed prologue
     const float* squares;           // [squares_tiles][16], left by the kernel above
     int squares_tiles;
-    int rotate;                     // tiles start their walk over K at different chunks
 };
 
 __device__ __forceinline__ float dg_silu(float g) {
@@ -136,15 +135,8 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
                 if (p.next_norm_weight) next_weight[r] = p.next_norm_weight[ok ? n : 0];
             }
         }
-        // Tiles walk K from different chunks on (and around): every workgroup reads the same rows of a,
-        // and in step they would all ask for the same cache lines at once. The start depends on the
-        // tile alone, so a row's sum does not depend on the batch or on timing.
-        const int chunks_total = (K + DG_CHUNK - 1) / DG_CHUNK;
-        const int rotate = p.rotate ? (int)((unsigned)tile * 5u % (unsigned)chunks_total) : 0;
 #pragma unroll 2
-        for (int chunk = wave; chunk < chunks_total; chunk += WAVES) {
-            const int turned = chunk + rotate;
-            const int k0 = (turned < chunks_total ? turned : turned - chunks_total) * DG_CHUNK;
+        for (int k0 = wave * DG_CHUNK; k0 < K; k0 += WAVES * DG_CHUNK) {
             bf16x8 wf[RT][4], af[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -337,8 +329,6 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
 }
 
 #define DG_MAX_BLOCKS 1024
-static int decode_rotate = 1;
-extern "C" void fw_gemm_decode_set_rotate(int on) { decode_rotate = on; }
 
 template <int RT, int WAVES, int ROWS, int PRO, int EPI, typename TO>
 static int launch(const DecodeGemmArgs& args, hipStream_t stream) {
@@ -385,7 +375,6 @@ extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_wei
     args.next_norm_weight = next_norm_weight; args.next_one_centered = next_one_centered;
     args.next_activations = (uint16_t*)next_activations; args.next_squares = next_squares;
     args.squares = squares; args.squares_tiles = squares_tiles;
-    args.rotate = decode_rotate;
     hipStream_t s = (hipStream_t)stream;
     const bool narrow = N < 256 * 16;       // fewer than one 16-feature tile per compute unit: use 8-feature tiles
     int status = -2;

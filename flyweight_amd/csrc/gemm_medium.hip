@@ -69,7 +69,7 @@ __device__ __forceinline__ float gm_silu(float g) {
 
 // MT: tiles of 16 rows of a. FW: waves side by side over features (4: 64 features, no split of
 // K inside the workgroup; 2: 32 features, the two halves of a 128-k chunk go to wave pairs).
-template <int MT, int FW, int MODE, typename TO>
+template <int MT, int FW, int MODE, typename TO, bool ROTATE>
 __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArgs p) {
     constexpr int KP = 4 / FW;                  // parts of K inside the workgroup
     constexpr int CHUNK = 64 * KP;              // k per iteration of the workgroup
@@ -121,9 +121,12 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
     // Workgroups walk their slice of K from different chunks on (and around): all of them read the
     // same rows of a, and in step they would ask one cache line of it at a time from every compute
     // unit at once. Where a workgroup starts depends on its tile alone, so the order of its sum
-    // over K does not depend on the batch or on timing.
-    const int rotate = p.rotate ? (int)((tile * 5u + blockIdx.y * 3u) % (unsigned)(chunks > 0 ? chunks : 1)) : 0;
+    // over K does not depend on the batch or on timing. It pays for a large W that is not split over
+    // workgroups (inside a decode step of 8 rows: gate|up 17.3 -> 16.5 us, the head 59.8 -> 50.3 us);
+    // the smaller products and those whose slices meet through the workspace lose a little by it.
+    const int rotate = ROTATE ? (int)((tile * 5u + blockIdx.y * 3u) % (unsigned)(chunks > 0 ? chunks : 1)) : 0;
     auto chunk_start = [&](const int c) {
+        if (!ROTATE) return k_begin + c * CHUNK;
         if (c >= chunks) return k_end;                  // past the slice: nothing of it is inside
         const int turned = c + rotate;
         return k_begin + (turned < chunks ? turned : turned - chunks) * CHUNK;
@@ -385,8 +388,6 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
 }
 
 // ----- host side ---------------------------------------------------------------------------
-static int medium_rotate = 1;
-extern "C" void fw_gemm_medium_set_rotate(int on) { medium_rotate = on; }
 
 struct MediumPlan {
     int mt, fw, tiles, splits, k_per_split;
@@ -431,12 +432,18 @@ extern "C" int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* worksp
     return 0;
 }
 
+template <int MT, int FW, bool ROTATE>
+static void medium_launch_as(const MediumArgs& args, int out_dtype, int mode, dim3 grid, hipStream_t stream) {
+    if (mode == GM_SWIGLU) gemm_medium_kernel<MT, FW, GM_SWIGLU, bf16_t, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
+    else if (mode == GM_ACCUMULATE) gemm_medium_kernel<MT, FW, GM_ACCUMULATE, float, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
+    else if (out_dtype == FW_F32) gemm_medium_kernel<MT, FW, GM_STORE, float, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
+    else gemm_medium_kernel<MT, FW, GM_STORE, bf16_t, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
+}
+
 template <int MT, int FW>
 static void medium_launch(const MediumArgs& args, int out_dtype, int mode, dim3 grid, hipStream_t stream) {
-    if (mode == GM_SWIGLU) gemm_medium_kernel<MT, FW, GM_SWIGLU, bf16_t><<<grid, GM_THREADS, 0, stream>>>(args);
-    else if (mode == GM_ACCUMULATE) gemm_medium_kernel<MT, FW, GM_ACCUMULATE, float><<<grid, GM_THREADS, 0, stream>>>(args);
-    else if (out_dtype == FW_F32) gemm_medium_kernel<MT, FW, GM_STORE, float><<<grid, GM_THREADS, 0, stream>>>(args);
-    else gemm_medium_kernel<MT, FW, GM_STORE, bf16_t><<<grid, GM_THREADS, 0, stream>>>(args);
+    if (args.rotate) medium_launch_as<MT, FW, true>(args, out_dtype, mode, grid, stream);
+    else medium_launch_as<MT, FW, false>(args, out_dtype, mode, grid, stream);
 }
 
 // mode 0: out = a . w^T (+ bias) stored as out_dtype; 1: out (float32) += a . w^T (+ bias);
@@ -472,7 +479,7 @@ extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, v
     args.next_norm_weight = next_norm_weight; args.next_one_centered = next_one_centered;
     args.next_activations = (uint16_t*)next_activations; args.next_squares = next_squares;
     args.squares = squares; args.squares_rows = squares_rows; args.eps = eps;
-    args.rotate = medium_rotate;
+    args.rotate = plan.splits == 1 && (long long)N * K * (mode == GM_SWIGLU ? 2 : 1) > (1ll << 24);
     const dim3 grid(plan.tiles, plan.splits);
     hipStream_t s = (hipStream_t)stream;
     if (plan.fw == 4) {
