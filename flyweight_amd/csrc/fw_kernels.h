@@ -67,13 +67,16 @@ int fw_gemm_mfma_split(const void* a, const void* w, const float* bias, void* ou
 // the kernel leaves them zero. Calls that overlap on one device need their own of both.
 // The accumulating product can leave what the norm after it needs, as fw_gemm_decode does
 // (next_activations [M][N] bfloat16, next_squares [squares_rows][16 for M <= 16, else 64]), and
-// any mode takes such prepared activations as a, with squares / squares_rows / eps.
+// any mode takes such prepared activations as a, with squares / squares_rows / eps. Mode 3 is the
+// gated short convolution for single-token rows (w = [B; C; x rows], taps [N][kernel_size], state
+// [slots][N][kernel_size - 1] read and shifted, seg_slot [M]), as fw_gemm_decode's epilogue 3.
 int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* workspace_bytes, int* counters, int* squares_rows);
 int fw_gemm_medium(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                    int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
                    int counters_len, const float* next_norm_weight, int next_one_centered,
                    void* next_activations, float* next_squares, const float* squares, int squares_rows,
-                   float eps, void* stream);
+                   float eps, const float* taps, const float* conv_bias, float* state, const int32_t* seg_slot,
+                   int kernel_size, void* stream);
 
 // Fused product for decode steps of up to 16 rows. prologue 0: a is bfloat16 [M][K]; 1: a is
 // float32 rows, RMS-normed with norm_weight/eps (rows gathered through row_index if given) inside

@@ -490,7 +490,9 @@ def prepare_device(device: torch.device) -> None:
 
 def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int,
                      next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False,
-                     squares: Optional[torch.Tensor] = None, eps: float = 0.0):
+                     squares: Optional[torch.Tensor] = None, eps: float = 0.0, taps: Optional[torch.Tensor] = None,
+                     conv_bias: Optional[torch.Tensor] = None, state: Optional[torch.Tensor] = None,
+                     seg_slot: Optional[torch.Tensor] = None):
     """The product for 1..64 rows with K split over workgroups (fw_gemm_medium). With
     ``squares`` ``a`` holds prepared activations (x * w of an RMS norm) and the rows' 1/rms is
     formed from those sums. With ``next_norm_weight`` (accumulating product) returns what the
@@ -514,7 +516,8 @@ def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tenso
                                     ctypes.c_size_t(need_bytes.value), _p(counters),
                                     0 if counters is None else counters.numel(), _p(next_norm_weight),
                                     int(next_one_centered), _p(next_activations), _p(next_squares), _p(squares),
-                                    0 if squares is None else squares.shape[0], ctypes.c_float(eps), _stream()))
+                                    0 if squares is None else squares.shape[0], ctypes.c_float(eps), _p(taps), _p(conv_bias),
+                                    _p(state), _p(seg_slot), 0 if taps is None else taps.shape[1], _stream()))
     if next_norm_weight is not None:
         return next_activations, next_squares
     return None
@@ -523,16 +526,18 @@ def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tenso
 def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, accumulate_into: Optional[torch.Tensor] = None,
                 squares: Optional[torch.Tensor] = None, eps: float = 0.0,
-                next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False):
+                next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False,
+                taps: Optional[torch.Tensor] = None, conv_bias: Optional[torch.Tensor] = None,
+                state: Optional[torch.Tensor] = None, seg_slot: Optional[torch.Tensor] = None):
     """The medium product with the fused decode product's conventions (EPILOGUE_STORE /
-    ACCUMULATE / SWIGLU): returns the output, or for an accumulation with ``next_norm_weight``
-    what the norm after it needs."""
-    _dev(a, w, bias, accumulate_into, squares, next_norm_weight)
+    ACCUMULATE / SWIGLU / CONV): returns the output, or for an accumulation with
+    ``next_norm_weight`` what the norm after it needs."""
+    _dev(a, w, bias, accumulate_into, squares, next_norm_weight, taps, conv_bias, state, seg_slot)
     _want(a, torch.bfloat16, "a")
     _want(w, torch.bfloat16, "w")
     M, K = a.shape
-    kinds = 2 if epilogue == EPILOGUE_SWIGLU else 1
-    if not 1 <= M <= MEDIUM_MAX_ROWS or w.shape[1] != K or w.shape[0] % kinds or K % 8 or epilogue not in (0, 1, 2):
+    kinds = {EPILOGUE_SWIGLU: 2, EPILOGUE_CONV: 3}.get(epilogue, 1)
+    if not 1 <= M <= MEDIUM_MAX_ROWS or w.shape[1] != K or w.shape[0] % kinds or K % 8 or epilogue not in (0, 1, 2, 3):
         raise KernelError(f"gemm_medium: a is {tuple(a.shape)}, w is {tuple(w.shape)}, epilogue {epilogue}")
     N = w.shape[0] // kinds
     if bias is not None and (bias.dtype != torch.float32 or bias.shape != (w.shape[0],)):
@@ -540,6 +545,8 @@ def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
     if next_norm_weight is not None and (epilogue != EPILOGUE_ACCUMULATE or next_norm_weight.dtype != torch.float32
                                          or next_norm_weight.shape != (N,)):
         raise KernelError("gemm_medium: only the accumulating product prepares the next norm, whose weight is float32 [N]")
+    if epilogue == EPILOGUE_CONV:
+        _check_conv_arguments("gemm_medium", M, N, taps, conv_bias, state, seg_slot)
     if epilogue == EPILOGUE_ACCUMULATE:
         _want(accumulate_into, torch.float32, "accumulate_into")
         if accumulate_into.shape != (M, N):
@@ -548,8 +555,27 @@ def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
         return accumulate_into if left is None else left
     out_dtype = torch.bfloat16 if epilogue == EPILOGUE_SWIGLU else (out_dtype or torch.bfloat16)
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    gemm_medium_into(a, w, bias, out, _code(out_dtype), epilogue, N, squares=squares, eps=eps)
+    gemm_medium_into(a, w, bias, out, _code(out_dtype), epilogue, N, squares=squares, eps=eps, taps=taps, conv_bias=conv_bias,
+                     state=state, seg_slot=seg_slot)
     return out
+
+
+def _check_conv_arguments(name: str, M: int, N: int, taps, conv_bias, state, seg_slot) -> None:
+    """What a convolution epilogue needs: taps float32 [N, L], state float32 [slots, N, L - 1],
+    seg_slot int32 of at least M entries, an optional bias float32 [N]."""
+    if taps is None or state is None or seg_slot is None:
+        raise KernelError(f"{name}: the convolution epilogue needs taps, state and slots")
+    _want(taps, torch.float32, "taps")
+    _want(state, torch.float32, "state")
+    _want(seg_slot, torch.int32, "seg_slot")
+    if taps.dim() != 2 or taps.shape[0] != N or not 2 <= taps.shape[1] <= 16:
+        raise KernelError(f"{name}: taps are {tuple(taps.shape)}, expected [{N}, 2..16]")
+    if state.dim() != 3 or state.shape[1:] != (N, taps.shape[1] - 1) or not state.is_contiguous() or not taps.is_contiguous():
+        raise KernelError(f"{name}: state is {tuple(state.shape)}, expected [slots, {N}, {taps.shape[1] - 1}]")
+    if seg_slot.numel() < M:
+        raise KernelError(f"{name}: {seg_slot.numel()} slots for {M} rows")
+    if conv_bias is not None and (conv_bias.dtype != torch.float32 or conv_bias.shape != (N,)):
+        raise KernelError(f"{name}: the convolution's bias must be float32 [{N}]")
 
 
 def gemm_deep(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,

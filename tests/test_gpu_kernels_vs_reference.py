@@ -217,3 +217,29 @@ def test_decode_attention_with_norm_rotation_and_cache_write_in_front(ops, ref, 
     q_h = ref.qk_norm_rope_kv_write(qkv, nh, nkv, hd, qw, kw, 1e-5, cos_h, sin_h, rotary, k_h, v_h, table, range(rows), contexts)
     want = ref.attention(q_h, nh, nkv, hd, k_h, v_h, table, range(rows), contexts, scale, window)
     close(one, want, torch.bfloat16, 2.0)
+
+
+@pytest.mark.parametrize("M,hidden,K,kernel,bias", [(20, 136, 264, 3, False), (64, 72, 1032, 4, True), (8, 200, 520, 2, True), (33, 2048, 2048, 3, False)])
+def test_products_with_the_short_convolution_behind_them(ops, ref, M, hidden, K, kernel, bias):
+    """in_proj with the gated convolution and the state shift in its epilogue, for single-token
+    rows of requests in scattered slots: the split-K product (any rows up to 64) and, up to 16
+    rows, the fused decode product, against the references of the product and of the convolution."""
+    a, a_h = rounded(RNG.normal(size=(M, K)), torch.bfloat16)
+    w, w_h = rounded(RNG.normal(size=(3 * hidden, K)) / math.sqrt(K), torch.bfloat16)
+    in_bias = RNG.normal(size=3 * hidden).astype(np.float32) * 0.1 if bias else None
+    conv_bias = RNG.normal(size=hidden).astype(np.float32) * 0.1 if bias else None
+    taps = RNG.normal(size=(hidden, kernel)).astype(np.float32) * 0.5
+    slots = RNG.permutation(M + 3)[:M]
+    state = RNG.normal(size=(M + 3, hidden, kernel - 1)).astype(np.float32)
+    want_state = state.copy()
+    want = ref.shortconv(ref.gemm(a_h, w_h, in_bias), taps, conv_bias, want_state, np.arange(M + 1), slots)
+    dev = lambda x: None if x is None else torch.tensor(x, device=DEV)      # noqa: E731
+    kernels = [ops.gemm_medium] + ([ops.gemm_decode] if M <= 16 else [])
+    for kernel_call in kernels:
+        state_d = dev(state)
+        out = kernel_call(a, w, ops.EPILOGUE_CONV, bias=dev(in_bias), out_dtype=torch.bfloat16, taps=dev(taps), conv_bias=dev(conv_bias),
+                          state=state_d, seg_slot=ints(slots))
+        close(out, want, torch.bfloat16, 2.0)
+        close(state_d, want_state, torch.bfloat16, 2.0)         # B * x comes from bfloat16 operands
+        untouched = [s for s in range(M + 3) if s not in slots.tolist()]
+        assert np.array_equal(state_d[untouched].cpu().numpy(), state[untouched])
