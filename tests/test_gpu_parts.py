@@ -399,6 +399,102 @@ def register_toy_router_and_positions():
             return ops.rope_table(ctx.encoding_pos, self.inv_freq)
 
 
+def toy_spec(base):
+    """Tiny A with a routed feed-forward and a stretched rotation in layer 1, scaled embeddings and
+    scaled, capped logits."""
+    from flyweight_amd.config import PartSpec
+    layer = base.layers[1]
+    position = PartSpec("toy_stretched_rotary", {"theta": 10000.0, "head_dim": 16, "stretch": TOY_STRETCH})
+    mixer = dataclasses.replace(layer.mixer, params={**layer.mixer.params, "position": position})
+    ffn = PartSpec("toy_top1_of_two", {"hidden_size": 64, "intermediate_size": 48}, prefix="model.layers.1.moe.")
+    return dataclasses.replace(base, layers=(base.layers[0], dataclasses.replace(layer, mixer=mixer, ffn=ffn)) + base.layers[2:],
+                               architecture="ToyForCausalLM", embedding_scale=1.5, logit_scale=0.5, logit_softcap=2.0)
+
+
+def toy_expected_logits(w, tokens, shift=0):
+    """Plain evaluation of ``toy_spec``'s model: (logits, first row whose routing is a close call)."""
+    from helpers import TINY_A
+    config = dict(TINY_A)
+    eps = config["norm_eps"]
+    x = 1.5 * w["model.embed_tokens.weight"][tokens]
+    T = len(tokens)
+    close_call = T
+    for i, is_attention in enumerate(plain.attention_layers(config)):
+        p = f"model.layers.{i}."
+        h = plain.rms_norm(x, w[p + "operator_norm.weight"], eps)
+        if is_attention:
+            positions = (np.arange(T) + shift) / (TOY_STRETCH if i == 1 else 1.0)
+            q, k, v = plain.attention_qkv(h, w, p + "self_attn.", config, positions)
+            x = x + plain.causal_attention(q, k, v, 0.25).reshape(T, -1) @ w[p + "self_attn.out_proj.weight"].T
+        else:
+            x = x + plain.short_conv_mixer(h, w, p + "conv.", config)
+        h = plain.rms_norm(x, w[p + "ffn_norm.weight"], eps)
+        if i == 1:
+            logits = TOY_ROUTER_GAIN * (h @ w[p + "moe.router.weight"].T)
+            share = np.exp(logits - logits.max(-1, keepdims=True))
+            share /= share.sum(-1, keepdims=True)
+            near = np.nonzero(np.abs(logits[:, 1] - logits[:, 0]) < TOY_AMBIGUOUS)[0]
+            close_call = int(near[0]) if len(near) else T
+            x = x.copy()
+            for t in range(T):
+                e = int(logits[t, 1] > logits[t, 0])
+                both = h[t] @ w[f"{p}moe.experts.{e}.gate_up.weight"].T
+                x[t] = x[t] + share[t, e] * ((plain.silu(both[:48]) * both[48:]) @ w[f"{p}moe.experts.{e}.down.weight"].T)
+        else:
+            x = x + plain.swiglu(h, w, p + "feed_forward.")
+    logits = 0.5 * (plain.rms_norm(x, w["model.embedding_norm.weight"], eps) @ w["model.embed_tokens.weight"].T)
+    return 2.0 * np.tanh(logits / 2.0), close_call
+
+
+def test_a_toy_architecture_is_registered_and_served_from_a_folder(tmp_path):
+    """An architecture of this file's own (its configuration class, its key names, its parts) goes
+    through the registry: a model folder is written from its configuration and a seed, opened by
+    name as any folder is, and generates through the runtime (scheduler, prompt portions, decode
+    steps) the tokens of a plain evaluation. Nothing of the package knows it."""
+    import flyweight_amd
+    from flyweight_amd.config import config_from_dict, register_architecture, registered_architectures
+    from flyweight_amd.weights import write_random_model
+    from helpers import TINY_A
+    register_toy_router_and_positions()
+
+    class ToyConfig:
+        """config.json of the toy: {"architectures": ["ToyForCausalLM"], "base": <an LFM2 config>}."""
+
+        def __init__(self, base):
+            self.base = base
+
+        @classmethod
+        def from_dict(cls, data):
+            return cls(config_from_dict(data["base"]))
+
+        def model_spec(self):
+            return toy_spec(self.base.model_spec())
+
+        def save(self, folder):
+            import json
+            with open(os.path.join(folder, "config.json"), "w") as handle:
+                json.dump({"architectures": ["ToyForCausalLM"], "base": self.base.to_dict()}, handle)
+
+    register_architecture("ToyForCausalLM", ToyConfig, replace=True)
+    assert "ToyForCausalLM" in registered_architectures()
+    folder = write_random_model(str(tmp_path / "toy3"), ToyConfig(config_from_dict(TINY_A)), seed=9, scale="fan_in")
+    model = flyweight_amd.Model(folder, dtype="float32")
+    assert isinstance(model.config, ToyConfig) and model.spec.architecture == "ToyForCausalLM"
+    from safetensors.torch import load_file
+    w = {n: t.double().numpy() for n, t in load_file(os.path.join(folder, "model.safetensors")).items()}
+    prompt = np.random.default_rng(TOY_TOKENS_SEED).integers(0, 256, 45).tolist()
+    expected, tokens = [], list(prompt)
+    for _ in range(6):
+        logits, _ = toy_expected_logits(w, tokens)
+        expected.append(plain.most_likely(logits[-1]))
+        tokens.append(expected[-1])
+    with flyweight_amd.Runtime(model, parallel_sequences=2, prefill_rows=16, max_batch_tokens=24) as runtime:
+        other = runtime.task_submit(prompt[:20], 3)         # a second request beside it: mixed steps
+        assert runtime.generate(prompt, 6) == expected
+        runtime.run()
+        assert runtime.task_error(other) is None and runtime.info["live_requests"] == 0
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_toy_routing_feed_forward_and_position_encoding_need_no_change_to_the_framework(tmp_path, dtype):
     """Layer 1 of tiny A gets a routed feed-forward and a stretched rotation, both defined in this
@@ -411,13 +507,7 @@ def test_toy_routing_feed_forward_and_position_encoding_need_no_change_to_the_fr
     from flyweight_amd.weights import load_tensors, random_tensors, write_file
     from helpers import TINY_A
     register_toy_router_and_positions()
-    base = config_from_dict(TINY_A).model_spec()
-    layer = base.layers[1]
-    position = PartSpec("toy_stretched_rotary", {"theta": 10000.0, "head_dim": 16, "stretch": TOY_STRETCH})
-    mixer = dataclasses.replace(layer.mixer, params={**layer.mixer.params, "position": position})
-    ffn = PartSpec("toy_top1_of_two", {"hidden_size": 64, "intermediate_size": 48}, prefix="model.layers.1.moe.")
-    spec = dataclasses.replace(base, layers=(base.layers[0], dataclasses.replace(layer, mixer=mixer, ffn=ffn)) + base.layers[2:],
-                               embedding_scale=1.5, logit_scale=0.5, logit_softcap=2.0)
+    spec = toy_spec(config_from_dict(TINY_A).model_spec())
     model = CausalLM(spec)
     folder = str(tmp_path / "toy2")
     os.makedirs(folder)
@@ -430,37 +520,7 @@ def test_toy_routing_feed_forward_and_position_encoding_need_no_change_to_the_fr
     eps = config["norm_eps"]
 
     def expected(tokens, shift=0):
-        """Logits, and the first row whose routing is a close call (rows from there on may differ
-        in bfloat16: top-1 routing is not continuous)."""
-        x = 1.5 * w["model.embed_tokens.weight"][tokens]
-        T = len(tokens)
-        close_call = T
-        for i, is_attention in enumerate(plain.attention_layers(config)):
-            p = f"model.layers.{i}."
-            h = plain.rms_norm(x, w[p + "operator_norm.weight"], eps)
-            if is_attention:
-                positions = (np.arange(T) + shift) / (TOY_STRETCH if i == 1 else 1.0)
-                q, k, v = plain.attention_qkv(h, w, p + "self_attn.", config, positions)
-                x = x + plain.causal_attention(q, k, v, 0.25).reshape(T, -1) @ w[p + "self_attn.out_proj.weight"].T
-            else:
-                x = x + plain.short_conv_mixer(h, w, p + "conv.", config)
-            h = plain.rms_norm(x, w[p + "ffn_norm.weight"], eps)
-            if i == 1:
-                logits = TOY_ROUTER_GAIN * (h @ w[p + "moe.router.weight"].T)
-                share = np.exp(logits - logits.max(-1, keepdims=True))
-                share /= share.sum(-1, keepdims=True)
-                near = np.nonzero(np.abs(logits[:, 1] - logits[:, 0]) < TOY_AMBIGUOUS)[0]
-                close_call = int(near[0]) if len(near) else T
-                x = x.copy()
-                for t in range(T):
-                    e = int(logits[t, 1] > logits[t, 0])
-                    both = h[t] @ w[f"{p}moe.experts.{e}.gate_up.weight"].T
-                    x[t] = x[t] + share[t, e] * ((plain.silu(both[:48]) * both[48:]) @ w[f"{p}moe.experts.{e}.down.weight"].T)
-                assert 0.2 < (logits[:, 1] > logits[:, 0]).mean() < 0.8       # both experts work
-            else:
-                x = x + plain.swiglu(h, w, p + "feed_forward.")
-        logits = 0.5 * (plain.rms_norm(x, w["model.embedding_norm.weight"], eps) @ w["model.embed_tokens.weight"].T)
-        return 2.0 * np.tanh(logits / 2.0), close_call
+        return toy_expected_logits(w, tokens, shift)
 
     tokens = np.random.default_rng(TOY_TOKENS_SEED).integers(0, 256, 100).tolist()
     want, sure = expected(tokens)
