@@ -258,6 +258,13 @@ def further_points(torch, args, points: dict) -> None:
                                         context=long_context + 2048)
     points["decode_b64_ctx32k_350m"] = round(64 * steps / seconds, 1)
     points["decode_b64_ctx32k_350m_frac"] = round(step_bytes / (seconds / steps) / 1e9 / HBM_PEAK_GBS, 4)
+    del model
+    torch.cuda.empty_cache()
+    # the two serving workloads at a quarter of their requests: whole jobs through the scheduler, tokens (prompt
+    # and generated) a second; `--workload` runs them at full size with a line of their own
+    for workload, requests in (("long-context", 16), ("mixed", 32)):
+        record = serving_run(torch, workload, requests)
+        points[f"serving_{workload.replace('-', '_')}_{requests}req"] = record["value"]
 
 
 def main() -> int:
