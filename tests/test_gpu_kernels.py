@@ -456,6 +456,33 @@ def test_the_prompt_product_of_one_round_of_tiles_over_a_long_k(ops, M, N, K):
     close(ops.gemm(a, w, out_dtype=torch.float32), want, torch.float32, 2.0)
 
 
+@pytest.mark.parametrize("M,N,K,mode,columns", [(256, 6144, 2048, 0, 64), (500, 6100, 1984, 0, 128), (130, 6144, 2048, 0, 64),
+                                                   (512, 2048, 2048, 1, 64), (300, 3072, 1024, 0, 64),
+                                                   (256, 2048, 8192, 1, 0), (600, 6144, 2048, 0, 0), (256, 1024, 2048, 0, 0)])
+def test_a_few_hundred_rows_go_to_the_tiles_whose_waves_split_k(ops, M, N, K, mode, columns):
+    """A decode step of a few hundred requests: storing and short accumulating products take those
+    tiles when they are not too few (equal, bit for bit, to the kernel called by name); a long K,
+    more rows or too few tiles stay with the other products."""
+    assert ops._deep_columns_few_rows(mode, M, N, K) == columns
+    a = as_dev(gen(M, K), torch.bfloat16)
+    w = as_dev(gen(N, K, seed=1, scale=K ** -0.5), torch.bfloat16)
+    want = back(a) @ back(w).T
+    if mode == 0:
+        got = ops.gemm(a, w, out_dtype=torch.float32)
+        close(got, want, torch.float32, 2.0)
+        if columns:
+            assert torch.equal(got, ops.gemm_deep(a, w, out_dtype=torch.float32, columns=columns))
+    else:
+        residual = gen(M, N, seed=3).float().to(DEV)
+        before = residual.cpu().double()
+        ops.gemm(a, w, accumulate_into=residual)
+        close(residual, before + want, torch.float32, 2.0)
+        if columns:
+            direct = before.float().to(DEV)
+            ops.gemm_deep(a, w, accumulate_into=direct, columns=columns)
+            assert torch.equal(direct, residual)
+
+
 def test_fast_gemm_rows_do_not_depend_on_the_batch(ops):
     a = as_dev(gen(300, 256), torch.bfloat16)
     w = as_dev(gen(200, 256, seed=1), torch.bfloat16)
