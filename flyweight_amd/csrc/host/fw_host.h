@@ -99,12 +99,14 @@ int fwh_scheduler_complete(void* scheduler, const int64_t* requests, const int* 
 // group_stride ints apart); returns the number of rows, or FWH_NOT_DECODE_ONLY and writes nothing.
 // fwh_scheduler_complete_ordered is fwh_scheduler_complete with the tokens given in the order
 // of the plan's segments that wanted logits.
-// fwh_plan_steps_ahead: how many further steps of exactly this batch are certain to follow such a
-// plan whatever tokens are drawn (at most `limit`): nobody waits for admission, no request of the
-// plan has stop tokens, and each has that many tokens to go within its budget and the context
-// beyond the one this plan produces. A caller may then run those steps on the device, feeding
-// each step's tokens to the next, before it hands any of them over. requests: the plan's requests
-// in row order (optional).
+// fwh_plan_steps_ahead: how many further steps of this batch are certain to follow such a plan
+// whatever tokens are drawn (at most `limit`), but for requests that draw one of their stop
+// tokens: nobody waits for admission, and each request has that many tokens to go within its
+// budget and the context beyond the one this plan produces. A caller may then run those steps on
+// the device, feeding each step's tokens to the next, before it hands any of them over; a request
+// that ends at a stop token is missing from the plans after it (the others keep their order), and
+// the tokens its row went on to draw are dropped. requests: the plan's requests in row order
+// (optional).
 #define FWH_NOT_DECODE_ONLY (-3)
 int fwh_plan_fill_decode(void* scheduler, int capacity, int* tokens, int* positions, int* slots, int table_stride,
                          int* tables, int group_stride);

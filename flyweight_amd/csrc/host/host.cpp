@@ -302,7 +302,7 @@ int fwh_plan_steps_ahead(void* scheduler, int limit, int64_t* requests, int capa
         int ahead = limit;
         for (const fwh::Segment& segment : plan.segments) {
             const fwh::Request* request = segment.request;
-            if (segment.count != 1 || !segment.wants_logits || !request->stop_tokens.empty() || request->cancelled) return 0;
+            if (segment.count != 1 || !segment.wants_logits || request->cancelled) return 0;
             const int budget = request->max_new_tokens - (int)request->generated.size() - 1;
             const int room = s->max_positions() - request->total() - 1;
             ahead = std::min({ahead, budget, room});

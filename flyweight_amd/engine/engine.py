@@ -12,6 +12,7 @@ from __future__ import annotations
 import time
 from typing import Callable, Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..cache import OutOfPages
@@ -208,20 +209,32 @@ class Runtime:
             if captured is not None:
                 began = time.perf_counter_ns()
                 try:
-                    tokens = self.stepper.replay_planned(captured, scheduler, self.decode_steps_per_turn)
+                    ran = self.stepper.replay_planned(captured, scheduler, self.decode_steps_per_turn)
                 except Exception as error:
                     return self._fail_step(scheduler.read_plan(counts), error)
-                if tokens is not None:
+                if ran is not None:
+                    tokens, row_requests = ran
                     self._counters["steps"] += len(tokens)
                     self._counters["decode_calls"] += counts[0] * len(tokens)
                     self._counters["decode_ns"] += time.perf_counter_ns() - began
                     events = scheduler.complete_ordered(tokens[0])
+                    # The steps that ran ahead: the scheduler makes the plan they ran by, then takes their
+                    # tokens. A request that ended on the way (a stop token) is missing from the later
+                    # plans, the others keep their order; what its row went on to draw is dropped.
+                    live = np.ones(counts[0], dtype=bool)
+                    checked = 0
                     for later in tokens[1:]:
-                        # the steps that ran ahead: the scheduler makes the plan they ran by, then takes their tokens
+                        ended = {task for task, _, kind in events[checked:] if kind in (EVENT_FINISHED, EVENT_ERROR)}
+                        checked = len(events)
+                        if ended:
+                            live &= np.array([request not in ended for request in row_requests], dtype=bool)
+                        rows = int(live.sum())
+                        if rows == 0:
+                            break
                         again = scheduler.plan_next()
-                        if again[0] != counts[0] or again[1] != counts[0] or any(again[2:6]):
+                        if again[0] != rows or again[1] != rows or any(again[2:6]):
                             raise EngineError("the scheduler's plan differs from the decode steps that ran ahead of it")
-                        events.extend(scheduler.complete_ordered(later))
+                        events.extend(scheduler.complete_ordered(np.ascontiguousarray(later[live])))
                     return events
         plan = scheduler.read_plan(counts)
         sampled: Dict[int, int] = {}

@@ -235,9 +235,10 @@ class Scheduler:
         return rows
 
     def steps_ahead(self, limit: int, rows: int):
-        """For a plain decode plan: how many further steps of exactly this batch are certain to
-        follow whatever tokens are drawn (nobody waits, no stop tokens, every request has the
-        budget), at most ``limit``; and the plan's requests (the host library's ids) in row order."""
+        """For a plain decode plan: how many further steps of this batch are certain to follow
+        whatever tokens are drawn (nobody waits, every request has the budget), at most ``limit``,
+        but for requests that draw a stop token: those are missing from the plans after it. And
+        the plan's requests (their ids) in row order."""
         requests = host.ids(rows)
         ahead = self._lib.fwh_plan_steps_ahead(self._native, int(limit), requests, rows)
         if ahead < 0:

@@ -447,16 +447,19 @@ class Stepper:
         captured.graph.replay()
         self.graph_replays += 1
 
-    def replay_planned(self, captured: "_CapturedDecode", scheduler, steps: int = 1) -> Optional[np.ndarray]:
+    def replay_planned(self, captured: "_CapturedDecode", scheduler, steps: int = 1):
         """Decode steps straight from the scheduler's plan (see ``StepContext.fill_from``): the
         pages are reserved by the plan and the lengths are committed when the scheduler completes
         it, so the cache manager is not asked again. Every token is the most likely one. With
         ``steps`` > 1 and a plan that is certain to repeat (``Scheduler.steps_ahead``), up to that
         many steps run back to back on the device (their pages reserved and their block tables
         uploaded before the first), each fed the tokens of the one before, and the host reads all
-        of them at once: it is then asked once per turn instead of once per step.
-        Returns the tokens, int32 [steps run, rows], or None if the plan is not a plain decode
-        step (nothing has run then)."""
+        of them at once: it is then asked once per turn instead of once per step. A request that
+        draws one of its stop tokens on the way has run on regardless (its row costs nothing beside
+        the others); the caller drops what it drew after it.
+        Returns (tokens, int32 [steps run, rows]; the plan's requests in row order if more than
+        one step ran, else None), or None if the plan is not a plain decode step (nothing has
+        run then)."""
         ctx = captured.ctx
         cache = self.cache
         rows = ctx.fill_from(scheduler, cache)
@@ -488,7 +491,7 @@ class Stepper:
         ran = ahead + 1
         self.steps += ran
         self.tokens_run += rows * ran
-        return drawn[:ran, :rows].cpu().numpy()
+        return drawn[:ran, :rows].cpu().numpy(), (list(natives[:rows]) if ahead else None)
 
     def _replay(self, captured: "_CapturedDecode", entries: Sequence[StepEntry], described=None) -> Optional[torch.Tensor]:
         cache = self.cache

@@ -197,8 +197,8 @@ def test_engine_tasks_equal_blocking_generation_and_survive_preemption(loaded):
 def test_decode_steps_that_run_ahead_of_the_host_give_the_same_tokens(loaded, dtype):
     """With several decode steps per turn the device feeds each step's tokens to the next and
     the host reads them in bursts: the same tokens in the same order as one step per turn (float32:
-    the plain model's), bursts cut short by the shortest budget, across page edges, and none for
-    a request that may stop on a token or while somebody still waits for a slot."""
+    the plain model's), bursts cut short by the shortest budget, across page edges, a request that stops on a token
+    in the middle of a burst, and no bursts while somebody still waits for a slot."""
     m = loaded("B", dtype)
     config, weights = m.plain_config, m.plain_weights
     prompts = [random_tokens(m.config.vocab_size, n, seed=40 + n) for n in (3, 60, 9, 30)]
@@ -226,11 +226,15 @@ def test_decode_steps_that_run_ahead_of_the_host_give_the_same_tokens(loaded, dt
         assert task_events[-1][2] == 1 and all(e[2] != 1 for e in task_events[:-1]), "finished is a request's last event"
     if dtype == "float32":
         assert ahead == [plain.greedy(config, weights, p, n) for p, n in zip(prompts, budgets)]
-    # a request with a stop token keeps the whole batch at one step per turn while it runs
-    stop = single[0][20]
-    stopped, burst, _ = run(4, stop_tokens=(stop,))
-    cut = single[0].index(stop) + 1
-    assert stopped[0] == single[0][:cut] and stopped[1:] == single[1:]
+    # a request that may stop on a token runs ahead like the others; when it draws that token, wherever
+    # in a turn, it ends there, what its row drew after it is dropped, and the others go on in order
+    for place in (17, 18, 19, 20):
+        stop = single[0][place]
+        stopped, burst, events = run(4, stop_tokens=(stop,))
+        cut = single[0].index(stop) + 1
+        assert stopped[0] == single[0][:cut] and stopped[1:] == single[1:] and burst == 4
+        for task_events in ([e for e in events if e[0] == task] for task in {e[0] for e in events}):
+            assert task_events[-1][2] == 1 and all(e[2] != 1 for e in task_events[:-1])
     # two slots for four requests: somebody waits until the last two run, only then steps run ahead
     queued, burst, _ = run(4, parallel=2)
     assert burst == 4 and [len(tokens) for tokens in queued] == budgets

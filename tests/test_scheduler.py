@@ -309,3 +309,49 @@ def test_a_failure_between_two_plans_is_not_lost():
     assert [e for e in seen[b.id]] == [(b.id, 0, EVENT_ERROR)]
     assert a.generated == expected_tokens([1] * 5, 3)
     assert scheduler.forget(b.id) and b.id not in scheduler.requests and not scheduler.forget(b.id)
+
+
+def test_steps_ahead_of_the_host_and_a_stop_token_in_the_middle_of_them():
+    """What a turn of several decode steps relies on: how many steps are certain to follow a plain
+    decode plan (the shortest budget, nobody waiting; a stop token does not forbid them), and
+    that a request which ends on the way is missing from the plans after it while the others keep
+    their rows' order."""
+    import numpy as np
+    cache, scheduler = make(num_pages=16, max_requests=4)
+    prompts = [[3, 4, 5], [9, 8], [20, 21, 22, 23]]
+    # the second request will stop at the third token it draws
+    stop = expected_tokens(prompts[1], 3)[2]
+    assert stop not in expected_tokens(prompts[1], 2)
+    budgets = [30, 30, 12]
+    requests = [scheduler.submit(p, n, stop_tokens=[stop] if i == 1 else []) for i, (p, n) in enumerate(zip(prompts, budgets))]
+    plan = scheduler.schedule()                         # the prompts
+    scheduler.complete(plan, {s.request.id: oracle(s.request.tokens) for s in plan.segments})
+    counts = scheduler.plan_next()                      # a plain decode plan of three rows
+    assert counts[0] == counts[1] == 3 and not any(counts[2:6])
+    ahead, rows = scheduler.steps_ahead(7, 3)
+    assert ahead == 7 and list(rows[:3]) == [r.id for r in requests]
+    assert scheduler.steps_ahead(100, 3)[0] == 12 - 1 - 1   # the shortest budget: one token drawn, one by this plan
+    # the device runs the turn on regardless of the stop token; the host then hands the steps over in order
+    sequences = [list(p) + expected_tokens(p, 1) for p in prompts]
+    live = [True, True, True]
+    for step in range(1 + 4):
+        if step:
+            counts = scheduler.plan_next()
+            assert counts[0] == counts[1] == sum(live) and not any(counts[2:6])
+        drawn = [oracle(sequence) for sequence in sequences]
+        for sequence, token in zip(sequences, drawn):
+            sequence.append(token)                      # every row goes on, whether its request still lives or not
+        events = scheduler.complete_ordered(np.array([t for t, alive in zip(drawn, live) if alive], dtype=np.int32))
+        owners = [e[0] for e in events if e[2] == EVENT_TOKEN]
+        assert owners == [r.id for r, alive in zip(requests, live) if alive], "the rows keep their order"
+        for e in events:
+            if e[2] == EVENT_FINISHED:
+                live[[r.id for r in requests].index(e[0])] = False
+        cache.check_invariants()
+    assert live == [True, False, True]
+    assert requests[1].generated == expected_tokens(prompts[1], 30, stop=(stop,)) and len(requests[1].generated) == 3
+    assert requests[0].generated == expected_tokens(prompts[0], 6) and requests[2].generated == expected_tokens(prompts[2], 6)
+    # somebody waiting for a slot: no steps ahead
+    for _ in range(3):
+        scheduler.submit([1, 2], 4)
+    assert scheduler.plan_next()[0] and scheduler.steps_ahead(4, 4)[0] == 0
