@@ -447,20 +447,25 @@ DEEP_MIN_K = 1024         # adding into the residual (2,048 x 2,048 x 2,048: 31 
 DEEP_MIN_K_STORE = 4096   # storing: no old values travel during the exchange at a tile's end, a short K gains nothing
 DEEP_ROUND = 256          # tiles of a round: one per compute unit
 DEEP_FILL = 0.85          # least share of the rounds' places that the tiles must fill (640 narrow tiles, 0.83: 193 vs 189 us)
+# adding into the residual, 2,048 features: 144 wide tiles (1,152 rows) K 8,192 72 vs 103 us, K 2,048 28 vs 35 us; 160
+# narrow tiles (576 rows) 46 vs 65 us and 16.5 vs 27 us; 576 narrow (2,304 rows) 120 vs 135 us; 128 narrow tiles lose
+DEEP_FILL_ADDING = 0.55
 
 
-def _fills_rounds(tiles: int) -> bool:
+def _round_fill(tiles: int) -> float:
+    """The share of the places in whole rounds over the chip that the tiles fill."""
     rounds = -(-tiles // DEEP_ROUND)
-    return tiles > 0 and tiles >= DEEP_FILL * rounds * DEEP_ROUND
+    return tiles / (rounds * DEEP_ROUND) if tiles > 0 else 0.0
 
 
 def _deep_columns(mode: int, M: int, N: int, K: int) -> int:
-    """The width of the tiles whose waves split K that serves this shape: 128 columns if they fill
-    whole rounds over the chip, else 64 if those do (an output of 1,024 features), else 0."""
-    for columns in (128, 64):
-        if _fills_rounds(library().fw_gemm_mfma_deep_tiles(mode, M, N, K, columns)):
-            return columns
-    return 0
+    """The width of the tiles whose waves split K that serves this shape: the width (128 or 64
+    columns) whose tiles fill their rounds over the chip better, the wider at a tie, if they fill
+    enough of them; else 0. A product that adds into the residual needs less (the other kernels
+    ask for the old values at the end of a tile, where nothing hides the read)."""
+    fills = {columns: _round_fill(library().fw_gemm_mfma_deep_tiles(mode, M, N, K, columns)) for columns in (128, 64)}
+    columns = 128 if fills[128] >= fills[64] else 64
+    return columns if fills[columns] >= (DEEP_FILL_ADDING if mode == 1 else DEEP_FILL) else 0
 
 
 DEEP_FEW_ROWS = 512       # up to here the tiles whose waves split K also serve a short K, if they are not too few

@@ -437,12 +437,15 @@ def test_tiles_whose_waves_split_k(ops, M, N, K, columns):
         ops.gemm_deep(a[:, :K - 8].contiguous(), w[:, :K - 8].contiguous())
 
 
-@pytest.mark.parametrize("M,N,K", [(2048, 2048, 4096), (1800, 1990, 4160), (2048, 1024, 2048)])
-def test_the_prompt_product_of_one_round_of_tiles_over_a_long_k(ops, M, N, K):
+@pytest.mark.parametrize("M,N,K,expected", [(2048, 2048, 4096, 128), (1800, 1990, 4160, 128), (2048, 1024, 2048, 64),
+                                            (1152, 2048, 2048, 128), (576, 2048, 1024, 64), (2304, 2048, 1024, 64)])
+def test_the_prompt_product_of_one_round_of_tiles_over_a_long_k(ops, M, N, K, expected):
     """What the dispatch sends to those tiles: about one 128 x 128 tile per compute unit and a
-    long K (the w2 product of a 2,048-token prompt)."""
+    long K (the w2 product of a 2,048-token prompt); for a product that adds into the residual
+    also rounds that are little more than half full, on the width that fills them better."""
     columns = ops._deep_columns(1, M, N, K)
-    assert columns == (64 if N == 1024 else 128) and K >= ops.DEEP_MIN_K
+    assert columns == expected and K >= ops.DEEP_MIN_K
+    assert ops._deep_columns(1, 512, 2048, 8192) == 0 and ops._deep_columns(0, 1152, 2048, 8192) == 0
     a = as_dev(gen(M, K), torch.bfloat16)
     w = as_dev(gen(N, K, seed=1, scale=K ** -0.5), torch.bfloat16)
     want = back(a) @ back(w).T
