@@ -41,7 +41,7 @@ int fw_gemm_skinny(const void* a, const void* w, const float* bias, void* out, i
                    int M, int N, int K, void* stream);
 int fw_gemm_mfma(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                  int M, int N, int K, void* stream);
-// The prompt product with 256 x 256 tiles, for shapes that give enough of them to fill the chip
+// The prompt product with 256 x 256 (or 256 x 192) tiles, for shapes that give enough of them to fill the chip
 // (fw_gemm_mfma_big_tiles says how many).
 int fw_gemm_mfma_big(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                      int M, int N, int K, void* stream);

@@ -369,10 +369,12 @@ static bool narrow_tiles_pay(int M, int N) {
     return 3 * fw_ceil_div(narrow, 256) < 4 * fw_ceil_div(wide, 256);
 }
 
-// How many 256 x 256 tiles a shape gives (the caller decides whether that fills the chip); 0 if
-// the kernel does not take the shape (K must be a multiple of 32).
+// How many tiles the kernel cuts a shape into, 256 x 256 or 256 x 192 as it will choose (the
+// caller decides whether that fills the chip); 0 if the kernel does not take the shape (K must be
+// a multiple of 32).
 extern "C" int fw_gemm_mfma_big_tiles(int mode, int M, int N, int K) {
     if (K <= 0 || K % BK) return 0;
+    if (mode != MB_SWIGLU && narrow_tiles_pay(M, N)) return fw_ceil_div(M, BT) * fw_ceil_div(N, 192);
     return fw_ceil_div(M, BT) * fw_ceil_div(N, mode == MB_SWIGLU ? BT / 2 : BT);
 }
 

@@ -470,7 +470,7 @@ def _deep_columns(mode: int, M: int, N: int, K: int) -> int:
 
 DEEP_FEW_ROWS = 512       # up to here the tiles whose waves split K also serve a short K, if they are not too few
 DEEP_FEW_TILES_WIDE = 192   # tiles of 128 columns from which those are taken, else
-DEEP_FEW_TILES = 96       # tiles of 64 columns from which those are (storing; adding into the residual: 128)
+DEEP_FEW_TILES = 96       # tiles of 64 columns from which those are
 
 
 def _deep_columns_few_rows(mode: int, M: int, N: int, K: int) -> int:
@@ -480,14 +480,15 @@ def _deep_columns_few_rows(mode: int, M: int, N: int, K: int) -> int:
     its compute unit keeps them coming. Measured against the products they replace, 8 in a row:
     storing 6,144 features at 256 rows 16.0 vs 21.0 us, at 128 rows 15.0 vs 18.6; 3,072 features at
     256 rows 15.0 vs 18.6, at 512 rows 15.9 vs 21.0 us; adding 2,048 features (K 2,048) at 512 rows
-    16.2 vs 23.0 us. With a long K (8,192) the product that cuts K over workgroups stays ahead."""
+    16.2 vs 23.0 us, at 320 rows 15.7 vs 21.5 us. With a long K (8,192) the product that cuts K over
+    workgroups is level with them."""
     if mode not in (0, 1) or M > DEEP_FEW_ROWS or K > (LONG_K if mode == 1 else 1 << 30):
         return 0
     wide = library().fw_gemm_mfma_deep_tiles(mode, M, N, K, 128)
     narrow = library().fw_gemm_mfma_deep_tiles(mode, M, N, K, 64)
     if mode == 0 and DEEP_FEW_TILES_WIDE <= wide <= DEEP_ROUND:
         return 128
-    if narrow >= (DEEP_FEW_TILES if mode == 0 else 128) and narrow <= 2 * DEEP_ROUND:
+    if DEEP_FEW_TILES <= narrow <= 2 * DEEP_ROUND:
         return 64
     return 0
 

@@ -364,10 +364,11 @@ def test_fast_gemm_every_epilogue(ops, M, N, K):
         close(ops.gemm_swiglu(a, w), act, torch.bfloat16, 0.4)
 
 
-@pytest.mark.parametrize("M,N,K", [(2048, 6144, 96), (1500, 8200, 160), (4000, 3100, 64), (1800, 6000, 2080)])
+@pytest.mark.parametrize("M,N,K", [(2048, 6144, 96), (1500, 8200, 160), (4000, 3100, 64), (1800, 6000, 2080), (1536, 6100, 96)])
 def test_large_tile_prompt_product(ops, M, N, K):
-    """Shapes with at least 192 tiles of 256 x 256 go to the large-tile kernel: every epilogue,
-    edges in both directions, few and many slabs. The first and the last shape give exactly one
+    """Shapes with at least 192 tiles of 256 x 256 (or of 256 x 192, where those are what the
+    kernel takes: the last shape has 144 of the wider) go to the large-tile kernel: every epilogue,
+    edges in both directions, few and many slabs. The first and the last two shapes give one
     round of tiles over the chip with tiles of 192 columns, which storing and accumulating
     products then take; the gated product keeps the 256 x 256 tiles."""
     assert ops.library().fw_gemm_mfma_big_tiles(0, M, N, K) >= ops.BIG_TILES_MIN and not ops.library().fw_gemm_mfma_big_tiles(0, M, N, K + 8)
@@ -460,7 +461,7 @@ def test_the_prompt_product_of_one_round_of_tiles_over_a_long_k(ops, M, N, K, ex
 
 
 @pytest.mark.parametrize("M,N,K,mode,columns", [(256, 6144, 2048, 0, 64), (500, 6100, 1984, 0, 128), (130, 6144, 2048, 0, 64),
-                                                   (512, 2048, 2048, 1, 64), (300, 3072, 1024, 0, 64),
+                                                   (512, 2048, 2048, 1, 64), (320, 2048, 2048, 1, 64), (300, 3072, 1024, 0, 64),
                                                    (256, 2048, 8192, 1, 0), (600, 6144, 2048, 0, 0), (256, 1024, 2048, 0, 0)])
 def test_a_few_hundred_rows_go_to_the_tiles_whose_waves_split_k(ops, M, N, K, mode, columns):
     """A decode step of a few hundred requests: storing and short accumulating products take those
