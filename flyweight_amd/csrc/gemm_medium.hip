@@ -438,7 +438,13 @@ static MediumPlan medium_plan(int M, int N, int K, int mode) {
         plan.tiles = fw_ceil_div(N, 32);
         const int chunk = 128;
         int splits = (256 + plan.tiles / 2) / plan.tiles;           // about one workgroup per compute unit
-        const int most = K / (2 * chunk) > 1 ? K / (2 * chunk) : 1; // at least two chunks per slice
+        // A slice costs its workgroup a start (the first loads' way from memory) and an end (its sums
+        // to the workspace, the ticket, the last one reading all of them: three trips to memory, 5-8 us)
+        // whatever its length, so K is only cut where a slice keeps at least nine chunks: at 64 rows
+        // and K 1,024 one slice against two or three 12.4 vs 21.1 us (gate|up of 4,608 features), 8.1 vs
+        // 13.2 (3,072 features), 7.4 vs 10.4 (1,024); K 2,048, 2,048 features 10.9 vs 12.0 us; K 4,608,
+        // 1,024 features 4 slices 14.1 vs 8 slices 15.7 us; K 8,192 stays at 4 slices (18.9 us; 1: 34.9).
+        const int most = K / (9 * chunk) > 1 ? K / (9 * chunk) : 1;
         splits = splits < 1 ? 1 : (splits > most ? most : splits);
         if (splits > 16) splits = 16;
         plan.k_per_split = fw_ceil_div(fw_ceil_div(K, splits), chunk) * chunk;
