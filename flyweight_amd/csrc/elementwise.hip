@@ -16,7 +16,7 @@ void fw_set_error(const char* format, ...) {
     va_end(args);
 }
 extern "C" const char* fw_last_error(void) { return fw_error_text; }
-extern "C" int fw_abi_version(void) { return 4; }
+extern "C" int fw_abi_version(void) { return 5; }
 
 // ---- embedding -------------------------------------------------------------------------
 // The reference gathers one row per token and widens it to float32
@@ -204,14 +204,6 @@ extern "C" int fw_rope_table(const int32_t* positions, const double* inv_freq, f
 // A candidate is ordered by (value descending, id ascending); NaN sorts last. The key packs
 // both so that one 64-bit max finds the winner, as the reference's fused LM-head argmax
 // does (native/include/flyweight_v2_qwen_kernels.hpp:2391-2405): ties go to the lowest id.
-__device__ __forceinline__ unsigned long long candidate_key(float value, int id) {
-    uint32_t bits = __float_as_uint(value);
-    uint32_t ordered;
-    if (value != value) ordered = 0u;                                   // NaN: below everything
-    else ordered = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u); // monotone in value
-    return ((unsigned long long)ordered << 32) | (unsigned long long)(0xffffffffu - (uint32_t)id);
-}
-
 __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
 #pragma unroll
     for (int offset = 32; offset > 0; offset >>= 1) {

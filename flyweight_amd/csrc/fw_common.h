@@ -157,3 +157,18 @@ __device__ __forceinline__ float block_sum(float v, float* scratch /* >= 16 floa
 }
 
 static inline int fw_ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
+
+// ---- candidates for the next token ----------------------------------------------------
+// A candidate is ordered by (value descending, id ascending); NaN sorts last. The key packs both
+// so that one 64-bit comparison orders two candidates (a greater key comes first) and ties go to
+// the lowest id, as the reference's fused LM-head argmax does
+// (native/include/flyweight_v2_qwen_kernels.hpp:2391-2405).
+__device__ __forceinline__ unsigned long long candidate_key(float value, int id) {
+    uint32_t bits = value == 0.0f ? 0u : __float_as_uint(value);        // -0 and +0 are one value: the lower id first
+    uint32_t ordered;
+    if (value != value) ordered = 0u;                                   // NaN: below everything
+    else ordered = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u); // monotone in value
+    return ((unsigned long long)ordered << 32) | (unsigned long long)(0xffffffffu - (uint32_t)id);
+}
+__device__ __forceinline__ int candidate_id(unsigned long long key) { return (int)(0xffffffffu - (uint32_t)(key & 0xffffffffull)); }
+

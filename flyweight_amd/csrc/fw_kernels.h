@@ -185,6 +185,14 @@ int fw_argmax_rows_static_max_rows(void);
 int fw_topk_rows(const float* logits, float* values, int32_t* ids, int rows, int vocab, int k,
                  void* stream);
 
+// The next token of every row, drawn on the device: settings float32 [rows][4] = temperature (0:
+// greedy, the best candidate, ties to the lowest id), top_k (0: all candidates), top_p, min_p;
+// states [rows]: the rows' xorshift64* generators, moved on by the rows that draw. also / advance
+// as in fw_argmax_rows. Candidates are taken in (value descending, id ascending) order and the
+// sums are float64, in that order.
+int fw_sample_rows(const float* logits, const float* settings, unsigned long long* states, int32_t* ids, int32_t* also,
+                   int32_t* advance, int rows, int vocab, void* stream);
+
 int fw_fill_zero(void* ptr, long long bytes, void* stream);
 
 #ifdef __cplusplus

@@ -47,6 +47,9 @@ int fwr_attention(const float* q, float* out, const float* k_pages, const float*
 // elementwise.hip argmax / top-k: order by value descending, then id ascending; NaN last
 int fwr_argmax_rows(const float* logits, int32_t* ids, int rows, int vocab);
 int fwr_topk_rows(const float* logits, float* values, int32_t* ids, int rows, int vocab, int k);
+// sampling.hip: settings [rows][4] = temperature (0: greedy), top_k (0: all), top_p, min_p; states: the
+// rows' xorshift64* generators, moved on by the rows that draw
+int fwr_sample_rows(const float* logits, const float* settings, unsigned long long* states, int32_t* ids, int rows, int vocab);
 // elementwise.hip scale_softcap: x * scale, then with cap > 0 cap * tanh(x / cap)
 int fwr_scale_softcap(float* x, long long count, float scale, float cap);
 

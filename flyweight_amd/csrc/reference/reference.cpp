@@ -246,6 +246,67 @@ int fwr_topk_rows(const float* logits, float* values, int32_t* ids, int rows, in
     return 0;
 }
 
+// native/src/v2_runtime.cpp:29500-29566 (the candidates), 29686-29743 (the cuts and the draw),
+// 29307-29314 (the generator): one row after the other, the whole row sorted, every sum in order
+int fwr_sample_rows(const float* logits, const float* settings, unsigned long long* states, int32_t* ids, int rows, int vocab) {
+    std::vector<int> order(vocab);
+    std::vector<double> p(vocab);
+    for (int r = 0; r < rows; ++r) {
+        const float* row = logits + (size_t)r * vocab;
+        const double temperature = settings[4 * r], top_p = settings[4 * r + 2], min_p = settings[4 * r + 3];
+        const long long top_k = (long long)settings[4 * r + 1];
+        for (int i = 0; i < vocab; ++i) order[i] = i;
+        std::sort(order.begin(), order.end(), [&](int a, int b) { return better(row[a], a, row[b], b); });
+        const int candidates = top_k > 0 && top_k < vocab ? (int)top_k : vocab;
+        ids[r] = order[0];
+        if (!(temperature > 0.0) || candidates == 1) continue;
+        const double best = (double)row[order[0]] / temperature;
+        double total = 0.0;
+        for (int i = 0; i < candidates; ++i) {
+            const double scaled = (double)row[order[i]] / temperature;
+            p[i] = std::isfinite(scaled) ? std::exp(scaled - best) : 0.0;
+            total += p[i];
+        }
+        if (!(total > 0.0) || !std::isfinite(total)) continue;
+        int keep = candidates;
+        if (top_p < 1.0) {
+            double share = 0.0;
+            for (int i = 0; i < candidates; ++i) {
+                share += p[i] / total;
+                if (share >= top_p) {
+                    keep = i + 1;
+                    break;
+                }
+            }
+        }
+        if (min_p > 0.0) {
+            const double least = min_p * p[0];
+            int kept = 1;
+            while (kept < keep && p[kept] >= least) ++kept;
+            keep = kept;
+        }
+        double kept_total = 0.0;
+        for (int i = 0; i < keep; ++i) kept_total += p[i];
+        unsigned long long x = states[r] ? states[r] : 0x9E3779B97F4A7C15ull;
+        x ^= x >> 12;
+        x ^= x << 25;
+        x ^= x >> 27;
+        states[r] = x;
+        const double u = (double)((x * 2685821657736338717ull) >> 11) * (1.0 / 9007199254740992.0);
+        const double threshold = u * kept_total;
+        double running = 0.0;
+        ids[r] = order[keep - 1];
+        for (int i = 0; i < keep; ++i) {
+            running += p[i];
+            if (threshold <= running) {
+                ids[r] = order[i];
+                break;
+            }
+        }
+    }
+    return 0;
+}
+
 int fwr_scale_softcap(float* x, long long count, float scale, float cap) {
     for (long long i = 0; i < count; ++i) {
         double value = (double)x[i] * scale;

@@ -16,7 +16,7 @@ import numpy as np
 import torch
 
 from ..cache import OutOfPages
-from ..sampling import GREEDY, SamplingConfig, sample_rows
+from ..sampling import GREEDY, SamplingConfig, pack_settings, sample_rows
 from .model import CausalLM, load_model, parse_dtype
 from .scheduler import (EVENT_ERROR, EVENT_FINISHED, EVENT_PREFILL, EVENT_TOKEN, Request, Scheduler,
                         SchedulerError)
@@ -204,16 +204,23 @@ class Runtime:
         # A plain decode step (one token for every request of the plan, every token the most likely
         # one, nothing else happened) that a captured step serves goes from the scheduler's plan to
         # the upload buffer and back without an object per request.
-        if counts[0] and counts[0] == counts[1] and not any(counts[2:6]) and scheduler.all_greedy:
+        if counts[0] and counts[0] == counts[1] and not any(counts[2:6]):
             captured = self.stepper.planned_decode(counts[0], counts[6] + self.decode_steps_per_turn - 1)
             if captured is not None:
                 began = time.perf_counter_ns()
+                settings_of = None if scheduler.all_greedy else self._sampling_of
                 try:
-                    ran = self.stepper.replay_planned(captured, scheduler, self.decode_steps_per_turn)
+                    ran = self.stepper.replay_planned(captured, scheduler, self.decode_steps_per_turn, settings_of)
                 except Exception as error:
                     return self._fail_step(scheduler.read_plan(counts), error)
                 if ran is not None:
-                    tokens, row_requests = ran
+                    tokens, row_requests, moved_on = ran
+                    if moved_on is not None:
+                        # the generators have drawn on the device: the requests' own copies follow
+                        for request, state in zip(row_requests, moved_on.tolist()):
+                            drawing = scheduler.requests[request]
+                            if not drawing.sampling.greedy:
+                                drawing.rng.state = state
                     self._counters["steps"] += len(tokens)
                     self._counters["decode_calls"] += counts[0] * len(tokens)
                     self._counters["decode_ns"] += time.perf_counter_ns() - began
@@ -272,6 +279,11 @@ class Runtime:
                 self._counters["decode_ns"] += elapsed
             break
         return scheduler.complete(plan, sampled)
+
+    def _sampling_of(self, row_requests, settings, states) -> None:
+        """Fills what the device sampler reads for the rows of a decode plan."""
+        requests = [self.scheduler.requests[request] for request in row_requests]
+        pack_settings([r.sampling for r in requests], [r.rng for r in requests], self.model.spec.vocab_size, settings, states)
 
     def _fail_step(self, plan, error: Exception) -> List[Tuple[int, int, int]]:
         """A step failed while it ran (or for a reason that names no request): what the cache

@@ -234,6 +234,13 @@ class Scheduler:
             raise SchedulerError(host.last_error())
         return rows
 
+    def plan_requests(self, rows: int, tokens: Optional[int] = None):
+        """The requests (ids) of the plan made last, in the order of its ``rows`` segments, which
+        hold ``tokens`` tokens together (default: one each)."""
+        owners, lengths, wants, flat = host.ids(rows), host.ints(rows), host.ints(rows), host.ints(tokens or rows)
+        self._lib.fwh_plan_segments(self._native, owners, lengths, wants, flat)
+        return owners
+
     def steps_ahead(self, limit: int, rows: int):
         """For a plain decode plan: how many further steps of this batch are certain to follow
         whatever tokens are drawn (nobody waits, every request has the budget), at most ``limit``,

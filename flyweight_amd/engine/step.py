@@ -447,7 +447,7 @@ class Stepper:
         captured.graph.replay()
         self.graph_replays += 1
 
-    def replay_planned(self, captured: "_CapturedDecode", scheduler, steps: int = 1):
+    def replay_planned(self, captured: "_CapturedDecode", scheduler, steps: int = 1, settings_of=None):
         """Decode steps straight from the scheduler's plan (see ``StepContext.fill_from``): the
         pages are reserved by the plan and the lengths are committed when the scheduler completes
         it, so the cache manager is not asked again. Every token is the most likely one. With
@@ -457,15 +457,26 @@ class Stepper:
         of them at once: it is then asked once per turn instead of once per step. A request that
         draws one of its stop tokens on the way has run on regardless (its row costs nothing beside
         the others); the caller drops what it drew after it.
-        Returns (tokens, int32 [steps run, rows]; the plan's requests in row order if more than
-        one step ran, else None), or None if the plan is not a plain decode step (nothing has
-        run then)."""
+        Every token is the most likely one unless ``settings_of`` is given: called with the plan's
+        requests in row order, it fills the sampling settings (float32 [rows, 4]) and generator
+        states (uint64 [rows]) handed to it, and the tokens are drawn on the device.
+        Returns (tokens, int32 [steps run, rows]; the plan's requests in row order; the generators'
+        states after the turn, uint64 [rows], or None), or None if the plan is not a plain decode
+        step (nothing has run then)."""
         ctx = captured.ctx
         cache = self.cache
         rows = ctx.fill_from(scheduler, cache)
         if rows < 0:
             return None
         ahead, natives = scheduler.steps_ahead(steps - 1, rows) if steps > 1 else (0, None)
+        if natives is None or (settings_of is not None and not ahead):
+            natives = scheduler.plan_requests(rows)       # (steps_ahead names them only when steps follow)
+        sampling = None
+        if settings_of is not None:
+            sampling = captured.sampling_buffers(self.device)
+            sampling.host_settings[:] = 0.0                 # the rows behind the plan's: greedy
+            settings_of(list(natives[:rows]), sampling.host_settings[:rows], sampling.host_states[:rows])
+            sampling.upload()
         if ahead:
             # Pages for all the steps of the turn now, and the block tables with them: a table that
             # already holds the page a later step will write to reads the same for the steps before.
@@ -483,15 +494,23 @@ class Stepper:
         # likely tokens writes them to the turn's record and to the next step's token ids, and moves
         # every row's position on by one.
         drawn = torch.empty((ahead + 1, ctx.num_rows), dtype=torch.int32, device=self.device)
+        def draw(step: int, **feed) -> None:
+            if sampling is None:
+                ops.argmax_rows(captured.logits, out=drawn[step], **feed)
+            else:
+                ops.sample_rows(captured.logits, sampling.settings, sampling.states, out=drawn[step], **feed)
+
         for step in range(ahead):
             self._run(captured)
-            ops.argmax_rows(captured.logits, out=drawn[step], also=ctx.token_ids, advance=ctx.row_pos)
+            draw(step, also=ctx.token_ids, advance=ctx.row_pos)
         self._run(captured)
-        ops.argmax_rows(captured.logits, out=drawn[ahead])
+        draw(ahead)
         ran = ahead + 1
         self.steps += ran
         self.tokens_run += rows * ran
-        return drawn[:ran, :rows].cpu().numpy(), (list(natives[:rows]) if ahead else None)
+        tokens = drawn[:ran, :rows].cpu().numpy()
+        moved_on = sampling.states[:rows].cpu().numpy().view(np.uint64) if sampling is not None else None
+        return tokens, list(natives[:rows]), moved_on
 
     def _replay(self, captured: "_CapturedDecode", entries: Sequence[StepEntry], described=None) -> Optional[torch.Tensor]:
         cache = self.cache
@@ -511,9 +530,32 @@ class Stepper:
         return captured.logits[wanted]
 
 
+class _SamplingBuffers:
+    """What the device sampler reads for a captured step's rows: settings float32 [rows, 4] and
+    generator states int64 [rows], on the device and in one pinned buffer on the host."""
+
+    def __init__(self, rows: int, device):
+        self._host = torch.zeros(3 * rows, dtype=torch.int64, pin_memory=True)
+        self._device = torch.zeros(3 * rows, dtype=torch.int64, device=device)
+        words = self._host.numpy()
+        self.host_settings = words[:2 * rows].view(np.float32).reshape(rows, 4)
+        self.host_states = words[2 * rows:].view(np.uint64)
+        self.settings = self._device[:2 * rows].view(torch.float32).view(rows, 4)
+        self.states = self._device[2 * rows:]
+
+    def upload(self) -> None:
+        self._device.copy_(self._host, non_blocking=True)
+
+
 class _CapturedDecode:
     def __init__(self, ctx: StepContext):
         self.ctx = ctx
         self.graph = None
         self.logits = None
         self.ran = False            # whether the step has run eagerly once
+        self._sampling = None
+
+    def sampling_buffers(self, device) -> _SamplingBuffers:
+        if self._sampling is None:
+            self._sampling = _SamplingBuffers(self.ctx.num_rows, device)
+        return self._sampling

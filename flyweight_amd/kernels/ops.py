@@ -19,7 +19,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _lib = None
 
@@ -386,6 +386,30 @@ def argmax_rows(logits: torch.Tensor, out: Optional[torch.Tensor] = None, also: 
                 raise KernelError(f"argmax_rows: {name} must be contiguous and hold {rows} ids")
     workspace = torch.empty((max(rows, 1), 64), dtype=torch.int64, device=logits.device)       # best key of each part
     _check(library().fw_argmax_rows(_p(logits), _p(ids), _p(also), _p(advance), _p(workspace), rows, vocab, _stream()))
+    return ids
+
+
+def sample_rows(logits: torch.Tensor, settings: torch.Tensor, states: torch.Tensor, out: Optional[torch.Tensor] = None,
+                also: Optional[torch.Tensor] = None, advance: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The next token of every row, drawn on the device (fw_sample_rows): ``settings`` float32
+    [rows, 4] = temperature (0: greedy), top_k (0: all), top_p, min_p; ``states`` int64 [rows], the
+    rows' xorshift64* generators, moved on in place by the rows that draw. ``out`` / ``also`` /
+    ``advance`` as for ``argmax_rows``."""
+    _dev(logits, settings, states)
+    _want(logits, torch.float32, "logits")
+    _want(settings, torch.float32, "settings")
+    _want(states, torch.int64, "states")
+    rows, vocab = logits.shape
+    if settings.numel() < 4 * rows or states.numel() < rows or not settings.is_contiguous() or not states.is_contiguous():
+        raise KernelError(f"sample_rows: settings must hold [{rows}, 4] and states [{rows}], contiguous")
+    ids = out if out is not None else torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    for name, target in (("out", out), ("also", also), ("advance", advance)):
+        if target is not None:
+            _dev(target)
+            _want(target, torch.int32, name)
+            if target.numel() < rows or not target.is_contiguous():
+                raise KernelError(f"sample_rows: {name} must be contiguous and hold {rows} ids")
+    _check(library().fw_sample_rows(_p(logits), _p(settings), _p(states), _p(ids), _p(also), _p(advance), rows, vocab, _stream()))
     return ids
 
 

@@ -154,6 +154,17 @@ def topk_rows(logits, k: int) -> Tuple[np.ndarray, np.ndarray]:
     return values, ids
 
 
+def sample_rows(logits, settings, states) -> Tuple[np.ndarray, np.ndarray]:
+    """The next token of every row and the generators' states afterwards (``states`` uint64 [rows]
+    is not changed): settings float32 [rows, 4] = temperature, top_k, top_p, min_p."""
+    logits = _f(logits)
+    settings = np.ascontiguousarray(settings, dtype=np.float32)
+    moved_on = np.ascontiguousarray(states, dtype=np.uint64).copy()
+    ids = np.empty(logits.shape[0], dtype=np.int32)
+    _check(library().fwr_sample_rows(_p(logits), _p(settings), _p(moved_on), _p(ids), logits.shape[0], logits.shape[1]))
+    return ids, moved_on
+
+
 def scale_softcap(x, scale: float = 1.0, cap: float = 0.0) -> np.ndarray:
     x = _f(x).copy()
     _check(library().fwr_scale_softcap(_p(x), ctypes.c_longlong(x.size), ctypes.c_float(scale), ctypes.c_float(cap)))

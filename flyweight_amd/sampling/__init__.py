@@ -1,5 +1,5 @@
-from .config import GREEDY, MAX_DEVICE_TOP_K, SamplingConfig, defaults
-from .sampler import XorShift64Star, draw_from_candidates, host_candidates, make_rng, sample_rows
+from .config import GREEDY, SamplingConfig, defaults
+from .sampler import XorShift64Star, draw_from_candidates, host_candidates, make_rng, pack_settings, sample_rows
 
-__all__ = ["GREEDY", "MAX_DEVICE_TOP_K", "SamplingConfig", "defaults", "XorShift64Star", "draw_from_candidates",
-           "host_candidates", "make_rng", "sample_rows"]
+__all__ = ["GREEDY", "SamplingConfig", "defaults", "XorShift64Star", "draw_from_candidates", "host_candidates", "make_rng",
+           "pack_settings", "sample_rows"]

@@ -10,9 +10,6 @@ import math
 from dataclasses import dataclass
 from typing import Optional
 
-MAX_DEVICE_TOP_K = 256
-
-
 @dataclass(frozen=True)
 class SamplingConfig:
     temperature: float = 0.8     # 0 is greedy: the best candidate, ties to the lowest id

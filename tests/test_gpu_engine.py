@@ -320,11 +320,65 @@ def test_seeded_sampling_does_not_depend_on_the_batch(loaded):
         want.append(plain.sample(logits.astype(np.float32), 0.8, 40, 0.95, 0.05, rng))
         context.append(want[-1])
     assert batch[ids[1]] == want
-    # top_k = 0 takes the host path over the whole vocabulary
+    # top_k = 0: the whole vocabulary; also the plain sampler's tokens
     full = _runtime(m, parallel_sequences=1)
     a = full.generate(prompts[1], 6, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, seed=3)
     b = full.generate(prompts[1], 6, temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, seed=3)
-    assert a == b and len(a) == 6
+    rng = plain.XorShift64Star(3)
+    context, want = list(prompts[1]), []
+    for _ in range(6):
+        logits = plain.forward(m.plain_config, m.plain_weights, context)[-1]
+        want.append(plain.sample(logits.astype(np.float32), 1.0, 0, 1.0, 0.0, rng))
+        context.append(want[-1])
+    assert a == b == want
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_drawn_tokens_come_from_recorded_steps_and_turns_like_the_most_likely_ones(loaded, dtype):
+    """Requests that draw their tokens (each with its own settings and seed, one of them greedy) run
+    through the recorded decode steps with the sampler behind them, one step or four per turn: the
+    same tokens either way, the same as each request alone, and in float32 the plain sampler's
+    given the plain model's logits. The generators end where the host's copies say."""
+    m = loaded("B", dtype)
+    prompts = [random_tokens(m.config.vocab_size, n, seed=70 + n) for n in (5, 33, 12, 64)]
+    settings = [dict(temperature=0.8, top_k=40, top_p=0.95, min_p=0.05, seed=11), dict(temperature=1.3, top_k=0, top_p=0.7, min_p=0.0, seed=12),
+                dict(temperature=0.0), dict(temperature=0.5, top_k=3, top_p=1.0, min_p=0.3, seed=14)]
+    budgets = [21, 30, 17, 26]
+
+    def run(steps_per_turn):
+        runtime = _runtime(m, parallel_sequences=4, prefill_rows=64, max_batch_tokens=128, decode_steps_per_turn=steps_per_turn)
+        ids = [runtime.task_submit(p, n, **kw) for p, n, kw in zip(prompts, budgets, settings)]
+        states = {}
+        bursts = []
+        while runtime.scheduler.has_work():
+            for task in ids:
+                request = runtime.scheduler.requests.get(task)
+                if request is not None:
+                    states[task] = request.rng.state
+            got = runtime.engine_step()
+            bursts.append(max([sum(1 for e in got if e[0] == task and e[2] == 0) for task in ids] + [0]))
+            for task, token, kind in got:
+                if kind == 0:
+                    states.setdefault(("tokens", task), []).append(token)
+        return [states[("tokens", task)] for task in ids], max(bursts), runtime.stepper.graph_replays
+
+    single, burst, replays = run(1)
+    assert burst == 1 and replays > 20, "the drawing requests ran through recorded steps"
+    ahead, burst, _ = run(4)
+    assert ahead == single and burst == 4
+    assert [len(tokens) for tokens in single] == budgets
+    for prompt, budget, kw, tokens in zip(prompts, budgets, settings, single):
+        alone = _runtime(m, parallel_sequences=1, prefill_rows=64)
+        if dtype == "float32":          # (in bfloat16 a prompt beside other rows may round to another of two near-equal logits)
+            assert alone.generate(prompt, budget, **kw) == tokens
+        if dtype == "float32" and kw.get("temperature", 0) > 0:
+            rng = plain.XorShift64Star(kw["seed"])
+            context, want = list(prompt), []
+            for _ in range(budget):
+                logits = plain.forward(m.plain_config, m.plain_weights, context)[-1]
+                want.append(plain.sample(logits.astype(np.float32), kw["temperature"], kw["top_k"], kw["top_p"], kw["min_p"], rng))
+                context.append(want[-1])
+            assert tokens == want
 
 
 def test_errors_are_reported_not_hidden(loaded):

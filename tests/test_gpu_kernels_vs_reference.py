@@ -72,6 +72,38 @@ def test_rows_kernels(ops, ref, dtype):
     assert found.cpu().tolist() == ref_ids.tolist() and np.array_equal(values.cpu().numpy(), ref_values)
 
 
+def test_sampler_draws_the_reference_samplers_tokens(ops, ref):
+    """The device sampler against the C++ one (whole row sorted, every sum in order): the same
+    tokens and the same generator states over random rows and settings, drawn three times in a
+    row; also into the places a following decode step reads (ids, positions)."""
+    from test_reference_kernels import sampling_cases
+    drawn = 0
+    for logits, settings, states in sampling_cases(60, seed=5):
+        rows = len(logits)
+        device_logits, device_settings = torch.tensor(logits, device=DEV), torch.tensor(settings, device=DEV)
+        device_states = torch.tensor(states.view(np.int64), device=DEV)
+        also = torch.full((rows,), -1, dtype=torch.int32, device=DEV)
+        positions = torch.arange(rows, dtype=torch.int32, device=DEV)
+        for draw in range(3):
+            want_ids, states = ref.sample_rows(logits, settings, states)
+            got = ops.sample_rows(device_logits, device_settings, device_states, also=also, advance=positions)
+            assert got.cpu().tolist() == want_ids.tolist() == also.cpu().tolist()
+            assert np.array_equal(device_states.cpu().numpy().view(np.uint64), states)
+            assert positions.cpu().tolist() == [r + draw + 1 for r in range(rows)]
+            drawn += rows
+    assert drawn > 500
+    # a vocabulary like a model's, rows that are greedy beside rows that draw
+    logits = (RNG.normal(size=(6, 65536)) * 3).astype(np.float32)
+    settings = np.array([[0, 0, 1, 0], [0.8, 40, 0.95, 0.05], [1.0, 0, 0.9, 0], [0.7, 1024, 1.0, 0.01], [2.0, 5000, 0.99, 0], [1.0, 0, 1.0, 0]],
+                        dtype=np.float32)
+    states = np.arange(1, 7, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15)
+    want_ids, want_states = ref.sample_rows(logits, settings, states)
+    device_states = torch.tensor(states.view(np.int64), device=DEV)
+    got = ops.sample_rows(torch.tensor(logits, device=DEV), torch.tensor(settings, device=DEV), device_states)
+    assert got.cpu().tolist() == want_ids.tolist() and got.cpu().tolist()[0] == int(logits[0].argmax())
+    assert np.array_equal(device_states.cpu().numpy().view(np.uint64), want_states) and want_states[0] == states[0]
+
+
 # rows that pick every product kernel: the fused decode product (<= 16), the split-K one (17..64),
 # the tiled prompt kernels (beyond), and the plain float32 kernel
 @pytest.mark.parametrize("dtype", DTYPES)

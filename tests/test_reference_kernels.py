@@ -128,6 +128,52 @@ def test_argmax_and_top_k_order():
     assert 5 not in ids[2].tolist() and ref.topk_rows(logits, 300)[1][2, -1] == 5        # NaN sorts last
 
 
+def sampling_cases(count, seed=0):
+    """Rows of logits with sampling settings and generator states that meet every branch of the
+    sampler: flat and peaked rows, ties, NaN and -inf, top_k from 1 to beyond the vocabulary."""
+    rng = np.random.default_rng(seed)
+    for trial in range(count):
+        vocab = int(rng.choice([5, 130, 1000, 1024, 1025, 4099]))
+        rows = int(rng.integers(1, 7))
+        logits = (rng.standard_normal((rows, vocab)) * [0.01, 1.0, 4.0, 12.0][trial % 4]).astype(np.float32)
+        if trial % 5 == 0:
+            logits[:, : max(1, vocab // 3)] = np.round(logits[:, : max(1, vocab // 3)])     # ties, and both zeros
+        if trial % 7 == 0:
+            logits[0, rng.integers(0, vocab)] = np.nan
+        if trial % 11 == 0:
+            logits[-1, rng.integers(0, vocab)] = -np.inf
+        settings = np.zeros((rows, 4), dtype=np.float32)
+        for r in range(rows):
+            settings[r] = (rng.choice([0.0, 0.3, 0.8, 1.0, 2.0]), rng.choice([0, 1, 2, 40, 256, 1024, 1500, vocab, vocab + 5]),
+                           rng.choice([1.0, 0.95, 0.5, 0.05]), rng.choice([0.0, 0.05, 0.5, 1.0]))
+        states = rng.integers(0, 2 ** 63 - 1, size=rows).astype(np.uint64)
+        states[0] = 0
+        yield logits, settings, states
+
+
+def test_sampler_against_the_plain_one_and_the_host_rules():
+    """The C++ sampler, the plain implementation's and the package's host rules draw the same
+    tokens and leave the generators in the same states, over random rows and settings."""
+    import plain_lfm2
+    from flyweight_amd.sampling import SamplingConfig, XorShift64Star, draw_from_candidates, host_candidates
+    drawn = 0
+    for logits, settings, states in sampling_cases(40):
+        ids, moved_on = ref.sample_rows(logits, settings, states)
+        for r in range(len(logits)):
+            temperature, top_k, top_p, min_p = (float(v) for v in settings[r])
+            top_k = int(top_k)
+            if not np.isnan(logits[r]).any():       # (the plain sampler says nothing about NaN; the engine's rule is: last)
+                plain_rng = plain_lfm2.XorShift64Star(int(states[r]))
+                assert ids[r] == plain_lfm2.sample(logits[r], temperature, top_k, top_p, min_p, plain_rng)
+            host_rng = XorShift64Star(int(states[r]))
+            values, order = host_candidates(logits[r], top_k if 0 < top_k < logits.shape[1] else 0)
+            config = SamplingConfig(temperature=temperature, top_k=top_k, top_p=top_p, min_p=min_p)
+            assert ids[r] == draw_from_candidates(values, order, config, host_rng)
+            assert int(moved_on[r]) == host_rng.state
+            drawn += int(moved_on[r]) != int(states[r])
+    assert drawn > 40
+
+
 def reference_forward(config, w, steps, num_pages=8):
     """A whole LFM2 from the C++ references alone: ``steps`` is a list of batches
     [(request, tokens)]; returns request -> logits of every token fed. Pages are handed out from
