@@ -60,9 +60,9 @@ def steps_per_turn(steps: int, warmup: int) -> int:
 
 
 def decode_run(torch, model, config, batch: int, steps: int, warmup: int, seed: int = 0, prompt: int = PROMPT,
-               context: int = CONTEXT):
-    """``batch`` requests with prompts of ``prompt`` tokens; returns (seconds for ``steps`` decode steps, mean
-    context, bytes the step must read)."""
+               context: int = CONTEXT, sampling: dict = None):
+    """``batch`` requests with prompts of ``prompt`` tokens (``sampling``: how they draw their tokens; default:
+    the most likely one); returns (seconds for ``steps`` decode steps, mean context, bytes the step must read)."""
     import numpy as np
     from flyweight_amd import Runtime
     from flyweight_amd.engine import accounting
@@ -79,7 +79,7 @@ def decode_run(torch, model, config, batch: int, steps: int, warmup: int, seed: 
                       max_batch_tokens=portion + batch, prefill_rows=portion, decode_steps_per_turn=turn).prepare()
     rng = np.random.default_rng(seed)
     for _ in range(batch):
-        runtime.task_submit(rng.integers(0, config.vocab_size, prompt).tolist(), new_tokens)
+        runtime.task_submit(rng.integers(0, config.vocab_size, prompt).tolist(), new_tokens, **(sampling or {}))
     # prompts: until every request has produced its first token
     while any(r.computed < len(r.prompt) for r in runtime.scheduler.requests.values()):
         runtime.engine_step()
@@ -243,6 +243,12 @@ def further_points(torch, args, points: dict) -> None:
         seconds, _, step_bytes = decode_run(torch, model, config, batch, steps, min(args.warmup, 8))
         points[name] = round(batch * steps / seconds, 1)
         points[name + "_frac"] = round(step_bytes / (seconds / steps) / 1e9 / HBM_PEAK_GBS, 4)
+    # requests that draw their tokens with the reference's command-line defaults, each from its own generator
+    drawing = dict(temperature=0.8, top_k=40, top_p=0.95, min_p=0.05)
+    for batch, steps in ((8, min(args.steps, 64)), (64, min(args.steps, 32))):
+        log(f"decode at batch {batch}, tokens drawn (temperature 0.8, top_k 40, top_p 0.95, min_p 0.05)")
+        seconds, _, _ = decode_run(torch, model, config, batch, steps, min(args.warmup, 8), sampling=drawing)
+        points[f"decode_b{batch}_drawn"] = round(batch * steps / seconds, 1)
     del model
     torch.cuda.empty_cache()
     long_context = 32768

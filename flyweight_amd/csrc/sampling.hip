@@ -319,7 +319,15 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
     double threshold = 0.0;
     unsigned long long moved_on = 0ull;
     int token = best_id;
-    for (int walk = 0; walk < 2; ++walk) {
+    // without cuts everything is kept: the kept sum is the sum over all candidates, and only the draw walks
+    // (with one batch the first walk costs less than a sum over the row)
+    const bool no_cuts = !(top_p < 1.0) && !(min_p > 0.0) && candidates > SAMPLE_BATCH;
+    if (no_cuts) {
+        unsigned long long floor_key = 0ull;
+        if (candidates < vocab) floor_key = sample_select(over_row, 0ull, ~0ull, (unsigned int)candidates, s);
+        mass_before = sample_total(row, vocab, floor_key, best_scaled, temperature, s);
+    }
+    for (int walk = no_cuts ? 1 : 0; walk < 2; ++walk) {
         unsigned long long ceiling = ~0ull;
         long long position = 0;
         const long long limit = walk == 0 ? candidates : keep;
