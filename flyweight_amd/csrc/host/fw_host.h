@@ -99,14 +99,16 @@ int fwh_scheduler_complete(void* scheduler, const int64_t* requests, const int* 
 // group_stride ints apart); returns the number of rows, or FWH_NOT_DECODE_ONLY and writes nothing.
 // fwh_scheduler_complete_ordered is fwh_scheduler_complete with the tokens given in the order
 // of the plan's segments that wanted logits.
-// fwh_plan_steps_ahead: how many further steps of this batch are certain to follow such a plan
-// whatever tokens are drawn (at most `limit`), but for requests that draw one of their stop
-// tokens: nobody waits for admission, and each request has that many tokens to go within its
-// budget and the context beyond the one this plan produces. A caller may then run those steps on
-// the device, feeding each step's tokens to the next, before it hands any of them over; a request
-// that ends at a stop token is missing from the plans after it (the others keep their order), and
-// the tokens its row went on to draw are dropped. requests: the plan's requests in row order
-// (optional).
+// fwh_plan_steps_ahead: how many further steps of this batch may follow such a plan before the
+// host looks again (at most `limit`): there is no place for a waiting request right now (no free
+// slot, or as many live requests as allowed), every request has that many positions left in the
+// context beyond the one this plan produces, and at least one request has that many tokens to go.
+// A caller may then run those steps on the device, feeding each step's tokens to the next, before
+// it hands any of them over, with fwh_scheduler_hold_admissions(steps) so that the plans it then
+// asks for are those steps. A request that ends on the way (a stop token, its last token) is
+// missing from the plans after it (the others keep their order), and the tokens its row went on to
+// draw are dropped; whoever waits is admitted by the first plan after the held ones. requests: the
+// plan's requests in row order (optional).
 #define FWH_NOT_DECODE_ONLY (-3)
 int fwh_plan_fill_decode(void* scheduler, int capacity, int* tokens, int* positions, int* slots, int table_stride,
                          int* tables, int group_stride);
@@ -117,6 +119,7 @@ int fwh_scheduler_complete_ordered(void* scheduler, const int* tokens, int count
 int fwh_request_info(void* scheduler, int64_t request, int info[9]);
 int fwh_request_generated(void* scheduler, int64_t request, int* tokens, int capacity);
 const char* fwh_request_error(void* scheduler, int64_t request);       // "" if none
+int fwh_scheduler_hold_admissions(void* scheduler, int plans);       // the next `plans` plans admit nobody
 int fwh_scheduler_forget(void* scheduler, int64_t request);            // drops a finished request's record
 
 #ifdef __cplusplus

@@ -38,7 +38,7 @@ int copy_ids(const std::vector<fwh::Request*>& from, int64_t* to) {
 extern "C" {
 
 const char* fwh_last_error(void) { return last_error.c_str(); }
-int fwh_abi_version(void) { return 2; }
+int fwh_abi_version(void) { return 3; }
 
 // ---- pools ---------------------------------------------------------------------------------
 void* fwh_pool_create(int size) {
@@ -297,16 +297,18 @@ int fwh_plan_steps_ahead(void* scheduler, int limit, int64_t* requests, int capa
         fwh::Scheduler* s = scheduler_of(scheduler);
         const fwh::Plan& plan = s->plan();
         if (plan.segments.empty() || !plan.preempted.empty() || !plan.failed.empty() || !plan.admitted.empty() ||
-            !plan.cancelled.empty() || !s->waiting().empty())
+            !plan.cancelled.empty() || s->place_for_admission())
             return 0;
-        int ahead = limit;
+        int ahead = limit, longest_budget = 0;
         for (const fwh::Segment& segment : plan.segments) {
             const fwh::Request* request = segment.request;
             if (segment.count != 1 || !segment.wants_logits || request->cancelled) return 0;
             const int budget = request->max_new_tokens - (int)request->generated.size() - 1;
             const int room = s->max_positions() - request->total() - 1;
-            ahead = std::min({ahead, budget, room});
+            longest_budget = std::max(longest_budget, budget);
+            ahead = std::min(ahead, room);
         }
+        ahead = std::min(ahead, longest_budget);       // no step in which nobody is left
         if (ahead < 0) ahead = 0;
         if (requests)
             for (size_t i = 0; i < plan.segments.size() && (int)i < capacity; ++i) requests[i] = plan.segments[i].request->id;
@@ -355,6 +357,10 @@ int fwh_request_generated(void* scheduler, int64_t request, int* tokens, int cap
 const char* fwh_request_error(void* scheduler, int64_t request) {
     const fwh::Request* r = scheduler_of(scheduler)->find(request);
     return r ? r->error.c_str() : "";
+}
+int fwh_scheduler_hold_admissions(void* scheduler, int plans) {
+    scheduler_of(scheduler)->hold_admissions(plans);
+    return 0;
 }
 int fwh_scheduler_forget(void* scheduler, int64_t request) { return scheduler_of(scheduler)->forget(request) ? 1 : 0; }
 

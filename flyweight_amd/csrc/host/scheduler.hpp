@@ -152,6 +152,13 @@ public:
         return true;
     }
     bool has_work() const { return !waiting_.empty() || !running_.empty(); }
+    // The next `plans` plans admit nobody: for a caller that has already run those steps on the
+    // device, with the requests that were running when it began.
+    void hold_admissions(int plans) { held_plans_ = plans > 0 ? plans : 0; }
+    // whether a waiting request could be admitted now as far as places go (slots, live requests)
+    bool place_for_admission() const {
+        return !waiting_.empty() && (int)running_.size() < max_live_ && cache_->slots().free_count() > 0;
+    }
     int preemptions() const { return preemptions_; }
     Request* find(int64_t id) {
         auto it = requests_.find(id);
@@ -192,8 +199,10 @@ public:
                 request->finished = true;
                 plan.cancelled.push_back(request);
             }
+        const bool admit = held_plans_ == 0;
+        if (held_plans_ > 0) --held_plans_;
         while (true) {
-            plan_once(plan);
+            plan_once(plan, admit);
             if (!plan.segments.empty() || running_.empty()) return plan;
             // every running request waits for pages and none can move
             if (running_.size() == 1) fail(running_[0], "out of cache pages: the request does not fit even alone", plan);
@@ -257,7 +266,7 @@ private:
         plan.preempted.push_back(victim);
     }
 
-    void plan_once(Plan& plan) {
+    void plan_once(Plan& plan, bool admit) {
         Cache& cache = *cache_;
         // 1. decode rows, oldest first; make room by preempting the newest
         for (Request* request : std::vector<Request*>(running_)) {
@@ -279,7 +288,7 @@ private:
         }
         // 3. admissions, in queue order, while everything a first portion needs is there;
         //    none in a step in which somebody had to give way
-        while (!waiting_.empty() && plan.preempted.empty() && plan.num_tokens < max_batch_tokens_ &&
+        while (admit && !waiting_.empty() && plan.preempted.empty() && plan.num_tokens < max_batch_tokens_ &&
                (int)running_.size() < max_live_ && cache.slots().free_count() > 0) {
             Request* request = waiting_.front();
             const int total = (int)request->prompt.size() + request->max_new_tokens;
@@ -320,6 +329,7 @@ private:
 
     Cache* cache_;
     int max_positions_, max_batch_tokens_, chunk_size_, max_live_, max_queued_, vocab_size_;
+    int held_plans_ = 0;
     std::deque<Request*> waiting_;
     std::vector<Request*> running_;         // in admission order, oldest first
     std::unordered_map<int64_t, std::unique_ptr<Request>> requests_;

@@ -225,23 +225,28 @@ class Runtime:
                     self._counters["decode_calls"] += counts[0] * len(tokens)
                     self._counters["decode_ns"] += time.perf_counter_ns() - began
                     events = scheduler.complete_ordered(tokens[0])
-                    # The steps that ran ahead: the scheduler makes the plan they ran by, then takes their
-                    # tokens. A request that ended on the way (a stop token) is missing from the later
-                    # plans, the others keep their order; what its row went on to draw is dropped.
+                    # The steps that ran ahead: the scheduler makes the plan they ran by (admitting nobody:
+                    # whoever waits comes in with the next turn), then takes their tokens. A request that
+                    # ended on the way (a stop token, its last token) is missing from the later plans, the
+                    # others keep their order; what its row went on to draw is dropped.
                     live = np.ones(counts[0], dtype=bool)
                     checked = 0
-                    for later in tokens[1:]:
-                        ended = {task for task, _, kind in events[checked:] if kind in (EVENT_FINISHED, EVENT_ERROR)}
-                        checked = len(events)
-                        if ended:
-                            live &= np.array([request not in ended for request in row_requests], dtype=bool)
-                        rows = int(live.sum())
-                        if rows == 0:
-                            break
-                        again = scheduler.plan_next()
-                        if again[0] != rows or again[1] != rows or any(again[2:6]):
-                            raise EngineError("the scheduler's plan differs from the decode steps that ran ahead of it")
-                        events.extend(scheduler.complete_ordered(np.ascontiguousarray(later[live])))
+                    scheduler.hold_admissions(len(tokens) - 1)
+                    try:
+                        for later in tokens[1:]:
+                            ended = {task for task, _, kind in events[checked:] if kind in (EVENT_FINISHED, EVENT_ERROR)}
+                            checked = len(events)
+                            if ended:
+                                live &= np.array([request not in ended for request in row_requests], dtype=bool)
+                            rows = int(live.sum())
+                            if rows == 0:
+                                break
+                            again = scheduler.plan_next()
+                            if again[0] != rows or again[1] != rows or any(again[2:6]):
+                                raise EngineError("the scheduler's plan differs from the decode steps that ran ahead of it")
+                            events.extend(scheduler.complete_ordered(np.ascontiguousarray(later[live])))
+                    finally:
+                        scheduler.hold_admissions(0)
                     return events
         plan = scheduler.read_plan(counts)
         sampled: Dict[int, int] = {}

@@ -234,6 +234,11 @@ class Scheduler:
             raise SchedulerError(host.last_error())
         return rows
 
+    def hold_admissions(self, plans: int) -> None:
+        """The next ``plans`` plans admit nobody (the steps they stand for have already run, with
+        the requests that were running); 0 ends the hold."""
+        self._lib.fwh_scheduler_hold_admissions(self._native, int(plans))
+
     def plan_requests(self, rows: int, tokens: Optional[int] = None):
         """The requests (ids) of the plan made last, in the order of its ``rows`` segments, which
         hold ``tokens`` tokens together (default: one each)."""
@@ -242,10 +247,11 @@ class Scheduler:
         return owners
 
     def steps_ahead(self, limit: int, rows: int):
-        """For a plain decode plan: how many further steps of this batch are certain to follow
-        whatever tokens are drawn (nobody waits, every request has the budget), at most ``limit``,
-        but for requests that draw a stop token: those are missing from the plans after it. And
-        the plan's requests (their ids) in row order."""
+        """For a plain decode plan: how many further steps of this batch may run before the host
+        looks again (no place for a waiting request right now, room in the context for every
+        request, tokens to go for at least one), at most ``limit``. Requests that end on the way
+        (a stop token, their last token) are missing from the plans after it. And the plan's
+        requests (their ids) in row order."""
         requests = host.ids(rows)
         ahead = self._lib.fwh_plan_steps_ahead(self._native, int(limit), requests, rows)
         if ahead < 0:

@@ -11,7 +11,7 @@ from .kernels.build import ensure_host_built
 
 ERROR, OUT_OF_PAGES, NO_PAGE = -1, -2, -1
 NOT_DECODE_ONLY = -3
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _LIB: Optional[ctypes.CDLL] = None
 _INTS, _IDS = POINTER(c_int), POINTER(c_int64)
@@ -67,6 +67,7 @@ _SIGNATURES = {
     "fwh_request_info": (c_int, [c_void_p, c_int64, _INTS]),
     "fwh_request_generated": (c_int, [c_void_p, c_int64, _INTS, c_int]),
     "fwh_request_error": (c_char_p, [c_void_p, c_int64]),
+    "fwh_scheduler_hold_admissions": (c_int, [c_void_p, c_int]),
     "fwh_scheduler_forget": (c_int, [c_void_p, c_int64]),
 }
 

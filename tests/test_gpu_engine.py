@@ -197,8 +197,8 @@ def test_engine_tasks_equal_blocking_generation_and_survive_preemption(loaded):
 def test_decode_steps_that_run_ahead_of_the_host_give_the_same_tokens(loaded, dtype):
     """With several decode steps per turn the device feeds each step's tokens to the next and
     the host reads them in bursts: the same tokens in the same order as one step per turn (float32:
-    the plain model's), bursts cut short by the shortest budget, across page edges, a request that stops on a token
-    in the middle of a burst, and no bursts while somebody still waits for a slot."""
+    the plain model's), bursts that go on past the requests that end in them (their last token, a stop token),
+    across page edges, and also while somebody waits for a slot that none of them has given up yet."""
     m = loaded("B", dtype)
     config, weights = m.plain_config, m.plain_weights
     prompts = [random_tokens(m.config.vocab_size, n, seed=40 + n) for n in (3, 60, 9, 30)]
@@ -235,7 +235,7 @@ def test_decode_steps_that_run_ahead_of_the_host_give_the_same_tokens(loaded, dt
         assert stopped[0] == single[0][:cut] and stopped[1:] == single[1:] and burst == 4
         for task_events in ([e for e in events if e[0] == task] for task in {e[0] for e in events}):
             assert task_events[-1][2] == 1 and all(e[2] != 1 for e in task_events[:-1])
-    # two slots for four requests: somebody waits until the last two run, only then steps run ahead
+    # two slots for four requests: the two that run do so in bursts while the others wait for their slots
     queued, burst, _ = run(4, parallel=2)
     assert burst == 4 and [len(tokens) for tokens in queued] == budgets
     if dtype == "float32":          # (in bfloat16 a prompt that runs beside other rows may round to another of two near-equal tokens)
@@ -258,7 +258,8 @@ def test_decode_steps_are_filled_up_to_the_sizes_that_are_kept(loaded, dtype):
         ids = [runtime.task_submit(p, n) for p, n in zip(prompts, budgets)]
         tokens = runtime.run()
         sizes = {batch for batch, _ in runtime.stepper._graphs}
-        assert {16, 8} <= sizes and not sizes & {9, 10, 11, 12, 13, 14, 15}, sizes
+        # (a turn of four steps goes on past the requests that end in it, so it need not meet every size)
+        assert 16 in sizes and (8 in sizes or steps_per_turn > 1) and not sizes & {9, 10, 11, 12, 13, 14, 15}, sizes
         runtime.stepper.cache.check_invariants()
         assert runtime.info["pages_free"] == runtime.num_pages and runtime.info["live_requests"] == 0
         # the same requests with every decode step at its exact size: rows are independent in every

@@ -311,33 +311,35 @@ def test_a_failure_between_two_plans_is_not_lost():
     assert scheduler.forget(b.id) and b.id not in scheduler.requests and not scheduler.forget(b.id)
 
 
-def test_steps_ahead_of_the_host_and_a_stop_token_in_the_middle_of_them():
-    """What a turn of several decode steps relies on: how many steps are certain to follow a plain
-    decode plan (the shortest budget, nobody waiting; a stop token does not forbid them), and
-    that a request which ends on the way is missing from the plans after it while the others keep
-    their rows' order."""
+def test_steps_ahead_of_the_host_and_requests_that_end_in_the_middle_of_them():
+    """What a turn of several decode steps relies on: how many steps may follow a plain decode plan
+    (room in the context, tokens to go for at least one request, no place for anybody who waits),
+    that a request which ends on the way (a stop token, its last token) is missing from the plans
+    after it while the others keep their rows' order, and that held plans admit nobody."""
     import numpy as np
-    cache, scheduler = make(num_pages=16, max_requests=4)
+    cache, scheduler = make(num_pages=16, max_requests=3)
     prompts = [[3, 4, 5], [9, 8], [20, 21, 22, 23]]
-    # the second request will stop at the third token it draws
+    # the second request will stop at the third token it draws, the third has seven tokens to draw
     stop = expected_tokens(prompts[1], 3)[2]
     assert stop not in expected_tokens(prompts[1], 2)
-    budgets = [30, 30, 12]
+    budgets = [30, 30, 7]
     requests = [scheduler.submit(p, n, stop_tokens=[stop] if i == 1 else []) for i, (p, n) in enumerate(zip(prompts, budgets))]
     plan = scheduler.schedule()                         # the prompts
     scheduler.complete(plan, {s.request.id: oracle(s.request.tokens) for s in plan.segments})
+    late = scheduler.submit([1, 2], 4)                  # every slot is taken: it waits
     counts = scheduler.plan_next()                      # a plain decode plan of three rows
     assert counts[0] == counts[1] == 3 and not any(counts[2:6])
     ahead, rows = scheduler.steps_ahead(7, 3)
     assert ahead == 7 and list(rows[:3]) == [r.id for r in requests]
-    assert scheduler.steps_ahead(100, 3)[0] == 12 - 1 - 1   # the shortest budget: one token drawn, one by this plan
-    # the device runs the turn on regardless of the stop token; the host then hands the steps over in order
+    assert scheduler.steps_ahead(100, 3)[0] == 30 - 1 - 1   # the longest budget: one token drawn, one by this plan
+    # the device runs the turn on whoever ends on the way; the host then hands the steps over in order
     sequences = [list(p) + expected_tokens(p, 1) for p in prompts]
     live = [True, True, True]
-    for step in range(1 + 4):
+    scheduler.hold_admissions(7)
+    for step in range(1 + 7):
         if step:
             counts = scheduler.plan_next()
-            assert counts[0] == counts[1] == sum(live) and not any(counts[2:6])
+            assert counts[0] == counts[1] == sum(live) and not any(counts[2:6]), "nobody is admitted while the turn is handed over"
         drawn = [oracle(sequence) for sequence in sequences]
         for sequence, token in zip(sequences, drawn):
             sequence.append(token)                      # every row goes on, whether its request still lives or not
@@ -348,10 +350,12 @@ def test_steps_ahead_of_the_host_and_a_stop_token_in_the_middle_of_them():
             if e[2] == EVENT_FINISHED:
                 live[[r.id for r in requests].index(e[0])] = False
         cache.check_invariants()
-    assert live == [True, False, True]
+    scheduler.hold_admissions(0)
+    assert live == [True, False, False] and not late.live
     assert requests[1].generated == expected_tokens(prompts[1], 30, stop=(stop,)) and len(requests[1].generated) == 3
-    assert requests[0].generated == expected_tokens(prompts[0], 6) and requests[2].generated == expected_tokens(prompts[2], 6)
-    # somebody waiting for a slot: no steps ahead
-    for _ in range(3):
-        scheduler.submit([1, 2], 4)
-    assert scheduler.plan_next()[0] and scheduler.steps_ahead(4, 4)[0] == 0
+    assert requests[2].generated == expected_tokens(prompts[2], 7)
+    assert requests[0].generated == expected_tokens(prompts[0], 9)
+    # the hold is over: who waited comes in, and while there is a place for somebody no steps run ahead
+    another = scheduler.submit([5, 6], 4)
+    counts = scheduler.plan_next()
+    assert counts[4] == 2 and late.live and another.live and scheduler.steps_ahead(4, 3)[0] == 0
