@@ -51,6 +51,7 @@ def log(text: str) -> None:
     print(f"[bench] {text}", file=sys.stderr, flush=True)
 
 
+DRAWING = dict(temperature=0.8, top_k=40, top_p=0.95, min_p=0.05)   # the reference's command-line defaults
 DECODE_STEPS_PER_TURN = 4      # decode steps the engine runs on the device before the host is asked again
 
 
@@ -244,7 +245,7 @@ def further_points(torch, args, points: dict) -> None:
         points[name] = round(batch * steps / seconds, 1)
         points[name + "_frac"] = round(step_bytes / (seconds / steps) / 1e9 / HBM_PEAK_GBS, 4)
     # requests that draw their tokens with the reference's command-line defaults, each from its own generator
-    drawing = dict(temperature=0.8, top_k=40, top_p=0.95, min_p=0.05)
+    drawing = DRAWING
     for batch, steps in ((8, min(args.steps, 64)), (64, min(args.steps, 32))):
         log(f"decode at batch {batch}, tokens drawn (temperature 0.8, top_k 40, top_p 0.95, min_p 0.05)")
         seconds, _, _ = decode_run(torch, model, config, batch, steps, min(args.warmup, 8), sampling=drawing)
@@ -282,6 +283,8 @@ def main() -> int:
     parser.add_argument("--skip-points", action="store_true", help="only the headline batch")
     parser.add_argument("--skip-further", action="store_true", help="without the points at further sizes")
     parser.add_argument("--only", choices=("decode", "prefill"), help="run one phase and print no JSON (for profiling)")
+    parser.add_argument("--drawn", action="store_true", help="with --only decode: the requests draw their tokens "
+                        "(temperature 0.8, top_k 40, top_p 0.95, min_p 0.05) instead of taking the most likely one")
     parser.add_argument("--workload", choices=("headline",) + tuple(WORKLOADS), default="headline",
                         help="headline: the LFM2-1.2B decode and prefill figures; the others: a whole serving run")
     parser.add_argument("--requests", type=int, help="requests of a serving workload (default: as the workload names)")
@@ -305,7 +308,7 @@ def main() -> int:
     model = Model.random(config, seed=0, dtype="bfloat16")
 
     if args.only == "decode":
-        elapsed, _, _ = decode_run(torch, model, config, args.batch, args.steps, args.warmup)
+        elapsed, _, _ = decode_run(torch, model, config, args.batch, args.steps, args.warmup, sampling=DRAWING if args.drawn else None)
         log(f"{args.batch * args.steps / elapsed:.1f} tokens/s")
         return 0
     log("prefill of 2,048 tokens")

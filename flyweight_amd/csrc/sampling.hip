@@ -9,11 +9,11 @@
 //
 // One workgroup of 1,024 threads per row. The sorted list is never made as a whole: candidates
 // come in batches of up to 1,024, the best that are below the last batch's smallest (a radix
-// select over the 64-bit keys: six passes over the row, counting in LDS), sorted in LDS, their p
-// formed by all threads, and one thread walks them in order with float64 sums, exactly as a
-// sequential program would. With top_k up to 1,024 (the usual case) that is one batch; a draw
-// over the whole vocabulary of a flat distribution takes as many batches as it walks through
-// (twice: once for the cuts and the kept sum, once for the draw).
+// select over the 64-bit keys: up to six passes over the row, counting in LDS), sorted in LDS,
+// their p formed by all threads, thread i holding candidate i and the running sums up to it (a
+// scan in a fixed order). With top_k up to 1,024 (the usual case) that is one batch, and up to 512
+// it is gathered without a select: everything at or above the k-th of the threads' own best. A
+// draw over the whole vocabulary of a flat distribution takes as many batches as it walks through.
 // A row whose temperature is 0 takes the best candidate and leaves its generator alone, so
 // greedy and sampled requests share one launch. Nothing is allocated; nothing crosses to the host.
 #include "fw_common.h"
@@ -293,20 +293,31 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
         sample_for_each(row, vocab, [&](float value, int id) { visit(candidate_key(value, id)); });
     };
 
-    // the sum over all candidates, which the shares of top_p are taken of
-    double total = 1.0;
+    // Up to 1,024 candidates are one batch. Everything at or above the bound is gathered at once; that
+    // is the wanted candidates and usually few more (only a row with very many equal values gives more
+    // than a batch holds: then the exact key of the last wanted candidate is selected first).
     bool first_batch_ready = false;
     int first_count = 0;
-    if (top_p < 1.0) {
-        if (candidates == vocab) {
-            total = sample_total(row, vocab, 0ull, best_scaled, temperature, s);
-        } else if (candidates <= SAMPLE_BATCH) {
+    if (candidates <= SAMPLE_BATCH) {
+        // (beyond half a batch the bound lies so low that what is above it seldom fits: 768 wanted of
+        // 65,536 evenly spread values leave some 1,400 above the 768th of the threads' best)
+        int count = 0;
+        const bool at_once = candidates <= SAMPLE_BATCH / 2;
+        if (at_once) count = sample_batch(row, vocab, bound, ~0ull, best_scaled, temperature, s);
+        if (!at_once || s.gathered > SAMPLE_BATCH) {
             const unsigned long long floor_key = sample_select(over_row, bound, ~0ull, (unsigned int)candidates, s);
-            first_count = sample_batch(row, vocab, floor_key, ~0ull, best_scaled, temperature, s);
-            first_batch_ready = true;
+            count = sample_batch(row, vocab, floor_key, ~0ull, best_scaled, temperature, s);
+        }
+        first_count = count < candidates ? count : (int)candidates;
+        first_batch_ready = true;
+    }
+    // the sum over all candidates, which the shares of top_p are taken of
+    double total = 1.0;
+    if (top_p < 1.0) {
+        if (first_batch_ready) {
             total = sample_running_sum((int)threadIdx.x < first_count ? s.p[threadIdx.x] : 0.0, s, true);
         } else {
-            const unsigned long long floor_key = sample_select(over_row, 0ull, ~0ull, (unsigned int)candidates, s);
+            const unsigned long long floor_key = candidates == vocab ? 0ull : sample_select(over_row, 0ull, ~0ull, (unsigned int)candidates, s);
             total = sample_total(row, vocab, floor_key, best_scaled, temperature, s);
         }
     }
@@ -352,10 +363,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
                 const unsigned int want = left < SAMPLE_BATCH ? (unsigned int)left : SAMPLE_BATCH;
                 const unsigned long long floor_key = sample_select(over_row, position == 0 ? bound : 0ull, ceiling, want, s);
                 count = sample_batch(row, vocab, floor_key, ceiling, best_scaled, temperature, s);
-                if (position == 0 && candidates <= SAMPLE_BATCH) {
-                    first_batch_ready = true;       // the only batch: the second walk finds it in LDS
-                    first_count = count;
-                }
             }
             if (count == 0) break;
             const int here = limit - position < count ? (int)(limit - position) : count;
