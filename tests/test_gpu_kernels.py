@@ -655,7 +655,7 @@ def test_attention_decode_on_the_matrix_cores(ops, nh, nkv, hd, window):
     again = ops.attention_decode(q, nh, nkv, hd, k_pages, v_pages, d(table), d(np.arange(rows)), d(positions), scale,
                                  max_context=1024, window=window)
     assert torch.equal(again, out)
-    # a row's result does not depend on the rest of the batch
+    # a row's result does not depend on the rest of the batch (of a batch so small that the keys are cut alike)
     alone = ops.attention_decode(q[5:6].contiguous(), nh, nkv, hd, k_pages, v_pages, d(table[5:6]), d([0]), d([positions[5]]),
                                  scale, max_context=lengths[5], window=window)
     assert torch.equal(alone[0], out[5])
