@@ -100,7 +100,7 @@ int fwh_scheduler_complete(void* scheduler, const int64_t* requests, const int* 
 // fwh_scheduler_complete_ordered is fwh_scheduler_complete with the tokens given in the order
 // of the plan's segments that wanted logits.
 // fwh_plan_steps_ahead: how many further steps of this batch may follow such a plan before the
-// host looks again (at most `limit`): there is no place for a waiting request right now (no free
+// host looks again (at most `limit`): the plan holds every running request, there is no place for a waiting request right now (no free
 // slot, or as many live requests as allowed), every request has that many positions left in the
 // context beyond the one this plan produces, and at least one request has that many tokens to go.
 // A caller may then run those steps on the device, feeding each step's tokens to the next, before

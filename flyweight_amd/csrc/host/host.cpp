@@ -297,8 +297,8 @@ int fwh_plan_steps_ahead(void* scheduler, int limit, int64_t* requests, int capa
         fwh::Scheduler* s = scheduler_of(scheduler);
         const fwh::Plan& plan = s->plan();
         if (plan.segments.empty() || !plan.preempted.empty() || !plan.failed.empty() || !plan.admitted.empty() ||
-            !plan.cancelled.empty() || s->place_for_admission())
-            return 0;
+            !plan.cancelled.empty() || s->place_for_admission() || plan.segments.size() != s->running().size())
+            return 0;       // (a running request that this plan leaves out, for want of pages or budget, may be in the next)
         int ahead = limit, longest_budget = 0;
         for (const fwh::Segment& segment : plan.segments) {
             const fwh::Request* request = segment.request;

@@ -604,3 +604,66 @@ def test_equal_logits_give_the_lowest_id_through_the_engine(folders, tmp_path, d
         if dtype == "float32":
             changed_config, changed = plain.read_folder(folder)
             assert plain.greedy(changed_config, changed, prompt, 1) == [expected]
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_a_random_load_under_every_setting_gives_each_request_what_it_gets_alone(loaded, seed):
+    """Forty requests (greedy ones, drawing ones, some with stop tokens, a few cancelled on the way)
+    arrive while others run, on few slots and so few pages that requests give way, in turns of one
+    and of four decode steps: every request that runs to its end gets the tokens it gets alone with
+    pages to spare (float32: nothing rounds differently), each has one last event, and the cache is
+    whole after every step and empty at the end."""
+    m = loaded("A", "float32")
+    rng = np.random.default_rng(100 + seed)
+    vocab = m.config.vocab_size
+    count = 40
+    prompts = [random_tokens(vocab, int(rng.integers(1, 90)), seed=500 + 50 * seed + i) for i in range(count)]
+    budgets = [int(rng.integers(1, 40)) for _ in range(count)]
+    settings = []
+    for i in range(count):
+        kind = int(rng.integers(0, 4))
+        drawn = {} if kind == 0 else dict(temperature=float(rng.choice([0.7, 1.0, 1.5])), top_k=int(rng.choice([0, 1, 5, 40])),
+                                          top_p=float(rng.choice([1.0, 0.9, 0.5])), min_p=float(rng.choice([0.0, 0.1])), seed=1000 + i)
+        settings.append(drawn)
+    alone = _runtime(m, parallel_sequences=1, prefill_rows=64)
+    wanted = [alone.generate(p, n, **kw) for p, n, kw in zip(prompts, budgets, settings)]
+    # a stop token for every third request: a token it will draw, where it draws one more than once
+    stops = [(wanted[i][len(wanted[i]) // 2],) if i % 3 == 0 and len(wanted[i]) > 2 else () for i in range(count)]
+    for i, stop in enumerate(stops):
+        if stop:
+            wanted[i] = wanted[i][:wanted[i].index(stop[0]) + 1]
+    cancel_at = {int(i): int(rng.integers(1, 6)) for i in rng.choice(count, 4, replace=False)}
+    gave_way = 0
+    for steps_per_turn in (1, 4):
+        runtime = _runtime(m, parallel_sequences=5, num_pages=6, prefill_rows=32, max_batch_tokens=48, decode_steps_per_turn=steps_per_turn)
+        todo = list(range(count))
+        ids, got, last, seen_tokens = {}, {}, {}, {}
+        engine_steps = 0
+        while todo or runtime.scheduler.has_work():
+            for _ in range(int(rng.integers(0, 3))):
+                if todo:
+                    i = todo.pop(0)
+                    ids[runtime.task_submit(prompts[i], budgets[i], stop_tokens=stops[i], **settings[i])] = i
+            for task, i in ids.items():
+                if i in cancel_at and seen_tokens.get(i, 0) >= cancel_at[i] and task not in last:
+                    runtime.task_cancel(task)
+            for task, value, kind in runtime.engine_step():
+                i = ids[task]
+                assert task not in last, "an event behind a request's last one"
+                if kind == 0:
+                    got.setdefault(i, []).append(value)
+                    seen_tokens[i] = seen_tokens.get(i, 0) + 1
+                elif kind in (1, 2):
+                    last[task] = kind
+            runtime.stepper.cache.check_invariants()
+            engine_steps += 1
+            assert engine_steps < 5000, "the load does not come to an end"
+        assert len(last) == count and all(kind == 1 for kind in last.values())
+        assert runtime.info["pages_free"] == runtime.num_pages and runtime.info["live_requests"] == 0
+        gave_way += runtime.info["preemptions"]
+        for i in range(count):
+            if i in cancel_at:
+                assert got.get(i, []) == wanted[i][:len(got.get(i, []))] and len(got.get(i, [])) >= min(cancel_at[i], len(wanted[i]))
+            else:
+                assert got.get(i, []) == wanted[i], (i, settings[i], stops[i])
+    assert gave_way > 0, "the pages were meant to run out"
