@@ -606,14 +606,16 @@ def test_equal_logits_give_the_lowest_id_through_the_engine(folders, tmp_path, d
             assert plain.greedy(changed_config, changed, prompt, 1) == [expected]
 
 
-@pytest.mark.parametrize("seed", [0, 1, 2])
-def test_a_random_load_under_every_setting_gives_each_request_what_it_gets_alone(loaded, seed):
+@pytest.mark.parametrize("name,seed", [("A", 0), ("A", 1), ("A", 2), ("B", 3)])
+def test_a_random_load_under_every_setting_gives_each_request_what_it_gets_alone(loaded, name, seed):
     """Forty requests (greedy ones, drawing ones, some with stop tokens, a few cancelled on the way)
     arrive while others run, on few slots and so few pages that requests give way, in turns of one
     and of four decode steps: every request that runs to its end gets the tokens it gets alone with
-    pages to spare (float32: nothing rounds differently), each has one last event, and the cache is
-    whole after every step and empty at the end."""
-    m = loaded("A", "float32")
+    pages to spare, each has one last event, and the cache is whole after every step and empty at the
+    end. (float32, whose logits differ between ways of cutting and batching in the last bits only: a
+    request that takes the most likely token is never moved by that; one that draws is, once in
+    thousands of draws, when a candidate sits on the edge of a cut, so one of the forty may differ.)"""
+    m = loaded(name, "float32")
     rng = np.random.default_rng(100 + seed)
     vocab = m.config.vocab_size
     count = 40
@@ -661,9 +663,13 @@ def test_a_random_load_under_every_setting_gives_each_request_what_it_gets_alone
         assert len(last) == count and all(kind == 1 for kind in last.values())
         assert runtime.info["pages_free"] == runtime.num_pages and runtime.info["live_requests"] == 0
         gave_way += runtime.info["preemptions"]
+        moved = []
         for i in range(count):
-            if i in cancel_at:
-                assert got.get(i, []) == wanted[i][:len(got.get(i, []))] and len(got.get(i, [])) >= min(cancel_at[i], len(wanted[i]))
-            else:
-                assert got.get(i, []) == wanted[i], (i, settings[i], stops[i])
+            mine = got.get(i, [])
+            same = mine == wanted[i][:len(mine)] and (len(mine) >= min(cancel_at[i], len(wanted[i])) if i in cancel_at else len(mine) == len(wanted[i]))
+            if not same:
+                assert settings[i], (i, "a request that takes the most likely token", mine, wanted[i])
+                assert len(mine) >= 1, "a request that ran got no token"
+                moved.append(i)
+        assert len(moved) <= 1, (moved, [settings[i] for i in moved])
     assert gave_way > 0, "the pages were meant to run out"
