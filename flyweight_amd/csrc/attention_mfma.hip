@@ -403,6 +403,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
 }
 
 // ---- decode ------------------------------------------------------------------------------------
+#define DECODE_WORKGROUPS 512        // two per compute unit: beyond, longer splits serve better than more of them
 // grid (rows, kv heads * head tiles, splits); four waves, each takes one page of the split's
 // SPLIT_PAGES, and their results are merged in LDS in the order of the keys. Columns are the
 // query heads of the kv group (16 per head tile). partial [rows][heads][max_splits][head_dim + 4]:
@@ -470,7 +471,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, float* partial, int* tickets,
     uint16_t* k_pages, uint16_t* v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ row_seg, const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads,
-    int head_dim, float scale_log2, int window, int max_splits, int rounds, const FusedProjections fused) {
+    int head_dim, float scale_log2, int window, int max_splits, const int32_t* __restrict__ decode_work, const FusedProjections fused) {
     __shared__ f32x4 shared_o[SPLIT_PAGES][HD / 16][64];
     __shared__ float shared_m[SPLIT_PAGES][16], shared_l[SPLIT_PAGES][16];
     __shared__ int ticket_shared;
@@ -484,8 +485,18 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     const int pos = row_pos[row];
     const int segment = row_seg[row];       // asked for together with the position, not behind the branch below
     const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
-    // splits are counted from the first page that holds a visible key; a split is `rounds` runs of
-    // SPLIT_PAGES pages (a long context of few rows: fewer, longer splits, and fewer parts to merge)
+    // Splits are counted from the first page that holds a visible key; a split is `rounds` runs of
+    // SPLIT_PAGES pages. One run each serves while the step's runs (decode_work: over all its rows;
+    // times the kv heads and head tiles) are no more than about two workgroups per compute unit;
+    // beyond, fewer and longer workgroups read the cache faster, and a row has fewer parts to merge (one
+    // workgroup for a whole row needs no merge at all). Counting the step's work, not the row's, gives
+    // a long row among short ones its share of the chip.
+    int rounds = 1;
+    if (decode_work) {
+        const long long workgroups = (long long)decode_work[0] * gridDim.y;
+        rounds = (int)(workgroups / DECODE_WORKGROUPS);
+        rounds = rounds < 1 ? 1 : rounds;
+    }
     const int pages_per_split = SPLIT_PAGES * rounds;
     const int first_block = first / PAGE + split * pages_per_split;
     const int last_block = pos / PAGE;
@@ -722,6 +733,8 @@ static int decode_check(int max_splits, int max_context, int* tickets, int ticke
     FW_REQUIRE(max_context >= 1, "attention_decode: max_context must be positive");
     int blocks = (max_context + PAGE - 1) / PAGE;
     if (window > 0 && (window + PAGE - 2) / PAGE + 1 < blocks) blocks = (window + PAGE - 2) / PAGE + 1;
+    FW_REQUIRE(max_splits * SPLIT_PAGES >= blocks, "attention_decode: %d splits of %d pages do not cover %d pages of context",
+               max_splits, SPLIT_PAGES, blocks);
     FW_REQUIRE((max_context + PAGE - 1) / PAGE <= table_stride, "attention_decode: a context of %d tokens exceeds the block table (%d pages)",
                max_context, table_stride);
     const int head_tiles = (num_heads / num_kv_heads + 15) / 16;
@@ -731,26 +744,23 @@ static int decode_check(int max_splits, int max_context, int* tickets, int ticke
     return 0;
 }
 
-static int decode_launch(const void* q, void* out, float* partial, int max_splits, int max_context, int* tickets, void* k_pages, void* v_pages,
+static int decode_launch(const void* q, void* out, float* partial, int max_splits, const int32_t* decode_work, int* tickets, void* k_pages, void* v_pages,
                          const int32_t* block_table, int table_stride, const int32_t* row_seg, const int32_t* row_pos, int rows,
                          int num_heads, int num_kv_heads, int head_dim, float scale, int window, const FusedProjections& fused,
                          void* stream) {
     if (rows == 0) return 0;
     const int head_tiles = (num_heads / num_kv_heads + 15) / 16;
     dim3 grid(rows, num_kv_heads * head_tiles, max_splits);
-    // the pages a row can see, shared out over the splits in runs of SPLIT_PAGES
-    int blocks = (max_context + PAGE - 1) / PAGE;
-    if (window > 0 && (window + PAGE - 2) / PAGE + 1 < blocks) blocks = (window + PAGE - 2) / PAGE + 1;
-    const int rounds = (blocks + max_splits * SPLIT_PAGES - 1) / (max_splits * SPLIT_PAGES);
+
 #define CALL(HD)                                                                                                              \
     if (fused.qkv)                                                                                                            \
         attention_decode_split_kernel<HD, true><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                          \
             (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
-            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits, rounds, fused); \
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits, decode_work, fused); \
     else                                                                                                                      \
         attention_decode_split_kernel<HD, false><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                         \
             (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
-            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits, rounds, fused)
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, scale * LOG2E, window, max_splits, decode_work, fused)
     FW_BY_HEAD_DIM(head_dim, CALL);
 #undef CALL
     FW_LAUNCH_CHECK("attention_decode");
@@ -758,20 +768,22 @@ static int decode_launch(const void* q, void* out, float* partial, int max_split
 }
 
 // One row per request. partial: float32 workspace of rows * heads * max_splits * (head_dim + 4).
-// max_context: no row's position reaches it (the caller knows; the kernel cannot check); the
-// pages such a row sees are shared out over max_splits workgroups in runs of 4 pages (as many runs
-// each as it takes: few rows of a long context do better with fewer, longer splits). tickets: rows * kv heads *
+// max_context: no row's position reaches it (the caller knows; the kernel cannot check);
+// max_splits must cover the keys such a row sees, in runs of 4 pages. decode_work: null, or one
+// int32 on the device: the runs of 4 pages that all the rows of the step see together (the sum over
+// the rows of ceil((position + 1) / 256)); with it a workgroup takes as many runs as bring the step
+// down to about 512 workgroups (it changes how the work is shared out, not what is computed). tickets: rows * kv heads *
 // ceil(group / 16) int32 counters, zero before the first call and left zero; calls that overlap on
 // one device need their own (and their own workspace).
 extern "C" int fw_attention_decode(const void* q, void* out, float* partial, int max_splits, int max_context,
-                                   int* tickets, int tickets_len, const void* k_pages,
+                                   const int32_t* decode_work, int* tickets, int tickets_len, const void* k_pages,
                                    const void* v_pages, const int32_t* block_table, int table_stride,
                                    const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                                    int num_kv_heads, int head_dim, float scale, int window, int page_size,
                                    int num_pages, void* stream) {
     if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, window,
                      page_size, num_pages)) return -1;
-    return decode_launch(q, out, partial, max_splits, max_context, tickets, const_cast<void*>(k_pages), const_cast<void*>(v_pages), block_table,
+    return decode_launch(q, out, partial, max_splits, decode_work, tickets, const_cast<void*>(k_pages), const_cast<void*>(v_pages), block_table,
                          table_stride, row_seg, row_pos, rows, num_heads, num_kv_heads, head_dim, scale, window, FusedProjections{}, stream);
 }
 
@@ -782,7 +794,7 @@ extern "C" int fw_attention_decode(const void* q, void* out, float* partial, int
 // (null with rotary_dim 0). Results as the two kernels one after the other give them.
 extern "C" int fw_attention_decode_fused(const float* qkv, const float* q_norm_weight, const float* k_norm_weight, float eps,
                                          const float* cos_table, const float* sin_table, int rotary_dim, int write_kv, void* out,
-                                         float* partial, int max_splits, int max_context, int* tickets, int tickets_len,
+                                         float* partial, int max_splits, int max_context, const int32_t* decode_work, int* tickets, int tickets_len,
                                          void* k_pages, void* v_pages, const int32_t* block_table, int table_stride,
                                          const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                                          int num_kv_heads, int head_dim, float scale, int window, int page_size, int num_pages,
@@ -797,6 +809,6 @@ extern "C" int fw_attention_decode_fused(const float* qkv, const float* q_norm_w
     FusedProjections fused;
     fused.qkv = qkv; fused.q_norm_weight = q_norm_weight; fused.k_norm_weight = k_norm_weight; fused.eps = eps;
     fused.cos_table = cos_table; fused.sin_table = sin_table; fused.rotary_dim = rotary_dim; fused.write_kv = write_kv;
-    return decode_launch(nullptr, out, partial, max_splits, max_context, tickets, k_pages, v_pages, block_table, table_stride, row_seg, row_pos,
+    return decode_launch(nullptr, out, partial, max_splits, decode_work, tickets, k_pages, v_pages, block_table, table_stride, row_seg, row_pos,
                          rows, num_heads, num_kv_heads, head_dim, scale, window, fused, stream);
 }

@@ -148,9 +148,11 @@ int fw_attention_prefill(const void* q, void* out, const void* k_pages, const vo
 // merged in order by the workgroup that finishes last. partial: float32 workspace
 // [rows][heads][max_splits][head_dim + 4]; max_context: an upper bound on position + 1 of every
 // row, known to the caller; tickets: rows * kv_heads * ceil(heads / kv_heads / 16) int32 counters,
-// zero before the first call and left zero.
+// zero before the first call and left zero. decode_work: null, or one int32 on the device, the runs
+// of 4 pages that all the rows of the step see together; with it a workgroup takes as many runs as
+// bring the step down to about 512 workgroups.
 int fw_attention_decode(const void* q, void* out, float* partial, int max_splits, int max_context,
-                        int* tickets, int tickets_len, const void* k_pages, const void* v_pages, const int32_t* block_table, int table_stride,
+                        const int32_t* decode_work, int* tickets, int tickets_len, const void* k_pages, const void* v_pages, const int32_t* block_table, int table_stride,
                         const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
                         int head_dim, float scale, int window, int page_size, int num_pages, void* stream);
 
@@ -160,7 +162,8 @@ int fw_attention_decode(const void* q, void* out, float* partial, int max_splits
 // the new key (normed, rotated) and value (write_kv 0: they are in the cache already).
 int fw_attention_decode_fused(const float* qkv, const float* q_norm_weight, const float* k_norm_weight, float eps,
                               const float* cos_table, const float* sin_table, int rotary_dim, int write_kv, void* out,
-                              float* partial, int max_splits, int max_context, int* tickets, int tickets_len, void* k_pages,
+                              float* partial, int max_splits, int max_context, const int32_t* decode_work, int* tickets,
+                              int tickets_len, void* k_pages,
                               void* v_pages, const int32_t* block_table, int table_stride, const int32_t* row_seg,
                               const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim, float scale,
                               int window, int page_size, int num_pages, void* stream);

@@ -99,7 +99,8 @@ class StepContext:
     encodings, and whatever index arrays the model's parts ask for (``Part.step_arrays``: built
     on the host from the batch, they travel in the same upload)."""
 
-    FIXED = 6       # tokens, positions, segment of each row, first row of each segment, slots, wanted rows
+    FIXED = 7       # tokens, positions, segment of each row, first row of each segment, slots, wanted rows, decode work
+    RUN_OF_KEYS = 256       # decode attention shares a row's keys out in runs of four pages
 
     def __init__(self, entries: Sequence[StepEntry], cache: CacheManager, device: torch.device, vocab_size: int,
                  max_positions: int, described=None, providers: Sequence = ()):
@@ -148,7 +149,11 @@ class StepContext:
         self.host_seg_slot = seg_slot
 
         tables = [cache.block_table_rows(g, self.requests, natives=natives) for g in range(len(cache.groups))]
-        pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows)]
+        # how many runs of keys the rows that go to the decode kernels see together: those kernels share
+        # the work out over the chip by it (a long row among short ones gets more workgroups)
+        single = self.num_rows if self.all_decode else self.decode_prefix
+        decode_work = [int(np.sum((row_pos[:single].astype(np.int64) + self.RUN_OF_KEYS) // self.RUN_OF_KEYS))]
+        pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows, decode_work)]
         pieces += [t.reshape(-1) for t in tables]
         if given_positions:
             pieces.append(np.concatenate(encoding_parts))
@@ -160,7 +165,7 @@ class StepContext:
         for piece in pieces:
             views.append(packed[offset:offset + piece.size])
             offset += piece.size
-        self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows = views[:self.FIXED]
+        self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows, self.decode_work = views[:self.FIXED]
         self.block_tables = [v.view(t.shape) for v, t in zip(views[self.FIXED:], tables)]
         at = self.FIXED + len(tables)
         # what the position encodings see: the places in the sequences, unless the entries say otherwise
@@ -213,7 +218,7 @@ class StepContext:
         self.host_seg_slot = [0] * batch
         extra = self._ask(providers)
         self.host_row_pos = self.host_seg_row0 = self.host_seg_slot = None     # not for captured steps
-        sizes = [batch, batch, batch, batch + 1, batch, batch] + [batch * table_stride] * groups
+        sizes = [batch, batch, batch, batch + 1, batch, batch, 1] + [batch * table_stride] * groups
         sizes += [array.size for _, _, array in extra]
         self.host_buffer = torch.empty(max(sum(sizes), 1), dtype=torch.int32, pin_memory=True)
         self.device_buffer = torch.zeros(max(sum(sizes), 1), dtype=torch.int32, device=device)
@@ -222,7 +227,7 @@ class StepContext:
             views.append(self.device_buffer[offset:offset + size])
             host_views.append(self.host_buffer[offset:offset + size].numpy())
             offset += size
-        self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows = views[:cls.FIXED]
+        self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows, self.decode_work = views[:cls.FIXED]
         self.encoding_pos = self.row_pos
         self.block_tables = [v.view(batch, table_stride) for v in views[cls.FIXED:cls.FIXED + groups]]
         self._host = host_views
@@ -254,6 +259,7 @@ class StepContext:
         host[0][:] = [int(e.tokens[0]) for e in entries]
         host[1][:] = starts
         host[4][:] = slots
+        self._count_decode_work()
         for g, rows in enumerate(self._host_tables):
             rows[:] = cache.block_table_rows(g, self.requests, stride=self._table_stride, natives=natives).reshape(-1)
         self.upload()
@@ -284,7 +290,12 @@ class StepContext:
         if rows < 0:
             return -1
         self.fill_up(rows, cache)
+        self._count_decode_work()
         return rows
+
+    def _count_decode_work(self) -> None:
+        host = self._host
+        host[6][0] = int(np.sum((host[1].astype(np.int64) + self.RUN_OF_KEYS) // self.RUN_OF_KEYS))
 
     def fill_up(self, rows: int, cache: CacheManager) -> None:
         """Rows behind the plan's (a step recorded for more requests than the plan has): token 0

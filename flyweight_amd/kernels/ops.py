@@ -19,7 +19,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _lib = None
 
@@ -810,26 +810,12 @@ def query_tiles(seg_row0):
     return tile_seg, tile_row0
 
 
-DECODE_WORKGROUPS = 512        # two per compute unit: beyond, longer splits serve better than more of them
-
-
-def decode_splits(max_context: int, window: int = 0, rows: int = 1, groups: int = 1) -> int:
-    """Into how many workgroups the keys that a row sees are cut, for ``rows`` rows of ``groups`` kv
-    heads (or tiles of 16 query heads) each: runs of 4 pages, one run each, while that gives no more
-    than 512 workgroups; beyond, as many runs each as bring the step down to about 512, down to one
-    workgroup per row and group, which then needs no merge at all. Measured (16 heads in 8 groups of
-    64 channels): 64 rows of 2,112 keys 51 vs 62 us, of 32,768 keys 689 vs 985 us; 256 rows of 2,112
-    keys 195 vs 266 us; 8 rows of 32,768 keys 96 vs 136 us; 1 row of 131,072 keys 56 vs 100 us.
-    The order in which a row's keys are summed then depends on the size of the batch, as the
-    products' does."""
+def decode_splits(max_context: int, window: int = 0) -> int:
+    """Into how many workgroups at most the keys that a row sees are cut: runs of 4 pages."""
     blocks = (max_context + PAGE_SIZE - 1) // PAGE_SIZE
     if window > 0:
         blocks = min(blocks, (window + PAGE_SIZE - 2) // PAGE_SIZE + 1)
-    runs_of_pages = max(1, (blocks + DECODE_SPLIT_PAGES - 1) // DECODE_SPLIT_PAGES)
-    wanted = max(1, -(-DECODE_WORKGROUPS // max(1, rows * groups)))
-    parts = min(runs_of_pages, wanted)
-    runs_each = -(-runs_of_pages // parts)
-    return -(-runs_of_pages // runs_each)
+    return max(1, (blocks + DECODE_SPLIT_PAGES - 1) // DECODE_SPLIT_PAGES)
 
 
 def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
@@ -860,10 +846,23 @@ def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     return out
 
 
+def _work(decode_work: Optional[torch.Tensor]):
+    if decode_work is not None:
+        _dev(decode_work)
+        _want(decode_work, torch.int32, "decode_work")
+        if decode_work.numel() < 1:
+            raise KernelError("attention_decode: decode_work holds one int32")
+    return _p(decode_work)
+
+
 def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                      v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
-                     scale: float, max_context: int, window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """One row per request; ``max_context`` bounds position + 1 of every row (the host knows it)."""
+                     scale: float, max_context: int, window: int = 0, out: Optional[torch.Tensor] = None,
+                     decode_work: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One row per request; ``max_context`` bounds position + 1 of every row (the host knows it).
+    ``decode_work``: one int32 on the device, the runs of 4 pages that the rows see together (the
+    sum of ceil((position + 1) / 256)): the kernel shares the work out by it (fewer, longer
+    workgroups once there are more than about 512); without it, one run per workgroup."""
     _dev(q, k_pages, v_pages, block_table, row_seg, row_pos)
     _want(q, torch.bfloat16, "q")
     rows = q.shape[0]
@@ -874,7 +873,7 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("attention: batch index arrays are too short")
-    splits = decode_splits(max_context, window, rows, num_kv_heads * (-(-(num_heads // num_kv_heads) // 16)))
+    splits = decode_splits(max_context, window)
     partial = torch.empty((rows, num_heads, splits, head_dim + 4), dtype=torch.float32, device=q.device)
     if out is None:
         out = torch.empty_like(q)
@@ -883,7 +882,7 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
     group = num_heads // num_kv_heads
     tickets = _medium_counters(q.device, rows * num_kv_heads * ((group + 15) // 16))
     _check(library().fw_attention_decode(
-        _p(q), _p(out), _p(partial), splits, int(max_context), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages),
+        _p(q), _p(out), _p(partial), splits, int(max_context), _work(decode_work), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages),
         _p(block_table),
         block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale),
         int(window), PAGE_SIZE, pages, _stream()))
@@ -894,7 +893,8 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
                            q_norm_weight: Optional[torch.Tensor], k_norm_weight: Optional[torch.Tensor], eps: float,
                            cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rotary_dim: int, k_pages: torch.Tensor,
                            v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
-                           scale: float, max_context: int, window: int = 0, write_kv: bool = True) -> torch.Tensor:
+                           scale: float, max_context: int, window: int = 0, write_kv: bool = True,
+                           decode_work: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One row per request, from the step's raw projections ``qkv`` (float32 [rows, (heads + 2 kv
     heads) * head_dim]): per-head norm and rotation of queries and keys, the new keys and values
     into their pages, and the split-key attention, in one kernel. Returns bfloat16 [rows, heads *
@@ -919,14 +919,14 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("attention: batch index arrays are too short")
-    splits = decode_splits(max_context, window, rows, num_kv_heads * (-(-(num_heads // num_kv_heads) // 16)))
+    splits = decode_splits(max_context, window)
     partial = torch.empty((rows, num_heads, splits, head_dim + 4), dtype=torch.float32, device=qkv.device)
     out = torch.empty((rows, num_heads * head_dim), dtype=torch.bfloat16, device=qkv.device)
     group = num_heads // num_kv_heads
     tickets = _medium_counters(qkv.device, rows * num_kv_heads * ((group + 15) // 16))
     _check(library().fw_attention_decode_fused(
         _p(qkv), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin), int(rotary_dim), int(write_kv), _p(out),
-        _p(partial), splits, int(max_context), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages), _p(block_table),
+        _p(partial), splits, int(max_context), _work(decode_work), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages), _p(block_table),
         block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, ctypes.c_float(scale), int(window),
         PAGE_SIZE, pages, _stream()))
     return out
@@ -950,7 +950,7 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
     fast = q.dtype == torch.bfloat16 and attention_is_tiled(head_dim)
     if fast and ctx.all_decode:
         return attention_decode(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                                ctx.row_pos, scale, ctx.max_context, window)
+                                ctx.row_pos, scale, ctx.max_context, window, decode_work=getattr(ctx, "decode_work", None))
     if fast:
         if tile_seg is None or tile_row0 is None:
             raise KernelError("attention: the tiled kernel needs the step's query tiles")
@@ -966,7 +966,7 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                                      tile_row0, ctx.seg_row0, ctx.row_pos, scale, window, heads_together=together)
         out = torch.empty_like(q)
         attention_decode(q[:single], num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                         ctx.row_pos, scale, ctx.max_context, window, out=out[:single])
+                         ctx.row_pos, scale, ctx.max_context, window, out=out[:single], decode_work=getattr(ctx, "decode_work", None))
         return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table,
                                  tile_seg[single:], tile_row0[single:], ctx.seg_row0, ctx.row_pos, scale, window,
                                  heads_together=together, out=out)

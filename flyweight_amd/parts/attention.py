@@ -120,7 +120,8 @@ class GQAttention(Mixer):
             attended = ops.attention_decode_fused(
                 qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight, self.qk_norm_eps,
                 cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table, ctx.row_seg, ctx.row_pos,
-                self.scale, ctx.max_context, int(self.window or 0), write_kv=cache.writes)
+                self.scale, ctx.max_context, int(self.window or 0), write_kv=cache.writes,
+                decode_work=getattr(ctx, "decode_work", None))
             return self.out.accumulate(attended, residual, then=getattr(ctx, "upcoming_norm", None))
         q = ops.qk_norm_rope_kv_write(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight,

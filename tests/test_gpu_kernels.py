@@ -655,7 +655,12 @@ def test_attention_decode_on_the_matrix_cores(ops, nh, nkv, hd, window):
     again = ops.attention_decode(q, nh, nkv, hd, k_pages, v_pages, d(table), d(np.arange(rows)), d(positions), scale,
                                  max_context=1024, window=window)
     assert torch.equal(again, out)
-    # a row's result does not depend on the rest of the batch (of a batch so small that the keys are cut alike)
+    # however the work is shared out, the result is the reference's: one run of pages per workgroup, a few, all
+    for work in (1, 40, 700, 5000, 1 << 20):
+        shared = ops.attention_decode(q, nh, nkv, hd, k_pages, v_pages, d(table), d(np.arange(rows)), d(positions), scale,
+                                      max_context=1024, window=window, decode_work=d([work]))
+        close(shared, want, torch.bfloat16)
+    # a row's result does not depend on the rest of the batch
     alone = ops.attention_decode(q[5:6].contiguous(), nh, nkv, hd, k_pages, v_pages, d(table[5:6]), d([0]), d([positions[5]]),
                                  scale, max_context=lengths[5], window=window)
     assert torch.equal(alone[0], out[5])
@@ -666,7 +671,7 @@ def test_attention_decode_on_the_matrix_cores(ops, nh, nkv, hd, window):
         partial = torch.empty(rows * nh * (hd + 4), device=DEV)
         status = ops.library().fw_attention_decode(
             ctypes.c_void_p(q.data_ptr()), ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(partial.data_ptr()), 1, 100000,
-            None, 0, ctypes.c_void_p(k_pages.data_ptr()), ctypes.c_void_p(v_pages.data_ptr()), ctypes.c_void_p(d(table).data_ptr()),
+            None, None, 0, ctypes.c_void_p(k_pages.data_ptr()), ctypes.c_void_p(v_pages.data_ptr()), ctypes.c_void_p(d(table).data_ptr()),
             table.shape[1], ctypes.c_void_p(d(np.arange(rows)).data_ptr()), ctypes.c_void_p(d(positions).data_ptr()), rows, nh,
             nkv, hd, ctypes.c_float(scale), 0, 64, 40, None)
         ops._check(status)
