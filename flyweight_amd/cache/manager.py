@@ -149,10 +149,23 @@ class CacheManager:
         self.spare_slot = max_requests
         # storage: each need allocates its own
         self.storage: Dict[int, object] = {}
+        self._state_together: List[Tuple[CacheNeed, object]] = []   # (need, what stands for its entries' storages)
         if device is not None:
             for entry, need in self.needs.items():
-                units = (num_pages if need.paged else max_requests) + 1
-                self.storage[entry] = need.allocate(units, page_size, dtype, device)
+                if need.paged:
+                    self.storage[entry] = need.allocate(num_pages + 1, page_size, dtype, device)
+            alike: List[Tuple[CacheNeed, List[int]]] = []       # fixed-size entries whose needs are equal
+            for entry, need in self.state_entries.items():
+                for other, entries in alike:
+                    if type(other) is type(need) and other == need:
+                        entries.append(entry)
+                        break
+                else:
+                    alike.append((need, [entry]))
+            for need, entries in alike:
+                storages, together = need.allocate_together(len(entries), max_requests + 1, page_size, dtype, device)
+                self.storage.update(zip(entries, storages))
+                self._state_together.append((need, together))
 
     def view(self, entry: int, block_table=None, writes: bool = True):
         """What the mixer that uses cache entry ``entry`` sees of it."""
@@ -237,9 +250,8 @@ class CacheManager:
     def start_slot(self, slot: int) -> None:
         """A slot's state is what a request starts with (zero, unless the need says otherwise)
         for the request that takes it."""
-        for entry, need in self.state_entries.items():
-            if entry in self.storage:
-                need.initial(self.storage[entry], slot)
+        for need, together in self._state_together:
+            need.initial_together(together, slot)
 
     def slot_of(self, request: Hashable) -> int:
         slot = self._lib.fwh_cache_slot_of(self._native, self._live_id(request))

@@ -48,6 +48,18 @@ class CacheNeed:
     def initial(self, storage: Any, slot: int) -> None:
         """Fixed-size needs: put slot ``slot`` into the state a request starts with."""
 
+    def allocate_together(self, count: int, units: int, page_size: int, dtype: torch.dtype, device: torch.device):
+        """Fixed-size needs: the storages of ``count`` cache entries whose needs equal this one, and
+        an object that stands for all of them (``initial_together`` gets it). A need that can
+        start a slot of all its entries with one launch overrides both; as they stand they go
+        entry by entry."""
+        storages = [self.allocate(units, page_size, dtype, device) for _ in range(count)]
+        return storages, storages
+
+    def initial_together(self, together: Any, slot: int) -> None:
+        for storage in together:
+            self.initial(storage, slot)
+
     def view(self, storage: Any, block_table: Optional[torch.Tensor], writes: bool) -> Any:
         raise NotImplementedError
 
@@ -91,6 +103,15 @@ class FixedState(CacheNeed):
 
     def initial(self, storage, slot):
         storage[slot].zero_()
+
+    def allocate_together(self, count, units, page_size, dtype, device):
+        # one tensor for the layers that keep the same state: a request's start clears its slot in
+        # all of them with one launch (a model of 22 such layers paid 22 before every admission)
+        whole = torch.zeros((count, units, *self.shape), dtype=self.dtype, device=device)
+        return [whole[index] for index in range(count)], whole
+
+    def initial_together(self, together, slot):
+        together[:, slot].zero_()
 
     def view(self, storage, block_table, writes):
         return CacheView(state=storage, writes=writes)

@@ -28,6 +28,8 @@ import ctypes
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
+
 from .. import host
 from ..cache import CacheManager
 from ..sampling import GREEDY, SamplingConfig, make_rng
@@ -99,7 +101,7 @@ class Request:
 @dataclass
 class PlannedSegment:
     request: Request
-    tokens: List[int]
+    tokens: Sequence[int]       # a piece of the plan's int32 array
     wants_logits: bool
 
 
@@ -284,9 +286,11 @@ class Scheduler:
         segments, tokens = counts[0], counts[1]
         plan = StepPlan(num_tokens=tokens, serial=self._serial)
         if segments:
-            owners, lengths, wants, flat = host.ids(segments), host.ints(segments), host.ints(segments), host.ints(tokens)
-            self._lib.fwh_plan_segments(self._native, owners, lengths, wants, flat)
-            flat, at = list(flat[:tokens]), 0
+            owners, lengths, wants = host.ids(segments), host.ints(segments), host.ints(segments)
+            # a segment's tokens are a piece of one int32 array: a prompt portion has thousands, and a
+            # Python object for each would cost the step more than its smaller kernels
+            flat, at = np.empty(max(tokens, 1), dtype=np.int32), 0
+            self._lib.fwh_plan_segments(self._native, owners, lengths, wants, flat.ctypes.data_as(ctypes.POINTER(ctypes.c_int)))
             for i in range(segments):
                 plan.segments.append(PlannedSegment(self.requests[owners[i]], flat[at:at + lengths[i]], bool(wants[i])))
                 at += lengths[i]

@@ -44,8 +44,9 @@ class StepEntry:
 def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int, max_positions: int):
     """What a step may not bring: no entries, an unknown or repeated request, no tokens, a token
     outside the vocabulary, a place outside the entry, a sequence past the model's limit.
-    Returns the requests' current lengths and slots (one call into the host library) and the
-    host library's ids of the requests, for the step's further calls."""
+    Returns the requests' current lengths and slots (one call into the host library), the
+    host library's ids of the requests, for the step's further calls, and the entries' tokens
+    as int32 arrays (None for a step of single tokens)."""
     if not entries:
         raise StepError("a step needs at least one entry")
     requests = [entry.request for entry in entries]
@@ -73,24 +74,61 @@ def check_entries(entries: Sequence[StepEntry], cache: CacheManager, vocab_size:
             for place in entry.want:
                 if int(place) != 0:
                     raise StepError(f"request {entry.request!r} wants logits at place {place} of 1 tokens", entry.request)
-        return lengths, slots, natives
+        return lengths, slots, natives, None
+    arrays = []         # each entry's tokens as one int32 array: made once, the step's upload takes them as they are
     for entry, start in zip(entries, lengths):
         n = len(entry.tokens)
         if n < 1:
             raise StepError(f"request {entry.request!r} brings no tokens", entry.request)
         if start + n > max_positions:
             raise StepError(f"request {entry.request!r} would reach {start + n} tokens; the context limit is {max_positions}", entry.request)
-        low, high = (min(entry.tokens), max(entry.tokens)) if n > 1 else (entry.tokens[0], entry.tokens[0])
-        if not (0 <= int(low) and int(high) < vocab_size):
-            bad = next(t for t in entry.tokens if not 0 <= int(t) < vocab_size)
+        try:
+            tokens = np.asarray(entry.tokens, dtype=np.int32)
+            if n == 1:          # the decoded tokens beside a prompt's portion: no reduction for one number
+                inside = tokens.ndim == 1 and 0 <= int(tokens[0]) < vocab_size
+            else:
+                inside = tokens.ndim == 1 and 0 <= int(tokens.min()) and int(tokens.max()) < vocab_size
+        except (OverflowError, TypeError, ValueError):
+            inside = False
+        if not inside:
+            bad = next((t for t in entry.tokens if not (isinstance(t, (int, np.integer)) and 0 <= int(t) < vocab_size)), entry.tokens[0])
             raise StepError(f"token id {bad} of request {entry.request!r} is outside the vocabulary (0..{vocab_size - 1})", entry.request)
+        arrays.append(tokens)
         for place in entry.want:
             if not 0 <= int(place) < n:
                 raise StepError(f"request {entry.request!r} wants logits at place {place} of {n} tokens", entry.request)
         if entry.positions is not None and (len(entry.positions) != n or min(entry.positions) < 0):
             raise StepError(f"request {entry.request!r} gives {len(entry.positions)} positions for {n} tokens, or a negative one",
                             entry.request)
-    return lengths, slots, natives
+    return lengths, slots, natives, arrays
+
+
+class _Staging:
+    """Pinned host memory that an eager step's index arrays pass through on their way to the
+    device: the copy is queued and the host goes on to the step's launches (from pageable
+    memory it would stand until the copy has run). One buffer serves every step: before it is
+    written again the copy of the step before must have left it."""
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self._host: Optional[torch.Tensor] = None
+        self._numpy: Optional[np.ndarray] = None
+        self._left = torch.cuda.Event()
+
+    def upload(self, pieces: Sequence[np.ndarray]) -> torch.Tensor:
+        total = sum(piece.size for piece in pieces)
+        if self._host is None or self._host.numel() < total:
+            if self._host is not None:
+                self._left.synchronize()
+            self._host = torch.empty(max(2 * total, 1 << 14), dtype=torch.int32, pin_memory=True)
+            self._numpy = self._host.numpy()
+        else:
+            self._left.synchronize()
+        np.concatenate(pieces, out=self._numpy[:total])
+        packed = torch.empty(total, dtype=torch.int32, device=self.device)
+        packed.copy_(self._host[:total], non_blocking=True)
+        self._left.record()
+        return packed
 
 
 class StepContext:
@@ -103,34 +141,37 @@ class StepContext:
     RUN_OF_KEYS = 256       # decode attention shares a row's keys out in runs of four pages
 
     def __init__(self, entries: Sequence[StepEntry], cache: CacheManager, device: torch.device, vocab_size: int,
-                 max_positions: int, described=None, providers: Sequence = ()):
-        """``described``: (lengths, slots) of the entries' requests if the caller has checked the
-        entries already (``check_entries``). ``providers``: the parts whose ``step_arrays`` this
-        step's upload carries."""
-        starts, slots, natives = described if described is not None else check_entries(entries, cache, vocab_size, max_positions)
-        # per-row arrays are put together from one numpy piece per entry: a prompt portion has
-        # thousands of rows, and a Python loop over them would take longer than some kernels
-        token_parts, pos_parts, seg_parts = [], [], []
-        seg_row0: List[int] = [0]
+                 max_positions: int, described=None, providers: Sequence = (), staging: Optional[_Staging] = None):
+        """``described``: what ``check_entries`` returned if the caller has checked the entries
+        already. ``providers``: the parts whose ``step_arrays`` this
+        step's upload carries. ``staging``: the pinned memory the upload passes through, if the
+        caller keeps some."""
+        starts, slots, natives, arrays = described if described is not None else check_entries(entries, cache, vocab_size, max_positions)
+        # per-row arrays are made by whole-array operations: a prompt portion has thousands of rows and
+        # a step dozens of entries, and a Python loop over either would take longer than some kernels
+        if arrays is None:
+            arrays = [np.asarray(entry.tokens, dtype=np.int32) for entry in entries]
+        counts = np.fromiter((array.size for array in arrays), dtype=np.int64, count=len(arrays))
+        first_rows = np.zeros(len(arrays) + 1, dtype=np.int64)
+        np.cumsum(counts, out=first_rows[1:])
+        starts_array = np.asarray(starts, dtype=np.int64)
+        tokens = np.concatenate(arrays)
+        row_seg = np.repeat(np.arange(len(arrays), dtype=np.int32), counts)
+        row_pos = (np.arange(len(tokens), dtype=np.int64) - np.repeat(first_rows[:-1] - starts_array, counts)).astype(np.int32)
+        seg_row0: List[int] = first_rows.tolist()
         seg_slot: List[int] = list(slots)
         want_rows: List[int] = []
+        for entry, row0 in zip(entries, seg_row0):
+            if len(entry.want):
+                want_rows.extend(row0 + int(place) for place in entry.want)
         self.requests: List[Hashable] = [entry.request for entry in entries]
-        self.new_lengths: List[int] = []
+        self.new_lengths: List[int] = (starts_array + counts).tolist()
         given_positions = any(entry.positions is not None for entry in entries)
         encoding_parts = []
-        for seg, (entry, start) in enumerate(zip(entries, starts)):
-            n = len(entry.tokens)
-            want_rows.extend(seg_row0[-1] + int(place) for place in entry.want)
-            token_parts.append(np.asarray(entry.tokens, dtype=np.int32))
-            pos_parts.append(np.arange(start, start + n, dtype=np.int32))
-            if given_positions:
-                encoding_parts.append(pos_parts[-1] if entry.positions is None else np.asarray(entry.positions, dtype=np.int32))
-            seg_parts.append(np.full(n, seg, dtype=np.int32))
-            seg_row0.append(seg_row0[-1] + n)
-            self.new_lengths.append(start + n)
-        tokens = np.concatenate(token_parts)
-        row_pos = np.concatenate(pos_parts)
-        row_seg = np.concatenate(seg_parts)
+        if given_positions:
+            for entry, row0, count in zip(entries, seg_row0, counts.tolist()):
+                encoding_parts.append(row_pos[row0:row0 + count] if entry.positions is None
+                                      else np.asarray(entry.positions, dtype=np.int32))
         self.num_rows = len(tokens)
         self.num_segments = len(entries)
         self.num_wanted = len(want_rows)
@@ -138,10 +179,7 @@ class StepContext:
         self.max_context = max(self.new_lengths)
         # segments of one token that a mixed step begins with (a scheduler puts the decoded tokens
         # first): mixers may give them to their decode kernels. Their rows are 0 .. n - 1.
-        self.decode_prefix = 0
-        if not self.all_decode:
-            while len(entries[self.decode_prefix].tokens) == 1:
-                self.decode_prefix += 1
+        self.decode_prefix = 0 if self.all_decode else int(np.argmax(counts != 1))
         self.device = device
         # the same on the host, for parts that plan their work there
         self.host_row_pos = row_pos
@@ -159,7 +197,7 @@ class StepContext:
             pieces.append(np.concatenate(encoding_parts))
         extra = self._ask(providers)
         pieces += [array for _, _, array in extra]
-        packed = torch.from_numpy(np.concatenate(pieces)).to(device)
+        packed = staging.upload(pieces) if staging is not None else torch.from_numpy(np.concatenate(pieces)).to(device)
         views = []
         offset = 0
         for piece in pieces:
@@ -250,7 +288,7 @@ class StepContext:
         host = self._host
         self.requests = [e.request for e in entries]
         if described is not None:
-            starts, slots, natives = described
+            starts, slots, natives = described[:3]
         else:
             natives = cache.natives_of(self.requests)
             starts, slots = cache.describe(self.requests, natives)
@@ -349,6 +387,7 @@ class Stepper:
         self.steps = 0
         self.tokens_run = 0
         self.providers = model.step_array_providers()      # parts whose index arrays travel with a step's upload
+        self._staging = _Staging(self.device) if self.device.type == "cuda" else None
         # decode steps (every segment one token) are captured in a HIP graph per batch size and
         # context bucket and replayed, if every part of the model allows it
         self.use_graphs = all(block.graph_safe for block in model.layers) and model.final_norm.graph_safe
@@ -380,7 +419,7 @@ class Stepper:
             if self.use_graphs and not ops.kernel_profile_active() and all(len(entry.tokens) == 1 and entry.positions is None for entry in entries):
                 return self._replay(self._decode_step(len(entries), max(new_lengths)), entries, described)
             ctx = StepContext(entries, cache, self.device, spec.vocab_size, self.context_limit, described=described,
-                              providers=self.providers)
+                              providers=self.providers, staging=self._staging)
             logits = self.model.forward(ctx, cache)
         except BaseException:
             # The lengths stay where they were and the pages reserved for this step go back. What

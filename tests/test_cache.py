@@ -5,7 +5,7 @@ import random
 import pytest
 import torch
 
-from flyweight_amd.cache import (CacheAccountingError, CacheManager, FixedState, NO_PAGE, OutOfPages, PagedKV,
+from flyweight_amd.cache import (CacheAccountingError, CacheManager, CacheNeed, FixedState, NO_PAGE, OutOfPages, PagedKV,
                                  PagePool, SlotPool)
 
 KV = PagedKV(num_kv_heads=2, head_dim=16)
@@ -130,6 +130,37 @@ def test_state_slot_is_zeroed_when_handed_out():
     cache.release("a")
     assert cache.admit("b") == slot     # LIFO: the same slot again
     assert float(cache.state[0][slot].abs().sum()) == 0.0
+
+
+def test_entries_with_equal_state_start_a_slot_together_and_others_on_their_own():
+    class Counted(FixedState):
+        """A need of a mixer's own: starts at 2, says so entry by entry (the inherited way)."""
+        def allocate_together(self, count, units, page_size, dtype, device):
+            return CacheNeed.allocate_together(self, count, units, page_size, dtype, device)
+
+        def initial_together(self, together, slot):
+            CacheNeed.initial_together(self, together, slot)
+
+        def initial(self, storage, slot):
+            storage[slot] = 2.0
+
+    needs = {0: FixedState((4, 2)), 1: FixedState((4, 2)), 2: FixedState((3,)), 5: FixedState((4, 2)), 7: Counted((4, 2)), 8: Counted((4, 2))}
+    cache = CacheManager(needs, num_pages=1, max_requests=3, device=torch.device("cpu"))
+    # the three equal entries lie in one tensor, the other shape and the other class apart
+    assert cache.state[0].data_ptr() != cache.state[1].data_ptr()
+    assert cache.state[0].untyped_storage().data_ptr() == cache.state[1].untyped_storage().data_ptr() == cache.state[5].untyped_storage().data_ptr()
+    assert cache.state[2].untyped_storage().data_ptr() != cache.state[0].untyped_storage().data_ptr()
+    assert cache.state[7].untyped_storage().data_ptr() != cache.state[8].untyped_storage().data_ptr()
+    first, second = cache.admit("a"), cache.admit("b")
+    for entry in needs:
+        cache.state[entry][first] = 7.0
+        cache.state[entry][second] = 9.0
+    cache.release("a")
+    assert cache.admit("c") == first
+    for entry in needs:
+        start = 2.0 if entry in (7, 8) else 0.0
+        assert bool((cache.state[entry][first] == start).all()), entry
+        assert bool((cache.state[entry][second] == 9.0).all()), entry       # the neighbour's slot is untouched
 
 
 def test_window_group_gives_back_the_pages_its_window_has_passed():

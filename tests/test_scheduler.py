@@ -32,7 +32,7 @@ def drive(scheduler, cache, max_steps=10000, log=None):
         assert plan.num_tokens <= scheduler.max_batch_tokens
         for segment in plan.segments:
             r = segment.request
-            assert r.live and segment.tokens == r.tokens[r.computed:r.computed + len(segment.tokens)]
+            assert r.live and list(segment.tokens) == r.tokens[r.computed:r.computed + len(segment.tokens)]
             assert cache.pages_missing(r.id, r.computed + len(segment.tokens)) == {0: 0}, "pages were not reserved"
             assert segment.wants_logits == (r.computed + len(segment.tokens) == len(r.tokens))
         sampled = {s.request.id: oracle(s.request.tokens) for s in plan.segments if s.wants_logits}
@@ -146,7 +146,7 @@ def test_out_of_pages_preempts_the_newest_and_never_the_oldest():
     # a preempted request recomputes prompt + generated as portions and asks for logits only at the end
     after = log[log.index(preempting[0]) + 1:]
     recompute = [s for p in after for s in p.segments if s.request is new and len(s.tokens) > 1]
-    assert recompute and recompute[0].tokens[:100] == [4] * 100
+    assert recompute and list(recompute[0].tokens[:100]) == [4] * 100
     assert cache.stats()["pages_free"] == 4
 
 
