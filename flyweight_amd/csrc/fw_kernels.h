@@ -41,11 +41,13 @@ int fw_gemm_skinny(const void* a, const void* w, const float* bias, void* out, i
                    int M, int N, int K, void* stream);
 int fw_gemm_mfma(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                  int M, int N, int K, void* stream);
-// The prompt product with 256 x 256 (or 256 x 192) tiles, for shapes that give enough of them to fill the chip
-// (fw_gemm_mfma_big_tiles says how many).
+// The prompt product with large tiles (256 x 256 or 256 x 192; storing products also 128 rows by as many columns,
+// where that fills the chip better), for shapes that give enough of them to fill the chip
+// (fw_gemm_mfma_big_tiles says how many, fw_gemm_mfma_big_plan also which).
 int fw_gemm_mfma_big(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                      int M, int N, int K, void* stream);
 int fw_gemm_mfma_big_tiles(int mode, int M, int N, int K);     // 0: the kernel does not take the shape
+int fw_gemm_mfma_big_plan(int mode, int M, int N, int K, int* rows, int* columns);     // the same, and the tile's edges
 // The prompt product with tiles of 128 rows and `columns` (128 or 64) columns whose four waves split
 // K (half the LDS traffic per flop of fw_gemm_mfma's tiles), for outputs too narrow for the
 // 256 x 256 tiles to fill the chip. Modes 0 and 1; K a multiple of 64 (fw_gemm_mfma_deep_tiles says

@@ -13,6 +13,11 @@
 //    not padded, their chunks are stored permuted against bank conflicts;
 //  * workgroups are numbered so that each XCD works on a compact group of tiles.
 //
+// A product whose 256-row tiles would leave compute units idle takes tiles of 128 rows (each wave
+// 64 rows): 2,048 rows by 3,072 features are 128 tiles of 256 x 192 but exactly 256 of 128 x 192.
+// Such a tile moves more bytes per flop through LDS and the memory path, so it is used only where
+// it fills the chip better.
+//
 // It needs enough tiles to fill the chip (the caller checks): 2,048 rows by 8,192 gated features
 // are 512 tiles. Epilogues as the other products: store, add into the residual stream, SwiGLU
 // (a tile holds 128 gate and the 128 up features of the same columns; a lane holds both of an
@@ -27,12 +32,12 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 
-#define BT 256                  // tile edge
+#define BT 256                  // tile edge (rows: of the tall tiles)
 #define BK 32                   // k per slab: an LDS row is 64 bytes, four 16-byte chunks
 #define BSTAGES 4               // slabs in LDS: one is multiplied, three are on their way
 #define BSLAB (BT * BK * 2)     // bytes of one operand's slab
 #define BGROUP_M 4
-#define B_LOADS 4               // wave-wide loads (16 rows of 64 bytes) per wave per operand per slab
+#define B_LOADS 4               // most wave-wide loads (16 rows of 64 bytes) per wave per operand per slab
 
 enum { MB_STORE = 0, MB_ACCUMULATE = 1, MB_SWIGLU = 2 };
 
@@ -55,17 +60,20 @@ __device__ __forceinline__ float from_neighbour(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
 }
 
-template <int TN>
+template <int TM, int TN>
 struct BigTile {
+    static constexpr int ROWS = 2 * TM * 32;               // rows of a tile
     static constexpr int WIDE = 2 * TN * 32;               // columns of a tile
-    static constexpr int W_LOADS = WIDE / 64;              // wave-wide loads per wave for a slab of w (16 rows each)
-    static constexpr int SLAB_LOADS = B_LOADS + W_LOADS;   // and for a slab of both operands
+    static constexpr int A_LOADS = ROWS / 64;              // wave-wide loads per wave for a slab of a (16 rows each)
+    static constexpr int W_LOADS = WIDE / 64;              // and for a slab of w
+    static constexpr int SLAB_LOADS = A_LOADS + W_LOADS;   // and for a slab of both operands
 };
 
 // K must be a multiple of BK (the loads go straight to LDS: nothing can be zeroed on the way).
 // TN: 32-column product tiles per wave, 4 (a 256 x 256 tile) or 3 (256 x 192: a width of 6,144
 // features gives 192 tiles of 256 columns for 256 compute units, but exactly 256 tiles of 192).
-template <int MODE, typename TO, int TN>
+// TM: 32-row product tiles per wave, 4 (256 rows a tile) or 2 (128 rows).
+template <int MODE, typename TO, int TN, int TM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void gemm_mfma_big_kernel(
     const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, const float* __restrict__ bias,
     TO* __restrict__ out, int M, int N, int K, int tiles_m, int tiles_n, int per_xcd, int up_offset) {
@@ -79,10 +87,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int group_size = tiles_m - first_m < BGROUP_M ? tiles_m - first_m : BGROUP_M;
     const int pid_m = first_m + (logical % width) % group_size;
     const int pid_n = (logical % width) / group_size;
-    static_assert(TN == 4 || (TN == 3 && MODE != MB_SWIGLU), "three column tiles per wave: store and accumulate only");
-    constexpr int WIDE = BigTile<TN>::WIDE, W_LOADS = BigTile<TN>::W_LOADS, SLAB_LOADS = BigTile<TN>::SLAB_LOADS;
+    static_assert((TN == 4 && TM == 4) || (MODE != MB_SWIGLU && (TN == 3 || TN == 4) && (TM == 2 || TM == 4)),
+                  "narrower or lower tiles: store and accumulate only");
+    constexpr int ROWS = BigTile<TM, TN>::ROWS, WIDE = BigTile<TM, TN>::WIDE;
+    constexpr int A_LOADS = BigTile<TM, TN>::A_LOADS, W_LOADS = BigTile<TM, TN>::W_LOADS, SLAB_LOADS = BigTile<TM, TN>::SLAB_LOADS;
     const int features = MODE == MB_SWIGLU ? BT / 2 : WIDE;
-    const int m0 = pid_m * BT, n0 = pid_n * features;
+    const int m0 = pid_m * ROWS, n0 = pid_n * features;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -96,8 +106,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const uint16_t* a_src[B_LOADS];
     const uint16_t* w_src[B_LOADS];     // W_LOADS of them are used (with w_src[W_LOADS] the host pass emitted no launch stub)
 #pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) {
-        const int row = (wave * B_LOADS + i) * 16 + (lane >> 2);
+    for (int i = 0; i < A_LOADS; ++i) {
+        const int row = (wave * A_LOADS + i) * 16 + (lane >> 2);
         const int chunk = (lane & 3) ^ ((row >> 2) & 3);
         int am = m0 + row;
         am = am < M ? am : M - 1;                       // rows past the end are computed and dropped
@@ -118,16 +128,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         unsigned char* stage = lds + (slab % BSTAGES) * 2 * BSLAB;
         const int k0 = slab * BK;
 #pragma unroll
-        for (int i = 0; i < B_LOADS; ++i)
-            __builtin_amdgcn_global_load_lds(a_src[i] + k0, reinterpret_cast<uint32_t*>(stage + (wave * B_LOADS + i) * 1024), 16, 0, 0);
+        for (int i = 0; i < A_LOADS; ++i)
+            __builtin_amdgcn_global_load_lds(a_src[i] + k0, reinterpret_cast<uint32_t*>(stage + (wave * A_LOADS + i) * 1024), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < W_LOADS; ++i)
             __builtin_amdgcn_global_load_lds(w_src[i] + k0, reinterpret_cast<uint32_t*>(stage + BSLAB + (wave * W_LOADS + i) * 1024), 16, 0, 0);
     };
 
-    f32x16 acc[4][TN];
+    f32x16 acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -135,7 +145,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
     // this wave's rows of the a slab, and its rows of the w slab: for SwiGLU the columns of a wave
     // are 64 gate features (tiles 0, 1) and the 64 up features of the same columns (tiles 2, 3)
-    const int a_row0 = wm * 128 + (lane & 31);
+    const int a_row0 = wm * (TM * 32) + (lane & 31);
     int b_row[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j)
@@ -146,15 +156,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
     for (int t = 0; t < BK / 16; ++t) slot[t] = ((2 * t + (lane >> 5)) ^ swizzle) * 16;
 
-    // operand registers of one k16 step: four row tiles of a, four column tiles of w
+    // operand registers of one k16 step: the wave's row tiles of a and column tiles of w
     struct Operands {
-        bf16x8 fa[4], fb[TN];
+        bf16x8 fa[TM], fb[TN];
     };
     auto read = [&](Operands& f, int slab, int t) {
         const unsigned char* sa = lds + (slab % BSTAGES) * 2 * BSLAB;
         const unsigned char* sb = sa + BSLAB;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < TM; ++i)
             f.fa[i] = *reinterpret_cast<const bf16x8*>(sa + (a_row0 + 32 * i) * (BK * 2) + slot[t]);
 #pragma unroll
         for (int j = 0; j < TN; ++j)
@@ -178,7 +188,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // Tells the compiler that these operands are needed HERE, so that it waits for their LDS reads
     // before the next reads are issued and not, for all reads together, in front of the MFMAs.
     auto arrived = [&](const Operands& f) {
-        asm volatile("" ::"v"(f.fa[0]), "v"(f.fa[1]), "v"(f.fa[2]), "v"(f.fa[3]), "v"(f.fb[0]), "v"(f.fb[1]), "v"(f.fb[2]), "v"(f.fb[TN - 1]));
+        asm volatile("" ::"v"(f.fa[0]), "v"(f.fa[1]), "v"(f.fa[TM - 2]), "v"(f.fa[TM - 1]), "v"(f.fb[0]), "v"(f.fb[1]), "v"(f.fb[2]), "v"(f.fb[TN - 1]));
     };
     // waits until at most `slabs` of this wave's requested slabs are still on their way (SLAB_LOADS loads each)
     auto wait_for_all_but = [&](int slabs) {
@@ -207,28 +217,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         // first half of step 0 of slab s, with the reads of step 1 between its MFMAs
         arrived(f0);
         read(f1, s, 1);
-        multiply(f0, 0, 2);
-        FW_INTERLEAVE(2 * TN, 1, 0x100)         // (with three column tiles one read of seven is left to the scheduler)
+        multiply(f0, 0, TM / 2);
+        FW_INTERLEAVE(TM / 2 * TN, 1, 0x100)    // (where the reads outnumber the MFMAs the rest is left to the scheduler)
         __builtin_amdgcn_sched_barrier(0);
         arrived(f1);                                        // slab s has been read
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * SLAB_LOADS) : "memory");   // slab s + 1 has landed; s + 2 and s + 3 may still fly
         __builtin_amdgcn_s_barrier();
         // second half, with the requests for slab s + 4 between its MFMAs
         request(s + BSTAGES);
-        multiply(f0, 2, 2);
-        FW_INTERLEAVE(2 * TN, 1, 0x020)
+        multiply(f0, TM / 2, TM / 2);
+        FW_INTERLEAVE(TM / 2 * TN, 1, 0x020)
         __builtin_amdgcn_sched_barrier(0);
         // step 1, with the reads of step 0 of slab s + 1 between its MFMAs
         read(f0, s + 1, 0);
-        multiply(f1, 0, 4);
-        FW_INTERLEAVE(2 * TN, 2, 0x100)
+        multiply(f1, 0, TM);
+        FW_INTERLEAVE(2 * TN, TM / 2, 0x100)
         __builtin_amdgcn_sched_barrier(0);
     }
     // the last slabs: nothing more to request
     for (; s < steps; ++s) {
         arrived(f0);
         read(f1, s, 1);
-        multiply(f0, 0, 4);
+        multiply(f0, 0, TM);
         __builtin_amdgcn_sched_barrier(0);
         arrived(f1);
         if (s + 1 < steps) {
@@ -236,7 +246,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             __builtin_amdgcn_s_barrier();
             read(f0, s + 1, 0);
         }
-        multiply(f1, 0, 4);
+        multiply(f1, 0, TM);
         __builtin_amdgcn_sched_barrier(0);
     }
 #undef FW_INTERLEAVE
@@ -249,16 +259,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // quick way: no bounds, no branches, pointers stepped by rows, and for bfloat16 two
     // neighbouring lanes swap one value each so that each stores a pair of columns as one word.
     // With one workgroup per compute unit nothing runs beside the epilogue, so its length counts.
-    const bool inside = m0 + BT <= M && n0 + features <= N && (sizeof(TO) == 4 || (N & 1) == 0);
+    const bool inside = m0 + ROWS <= M && n0 + features <= N && (sizeof(TO) == 4 || (N & 1) == 0);
     const bool odd = lane & 1;
     if constexpr (MODE == MB_SWIGLU) {
         if (inside) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                uint16_t* pair = reinterpret_cast<uint16_t*>(out) + (size_t)(m0 + wm * 128 + row_base) * N +
+                uint16_t* pair = reinterpret_cast<uint16_t*>(out) + (size_t)(m0 + wm * (TM * 32) + row_base) * N +
                                  (n0 + wn * 64 + j * 32 + (col & ~1));
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
+                for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int q = 0; q < 4; ++q)
 #pragma unroll
@@ -279,10 +289,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             const int n = n0 + wn * 64 + j * 32 + col;
             if (n >= N) continue;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int m = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + row_base + (r & 3);
+                    const int m = m0 + wm * (TM * 32) + i * 32 + 8 * (r >> 2) + row_base + (r & 3);
                     if (m < M) store_from_float(out, (size_t)m * N + n, silu_quick(acc[i][j][r]) * acc[i][j + 2][r]);
                 }
         }
@@ -294,9 +304,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             const int n = n0 + wn * (TN * 32) + j * 32 + col;
             const float b = bias ? bias[n] : 0.0f;
             if constexpr (sizeof(TO) == 4) {
-                float* column = reinterpret_cast<float*>(out) + (size_t)(m0 + wm * 128 + row_base) * N + n;
+                float* column = reinterpret_cast<float*>(out) + (size_t)(m0 + wm * (TM * 32) + row_base) * N + n;
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
+                for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         float* to = column + (size_t)(i * 32 + 8 * (r >> 2) + (r & 3)) * N;
@@ -305,9 +315,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                         *to = value;
                     }
             } else {
-                uint16_t* pair = reinterpret_cast<uint16_t*>(out) + (size_t)(m0 + wm * 128 + row_base) * N + (n & ~1);
+                uint16_t* pair = reinterpret_cast<uint16_t*>(out) + (size_t)(m0 + wm * (TM * 32) + row_base) * N + (n & ~1);
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
+                for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int q = 0; q < 4; ++q)
 #pragma unroll
@@ -328,10 +338,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         if (n >= N) continue;
         const float b = bias ? bias[n] : 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm * 128 + i * 32 + 8 * (r >> 2) + row_base + (r & 3);
+                const int m = m0 + wm * (TM * 32) + i * 32 + 8 * (r >> 2) + row_base + (r & 3);
                 if (m >= M) continue;
                 const size_t at = (size_t)m * N + n;
                 float value = acc[i][j][r] + b;
@@ -341,15 +351,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
 }
 
-template <int MODE, typename TO, int TN = 4>
+template <int MODE, typename TO, int TN = 4, int TM = 4>
 static int launch_big(const void* a, const void* w, const float* bias, void* out, int M, int N, int K, hipStream_t stream) {
     const int features = MODE == MB_SWIGLU ? BT / 2 : 2 * TN * 32;
-    const int tiles_m = fw_ceil_div(M, BT), tiles_n = fw_ceil_div(N, features);
+    const int tiles_m = fw_ceil_div(M, 2 * TM * 32), tiles_n = fw_ceil_div(N, features);
     const int per_xcd = fw_ceil_div((long long)tiles_m * tiles_n, 8);
     const int lds_bytes = BSTAGES * 2 * BSLAB;
     static bool configured = false;     // per instantiation
     if (!configured) {
-        hipError_t status = hipFuncSetAttribute((const void*)gemm_mfma_big_kernel<MODE, TO, TN>,
+        hipError_t status = hipFuncSetAttribute((const void*)gemm_mfma_big_kernel<MODE, TO, TN, TM>,
                                                 hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (status != hipSuccess) {
             fw_set_error("gemm_mfma_big: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(status));
@@ -357,25 +367,64 @@ static int launch_big(const void* a, const void* w, const float* bias, void* out
         }
         configured = true;
     }
-    gemm_mfma_big_kernel<MODE, TO, TN><<<per_xcd * 8, 256, lds_bytes, stream>>>(
+    gemm_mfma_big_kernel<MODE, TO, TN, TM><<<per_xcd * 8, 256, lds_bytes, stream>>>(
         (const uint16_t*)a, (const uint16_t*)w, bias, (TO*)out, M, N, K, tiles_m, tiles_n, per_xcd, N);
     return 0;
 }
 
-// Whether tiles of 192 columns serve a storing or accumulating product better than tiles of 256:
-// rounds of tiles over the chip's 256 compute units, a narrow tile counting three quarters.
-static bool narrow_tiles_pay(int M, int N) {
-    const long long wide = (long long)fw_ceil_div(M, BT) * fw_ceil_div(N, BT), narrow = (long long)fw_ceil_div(M, BT) * fw_ceil_div(N, 192);
-    return 3 * fw_ceil_div(narrow, 256) < 4 * fw_ceil_div(wide, 256);
+// The tile a storing or accumulating product is cut into: 256 or 128 rows by 256 or 192 columns,
+// whichever takes the least time by this count: rounds of tiles over the chip's 256 compute units
+// times the tile's area, a tile of 128 rows counting a quarter more than its area (it moves more
+// bytes per flop). Gated products (SwiGLU) keep 256 x 256, and accumulating ones 256 rows: their
+// epilogue reads the old values where nothing hides the read, and twice the tiles for the same
+// output pay that twice as often (2,048 x 3,072 x 2,048: storing 50.9 -> 35.6 us with tiles of
+// 128 x 192, accumulating 51.6 -> 58.5 us).
+struct BigPlan {
+    int rows, columns, tiles;
+};
+static BigPlan big_plan(int mode, int M, int N) {
+    if (mode == MB_SWIGLU) return {BT, BT / 2, fw_ceil_div(M, BT) * fw_ceil_div(N, BT / 2)};
+    BigPlan best = {0, 0, 0};
+    long long best_cost = 0;
+    for (int rows = BT; rows >= (mode == MB_STORE ? BT / 2 : BT); rows /= 2)
+        for (int columns = BT; columns >= 192; columns -= 64) {
+            const long long tiles = (long long)fw_ceil_div(M, rows) * fw_ceil_div(N, columns);
+            const long long cost = fw_ceil_div(tiles, 256) * (rows / 32) * (columns / 32) * (rows == BT ? 4 : 5);
+            if (best.tiles == 0 || cost < best_cost) {
+                best = {rows, columns, (int)(tiles < (1ll << 30) ? tiles : (1ll << 30))};
+                best_cost = cost;
+            }
+        }
+    return best;
 }
 
-// How many tiles the kernel cuts a shape into, 256 x 256 or 256 x 192 as it will choose (the
-// caller decides whether that fills the chip); 0 if the kernel does not take the shape (K must be
-// a multiple of 32).
+// How many tiles the kernel cuts a shape into, by the tile it will choose (the caller decides
+// whether that fills the chip); 0 if the kernel does not take the shape (K must be a multiple
+// of 32).
 extern "C" int fw_gemm_mfma_big_tiles(int mode, int M, int N, int K) {
-    if (K <= 0 || K % BK) return 0;
-    if (mode != MB_SWIGLU && narrow_tiles_pay(M, N)) return fw_ceil_div(M, BT) * fw_ceil_div(N, 192);
-    return fw_ceil_div(M, BT) * fw_ceil_div(N, mode == MB_SWIGLU ? BT / 2 : BT);
+    if (K <= 0 || K % BK || M < 1 || N < 1) return 0;
+    return big_plan(mode, M, N).tiles;
+}
+
+// The same with the tile's edges: what the caller needs to tell how much of the tiles the output fills.
+extern "C" int fw_gemm_mfma_big_plan(int mode, int M, int N, int K, int* rows, int* columns) {
+    if (K <= 0 || K % BK || M < 1 || N < 1) return 0;
+    const BigPlan plan = big_plan(mode, M, N);
+    if (rows) *rows = plan.rows;
+    if (columns) *columns = plan.columns;
+    return plan.tiles;
+}
+
+template <int MODE, typename TO>
+static int launch_planned(const BigPlan& plan, const void* a, const void* w, const float* bias, void* out, int M, int N, int K,
+                          hipStream_t stream) {
+    if (plan.rows == BT || MODE != MB_STORE)
+        return plan.columns == BT ? launch_big<MODE, TO, 4, 4>(a, w, bias, out, M, N, K, stream)
+                                  : launch_big<MODE, TO, 3, 4>(a, w, bias, out, M, N, K, stream);
+    if constexpr (MODE == MB_STORE)
+        return plan.columns == BT ? launch_big<MODE, TO, 4, 2>(a, w, bias, out, M, N, K, stream)
+                                  : launch_big<MODE, TO, 3, 2>(a, w, bias, out, M, N, K, stream);
+    return -1;
 }
 
 // Same contract as fw_gemm_mfma.
@@ -387,17 +436,14 @@ extern "C" int fw_gemm_mfma_big(const void* a, const void* w, const float* bias,
     FW_REQUIRE(mode != MB_SWIGLU || (out_dtype == FW_BF16 && bias == nullptr), "gemm_mfma_big: SwiGLU stores bfloat16 and takes no bias");
     FW_REQUIRE(out_dtype == FW_F32 || out_dtype == FW_BF16, "gemm_mfma_big: unknown out dtype %d", out_dtype);
     FW_REQUIRE(((uintptr_t)a % 16 == 0) && ((uintptr_t)w % 16 == 0), "gemm_mfma_big: operands must be 16-byte aligned");
-    FW_REQUIRE((long long)fw_ceil_div(M, BT) * fw_ceil_div(N, BT / 2) < (1ll << 30), "gemm_mfma_big: too many tiles");
+    FW_REQUIRE((long long)fw_ceil_div(M, BT / 2) * fw_ceil_div(N, BT / 2) < (1ll << 30), "gemm_mfma_big: too many tiles");
     hipStream_t s = (hipStream_t)stream;
+    const BigPlan plan = big_plan(mode, M, N);
     int status;
-    const bool narrow = mode != MB_SWIGLU && narrow_tiles_pay(M, N);
     if (mode == MB_SWIGLU) status = launch_big<MB_SWIGLU, bf16_t>(a, w, nullptr, out, M, N, K, s);
-    else if (mode == MB_ACCUMULATE) status = narrow ? launch_big<MB_ACCUMULATE, float, 3>(a, w, bias, out, M, N, K, s)
-                                                    : launch_big<MB_ACCUMULATE, float>(a, w, bias, out, M, N, K, s);
-    else if (out_dtype == FW_F32) status = narrow ? launch_big<MB_STORE, float, 3>(a, w, bias, out, M, N, K, s)
-                                                  : launch_big<MB_STORE, float>(a, w, bias, out, M, N, K, s);
-    else status = narrow ? launch_big<MB_STORE, bf16_t, 3>(a, w, bias, out, M, N, K, s)
-                         : launch_big<MB_STORE, bf16_t>(a, w, bias, out, M, N, K, s);
+    else if (mode == MB_ACCUMULATE) status = launch_planned<MB_ACCUMULATE, float>(plan, a, w, bias, out, M, N, K, s);
+    else if (out_dtype == FW_F32) status = launch_planned<MB_STORE, float>(plan, a, w, bias, out, M, N, K, s);
+    else status = launch_planned<MB_STORE, bf16_t>(plan, a, w, bias, out, M, N, K, s);
     if (status != 0) return status;
     FW_LAUNCH_CHECK("gemm_mfma_big");
     return 0;

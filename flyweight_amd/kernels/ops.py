@@ -19,7 +19,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _lib = None
 
@@ -446,6 +446,12 @@ def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out
         _check(library().fw_gemm_mfma_deep(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K,
                                            _deep_columns(mode, M, N, K), _stream()))
         return
+    elif _deep_columns_few_rows(mode, M, N, K, one_round=True):
+        _check(library().fw_gemm_mfma_deep(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K,
+                                           _deep_columns_few_rows(mode, M, N, K), _stream()))
+        return
+    elif M > BIG_MIN_ROWS and _big_tiles_store_well(mode, M, N, K):
+        entry = library().fw_gemm_mfma_big      # fewer large tiles than compute units, but every other way takes two rounds
     elif _deep_columns_few_rows(mode, M, N, K):
         _check(library().fw_gemm_mfma_deep(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K,
                                            _deep_columns_few_rows(mode, M, N, K), _stream()))
@@ -497,7 +503,23 @@ DEEP_FEW_TILES_WIDE = 192   # tiles of 128 columns from which those are taken, e
 DEEP_FEW_TILES = 96       # tiles of 64 columns from which those are
 
 
-def _deep_columns_few_rows(mode: int, M: int, N: int, K: int) -> int:
+BIG_TILES_MIN_STORE = 96      # large tiles from which a storing product takes them, if the output fills
+BIG_FILL_STORE = 0.95         # at least this share of them
+
+
+def _big_tiles_store_well(mode: int, M: int, N: int, K: int) -> bool:
+    """A storing product that no kernel serves in one round of small tiles takes the large
+    tiles from 96 of them on if they are well filled: 768 x 3,072 (K 1,024) 18.7 -> 14.9 us,
+    512 x 4,608 21.1 -> 14.6 us, 1,024 x 3,072 (K 2,048) 29.5 -> 25.0 us; 2,048 x 1,024 (96 tiles
+    of 192 columns, an eighth of them outside the output) would lose, 14.1 -> 17.5 us."""
+    if mode != 0:
+        return False
+    rows, columns = ctypes.c_int(0), ctypes.c_int(0)
+    tiles = library().fw_gemm_mfma_big_plan(mode, M, N, K, ctypes.byref(rows), ctypes.byref(columns))
+    return tiles >= BIG_TILES_MIN_STORE and M * N >= BIG_FILL_STORE * tiles * rows.value * columns.value
+
+
+def _deep_columns_few_rows(mode: int, M: int, N: int, K: int, one_round: bool = False) -> int:
     """A few hundred rows (decode steps of that many requests, short prompts) give the 128 x 128
     tiles of the register-staged product less than a round over the chip; the tiles whose waves
     split K bring their operands straight into LDS, three slabs ahead, and a workgroup alone on
@@ -512,7 +534,7 @@ def _deep_columns_few_rows(mode: int, M: int, N: int, K: int) -> int:
     narrow = library().fw_gemm_mfma_deep_tiles(mode, M, N, K, 64)
     if mode == 0 and DEEP_FEW_TILES_WIDE <= wide <= DEEP_ROUND:
         return 128
-    if DEEP_FEW_TILES <= narrow <= 2 * DEEP_ROUND:
+    if DEEP_FEW_TILES <= narrow <= (1 if one_round else 2) * DEEP_ROUND:
         return 64
     return 0
 

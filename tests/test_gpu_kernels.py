@@ -364,14 +364,17 @@ def test_fast_gemm_every_epilogue(ops, M, N, K):
         close(ops.gemm_swiglu(a, w), act, torch.bfloat16, 0.4)
 
 
-@pytest.mark.parametrize("M,N,K", [(2048, 6144, 96), (1500, 8200, 160), (4000, 3100, 64), (1800, 6000, 2080), (1536, 6100, 96)])
-def test_large_tile_prompt_product(ops, M, N, K):
-    """Shapes with at least 192 tiles of 256 x 256 (or of 256 x 192, where those are what the
-    kernel takes: the last shape has 144 of the wider) go to the large-tile kernel: every epilogue,
-    edges in both directions, few and many slabs. The first and the last two shapes give one
-    round of tiles over the chip with tiles of 192 columns, which storing and accumulating
-    products then take; the gated product keeps the 256 x 256 tiles."""
-    assert ops.library().fw_gemm_mfma_big_tiles(0, M, N, K) >= ops.BIG_TILES_MIN and not ops.library().fw_gemm_mfma_big_tiles(0, M, N, K + 8)
+@pytest.mark.parametrize("M,N,K,tiles", [(2048, 6144, 96, 256), (1500, 8200, 160, 198), (4000, 3100, 64, 208), (1800, 6000, 2080, 256),
+                                         (1536, 6100, 96, 192), (2048, 3072, 96, 256), (1990, 3000, 2080, 256), (1900, 4000, 160, 240)])
+def test_large_tile_prompt_product(ops, M, N, K, tiles):
+    """Shapes that the large-tile kernel cuts into at least 192 tiles go to it: every epilogue,
+    edges in both directions, few and many slabs. ``tiles`` tells which tile a storing or
+    accumulating product takes: 256 x 256 (the second and third shape), 256 x 192 (the first,
+    fourth and fifth: one round over the chip with the narrower tile), 128 x 192 (the sixth and
+    seventh: 128 tiles of 256 rows, 256 of 128) and 128 x 256 (the last); the gated product keeps
+    the 256 x 256 tiles."""
+    assert ops.library().fw_gemm_mfma_big_tiles(0, M, N, K) == tiles and tiles >= ops.BIG_TILES_MIN
+    assert not ops.library().fw_gemm_mfma_big_tiles(0, M, N, K + 8)
     a = as_dev(gen(M, K), torch.bfloat16)
     w = as_dev(gen(N, K, seed=1, scale=K ** -0.5), torch.bfloat16)
     bias = gen(N, seed=2).float().to(DEV)
