@@ -102,15 +102,25 @@ class CausalLM:
         x = ops.embed_rows(self.embedding, ctx.token_ids, scale=self.spec.embedding_scale)
         schedule = self.spec.schedule
         ctx.prepared = None
+        # A step of single tokens: the final norm reads every row as it is, like a layer's first norm, so
+        # the last layer's last product may prepare it; rows that nobody wants cost the head nothing
+        # it would not read anyway, and are dropped behind it. (A recorded step computes every row too:
+        # what it gives and what the launches give stay bit for bit the same.)
+        every_row = bool(ctx.all_decode)
         for at, entry in enumerate(schedule):
             # the norm that reads the residual after this layer, for the layer's last product
-            following = self.layers[schedule[at + 1].layer] if at + 1 < len(schedule) else None
-            ctx.norm_after_block = getattr(following, "mixer_norm", None)
+            if at + 1 < len(schedule):
+                ctx.norm_after_block = getattr(self.layers[schedule[at + 1].layer], "mixer_norm", None)
+            else:
+                ctx.norm_after_block = self.final_norm if every_row else None
             self.layers[entry.layer].forward(x, ctx, ctx.cache_view(cache, entry))
-        ctx.prepared = ctx.norm_after_block = None
+        prepared, ctx.prepared, ctx.norm_after_block = ctx.prepared, None, None
         if ctx.num_wanted == 0:
             return None
-        logits = self.head.forward(LazyNorm(self.final_norm, x, ctx, row_index=ctx.want_rows), out_dtype=torch.float32)
+        final = LazyNorm(self.final_norm, x, ctx, prepared=prepared) if every_row else LazyNorm(self.final_norm, x, ctx, row_index=ctx.want_rows)
+        logits = self.head.forward(final, out_dtype=torch.float32)
+        if every_row and not getattr(ctx, "wants_every_row", False):
+            logits = logits[ctx.want_rows.long()]
         if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0.0:
             ops.scale_softcap_(logits, self.spec.logit_scale, self.spec.logit_softcap)
         return logits

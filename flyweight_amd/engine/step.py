@@ -175,6 +175,7 @@ class StepContext:
         self.num_rows = len(tokens)
         self.num_segments = len(entries)
         self.num_wanted = len(want_rows)
+        self.wants_every_row = want_rows == list(range(self.num_rows))      # in order: the logits' rows are the step's rows
         self.all_decode = self.num_rows == self.num_segments
         self.max_context = max(self.new_lengths)
         # segments of one token that a mixed step begins with (a scheduler puts the decoded tokens
@@ -245,6 +246,7 @@ class StepContext:
         depend on more than that (on positions, say) must not call itself ``graph_safe``."""
         self = cls.__new__(cls)
         self.num_rows = self.num_segments = self.num_wanted = batch
+        self.wants_every_row = True
         self.all_decode = True
         self.decode_prefix = 0
         self.max_context = max_context          # bounds the split-key grid, not the result
