@@ -218,7 +218,7 @@ __device__ int sample_batch(const float* __restrict__ row, int vocab, unsigned l
     if ((int)threadIdx.x < count) {
         const double scaled = (double)row[candidate_id(s.keys[threadIdx.x])] / temperature;
         const double p = exp(scaled - best_scaled);
-        s.p[threadIdx.x] = (scaled - scaled == 0.0) ? p : 0.0;       // not finite: no share
+        s.p[threadIdx.x] = __builtin_isfinite(scaled) ? p : 0.0;     // not finite: no share
     }
     __syncthreads();
     return count;
@@ -231,7 +231,7 @@ __device__ double sample_total(const float* __restrict__ row, int vocab, unsigne
     sample_for_each(row, vocab, [&](float value, int id) {
         if (candidate_key(value, id) >= floor_key) {
             const double scaled = (double)value / temperature;
-            if (scaled - scaled == 0.0) mine += exp(scaled - best_scaled);
+            if (__builtin_isfinite(scaled)) mine += exp(scaled - best_scaled);
         }
     });
 #pragma unroll
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
     };
     const long long candidates = (top_k > 0 && top_k < vocab) ? top_k : vocab;
     const double best_scaled = (double)row[best_id] / temperature;
-    if (!(temperature > 0.0) || candidates == 1 || !(best_scaled - best_scaled == 0.0)) {
+    if (!(temperature > 0.0) || candidates == 1 || !__builtin_isfinite(best_scaled)) {
         leave(best_id);         // greedy, one candidate, or a best value that is not finite (no share is): the generator rests
         return;
     }
