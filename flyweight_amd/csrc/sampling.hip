@@ -133,6 +133,9 @@ __device__ void sample_sort(unsigned long long* keys, int slots) {
 template <typename Each>
 __device__ unsigned long long sample_select(Each each, unsigned long long lower, unsigned long long ceiling, unsigned int count,
                                             SampleShared& s) {
+    // a call may follow another directly: every wave must have read the last call's prefix, wanted
+    // and exact before they are set anew
+    __syncthreads();
     if (threadIdx.x == 0) {
         s.prefix = 0ull;
         s.wanted = count;

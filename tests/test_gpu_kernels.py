@@ -269,6 +269,67 @@ def test_attention_over_scattered_pages(ops, dtype, nh, nkv, hd, window):
     close(out, want, dtype)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 16, 0), (32, 8, 64, 0), (3, 1, 48, 0), (5, 1, 24, 0), (8, 2, 128, 100), (2, 1, 256, 0)])
+def test_where_the_pages_lie_changes_no_bit_of_any_attention_kernel(ops, nh, nkv, hd, window):
+    """The paging contract of the reference (native/tests/paged_kv_contract.cpp:89-242): the
+    same keys and values under the block table {9, 2, 14, 5} of a pool of 16 pages and under the
+    identity table {0, 1, 2, 3} give the same result bit for bit, from every attention kernel:
+    the wave-per-row one in both precisions, the tiled one (one head and four heads of a group per
+    workgroup), the split-key one, and the one that also forms and writes the step's keys."""
+    T = 250
+    scattered, identity = [9, 2, 14, 5], [0, 1, 2, 3]
+    keys, values = gen(T, nkv, hd).to(torch.bfloat16).double(), gen(T, nkv, hd, seed=1).to(torch.bfloat16).double()
+    scale = 1 / math.sqrt(hd)
+    d = lambda a: torch.tensor(np.asarray(a, dtype=np.int32), device=DEV)       # noqa: E731
+    positions = [0, 1, 62, 63, 64, 65, 127, 128, 129, 200, 249]
+    rows = len(positions)
+    tiled = ops.attention_is_tiled(hd)
+
+    def every_kernel(table_row, dtype):
+        """name -> result of each kernel that takes this head size and precision, over pages
+        laid out by ``table_row``; what no table names is not a number."""
+        k_pages, v_pages = paged(keys, values, table_row, 16, dtype)
+        table = d([table_row])
+        q = as_dev(gen(rows, nh * hd, seed=2), dtype)
+        found = {"generic": ops.attention_generic(q, nh, nkv, hd, k_pages, v_pages, table, d(np.zeros(rows)), d(positions), scale, window)}
+        if dtype != torch.bfloat16 or not tiled:
+            return found
+        # a portion of the sequence: rows 120..249 of the one request, in tiles of 64
+        portion = list(range(120, T))
+        qp = as_dev(gen(len(portion), nh * hd, seed=3), dtype)
+        tile_seg, tile_row0 = ops.query_tiles([0, len(portion)])
+        for together in (1, 4) if hd <= 64 else (1,):
+            found[f"tiled, {together} heads"] = ops.attention_prefill(
+                qp, nh, nkv, hd, k_pages, v_pages, table, d(tile_seg), d(tile_row0), d([0, len(portion)]), d(portion), scale, window,
+                heads_together=together)
+        # decode: one row per request, four requests that share the one table row's pages at different lengths
+        lengths = [250, 129, 64, 1]
+        tables = d([table_row] * len(lengths))
+        qd = as_dev(gen(len(lengths), nh * hd, seed=4), dtype)
+        found["split-key"] = ops.attention_decode(qd, nh, nkv, hd, k_pages, v_pages, tables, d(np.arange(len(lengths))),
+                                                  d([n - 1 for n in lengths]), scale, max_context=256, window=window)
+        # the fused kernel writes the row's own key and value first: one request at position 249
+        qkv = gen(1, (nh + 2 * nkv) * hd, seed=5).float().to(DEV)
+        weight = (1 + 0.1 * gen(hd, seed=6)).float().to(DEV)
+        inv = 1e4 ** (-torch.arange(hd // 2, dtype=torch.float64) * 2 / hd)
+        angle = torch.tensor([T - 1], dtype=torch.float64)[:, None] * inv[None]
+        found["fused"] = ops.attention_decode_fused(qkv, nh, nkv, hd, weight, weight, 1e-5, torch.cos(angle).float().to(DEV),
+                                                    torch.sin(angle).float().to(DEV), hd, k_pages, v_pages, table, d([0]), d([T - 1]),
+                                                    scale, max_context=256, window=window)
+        page = table_row[(T - 1) // 64]
+        found["fused: the key it wrote"] = k_pages[page, :, (T - 1) % 64, :].clone()
+        found["fused: the value it wrote"] = v_pages[page, :, :, (T - 1) % 64].clone()
+        return found
+
+    for dtype in DTYPES:
+        here, there = every_kernel(scattered, dtype), every_kernel(identity, dtype)
+        assert here.keys() == there.keys()
+        assert ("split-key" in here) == (dtype == torch.bfloat16 and tiled)
+        for name in here:
+            assert torch.isfinite(here[name].float()).all(), f"{name} ({dtype}) read a page that no table names"
+            assert torch.equal(here[name], there[name]), f"{name} ({dtype}) depends on where the pages lie"
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_finds_one_far_key_and_the_edges_of_a_window(ops, dtype):
     """One key is made to match the query far better than all others, so the output is

@@ -1,5 +1,6 @@
 """Random tiny configurations against the plain implementation: head sizes in steps of 16 up to
-256, any number of heads and groups, widths and vocabularies that are no power of two, two to five
+256 (and, listed by hand, head sizes and widths that the matrix-core kernels do not take), any
+number of heads and groups, widths and vocabularies that are no power of two, two to five
 layers in any arrangement of the two mixers, two to six taps with and without biases, tied and
 untied heads. Each is stepped whole, in portions with single tokens between them, and as two
 requests of which one decodes beside portions of the other, in float32 and in bfloat16."""
@@ -37,15 +38,13 @@ def random_config(rng) -> dict:
         tie_word_embeddings=bool(rng.integers(0, 2)), max_position_embeddings=512, layer_types=types)
 
 
-@pytest.mark.parametrize("seed", range(12))
-def test_a_random_configuration_matches_the_plain_model(seed):
+def check_configuration(config: dict, seed: int, what: str) -> None:
+    """One configuration against the plain model: whole, in portions, and as two requests of which
+    one decodes beside portions of the other, in float32 and in bfloat16."""
     from flyweight_amd.config import config_from_dict
     from flyweight_amd.engine import StepEntry, Stepper, load_model
     from flyweight_amd.weights import write_random_model
-    rng = np.random.default_rng(1000 + seed)
-    config = random_config(rng)
-    what = (f"head_dim {config['hidden_size'] // config['num_attention_heads']} heads {config['num_attention_heads']}/"
-            f"{config['num_key_value_heads']} layers {config['layer_types']} taps {config['conv_L_cache']}")
+    rng = np.random.default_rng(5000 + seed)
     with tempfile.TemporaryDirectory() as folder:
         write_random_model(folder, config_from_dict(config), seed=seed, scale="fan_in")
         plain_config, plain_weights = plain.read_folder(folder)
@@ -88,6 +87,37 @@ def test_a_random_configuration_matches_the_plain_model(seed):
             stepper.release("b")
             stepper.cache.check_invariants()
             assert stepper.cache.groups[0].pool.in_use == 0
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_a_random_configuration_matches_the_plain_model(seed):
+    config = random_config(np.random.default_rng(1000 + seed))
+    what = (f"head_dim {config['hidden_size'] // config['num_attention_heads']} heads {config['num_attention_heads']}/"
+            f"{config['num_key_value_heads']} layers {config['layer_types']} taps {config['conv_L_cache']}")
+    check_configuration(config, seed, what)
+
+
+# Head sizes that are no multiple of 16 leave the matrix-core attention (bfloat16 too runs on the
+# wave-per-row kernel, its rotation's partner lane half a head away where half is no power of
+# two), widths that are no multiple of 8 leave the matrix-core products (rows of bfloat16 are
+# then not 16-byte aligned), and a feed-forward width that is no multiple of 8 does the same to
+# the product that reads it: (head size, heads, kv heads, feed-forward width).
+ODD_SIZES = [(8, 4, 2, 72), (24, 3, 1, 100), (40, 2, 2, 160), (72, 2, 1, 52), (136, 2, 1, 200),
+             (20, 3, 1, 90), (10, 5, 5, 36), (18, 3, 3, 70), (6, 6, 2, 44)]
+
+
+@pytest.mark.parametrize("head_dim,heads,kv_heads,intermediate", ODD_SIZES)
+def test_head_sizes_and_widths_that_the_matrix_core_kernels_do_not_take(head_dim, heads, kv_heads, intermediate):
+    seed = head_dim
+    rng = np.random.default_rng(seed)
+    config = dict(
+        architectures=["Lfm2ForCausalLM"], model_type="lfm2", vocab_size=int(rng.choice([131, 257, 500])),
+        hidden_size=heads * head_dim, num_hidden_layers=3, num_attention_heads=heads, num_key_value_heads=kv_heads,
+        intermediate_size=intermediate, block_auto_adjust_ff_dim=False, norm_eps=float(rng.choice([1e-5, 1e-6])),
+        rope_theta=float(rng.choice([1e4, 1e6])), conv_L_cache=int(rng.integers(2, 5)), conv_bias=bool(rng.integers(0, 2)),
+        tie_word_embeddings=bool(rng.integers(0, 2)), max_position_embeddings=512,
+        layer_types=["full_attention", "conv", "full_attention"])
+    check_configuration(config, seed, f"head_dim {head_dim} heads {heads}/{kv_heads} hidden {heads * head_dim} ffn {intermediate}")
 
 
 @pytest.mark.parametrize("hidden,heads,intermediate", [(2048, 32, 12288), (1024, 16, 6656)])
