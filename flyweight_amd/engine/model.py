@@ -89,7 +89,7 @@ class CausalLM:
         (``Part.step_arrays``), one for each distinct key."""
         found: Dict = {}
         for block in self.layers:
-            for part in getattr(block, "parts", tuple)():
+            for part in block.parts():
                 key = part.step_arrays_key()
                 if key is not None:
                     found.setdefault(key, part)
@@ -101,20 +101,19 @@ class CausalLM:
         [wanted, vocab] for ``ctx.want_rows`` (None when nothing is wanted)."""
         x = ops.embed_rows(self.embedding, ctx.token_ids, scale=self.spec.embedding_scale)
         schedule = self.spec.schedule
-        ctx.prepared = None
         # A step of single tokens: the final norm reads every row as it is, like a layer's first norm, so
         # the last layer's last product may prepare it; rows that nobody wants cost the head nothing
         # it would not read anyway, and are dropped behind it. (A recorded step computes every row too:
         # what it gives and what the launches give stay bit for bit the same.)
         every_row = bool(ctx.all_decode)
+        prepared = None
         for at, entry in enumerate(schedule):
             # the norm that reads the residual after this layer, for the layer's last product
             if at + 1 < len(schedule):
-                ctx.norm_after_block = getattr(self.layers[schedule[at + 1].layer], "mixer_norm", None)
+                norm_after = self.layers[schedule[at + 1].layer].first_norm()
             else:
-                ctx.norm_after_block = self.final_norm if every_row else None
-            self.layers[entry.layer].forward(x, ctx, ctx.cache_view(cache, entry))
-        prepared, ctx.prepared, ctx.norm_after_block = ctx.prepared, None, None
+                norm_after = self.final_norm if every_row else None
+            prepared = self.layers[entry.layer].forward(x, ctx, ctx.cache_view(cache, entry), prepared=prepared, norm_after=norm_after)
         if ctx.num_wanted == 0:
             return None
         final = LazyNorm(self.final_norm, x, ctx, prepared=prepared) if every_row else LazyNorm(self.final_norm, x, ctx, row_index=ctx.want_rows)

@@ -56,9 +56,19 @@ class Part:
 
     def step_arrays(self, batch) -> Dict[str, "numpy.ndarray"]:
         """name -> int32 array, from ``batch.host_seg_row0`` (first row of each segment, and the
-        end), ``batch.host_row_pos``, ``batch.decode_prefix``, ``batch.num_rows``. For a recorded
-        decode step this is asked once, for segments of one row each."""
+        end), ``batch.host_row_pos``, ``batch.host_seg_slot``, ``batch.decode_prefix``,
+        ``batch.all_decode``, ``batch.num_rows``. For a recorded decode step this is asked once, for
+        segments of one row each at position 0: it fixes the arrays' names and sizes, which may
+        depend on the number of rows alone; what depends on positions or slots is then brought
+        up to date by ``refresh_step_arrays`` before every replay."""
         return {}
+
+    def refresh_step_arrays(self, batch, arrays: Dict[str, "numpy.ndarray"]) -> None:
+        """For a recorded decode step, before each of its uploads: ``arrays`` are the host
+        copies of what ``step_arrays`` returned (name -> int32 numpy array, to be changed in
+        place), ``batch`` has this replay's ``host_row_pos`` and ``host_seg_slot``. When several
+        steps run back to back on the device this is called before the first of them only.
+        The default leaves the arrays as they were built."""
 
 
 class Norm(Part):
@@ -89,6 +99,42 @@ class Mixer(Part):
 class FeedForward(Part):
     def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx):
         """Adds to ``residual`` in place; the return value is as for a mixer."""
+        raise NotImplementedError
+
+
+class Block:
+    """The arrangement of parts in a layer. ``forward(x, ctx, cache, prepared, norm_after)``
+    updates the float32 residual rows ``x`` in place. The model hands over what the layer before
+    prepared for this block's ``first_norm()`` (``prepared``, may be None) and names the norm that
+    reads the residual after this block (``norm_after``, may be None); the block returns what its
+    last product prepared for that norm, or None. An arrangement that ignores both is right, only
+    slower: the norms then run as kernels of their own."""
+
+    graph_safe = False
+
+    def parts(self):
+        """Every part of the block (the model asks them for tensors and step arrays)."""
+        return ()
+
+    def first_norm(self):
+        """The norm that reads the residual stream first in this block, if the block begins with
+        one that a product before it may prepare; else None."""
+        return None
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        declared: Dict[str, TensorDecl] = {}
+        for part in self.parts():
+            declared.update(part.tensors())
+        return declared
+
+    def bind(self, tensors, dtype, device) -> None:
+        for part in self.parts():
+            part.bind(tensors, dtype, device)
+
+    def cache_need(self):
+        return None
+
+    def forward(self, x, ctx, cache, prepared=None, norm_after=None):
         raise NotImplementedError
 
 

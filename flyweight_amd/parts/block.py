@@ -7,15 +7,12 @@ arrangement (post-norm, parallel mixer and feed-forward) is another class regist
 
 from __future__ import annotations
 
-from typing import Dict
-
-from ..weights.loader import TensorDecl
-from .base import build_part, register_block
+from .base import Block, build_part, register_block
 from .norm import LazyNorm
 
 
 @register_block("pre_norm_residual")
-class PreNormResidualBlock:
+class PreNormResidualBlock(Block):
     def __init__(self, spec):
         self.spec = spec
         self.mixer_norm = build_part("norm", spec.mixer_norm)
@@ -26,15 +23,8 @@ class PreNormResidualBlock:
     def parts(self):
         return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
 
-    def tensors(self) -> Dict[str, TensorDecl]:
-        declared: Dict[str, TensorDecl] = {}
-        for part in self.parts():
-            declared.update(part.tensors())
-        return declared
-
-    def bind(self, tensors, dtype, device) -> None:
-        for part in self.parts():
-            part.bind(tensors, dtype, device)
+    def first_norm(self):
+        return self.mixer_norm
 
     def cache_need(self):
         return self.mixer.cache_need()
@@ -44,15 +34,16 @@ class PreNormResidualBlock:
         position = getattr(self.mixer, "position", None)
         return all(part.graph_safe for part in self.parts()) and (position is None or position.graph_safe)
 
-    def forward(self, x, ctx, cache) -> None:
+    def forward(self, x, ctx, cache, prepared=None, norm_after=None):
         """``x`` [rows, hidden] float32 is updated in place."""
         # A part that can take the norm into its own first kernel gets it unevaluated. A part is
         # told which norm reads the residual after it (ctx.upcoming_norm) and may return what its
         # last product prepared for that norm; a part that returns nothing costs a plain norm.
-        h = LazyNorm(self.mixer_norm, x, ctx, prepared=getattr(ctx, "prepared", None))
+        h = LazyNorm(self.mixer_norm, x, ctx, prepared=prepared)
         ctx.upcoming_norm = self.ffn_norm
         prepared = self.mixer.forward(h if getattr(self.mixer, "accepts_lazy_norm", False) else h.tensor(), x, ctx, cache)
         h = LazyNorm(self.ffn_norm, x, ctx, prepared=prepared)
-        ctx.upcoming_norm = getattr(ctx, "norm_after_block", None)
-        ctx.prepared = self.ffn.forward(h if getattr(self.ffn, "accepts_lazy_norm", False) else h.tensor(), x, ctx)
+        ctx.upcoming_norm = norm_after
+        prepared = self.ffn.forward(h if getattr(self.ffn, "accepts_lazy_norm", False) else h.tensor(), x, ctx)
         ctx.upcoming_norm = None
+        return prepared

@@ -40,12 +40,15 @@ CONFIGS = {"A": TINY_A, "B": TINY_B}
 # gated parts multiply up to three rounded numbers. Measured with the straightforward
 # kernels over rows of both tiny models: float32 (rounding 6e-8) is off by at most 4e-6 and
 # 6e-7 in the root mean square; bfloat16 (rounding 2e-3 at every stored activation, four to
-# seven per layer) by 4.5e-2 and 1.1e-2, the same pattern 2^13 times larger. The limits sit
-# about five times above the float32 figures and twice above the bfloat16 ones. The float32
-# run of the same code is what shows the logic right; the bfloat16 limits only have to tell
-# rounding from a fault, and the tests make faults large on purpose.
-MAX_TOL = {"float32": 2e-5, "bfloat16": 1e-1}
-RMS_TOL = {"float32": 4e-6, "bfloat16": 2.5e-2}
+# seven per layer) by 4.5e-2 and 1.1e-2, the same pattern 2^13 times larger. Over every
+# comparison of the GPU tests (some six hundred, many of a single row, whose root mean square
+# is over one row only) the largest are 1.7e-5 and 1.9e-6 in float32, 5.5e-2 and 1.4e-2 in
+# bfloat16. The limits sit a fifth to a quarter above those: a bfloat16 fault of a few per
+# cent of the logits does not pass. The float32 run of the same code is what shows the logic
+# right; the bfloat16 limits have to tell rounding from a fault, and the tests make faults
+# large on purpose.
+MAX_TOL = {"float32": 2e-5, "bfloat16": 7e-2}
+RMS_TOL = {"float32": 4e-6, "bfloat16": 1.8e-2}
 
 
 def make_model(folder: str, name: str, seed: int = 0, scale: str = "fan_in") -> str:

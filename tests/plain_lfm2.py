@@ -197,6 +197,72 @@ def forward(config: dict, w: Dict[str, np.ndarray], tokens: Sequence[int]) -> np
     return h @ head.T
 
 
+# ----- long sequences: the same formulas, by blocks, and only the rows that are compared -----
+def causal_attention_rows(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, first_row: int,
+                          block: int = 512) -> np.ndarray:
+    """``causal_attention`` for the rows from ``first_row`` on only (q holds those rows alone:
+    [T - first_row, nh, hd]; k and v all T), a block of rows against all their keys at a time
+    instead of row by row. Same formulas and citations as ``causal_attention``; the test of the
+    plain model holds the two against each other. (The sums run in float64 through torch's
+    threaded routines: tens of thousands of keys per row, thousands of rows.)"""
+    import torch
+    R, nh, hd = q.shape
+    T, nkv = k.shape[0], k.shape[1]
+    assert first_row + R == T
+    group = nh // nkv
+    out = np.zeros_like(q)
+    keys, values = torch.from_numpy(np.ascontiguousarray(k)), torch.from_numpy(np.ascontiguousarray(v))
+    for start in range(0, R, block):
+        rows = min(block, R - start)
+        last_key = first_row + start + rows             # keys below this index are seen by some row of the block
+        position = torch.arange(first_row + start, first_row + start + rows)[:, None]
+        hidden = torch.arange(last_key)[None, :] > position        # [rows, keys]: the future
+        for kv in range(nkv):
+            queries = torch.from_numpy(np.ascontiguousarray(q[start:start + rows, kv * group:(kv + 1) * group]))   # [rows, group, hd]
+            scores = torch.einsum("rgd,sd->rgs", queries, keys[:last_key, kv]) * scale
+            scores.masked_fill_(hidden[:, None, :], float("-inf"))
+            p = torch.softmax(scores, dim=-1)
+            out[start:start + rows, kv * group:(kv + 1) * group] = torch.einsum("rgs,sd->rgd", p, values[:last_key, kv]).numpy()
+    return out
+
+
+def forward_tail(config: dict, w: Dict[str, np.ndarray], tokens: Sequence[int], last: int) -> np.ndarray:
+    """Logits of the last ``last`` positions of a long sequence, [last, vocab]: ``forward``, with
+    attention by blocks and, from the last attention layer on, only the rows that the wanted ones
+    depend on (each short convolution behind it reaches L - 1 rows further back)."""
+    eps = config["norm_eps"]
+    T = len(tokens)
+    kinds = attention_layers(config)
+    taps = config["conv_L_cache"]
+    last_attention = max((i for i, a in enumerate(kinds) if a), default=-1)
+    convs_behind = sum(1 for a in kinds[last_attention + 1:] if not a)
+    first = max(0, T - last - convs_behind * (taps - 1)) if last_attention >= 0 else 0      # the rows kept from that layer on
+    x = w["model.embed_tokens.weight"][np.asarray(tokens, dtype=np.int64)]
+    kept_from = 0
+    for index, is_attention in enumerate(kinds):
+        base = f"model.layers.{index}."
+        h = rms_norm(x, w[base + "operator_norm.weight"], eps)
+        if is_attention:
+            prefix = base + "self_attn."
+            q, k, v = attention_qkv(h, w, prefix, config, np.arange(T))
+            rows_from = first if index == last_attention else 0
+            out = causal_attention_rows(q[rows_from:], k, v, 1.0 / math.sqrt(q.shape[-1]), rows_from)
+            if index == last_attention:
+                x, kept_from = x[first:], first
+            x = x + out.reshape(out.shape[0], -1) @ w[prefix + "out_proj.weight"].T
+        else:
+            # behind the last attention layer the kept rows begin in mid-sequence: the first L - 1 of them
+            # see zeros where their forerunners were, and are among the rows dropped at the end
+            x = x + short_conv_mixer(h, w, base + "conv.", config)
+        h = rms_norm(x, w[base + "ffn_norm.weight"], eps)
+        x = x + swiglu(h, w, base + "feed_forward.")
+    assert T - kept_from >= last
+    h = rms_norm(x[-last:], w["model.embedding_norm.weight"], eps)
+    tied = config.get("tie_word_embeddings", config.get("tie_embedding", True))
+    head = w["model.embed_tokens.weight"] if tied else w["lm_head.weight"]
+    return h @ head.T
+
+
 def most_likely(logits: np.ndarray) -> int:
     """The largest logit's id; among equal ones the lowest id wins
     (native/include/flyweight_v2_qwen_kernels.hpp:2391-2405: the key orders by value, then by

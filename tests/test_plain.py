@@ -297,3 +297,24 @@ def test_the_mixer_scales_scores_by_one_over_root_head_dim(hd):
     lib = F.scaled_dot_product_attention(tq, tk.repeat_interleave(2, 1), tv.repeat_interleave(2, 1), is_causal=True)
     np.testing.assert_allclose(plain.attention_mixer(h, w, "a.", config), lib[0].transpose(0, 1).reshape(7, 4 * hd).numpy(),
                                rtol=1e-10, atol=1e-12)
+
+
+def test_attention_by_blocks_and_the_tail_of_a_sequence_equal_the_row_by_row_model(tmp_path):
+    """The long-context tests compare with ``forward_tail``: attention by blocks of rows, and
+    behind the last attention layer only the rows that the wanted ones depend on. Both must give
+    what the row-by-row functions give: blocks that end inside the sequence, a first row in
+    mid-sequence, groups of heads, and both tiny models whole (in B two convolution layers
+    follow the last attention layer and reach six rows back)."""
+    T, nh, nkv, hd = 150, 6, 2, 16
+    q, k, v = RNG.standard_normal((T, nh, hd)), RNG.standard_normal((T, nkv, hd)), RNG.standard_normal((T, nkv, hd))
+    whole = plain.causal_attention(q, k, v, 0.3)
+    for first_row, block in ((0, 64), (0, 150), (97, 16), (149, 512)):
+        rows = plain.causal_attention_rows(q[first_row:], k, v, 0.3, first_row, block=block)
+        np.testing.assert_allclose(rows, whole[first_row:], rtol=1e-11, atol=1e-13)
+    for name in ("A", "B"):
+        folder = make_model(str(tmp_path / name), name, seed=5)
+        config, w = plain.read_folder(folder)
+        tokens = random_tokens(config["vocab_size"], 90, 2)
+        logits = plain.forward(config, w, tokens)
+        for last in (1, 17, 90):
+            np.testing.assert_allclose(plain.forward_tail(config, w, tokens, last), logits[-last:], rtol=1e-9, atol=1e-11)
