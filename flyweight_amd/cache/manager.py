@@ -99,16 +99,16 @@ class PageGroup:
 
 
 class CacheManager:
-    def __init__(self, needs: Mapping[int, object], num_pages: int, max_requests: int, page_size: int = 64,
+    def __init__(self, needs: Mapping[int, object], num_pages, max_requests: int, page_size: int = 64,
                  max_pages_per_request: Optional[int] = None, dtype: torch.dtype = torch.float32,
                  device: Optional[torch.device] = None):
         """``needs``: cache entry id -> a :class:`CacheNeed` (``PagedKV``, ``FixedState`` or a
-        class of the mixer's own). ``num_pages``: pages of every page group. ``device`` None keeps
-        the bookkeeping only (no storage)."""
+        class of the mixer's own). ``num_pages``: pages of every page group, or a mapping from a
+        group's key (``need.group_key()``) to the pages of that group, with ``None`` as the key of
+        all others: a group that keeps a window of keys needs far fewer pages than one that keeps
+        them all. ``device`` None keeps the bookkeeping only (no storage)."""
         self.page_size = page_size
-        self.num_pages = num_pages
         self.max_requests = max_requests
-        self.max_pages_per_request = max_pages_per_request or num_pages
         self.dtype = dtype
         self.device = device
         self.groups: List[PageGroup] = []
@@ -128,11 +128,32 @@ class CacheManager:
                 self.entry_group[entry] = list(grouped).index(need.group_key())
             else:
                 self.state_entries[entry] = need
+        # pages of each group
+        if isinstance(num_pages, Mapping):
+            unknown = [key for key in num_pages if key is not None and key not in grouped]
+            if unknown:
+                raise ValueError(f"pages are given for page groups that do not exist: {unknown}; the groups are {list(grouped)}")
+            missing = [key for key in grouped if key not in num_pages and None not in num_pages]
+            if missing:
+                raise ValueError(f"no number of pages is given for the page groups {missing}")
+            self.group_pages = [int(num_pages[key] if key in num_pages else num_pages[None]) for key in grouped]
+            default_pages = int(num_pages[None]) if None in num_pages else max(self.group_pages, default=1)
+        else:
+            self.group_pages = [int(num_pages)] * len(grouped)
+            default_pages = int(num_pages)
+        # what bounds one sequence: the smallest pool among the groups that keep every key
+        keeping_all = [pages for pages, (need, _) in zip(self.group_pages, grouped.values()) if not need.window]
+        self.num_pages = min(keeping_all) if keeping_all else (max(self.group_pages) if self.group_pages else default_pages)
+        self.max_pages_per_request = max_pages_per_request or max(self.group_pages, default=default_pages)
         # the bookkeeping lives in the host library
         self._lib = host.library()
         windows = (ctypes.c_int * max(len(grouped), 1))(*[int(need.window or 0) for need, _ in grouped.values()])
-        self._native = self._lib.fwh_cache_create(len(grouped), windows, num_pages, max_requests, page_size,
-                                                  self.max_pages_per_request)
+        if grouped:
+            pages = (ctypes.c_int * len(grouped))(*self.group_pages)
+            self._native = self._lib.fwh_cache_create_sized(len(grouped), windows, pages, max_requests, page_size,
+                                                            self.max_pages_per_request)
+        else:
+            self._native = self._lib.fwh_cache_create(0, windows, default_pages, max_requests, page_size, self.max_pages_per_request)
         if not self._native:
             raise ValueError(host.last_error())
         for index, (key, (need, entries)) in enumerate(grouped.items()):
@@ -143,9 +164,10 @@ class CacheManager:
         self._ids: Dict[Hashable, int] = {}         # keys that are not small integers -> ids of the host library
         self._keys: Dict[int, Hashable] = {}
         self._next_named = _FIRST_NAMED_ID
-        # One page and one slot lie behind those the pools hand out: rows that only fill a step up to
-        # a size it was recorded for (see Stepper.planned_decode) write there, and nobody reads it.
-        self.spare_page = num_pages
+        # One page of every group and one slot lie behind those the pools hand out: rows that only fill
+        # a step up to a size it was recorded for (see Stepper.planned_decode) write there, and nobody
+        # reads it.
+        self.spare_pages = list(self.group_pages)
         self.spare_slot = max_requests
         # storage: each need allocates its own
         self.storage: Dict[int, object] = {}
@@ -153,7 +175,7 @@ class CacheManager:
         if device is not None:
             for entry, need in self.needs.items():
                 if need.paged:
-                    self.storage[entry] = need.allocate(num_pages + 1, page_size, dtype, device)
+                    self.storage[entry] = need.allocate(self.group_pages[self.entry_group[entry]] + 1, page_size, dtype, device)
             alike: List[Tuple[CacheNeed, List[int]]] = []       # fixed-size entries whose needs are equal
             for entry, need in self.state_entries.items():
                 for other, entries in alike:
@@ -381,7 +403,7 @@ class CacheManager:
 
     def stats(self) -> Dict[str, int]:
         return {
-            "pages_total": self.num_pages,
+            "pages_total": self.num_pages,        # of the tightest group that keeps every key
             "pages_free": self.free_pages() if self.groups else self.num_pages,
             "pages_peak": max((g.pool.peak_in_use for g in self.groups), default=0),
             "slots_free": self.slots.free_count,

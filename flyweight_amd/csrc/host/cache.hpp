@@ -65,12 +65,26 @@ struct Live {
 
 class Cache {
 public:
-    Cache(const std::vector<int>& windows, int num_pages, int max_requests, int page_size, int max_pages_per_request)
-        : page_size_(page_size), num_pages_(num_pages), max_requests_(max_requests),
-          max_pages_per_request_(max_pages_per_request > 0 ? max_pages_per_request : num_pages), slots_(max_requests) {
-        if (page_size <= 0 || num_pages <= 0) throw std::invalid_argument("page size and page count must be positive");
+    // pages: one pool size for every group, or one per group (a group that keeps a window of keys
+    // needs far fewer pages than one that keeps them all).
+    Cache(const std::vector<int>& windows, const std::vector<int>& pages, int max_requests, int page_size, int max_pages_per_request)
+        : page_size_(page_size), max_requests_(max_requests), slots_(max_requests) {
+        if (pages.size() != 1 && pages.size() != windows.size())
+            throw std::invalid_argument("page counts: one for all groups or one per group");
         groups_.reserve(windows.size());
-        for (int window : windows) groups_.emplace_back(window, num_pages);
+        int largest = 0;
+        num_pages_ = 0;
+        for (size_t g = 0; g < windows.size() || g < 1; ++g) {
+            const int count = pages[pages.size() == 1 ? 0 : g];
+            if (page_size <= 0 || count <= 0) throw std::invalid_argument("page size and page count must be positive");
+            largest = count > largest ? count : largest;
+            // what bounds a sequence: the smallest pool among the groups that keep every key
+            const bool keeps_all = g >= windows.size() || windows[g] <= 0;
+            if (keeps_all && (num_pages_ == 0 || count < num_pages_)) num_pages_ = count;
+            if (g < windows.size()) groups_.emplace_back(windows[g], count);
+        }
+        if (num_pages_ == 0) num_pages_ = largest;
+        max_pages_per_request_ = max_pages_per_request > 0 ? max_pages_per_request : largest;
     }
 
     int page_size() const { return page_size_; }
@@ -217,7 +231,7 @@ public:
     // No page lost, none held twice; slots likewise.
     void check() const {
         for (const Group& group : groups_) {
-            std::vector<char> seen(num_pages_, 0);
+            std::vector<char> seen(group.pool.size(), 0);
             int held = 0;
             for (const auto& entry : group.tables) {
                 if (!live_.count(entry.first)) throw AccountingError("block tables and live requests differ");

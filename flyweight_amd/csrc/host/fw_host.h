@@ -33,6 +33,9 @@ int fwh_pool_is_held(void* pool, int id);
 // ---- the cache: page groups (window 0: every key is kept), block tables, slots --------------------
 void* fwh_cache_create(int num_groups, const int* windows, int num_pages, int max_requests, int page_size,
                        int max_pages_per_request);
+// the same with a pool size per group (a group that keeps a window needs fewer pages than one that keeps every key)
+void* fwh_cache_create_sized(int num_groups, const int* windows, const int* pages, int max_requests, int page_size,
+                             int max_pages_per_request);
 void fwh_cache_destroy(void* cache);
 void* fwh_cache_group_pool(void* cache, int group);     // borrowed: lives as long as the cache
 void* fwh_cache_slot_pool(void* cache);

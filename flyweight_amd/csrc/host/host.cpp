@@ -38,7 +38,7 @@ int copy_ids(const std::vector<fwh::Request*>& from, int64_t* to) {
 extern "C" {
 
 const char* fwh_last_error(void) { return last_error.c_str(); }
-int fwh_abi_version(void) { return 3; }
+int fwh_abi_version(void) { return 4; }
 
 // ---- pools ---------------------------------------------------------------------------------
 void* fwh_pool_create(int size) {
@@ -59,7 +59,19 @@ void* fwh_cache_create(int num_groups, const int* windows, int num_pages, int ma
                        int max_pages_per_request) {
     void* made = nullptr;
     guarded([&] {
-        made = new fwh::Cache(std::vector<int>(windows, windows + num_groups), num_pages, max_requests, page_size, max_pages_per_request);
+        made = new fwh::Cache(std::vector<int>(windows, windows + num_groups), std::vector<int>{num_pages}, max_requests, page_size,
+                              max_pages_per_request);
+        return 0;
+    });
+    return made;
+}
+void* fwh_cache_create_sized(int num_groups, const int* windows, const int* pages, int max_requests, int page_size,
+                             int max_pages_per_request) {
+    void* made = nullptr;
+    guarded([&] {
+        if (num_groups < 1) throw std::invalid_argument("a cache sized per group needs at least one group");
+        made = new fwh::Cache(std::vector<int>(windows, windows + num_groups), std::vector<int>(pages, pages + num_groups), max_requests,
+                              page_size, max_pages_per_request);
         return 0;
     });
     return made;

@@ -46,12 +46,15 @@ void pools() {
     EXPECT(fwh_pool_create(0) == nullptr && std::strlen(fwh_last_error()) > 0);
 }
 
-// Random lifetimes over a cache with one plain and one windowed group; a model of lengths is kept
-// beside it and the library's own check runs after every change.
+// Random lifetimes over a cache with one plain and one windowed group (on odd seeds the windowed
+// group has a smaller pool of its own); a model of lengths is kept beside it and the library's
+// own check runs after every change.
 void cache_lifetimes(uint64_t seed) {
     const int pages = 24, slots = 5, page = 64, window = 100;
+    const int windowed_pages = seed % 2 ? 9 : pages;
     const int windows[2] = {0, window};
-    void* cache = fwh_cache_create(2, windows, pages, slots, page, 0);
+    const int sizes[2] = {pages, windowed_pages};
+    void* cache = seed % 2 ? fwh_cache_create_sized(2, windows, sizes, slots, page, 0) : fwh_cache_create(2, windows, pages, slots, page, 0);
     EXPECT(cache != nullptr);
     Random random(seed);
     std::map<int64_t, int> length;      // live request -> committed length
@@ -107,11 +110,12 @@ void cache_lifetimes(uint64_t seed) {
             const int windowed = fwh_cache_table(cache, entry.first, 1, table, 64);
             const int passed = entry.second - window + 1 > 0 ? (entry.second - window + 1) / page : 0;
             for (int b = 0; b < windowed && b < 64; ++b) EXPECT((table[b] == FWH_NO_PAGE) == (b < passed));
+            for (int b = 0; b < windowed && b < 64; ++b) EXPECT(table[b] < windowed_pages);
         }
     }
     for (const auto& entry : length) EXPECT(fwh_cache_release(cache, entry.first) == 0);
     EXPECT(fwh_pool_free_count(fwh_cache_group_pool(cache, 0)) == pages);
-    EXPECT(fwh_pool_free_count(fwh_cache_group_pool(cache, 1)) == pages);
+    EXPECT(fwh_pool_free_count(fwh_cache_group_pool(cache, 1)) == windowed_pages);
     EXPECT(fwh_pool_free_count(fwh_cache_slot_pool(cache)) == slots);
     fwh_cache_destroy(cache);
 }

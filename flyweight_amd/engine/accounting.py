@@ -87,7 +87,7 @@ def cache_bytes_per_token(cache) -> int:
     total = 0
     for entry, need in cache.needs.items():
         if need.paged:
-            total += _bytes(_tensors([cache.storage[entry]])) // ((cache.num_pages + 1) * cache.page_size)
+            total += _bytes(_tensors([cache.storage[entry]])) // ((cache.group_pages[cache.entry_group[entry]] + 1) * cache.page_size)
     return total
 
 

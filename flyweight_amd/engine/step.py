@@ -135,10 +135,10 @@ class StepContext:
     """The batch as the kernels see it: per-row and per-segment index arrays on the
     device (one upload), block tables per page group, per-step tables of the position
     encodings, and whatever index arrays the model's parts ask for (``Part.step_arrays``: built
-    on the host from the batch, they travel in the same upload)."""
+    on the host from the batch, they travel in the same upload; a recorded step lets the parts
+    bring theirs up to date before every replay, ``Part.refresh_step_arrays``)."""
 
-    FIXED = 7       # tokens, positions, segment of each row, first row of each segment, slots, wanted rows, decode work
-    RUN_OF_KEYS = 256       # decode attention shares a row's keys out in runs of four pages
+    FIXED = 6       # tokens, positions, segment of each row, first row of each segment, slots, wanted rows
 
     def __init__(self, entries: Sequence[StepEntry], cache: CacheManager, device: torch.device, vocab_size: int,
                  max_positions: int, described=None, providers: Sequence = (), staging: Optional[_Staging] = None):
@@ -188,11 +188,7 @@ class StepContext:
         self.host_seg_slot = seg_slot
 
         tables = [cache.block_table_rows(g, self.requests, natives=natives) for g in range(len(cache.groups))]
-        # how many runs of keys the rows that go to the decode kernels see together: those kernels share
-        # the work out over the chip by it (a long row among short ones gets more workgroups)
-        single = self.num_rows if self.all_decode else self.decode_prefix
-        decode_work = [int(np.sum((row_pos[:single].astype(np.int64) + self.RUN_OF_KEYS) // self.RUN_OF_KEYS))]
-        pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows, decode_work)]
+        pieces = [np.asarray(a, dtype=np.int32) for a in (tokens, row_pos, row_seg, seg_row0, seg_slot, want_rows)]
         pieces += [t.reshape(-1) for t in tables]
         if given_positions:
             pieces.append(np.concatenate(encoding_parts))
@@ -204,7 +200,7 @@ class StepContext:
         for piece in pieces:
             views.append(packed[offset:offset + piece.size])
             offset += piece.size
-        self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows, self.decode_work = views[:self.FIXED]
+        self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows = views[:self.FIXED]
         self.block_tables = [v.view(t.shape) for v, t in zip(views[self.FIXED:], tables)]
         at = self.FIXED + len(tables)
         # what the position encodings see: the places in the sequences, unless the entries say otherwise
@@ -226,12 +222,18 @@ class StepContext:
                 asked.append((key, name, np.ascontiguousarray(array, dtype=np.int32).reshape(-1)))
         return asked
 
+    def _refresh_parts(self) -> None:
+        """A recorded step: the parts bring their own arrays up to date with this replay's
+        positions and slots, in the pinned buffer that the upload takes."""
+        for part, arrays in self._provider_arrays:
+            part.refresh_step_arrays(self, arrays)
+
     def step_arrays(self, part) -> Dict[str, torch.Tensor]:
         """The device copies of what ``part.step_arrays`` built for this step. A part that was
         not among the step's providers gets them made now, with an upload of their own."""
         key = part.step_arrays_key()
         if key not in self._arrays:
-            if self.host_seg_row0 is None:
+            if getattr(self, "_provider_arrays", None) is not None:
                 raise StepError("a recorded step holds only the arrays of the parts it was built with")
             self._arrays[key] = {name: torch.from_numpy(np.ascontiguousarray(array, dtype=np.int32)).to(self.device)
                                  for name, array in part.step_arrays(self).items()}
@@ -242,8 +244,9 @@ class StepContext:
                          table_stride: int, providers: Sequence = ()) -> "StepContext":
         """A context of ``batch`` single-token segments whose index arrays live in ONE
         persistent device buffer, refreshed before every replay of the captured step. The parts'
-        own arrays are built once, for ``batch`` segments of one row each: a part whose arrays
-        depend on more than that (on positions, say) must not call itself ``graph_safe``."""
+        own arrays are built once, for ``batch`` segments of one row each at position 0 (that fixes
+        their sizes), and brought up to date by the parts before every upload
+        (``Part.refresh_step_arrays``)."""
         self = cls.__new__(cls)
         self.num_rows = self.num_segments = self.num_wanted = batch
         self.wants_every_row = True
@@ -257,8 +260,7 @@ class StepContext:
         self.host_seg_row0 = list(range(batch + 1))
         self.host_seg_slot = [0] * batch
         extra = self._ask(providers)
-        self.host_row_pos = self.host_seg_row0 = self.host_seg_slot = None     # not for captured steps
-        sizes = [batch, batch, batch, batch + 1, batch, batch, 1] + [batch * table_stride] * groups
+        sizes = [batch, batch, batch, batch + 1, batch, batch] + [batch * table_stride] * groups
         sizes += [array.size for _, _, array in extra]
         self.host_buffer = torch.empty(max(sum(sizes), 1), dtype=torch.int32, pin_memory=True)
         self.device_buffer = torch.zeros(max(sum(sizes), 1), dtype=torch.int32, device=device)
@@ -267,21 +269,28 @@ class StepContext:
             views.append(self.device_buffer[offset:offset + size])
             host_views.append(self.host_buffer[offset:offset + size].numpy())
             offset += size
-        self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows, self.decode_work = views[:cls.FIXED]
+        self.token_ids, self.row_pos, self.row_seg, self.seg_row0, self.seg_slot, self.want_rows = views[:cls.FIXED]
         self.encoding_pos = self.row_pos
         self.block_tables = [v.view(batch, table_stride) for v in views[cls.FIXED:cls.FIXED + groups]]
         self._host = host_views
         self._host_tables = host_views[cls.FIXED:cls.FIXED + groups]
         self._table_stride = table_stride
+        # what the parts see of a replay on the host: its positions and slots, where the upload takes them
+        self.host_row_pos = host_views[1]
+        self.host_seg_slot = host_views[4]
         # what never changes between replays
         rows = np.arange(batch, dtype=np.int32)
+        host_views[1][:] = 0
         host_views[2][:] = rows
         host_views[3][:] = np.arange(batch + 1, dtype=np.int32)
         host_views[5][:] = rows
         self._arrays = {}
+        by_part: Dict = {}
         for (key, name, array), view, host_view in zip(extra, views[cls.FIXED + groups:], host_views[cls.FIXED + groups:]):
             host_view[:] = array
             self._arrays.setdefault(key, {})[name] = view
+            by_part.setdefault(key, {})[name] = host_view
+        self._provider_arrays = [(part, by_part.get(part.step_arrays_key(), {})) for part in providers]
         self._position_tables = {}
         return self
 
@@ -299,9 +308,9 @@ class StepContext:
         host[0][:] = [int(e.tokens[0]) for e in entries]
         host[1][:] = starts
         host[4][:] = slots
-        self._count_decode_work()
         for g, rows in enumerate(self._host_tables):
             rows[:] = cache.block_table_rows(g, self.requests, stride=self._table_stride, natives=natives).reshape(-1)
+        self._refresh_parts()
         self.upload()
 
     def wait_uploaded(self) -> None:
@@ -330,12 +339,8 @@ class StepContext:
         if rows < 0:
             return -1
         self.fill_up(rows, cache)
-        self._count_decode_work()
+        self._refresh_parts()
         return rows
-
-    def _count_decode_work(self) -> None:
-        host = self._host
-        host[6][0] = int(np.sum((host[1].astype(np.int64) + self.RUN_OF_KEYS) // self.RUN_OF_KEYS))
 
     def fill_up(self, rows: int, cache: CacheManager) -> None:
         """Rows behind the plan's (a step recorded for more requests than the plan has): token 0
@@ -346,8 +351,8 @@ class StepContext:
         host[0][rows:] = 0
         host[1][rows:] = 0
         host[4][rows:] = cache.spare_slot
-        for table in self._host_tables:
-            table[rows * self._table_stride:] = cache.spare_page
+        for group, table in enumerate(self._host_tables):
+            table[rows * self._table_stride:] = cache.spare_pages[group]
 
     def position_tables(self, part):
         key = part.key()
@@ -369,9 +374,10 @@ class Stepper:
     """Owns the model's cache and runs steps. ``admit`` a request before its first step,
     ``release`` it when it ends."""
 
-    def __init__(self, model: CausalLM, num_pages: int, max_requests: int, page_size: int = 64,
+    def __init__(self, model: CausalLM, num_pages, max_requests: int, page_size: int = 64,
                  context_limit: Optional[int] = None):
-        """``context_limit``: the most tokens one request may reach here, at most the model's
+        """``num_pages``: cache pages per page group, one number or a mapping by group
+        (``CacheManager``). ``context_limit``: the most tokens one request may reach here, at most the model's
         own limit (the default). Block tables and everything sized by a sequence's length follow
         this number, not the model's: a model that allows 128,000 positions costs a run of 4,096
         no more than one that allows 4,096."""

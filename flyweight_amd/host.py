@@ -11,7 +11,7 @@ from .kernels.build import ensure_host_built
 
 ERROR, OUT_OF_PAGES, NO_PAGE = -1, -2, -1
 NOT_DECODE_ONLY = -3
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _LIB: Optional[ctypes.CDLL] = None
 _INTS, _IDS = POINTER(c_int), POINTER(c_int64)
@@ -28,6 +28,7 @@ _SIGNATURES = {
     "fwh_pool_peak": (c_int, [c_void_p]),
     "fwh_pool_is_held": (c_int, [c_void_p, c_int]),
     "fwh_cache_create": (c_void_p, [c_int, _INTS, c_int, c_int, c_int, c_int]),
+    "fwh_cache_create_sized": (c_void_p, [c_int, _INTS, _INTS, c_int, c_int, c_int]),
     "fwh_cache_destroy": (None, [c_void_p]),
     "fwh_cache_group_pool": (c_void_p, [c_void_p, c_int]),
     "fwh_cache_slot_pool": (c_void_p, [c_void_p]),

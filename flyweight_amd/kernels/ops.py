@@ -962,17 +962,18 @@ def attention_is_tiled(head_dim: int) -> bool:
 
 def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
               v_pages: torch.Tensor, block_table: torch.Tensor, ctx, scale: float, window: int = 0,
-              tile_seg: Optional[torch.Tensor] = None, tile_row0: Optional[torch.Tensor] = None) -> torch.Tensor:
+              tile_seg: Optional[torch.Tensor] = None, tile_row0: Optional[torch.Tensor] = None,
+              decode_work: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bfloat16 with a head size in steps of 16 runs on the matrix cores: the split-key decode
     kernel for segments of one row (all of them, or those a mixed step begins with: a single row
     would hold a 64-row tile of the prompt kernel and walk its whole context alone), the tiled
     kernel for the rest (``tile_seg``, ``tile_row0``: the tiles of ``query_tiles`` in the order
-    workgroups take them, those of the leading single rows in front); float32 and everything
-    else on the generic kernel."""
+    workgroups take them, those of the leading single rows in front; ``decode_work``: see
+    ``attention_decode``); float32 and everything else on the generic kernel."""
     fast = q.dtype == torch.bfloat16 and attention_is_tiled(head_dim)
     if fast and ctx.all_decode:
         return attention_decode(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                                ctx.row_pos, scale, ctx.max_context, window, decode_work=getattr(ctx, "decode_work", None))
+                                ctx.row_pos, scale, ctx.max_context, window, decode_work=decode_work)
     if fast:
         if tile_seg is None or tile_row0 is None:
             raise KernelError("attention: the tiled kernel needs the step's query tiles")
@@ -988,7 +989,7 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                                      tile_row0, ctx.seg_row0, ctx.row_pos, scale, window, heads_together=together)
         out = torch.empty_like(q)
         attention_decode(q[:single], num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                         ctx.row_pos, scale, ctx.max_context, window, out=out[:single], decode_work=getattr(ctx, "decode_work", None))
+                         ctx.row_pos, scale, ctx.max_context, window, out=out[:single], decode_work=decode_work)
         return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table,
                                  tile_seg[single:], tile_row0[single:], ctx.seg_row0, ctx.row_pos, scale, window,
                                  heads_together=together, out=out)

@@ -91,11 +91,21 @@ class GQAttention(Mixer):
         self.q_norm_weight = tensors[self._name("q_norm")] if self.qk_norm else None
         self.k_norm_weight = tensors[self._name("k_norm")] if self.qk_norm else None
 
-    # The prompt kernel on the matrix cores works on tiles of up to 64 rows of one segment; which
-    # tiles there are, and in which order workgroups take them, is this part's business.
+    # The kernels on the matrix cores need index arrays of this part's own. The prompt kernel works
+    # on tiles of up to 64 rows of one segment: which tiles there are, and in which order workgroups
+    # take them. The split-key decode kernel shares a step's work out over the chip by the number of
+    # runs of keys (four pages each) that all the rows it serves see together: a long row among
+    # short ones gets more workgroups, and a recorded step adapts as its requests grow.
+    RUN_OF_KEYS = ops.DECODE_SPLIT_PAGES * ops.PAGE_SIZE
+
     def step_arrays_key(self):
         fast = getattr(self, "dtype", None) == torch.bfloat16 and ops.attention_is_tiled(self.head_dim)
-        return ("query_tiles", ops.QUERY_TILE) if fast else None
+        return ("query_tiles", ops.QUERY_TILE, self.RUN_OF_KEYS) if fast else None
+
+    def _decode_work(self, batch) -> int:
+        single = batch.num_rows if batch.all_decode else batch.decode_prefix    # the rows that go to the decode kernel
+        positions = np.asarray(batch.host_row_pos[:single], dtype=np.int64)
+        return int(np.sum((positions + self.RUN_OF_KEYS) // self.RUN_OF_KEYS))
 
     def step_arrays(self, batch):
         seg_row0 = batch.host_seg_row0
@@ -103,32 +113,36 @@ class GQAttention(Mixer):
         # Workgroups start in the order of the tiles: those that see the most keys go first, the short
         # ones fill in behind. The tiles of the leading single rows stay in front (they go to the
         # decode kernel and their tiles are skipped).
-        if len(tile_seg) - batch.decode_prefix > 1:
+        if len(tile_seg) - batch.decode_prefix > 1 and not batch.all_decode:
             tile_seg, tile_row0 = np.asarray(tile_seg, dtype=np.int32), np.asarray(tile_row0, dtype=np.int32)
             tile_end = np.minimum(tile_row0 + ops.QUERY_TILE, np.asarray(seg_row0, dtype=np.int32)[tile_seg + 1])
             keys_seen = batch.host_row_pos[tile_end - 1].astype(np.int64)
             keys_seen[:batch.decode_prefix] = np.iinfo(np.int64).max
             order = np.argsort(-keys_seen, kind="stable")
             tile_seg, tile_row0 = tile_seg[order], tile_row0[order]
-        return {"tile_seg": np.asarray(tile_seg, dtype=np.int32), "tile_row0": np.asarray(tile_row0, dtype=np.int32)}
+        return {"tile_seg": np.asarray(tile_seg, dtype=np.int32), "tile_row0": np.asarray(tile_row0, dtype=np.int32),
+                "decode_work": np.asarray([self._decode_work(batch)], dtype=np.int32)}
+
+    def refresh_step_arrays(self, batch, arrays) -> None:
+        arrays["decode_work"][0] = self._decode_work(batch)     # the tiles of single rows never change
 
     def forward(self, h, residual, ctx, cache):
         qkv = self.qkv.forward(h, out_dtype=torch.float32)      # normed, rotated and rounded once, below
         cos, sin = ctx.position_tables(self.position)
+        own = ctx.step_arrays(self) if self.step_arrays_key() is not None else {}
         if ctx.all_decode and ctx.num_rows <= self.FUSED_DECODE_ROWS and qkv.dtype == torch.float32 and self.step_arrays_key() is not None:
             # a few single-token segments on the matrix cores: norm, rotation, cache write and attention in one kernel
             attended = ops.attention_decode_fused(
                 qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight, self.qk_norm_eps,
                 cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table, ctx.row_seg, ctx.row_pos,
                 self.scale, ctx.max_context, int(self.window or 0), write_kv=cache.writes,
-                decode_work=getattr(ctx, "decode_work", None))
+                decode_work=own.get("decode_work"))
             return self.out.accumulate(attended, residual, then=getattr(ctx, "upcoming_norm", None))
         q = ops.qk_norm_rope_kv_write(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight,
             self.qk_norm_eps, cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table,
             ctx.row_seg, ctx.row_pos, write_kv=cache.writes)
-        tiles = ctx.step_arrays(self) if self.step_arrays_key() is not None else {}
         attended = ops.attention(q, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
                                  cache.block_table, ctx, self.scale, int(self.window or 0),
-                                 tile_seg=tiles.get("tile_seg"), tile_row0=tiles.get("tile_row0"))
+                                 tile_seg=own.get("tile_seg"), tile_row0=own.get("tile_row0"), decode_work=own.get("decode_work"))
         return self.out.accumulate(attended, residual, then=getattr(ctx, "upcoming_norm", None))

@@ -185,6 +185,40 @@ def test_window_group_gives_back_the_pages_its_window_has_passed():
     assert table.shape == (1, 4) and table.dtype.name == "int32" and (table >= 0).all()
 
 
+def test_page_groups_are_sized_apart():
+    """A group that keeps a window of keys beside one that keeps them all: each has a pool of its
+    own size, a sequence is bounded by the group that keeps everything, and the windowed group
+    serves it from a handful of pages that it keeps giving back."""
+    window, full = PagedKV(1, 16, window=70), PagedKV(1, 16)
+    cache = CacheManager({0: window, 1: full}, num_pages={window.group_key(): 3, full.group_key(): 10}, max_requests=2)
+    windowed_group, full_group = cache.groups
+    assert (windowed_group.pool.num_pages, full_group.pool.num_pages) == (3, 10)
+    assert cache.num_pages == 10 and cache.group_pages == [3, 10] and cache.spare_pages == [3, 10]
+    cache.admit("r")
+    for length in range(60, 640, 60):       # portions of 60 tokens: the window never needs more than 3 pages at once
+        cache.reserve("r", length)
+        cache.commit("r", length)
+        cache.check_invariants()
+    assert full_group.pool.in_use == 10 and windowed_group.pool.in_use <= 3
+    with pytest.raises(OutOfPages):
+        cache.reserve("r", 641)             # the eleventh page of the group that keeps every key
+    cache.release("r")
+    assert windowed_group.pool.in_use == 0 and full_group.pool.in_use == 0
+    # a portion that the windowed group cannot hold at once is refused whole: neither group changes
+    cache.admit("s")
+    with pytest.raises(OutOfPages):
+        cache.reserve("s", 4 * 64)
+    assert windowed_group.pool.in_use == 0 and full_group.pool.in_use == 0
+    cache.check_invariants()
+    # one number for the others, and names that match no group are refused
+    other = CacheManager({0: window, 1: full}, num_pages={window.group_key(): 2, None: 7}, max_requests=1)
+    assert other.group_pages == [2, 7]
+    with pytest.raises(ValueError, match="do not exist"):
+        CacheManager({0: full}, num_pages={window.group_key(): 2, None: 7}, max_requests=1)
+    with pytest.raises(ValueError, match="no number of pages"):
+        CacheManager({0: window, 1: full}, num_pages={window.group_key(): 2}, max_requests=1)
+
+
 def test_misuse_is_refused():
     cache = CacheManager({0: KV}, num_pages=2, max_requests=1)
     cache.admit("a")

@@ -333,6 +333,110 @@ def test_a_toy_mixer_with_its_own_state_is_registered_built_and_stepped(tmp_path
     assert np.abs(again - expected(a[:20])).max() <= tolerance * np.abs(expected(a[:20])).max()
 
 
+def register_toy_gate():
+    from flyweight_amd.parts import Linear, Mixer, register_mixer
+    from flyweight_amd.weights import TensorDecl
+
+    @register_mixer("toy_position_gate")
+    class PositionGate(Mixer):
+        """out_t = W . (h_t * (1 + position_t mod 5)): the factor is built on the host from the rows'
+        positions, an index array of the part's own that travels with every step's upload. The
+        part launches device work only, so decode steps of a model that holds it are recorded;
+        before each replay it brings its array up to date."""
+        graph_safe = True
+        refreshed = 0
+
+        def __init__(self, spec):
+            super().__init__(spec)
+            self.hidden = int(spec["hidden_size"])
+
+        def tensors(self):
+            return {self.prefix + "mix.weight": TensorDecl((self.hidden, self.hidden))}
+
+        def bind(self, tensors, dtype, device):
+            super().bind(tensors, dtype, device)
+            self.mix = Linear(tensors[self.prefix + "mix.weight"])
+
+        def step_arrays_key(self):
+            return ("toy_position_gate",)
+
+        def step_arrays(self, batch):
+            return {"gate": 1 + np.asarray(batch.host_row_pos, dtype=np.int32) % 5}
+
+        def refresh_step_arrays(self, batch, arrays):
+            arrays["gate"][:] = 1 + np.asarray(batch.host_row_pos, dtype=np.int32) % 5
+            type(self).refreshed += 1
+
+        def forward(self, h, residual, ctx, cache):
+            gate = ctx.step_arrays(self)["gate"]
+            self.mix.accumulate((h.float() * gate[:, None].float()).to(h.dtype), residual)
+    return PositionGate
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_toy_mixer_whose_index_array_depends_on_positions_is_replayed_from_recorded_steps(tmp_path, dtype):
+    """A part's own index arrays may depend on the rows' positions and still ride in recorded
+    decode steps: the step asks the part to refresh them before every replay. The logits are
+    those of the plain computation, and bit for bit those of the same steps launched one by one."""
+    from flyweight_amd.config import PartSpec, ScheduleEntry, config_from_dict
+    from flyweight_amd.engine import CausalLM, StepEntry, Stepper
+    from flyweight_amd.engine.model import parse_dtype
+    from flyweight_amd.weights import load_tensors, random_tensors, write_file
+    from helpers import TINY_A
+    gate_class = register_toy_gate()
+    base = config_from_dict(TINY_A).model_spec()
+    toy_layer = dataclasses.replace(base.layers[0], mixer=PartSpec("toy_position_gate", {"hidden_size": 64}, prefix="model.layers.0.toy."))
+    spec = dataclasses.replace(base, layers=(toy_layer,) + base.layers[1:], schedule=(
+        ScheduleEntry(0, cache=None), ScheduleEntry(1, cache=1), ScheduleEntry(2, cache=2), ScheduleEntry(3, cache=3)))
+    model = CausalLM(spec)
+    folder = str(tmp_path / "gate")
+    os.makedirs(folder)
+    write_file(os.path.join(folder, "model.safetensors"), random_tensors(model.tensors(), 6, scale="fan_in"))
+    torch_dtype = parse_dtype(dtype)
+    tensors = load_tensors(folder, model.tensors(), torch_dtype, DEV)
+    model.bind(tensors, torch_dtype, DEV)
+    w = {n: t.double().cpu().numpy() for n, t in tensors.items()}
+    config = dict(TINY_A)
+    eps = config["norm_eps"]
+
+    def expected(tokens):
+        x = w["model.embed_tokens.weight"][tokens]
+        h = plain.rms_norm(x, w["model.layers.0.operator_norm.weight"], eps)
+        x = x + (h * (1 + np.arange(len(tokens)) % 5)[:, None]) @ w["model.layers.0.toy.mix.weight"].T
+        x = x + plain.swiglu(plain.rms_norm(x, w["model.layers.0.ffn_norm.weight"], eps), w, "model.layers.0.feed_forward.")
+        for index, is_attention in ((1, True), (2, False), (3, True)):
+            p = f"model.layers.{index}."
+            h = plain.rms_norm(x, w[p + "operator_norm.weight"], eps)
+            x = x + (plain.attention_mixer(h, w, p + "self_attn.", config) if is_attention else plain.short_conv_mixer(h, w, p + "conv.", config))
+            x = x + plain.swiglu(plain.rms_norm(x, w[p + "ffn_norm.weight"], eps), w, p + "feed_forward.")
+        return plain.rms_norm(x, w["model.embedding_norm.weight"], eps) @ w["model.embed_tokens.weight"].T
+
+    rng = np.random.default_rng(3)
+    a, b = rng.integers(0, 256, 40).tolist(), rng.integers(0, 256, 33).tolist()
+
+    def run(recorded: bool):
+        stepper = Stepper(model, num_pages=4, max_requests=2)
+        assert stepper.use_graphs           # every part of the model, the toy too, allows recording
+        stepper.use_graphs = recorded
+        stepper.admit("a"); stepper.admit("b")
+        got = {"a": [stepper.step([StepEntry("a", a[:20], list(range(20)))]).cpu().numpy()],
+               "b": [stepper.step([StepEntry("b", b[:13], list(range(13)))]).cpu().numpy()]}
+        for i in range(20):         # twenty decode steps of both requests, whose positions differ by seven
+            out = stepper.step([StepEntry("a", a[20 + i:21 + i], [0]), StepEntry("b", b[13 + i:14 + i], [0])]).cpu().numpy()
+            got["a"].append(out[:1]); got["b"].append(out[1:])
+        return stepper, {name: np.concatenate(rows) for name, rows in got.items()}
+
+    before = gate_class.refreshed
+    stepper, recorded = run(True)
+    assert stepper.graph_replays >= 18 and gate_class.refreshed - before == 20
+    _, launched = run(False)
+    tolerance = {"float32": 2e-5, "bfloat16": 3e-2}[dtype]
+    for name, tokens in (("a", a), ("b", b)):
+        want = expected(tokens)
+        assert np.abs(recorded[name] - want).max() <= tolerance * np.abs(want).max()
+        assert np.array_equal(recorded[name], launched[name])
+
+
 # ----- a toy feed-forward with routing and a toy position encoding -----------------------------
 TOY_STRETCH = 4.0
 TOY_ROUTER_GAIN = 8.0       # router logits far apart: few rows sit near the border between the experts
