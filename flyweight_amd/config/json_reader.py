@@ -36,6 +36,9 @@ class Number(float):
         return self
 
 
+MAX_INTEGER_DIGITS = 64
+
+
 class _Parser:
     def __init__(self, data: bytes):
         self.data = data
@@ -146,6 +149,7 @@ class _Parser:
                 pieces.append(_ESCAPES[e])
                 self.at += 2
             elif e == ord("u"):
+                escape = self.at
                 code = self._hex4(self.at + 2)
                 self.at += 6
                 if 0xD800 <= code < 0xDC00 and data[self.at:self.at + 2] == b"\\u":     # a surrogate pair
@@ -153,6 +157,8 @@ class _Parser:
                     if 0xDC00 <= low < 0xE000:
                         code = 0x10000 + ((code - 0xD800) << 10) + (low - 0xDC00)
                         self.at += 6
+                if 0xD800 <= code < 0xE000:
+                    self.fail("half of a surrogate pair stands alone", escape)      # no character: it could not be written out again
                 pieces.append(chr(code))
             else:
                 self.fail("unknown escape in a string")
@@ -166,12 +172,10 @@ class _Parser:
 
     def _hex4(self, at: int) -> int:
         digits = self.data[at:at + 4]
-        try:
-            if len(digits) != 4:
-                raise ValueError
-            return int(digits, 16)
-        except ValueError:
+        # (int(..., 16) alone would also take a sign, blanks and underscores)
+        if len(digits) != 4 or any(d not in b"0123456789abcdefABCDEF" for d in digits):
             self.fail("\\u needs four hexadecimal digits", at)
+        return int(digits, 16)
 
     def number(self) -> Union[int, Number]:
         data, start = self.data, self.at
@@ -204,7 +208,13 @@ class _Parser:
                 self.fail("a number needs digits in its exponent", start)
         self.at = at
         literal = data[start:at].decode("ascii")
-        return int(literal) if whole else Number(literal)
+        if not whole:
+            return Number(literal)
+        # Whole numbers are exact at any size a file can mean (64-bit offsets and beyond); a run of
+        # thousands of digits means nothing, and converting it takes time that grows with its square.
+        if at - digits > MAX_INTEGER_DIGITS:
+            self.fail(f"a whole number of more than {MAX_INTEGER_DIGITS} digits", start)
+        return int(literal)
 
 
 def parse(document: Union[bytes, bytearray, memoryview, str]) -> Any:

@@ -116,6 +116,9 @@ int fwh_scheduler_complete(void* scheduler, const int64_t* requests, const int* 
 int fwh_plan_fill_decode(void* scheduler, int capacity, int* tokens, int* positions, int* slots, int table_stride,
                          int* tables, int group_stride);
 int fwh_plan_steps_ahead(void* scheduler, int limit, int64_t* requests, int capacity);
+// For each segment of the plan made last, in order: the tokens its request may still generate
+// after the one this plan gives it (0: the plan's token is its last). Returns the number written.
+int fwh_plan_budgets(void* scheduler, int* budgets, int capacity);
 int fwh_scheduler_complete_ordered(void* scheduler, const int* tokens, int count, int64_t* event_requests,
                                    int* event_values, int* event_kinds, int capacity);
 // info: computed, live, finished, cancelled, admitted_at, preemptions, prompt length, generated length, max_new_tokens

@@ -38,7 +38,7 @@ int copy_ids(const std::vector<fwh::Request*>& from, int64_t* to) {
 extern "C" {
 
 const char* fwh_last_error(void) { return last_error.c_str(); }
-int fwh_abi_version(void) { return 4; }
+int fwh_abi_version(void) { return 5; }
 
 // ---- pools ---------------------------------------------------------------------------------
 void* fwh_pool_create(int size) {
@@ -325,6 +325,19 @@ int fwh_plan_steps_ahead(void* scheduler, int limit, int64_t* requests, int capa
         if (requests)
             for (size_t i = 0; i < plan.segments.size() && (int)i < capacity; ++i) requests[i] = plan.segments[i].request->id;
         return ahead;
+    });
+}
+int fwh_plan_budgets(void* scheduler, int* budgets, int capacity) {
+    return guarded([&] {
+        const fwh::Plan& plan = scheduler_of(scheduler)->plan();
+        int rows = 0;
+        for (const fwh::Segment& segment : plan.segments) {
+            if (rows >= capacity) break;
+            const fwh::Request* request = segment.request;
+            const int budget = request->max_new_tokens - (int)request->generated.size() - (segment.wants_logits ? 1 : 0);
+            budgets[rows++] = budget > 0 ? budget : 0;
+        }
+        return rows;
     });
 }
 int fwh_scheduler_complete_ordered(void* scheduler, const int* tokens, int count, int64_t* event_requests,

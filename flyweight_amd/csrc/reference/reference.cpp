@@ -259,7 +259,7 @@ int fwr_sample_rows(const float* logits, const float* settings, unsigned long lo
         std::sort(order.begin(), order.end(), [&](int a, int b) { return better(row[a], a, row[b], b); });
         const int candidates = top_k > 0 && top_k < vocab ? (int)top_k : vocab;
         ids[r] = order[0];
-        if (!(temperature > 0.0) || candidates == 1) continue;
+        if (!(temperature > 0.0)) continue;       // (a single candidate is drawn like any list: the generator moves on)
         const double best = (double)row[order[0]] / temperature;
         double total = 0.0;
         for (int i = 0; i < candidates; ++i) {

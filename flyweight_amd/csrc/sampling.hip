@@ -18,7 +18,8 @@
 // 0.9 against 137 us when each walk selected its own first 1,024). A draw over the whole
 // vocabulary of a flat distribution takes as many batches as it walks through.
 // A row whose temperature is 0 takes the best candidate and leaves its generator alone, so
-// greedy and sampled requests share one launch. Nothing is allocated; nothing crosses to the host.
+// greedy and sampled requests share one launch; a drawing row with a single candidate (top_k 1)
+// moves its generator on like any other draw. Nothing is allocated; nothing crosses to the host.
 #include "fw_common.h"
 #include "fw_kernels.h"
 
@@ -285,8 +286,20 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
     };
     const long long candidates = (top_k > 0 && top_k < vocab) ? top_k : vocab;
     const double best_scaled = (double)row[best_id] / temperature;
-    if (!(temperature > 0.0) || candidates == 1 || !__builtin_isfinite(best_scaled)) {
-        leave(best_id);         // greedy, one candidate, or a best value that is not finite (no share is): the generator rests
+    if (!(temperature > 0.0) || !__builtin_isfinite(best_scaled)) {
+        leave(best_id);         // greedy, or a best value that is not finite (no share is): the generator rests
+        return;
+    }
+    if (candidates == 1) {
+        // one candidate is drawn like any list (native/src/v2_runtime.cpp:29722-29733): the generator moves on
+        if (threadIdx.x == 0) {
+            unsigned long long x = states[r] ? states[r] : 0x9E3779B97F4A7C15ull;
+            x ^= x >> 12;
+            x ^= x << 25;
+            x ^= x >> 27;
+            states[r] = x;
+        }
+        leave(best_id);
         return;
     }
     // The k-th best of the threads' best candidates (1,024 different ones) lies at or below the row's

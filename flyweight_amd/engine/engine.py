@@ -224,31 +224,18 @@ class Runtime:
                     self._counters["steps"] += len(tokens)
                     self._counters["decode_calls"] += counts[0] * len(tokens)
                     self._counters["decode_ns"] += time.perf_counter_ns() - began
-                    events = scheduler.complete_ordered(tokens[0])
-                    # The steps that ran ahead: the scheduler makes the plan they ran by (admitting nobody:
-                    # whoever waits comes in with the next turn), then takes their tokens. A request that
-                    # ended on the way (a stop token, its last token) is missing from the later plans, the
-                    # others keep their order; what its row went on to draw is dropped.
-                    live = np.ones(counts[0], dtype=bool)
-                    checked = 0
-                    scheduler.hold_admissions(len(tokens) - 1)
-                    try:
-                        for later in tokens[1:]:
-                            ended = {task for task, _, kind in events[checked:] if kind in (EVENT_FINISHED, EVENT_ERROR)}
-                            checked = len(events)
-                            if ended:
-                                live &= np.array([request not in ended for request in row_requests], dtype=bool)
-                            rows = int(live.sum())
-                            if rows == 0:
-                                break
-                            again = scheduler.plan_next()
-                            if again[0] != rows or again[1] != rows or any(again[2:6]):
-                                raise EngineError("the scheduler's plan differs from the decode steps that ran ahead of it")
-                            events.extend(scheduler.complete_ordered(np.ascontiguousarray(later[live])))
-                    finally:
-                        scheduler.hold_admissions(0)
-                    return events
-        plan = scheduler.read_plan(counts)
+                    events, differing = scheduler.complete_turn(tokens, row_requests)
+                    if differing is None:
+                        return events
+                    # a later plan was not the step that ran: the turn's requests have ended with an
+                    # error; what else that plan holds runs now
+                    self._counters["failed_steps"] = self._counters.get("failed_steps", 0) + 1
+                    return events + self._run_plan(differing)
+        return self._run_plan(scheduler.read_plan(counts))
+
+    def _run_plan(self, plan) -> List[Tuple[int, int, int]]:
+        """Runs a plan's segments as one step through the step function and completes it."""
+        scheduler = self.scheduler
         sampled: Dict[int, int] = {}
         while plan.segments:
             entries = [StepEntry(s.request.id, s.tokens, [len(s.tokens) - 1] if s.wants_logits else [])

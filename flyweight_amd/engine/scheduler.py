@@ -260,6 +260,15 @@ class Scheduler:
             raise SchedulerError(host.last_error())
         return ahead, requests
 
+    def plan_budgets(self, rows: int) -> np.ndarray:
+        """For each of the ``rows`` segments of the plan made last: how many tokens its request may
+        still generate after the one this plan gives it (int32)."""
+        out = host.ints(rows)
+        made = self._lib.fwh_plan_budgets(self._native, out, rows)
+        if made != rows:
+            raise SchedulerError(host.last_error() if made < 0 else f"the plan has {made} segments, not {rows}")
+        return np.frombuffer(out, dtype=np.int32, count=rows)
+
     def complete_ordered(self, tokens) -> List[Tuple[int, int, int]]:
         """``complete`` for the plan made last, the tokens (int32 numpy array) in the order of
         its segments that wanted logits."""
@@ -272,6 +281,50 @@ class Scheduler:
         if made < 0:
             raise SchedulerError(host.last_error())
         return self._events(event_owner, event_value, event_kind, made)
+
+    TURN_DIFFERS = "the scheduler's plan differs from the decode steps that ran ahead of it"
+
+    def complete_turn(self, tokens, row_requests: Sequence[int]):
+        """Finishes a turn of decode steps that ran back to back on the device: ``tokens`` int32
+        [steps, at least the plan's rows], ``row_requests`` the ids of the plan made last in row
+        order. The first step's tokens complete that plan; for every further step the scheduler
+        makes the plan it ran by (admitting nobody: whoever waits comes in with the next turn) and
+        takes its tokens. A request that ended on the way (a stop token, its last token) is
+        missing from the later plans, the others keep their order; what its row went on to draw is
+        dropped. Returns (events, None).
+
+        If a later plan is not the step that ran (somebody was cancelled or gave way meanwhile),
+        the requests still live in the turn end with an error: their fixed-size state on the
+        device is several tokens ahead of the scheduler's lengths and cannot be wound back. The
+        rest of that plan stands; it is returned for the caller to run: (events, plan)."""
+        rows = len(row_requests)
+        events = self.complete_ordered(np.ascontiguousarray(tokens[0][:rows]))
+        live = np.ones(rows, dtype=bool)
+        checked = 0
+        self.hold_admissions(len(tokens) - 1)
+        try:
+            for later in tokens[1:]:
+                ended = {task for task, _, kind in events[checked:] if kind in (EVENT_FINISHED, EVENT_ERROR)}
+                checked = len(events)
+                if ended:
+                    live &= np.array([request not in ended for request in row_requests], dtype=bool)
+                going = int(live.sum())
+                if going == 0:
+                    break
+                again = self.plan_next()
+                if again[0] != going or again[1] != going or any(again[2:6]):
+                    plan = self.read_plan(again)
+                    ahead = [request for request, alive in zip(row_requests, live) if alive]
+                    for request in ahead:
+                        if self.fail(request, self.TURN_DIFFERS):
+                            plan.failed.append(self.requests[request])
+                    plan.segments = [s for s in plan.segments if s.request.id not in set(ahead)]
+                    plan.preempted = [r for r in plan.preempted if r.id not in set(ahead)]
+                    return events, plan
+                events.extend(self.complete_ordered(np.ascontiguousarray(later[:rows][live])))
+        finally:
+            self.hold_admissions(0)
+        return events, None
 
     def _events(self, owners, values, kinds, count: int) -> List[Tuple[int, int, int]]:
         events = list(zip(owners[:count], values[:count], kinds[:count]))

@@ -538,15 +538,26 @@ class Stepper:
         if ahead:
             # Pages for all the steps of the turn now, and the block tables with them: a table that
             # already holds the page a later step will write to reads the same for the steps before.
+            # A request whose last token comes earlier in the turn gets pages up to that token only:
+            # its row runs on beside the others (that costs nothing), and what it then writes goes to
+            # the spare page, which its table names behind the pages it holds.
             positions = ctx._host[1]
             stride = ctx._table_stride
+            going = np.minimum(scheduler.plan_budgets(rows), ahead).astype(np.int64)     # further steps each row takes part in
+            reach = positions[:rows].astype(np.int64) + 1 + going
             try:
-                cache.reserve_all((), (positions[:rows] + 1 + ahead).tolist(), natives=natives, count=rows)
+                cache.reserve_all((), reach.tolist(), natives=natives, count=rows)
             except OutOfPages:
                 ahead = 0                   # one step; the scheduler will decide who gives way
             else:
+                ending = going < ahead
                 for g in range(len(cache.groups)):
-                    ctx._host_tables[g][:rows * stride] = cache.block_table_rows(g, (), stride=stride, natives=natives, count=rows).reshape(-1)
+                    table = cache.block_table_rows(g, (), stride=stride, natives=natives, count=rows)
+                    if ending.any():
+                        held = (reach + cache.page_size - 1) // cache.page_size
+                        behind = (np.arange(stride)[None, :] >= held[:, None]) & ending[:, None]
+                        table[behind] = cache.spare_pages[g]
+                    ctx._host_tables[g][:rows * stride] = table.reshape(-1)
         ctx.upload()
         # Nothing crosses to the host between the steps of a turn: the kernel that finds a step's most
         # likely tokens writes them to the turn's record and to the next step's token ids, and moves

@@ -11,7 +11,7 @@ from .kernels.build import ensure_host_built
 
 ERROR, OUT_OF_PAGES, NO_PAGE = -1, -2, -1
 NOT_DECODE_ONLY = -3
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _LIB: Optional[ctypes.CDLL] = None
 _INTS, _IDS = POINTER(c_int), POINTER(c_int64)
@@ -65,6 +65,7 @@ _SIGNATURES = {
     "fwh_plan_fill_decode": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int]),
     "fwh_scheduler_complete_ordered": (c_int, [c_void_p, _INTS, c_int, _IDS, _INTS, _INTS, c_int]),
     "fwh_plan_steps_ahead": (c_int, [c_void_p, c_int, _IDS, c_int]),
+    "fwh_plan_budgets": (c_int, [c_void_p, _INTS, c_int]),
     "fwh_request_info": (c_int, [c_void_p, c_int64, _INTS]),
     "fwh_request_generated": (c_int, [c_void_p, c_int64, _INTS, c_int]),
     "fwh_request_error": (c_char_p, [c_void_p, c_int64]),

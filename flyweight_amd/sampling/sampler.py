@@ -50,8 +50,10 @@ def make_rng(seed: Optional[int], request_number: int) -> XorShift64Star:
 
 def draw_from_candidates(values: Sequence[float], ids: Sequence[int], config: SamplingConfig,
                          rng: XorShift64Star) -> int:
-    """``values`` sorted descending (ties by ascending id), ``ids`` alongside."""
-    if config.greedy or len(ids) == 1:
+    """``values`` sorted descending (ties by ascending id), ``ids`` alongside. A list of one
+    candidate is drawn like any other: the generator moves on, as the reference's does
+    (native/src/v2_runtime.cpp:29722-29733)."""
+    if config.greedy:
         return int(ids[0])
     scaled = np.asarray(values, dtype=np.float64) / config.temperature
     probabilities = np.where(np.isfinite(scaled), np.exp(scaled - scaled[0]), 0.0)

@@ -162,10 +162,13 @@ def test_json_reader_values_and_what_it_refuses():
     for bad, offset, what in (('{"a": 1} x', 9, "follows"), ('{"a": 1,}', 8, "key"), ("[1 2]", 3, "','"), ('{"a" 1}', 5, "':'"),
                               ('"abc', 0, "not closed"), ("01", 0, "leading zero"), ("[1.]", 1, "behind its point"),
                               ('{"a": 1, "a": 2}', 9, "twice"), ("tru", 0, "expected a value"), ("", 0, "ends here"),
-                              ('"\\x"', 1, "escape")):
+                              ('"\\x"', 1, "escape"), ('"\\u+1a2"', 3, "four hexadecimal"), ('"\\u1_2a"', 3, "four hexadecimal"),
+                              ('"\\u 1a2"', 3, "four hexadecimal"), ('"a\\ud800"', 2, "surrogate"), ('"\\udc00\\ud800"', 1, "surrogate"),
+                              ('"\\ud83dx"', 1, "surrogate"), ("[" + "9" * 65 + "]", 1, "more than 64 digits")):
         with pytest.raises(json_reader.JsonError, match=what) as caught:
             json_reader.parse(bad)
         assert caught.value.offset == offset, (bad, caught.value.offset)
+    assert json_reader.parse("-" + "9" * 64) == -int("9" * 64)
     deep = "[" * 64 + "]" * 64
     assert json_reader.parse(deep) is not None
     with pytest.raises(json_reader.JsonError, match="deeper than 64"):

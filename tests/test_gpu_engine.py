@@ -243,6 +243,39 @@ def test_decode_steps_that_run_ahead_of_the_host_give_the_same_tokens(loaded, dt
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_a_turn_reserves_pages_only_up_to_each_requests_last_token(loaded, dtype):
+    """Two pages for two requests. One of them ends with the turn's first step, two tokens short
+    of its page's end; its row runs on beside the other for three more steps. Pages for those
+    steps would be a second page for it, which the pool does not have: the turn reserves up to its
+    last token only, names the spare page behind the one it holds, and runs ahead all the same.
+    The other request's tokens are what it draws one step per turn."""
+    m = loaded("B", dtype)
+    prompts = [random_tokens(m.config.vocab_size, n, seed=70 + n) for n in (62, 10)]
+    budgets = [2, 30]
+
+    def run(steps_per_turn):
+        runtime = _runtime(m, parallel_sequences=2, num_pages=2, prefill_rows=64, max_batch_tokens=128,
+                           decode_steps_per_turn=steps_per_turn)
+        ids = [runtime.task_submit(p, n) for p, n in zip(prompts, budgets)]
+        events, bursts = [], []
+        while runtime.scheduler.has_work():
+            got = runtime.engine_step()
+            bursts.append(sum(1 for e in got if e[0] == ids[1] and e[2] == 0))
+            events += got
+        runtime.stepper.cache.check_invariants()
+        assert runtime.info["pages_free"] == 2 and runtime.info["live_requests"] == 0 and runtime.scheduler.preemptions == 0
+        return [[e[1] for e in events if e[0] == task and e[2] == 0] for task in ids], bursts
+
+    single, bursts = run(1)
+    assert max(bursts) == 1 and [len(tokens) for tokens in single] == budgets
+    ahead, bursts = run(4)
+    assert ahead == single
+    assert bursts[:2] == [1, 4], "the first decode turn ran four steps although one request ended in its first"
+    if dtype == "float32":
+        assert ahead == [plain.greedy(m.plain_config, m.plain_weights, p, n) for p, n in zip(prompts, budgets)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_decode_steps_are_filled_up_to_the_sizes_that_are_kept(loaded, dtype):
     """Eleven requests that end one by one: the engine's decode steps run at the kept sizes (16,
     then 8, then every size below), the rows behind the plan's filled up with a token of nobody's

@@ -165,6 +165,8 @@ def test_sampler_against_the_plain_one_and_the_host_rules():
             if not np.isnan(logits[r]).any():       # (the plain sampler says nothing about NaN; the engine's rule is: last)
                 plain_rng = plain_lfm2.XorShift64Star(int(states[r]))
                 assert ids[r] == plain_lfm2.sample(logits[r], temperature, top_k, top_p, min_p, plain_rng)
+                # the generator moves on once per drawn token, also when top_k leaves one candidate
+                assert plain_rng.state == int(moved_on[r]) and (plain_rng.state != int(states[r])) == (temperature > 0)
             host_rng = XorShift64Star(int(states[r]))
             values, order = host_candidates(logits[r], top_k if 0 < top_k < logits.shape[1] else 0)
             config = SamplingConfig(temperature=temperature, top_k=top_k, top_p=top_p, min_p=min_p)

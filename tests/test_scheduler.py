@@ -359,3 +359,77 @@ def test_steps_ahead_of_the_host_and_requests_that_end_in_the_middle_of_them():
     another = scheduler.submit([5, 6], 4)
     counts = scheduler.plan_next()
     assert counts[4] == 2 and late.live and another.live and scheduler.steps_ahead(4, 3)[0] == 0
+
+
+def test_a_turn_whose_later_plan_differs_ends_its_requests_and_nobody_else():
+    """``complete_turn`` hands a turn of decode steps that ran ahead over to the scheduler. If
+    the plan the scheduler makes for a later step is not the step that ran (here: a request is
+    cancelled between the turn's run and its handing over), the requests still live in the
+    turn end with an error (their state on the device is ahead of the scheduler's lengths),
+    everything they held comes back, the tokens handed over before are kept, and whoever
+    waited goes on afterwards. A turn whose plans agree gives the events of its single steps,
+    and the budgets that bound a turn's reservations are the tokens each request has to go."""
+    import numpy as np
+    cache, scheduler = make(num_pages=16, max_requests=3)
+    prompts = [[3, 4, 5], [9, 8], [20, 21, 22, 23]]
+    requests = [scheduler.submit(p, n) for p, n in zip(prompts, (30, 3, 30))]
+    plan = scheduler.schedule()
+    scheduler.complete(plan, {s.request.id: oracle(s.request.tokens) for s in plan.segments})
+    late = scheduler.submit([1, 2], 4)                  # every slot is taken: it waits
+    sequences = [list(p) + expected_tokens(p, 1) for p in prompts]
+
+    def turn(steps):
+        """What the device would draw in ``steps`` steps of all three rows."""
+        drawn = np.zeros((steps, 3), dtype=np.int32)
+        for step in range(steps):
+            for row, sequence in enumerate(sequences):
+                drawn[step, row] = oracle(sequence)
+                sequence.append(int(drawn[step, row]))
+        return drawn
+
+    # a turn that goes through: the second request ends on its third token, in the turn's second step
+    counts = scheduler.plan_next()
+    assert counts[0] == counts[1] == 3 and not any(counts[2:6])
+    assert scheduler.plan_budgets(3).tolist() == [30 - 2, 3 - 2, 30 - 2]
+    ahead, rows = scheduler.steps_ahead(3, 3)
+    assert ahead == 3
+    events, differing = scheduler.complete_turn(turn(4), list(rows[:3]))
+    assert differing is None
+    assert [e[0] for e in events if e[2] == EVENT_TOKEN] == [1, 2, 3, 1, 2, 3, 1, 3, 1, 3]
+    assert (requests[1].id, 3, EVENT_FINISHED) in events and not late.live
+    cache.check_invariants()
+    # the next turn: one slot is free now, so the scheduler would admit; a turn only starts when it says so
+    counts = scheduler.plan_next()
+    assert counts[4] == 1 and late.live
+    plan = scheduler.read_plan(counts)
+    scheduler.complete(plan, {s.request.id: oracle(s.request.tokens) for s in plan.segments if s.wants_logits})
+    for sequence, request in zip(sequences, requests):
+        if not request.finished:
+            sequence[:] = request.tokens
+    # a turn of the three running requests, one of which is cancelled while the device runs ahead
+    counts = scheduler.plan_next()
+    assert counts[0] == counts[1] == 3 and not any(counts[2:6])
+    ahead, rows = scheduler.steps_ahead(3, 3)
+    assert ahead == 3 and list(rows[:3]) == [requests[0].id, requests[2].id, late.id]
+    sequences = [requests[0].tokens, requests[2].tokens, late.tokens]
+    drawn = turn(4)
+    before = {r.id: len(r.generated) for r in (requests[0], requests[2], late)}
+    assert scheduler.cancel(requests[2].id)
+    events, differing = scheduler.complete_turn(drawn, list(rows[:3]))
+    assert differing is not None and not differing.segments
+    # the first step's tokens were handed over as drawn; then the plans parted
+    assert [e for e in events if e[2] == EVENT_TOKEN] == [(requests[0].id, int(drawn[0, 0]), EVENT_TOKEN),
+                                                            (requests[2].id, int(drawn[0, 1]), EVENT_TOKEN),
+                                                            (late.id, int(drawn[0, 2]), EVENT_TOKEN)]
+    events = scheduler.complete(differing, {})
+    kinds = {e[0]: e[2] for e in events}
+    assert kinds == {requests[0].id: EVENT_ERROR, late.id: EVENT_ERROR, requests[2].id: EVENT_FINISHED}
+    assert "ran ahead" in requests[0].error and "ran ahead" in late.error and requests[2].error is None
+    assert all(len(r.generated) == before[r.id] + 1 for r in (requests[0], requests[2], late))
+    assert not scheduler.has_work() and len(cache.requests) == 0
+    assert cache.groups[0].pool.in_use == 0 and cache.slots.free_count == 3
+    cache.check_invariants()
+    # the scheduler is as good as new
+    fresh = scheduler.submit([7, 7, 7], 5)
+    seen = drive(scheduler, cache)
+    assert [e[1] for e in seen[fresh.id] if e[2] == EVENT_TOKEN] == expected_tokens([7, 7, 7], 5)
