@@ -15,6 +15,8 @@ from typing import Any, Optional, Tuple
 
 import torch
 
+from ..kernels import ops
+
 
 @dataclass
 class CacheView:
@@ -102,7 +104,10 @@ class FixedState(CacheNeed):
         return torch.zeros((units, *self.shape), dtype=self.dtype, device=device)
 
     def initial(self, storage, slot):
-        storage[slot].zero_()
+        if storage.is_cuda:
+            ops.fill_zero(storage[slot])
+        else:
+            storage[slot].zero_()
 
     def allocate_together(self, count, units, page_size, dtype, device):
         # one tensor for the layers that keep the same state: a request's start clears its slot in
@@ -111,7 +116,10 @@ class FixedState(CacheNeed):
         return [whole[index] for index in range(count)], whole
 
     def initial_together(self, together, slot):
-        together[:, slot].zero_()
+        if together.is_cuda:
+            ops.fill_zero_pieces(together[0, slot], together.shape[0], together.stride(0) * together.element_size())
+        else:
+            together[:, slot].zero_()
 
     def view(self, storage, block_table, writes):
         return CacheView(state=storage, writes=writes)

@@ -16,7 +16,7 @@ void fw_set_error(const char* format, ...) {
     va_end(args);
 }
 extern "C" const char* fw_last_error(void) { return fw_error_text; }
-extern "C" int fw_abi_version(void) { return 7; }
+extern "C" int fw_abi_version(void) { return 8; }
 
 // ---- embedding -------------------------------------------------------------------------
 // The reference gathers one row per token and widens it to float32
@@ -224,39 +224,6 @@ __device__ __forceinline__ unsigned long long block_max_u64(unsigned long long v
     return best;
 }
 
-// One block per row; `k` rounds, each picks the best key strictly below the last winner.
-__global__ void topk_rows_kernel(const float* __restrict__ logits, float* __restrict__ values,
-                                 int32_t* __restrict__ ids, int vocab, int k) {
-    __shared__ unsigned long long scratch[16];
-    const int row = blockIdx.x;
-    const float* source = logits + (size_t)row * vocab;
-    unsigned long long ceiling = ~0ull;
-    for (int round = 0; round < k; ++round) {
-        unsigned long long best = 0;
-        for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-            const unsigned long long key = candidate_key(source[i], i);
-            if (key < ceiling && key > best) best = key;
-        }
-        best = block_max_u64(best, scratch);
-        if (threadIdx.x == 0) {
-            const int id = (int)(0xffffffffu - (uint32_t)(best & 0xffffffffull));
-            ids[(size_t)row * k + round] = id;
-            if (values) values[(size_t)row * k + round] = source[id];
-        }
-        ceiling = best;
-    }
-}
-
-extern "C" int fw_topk_rows(const float* logits, float* values, int32_t* ids, int rows, int vocab, int k,
-                            void* stream) {
-    FW_REQUIRE(rows >= 0 && vocab > 0, "topk_rows: bad sizes rows=%d vocab=%d", rows, vocab);
-    FW_REQUIRE(k >= 1 && k <= vocab && k <= 256, "topk_rows: k must be in 1..min(256, vocab), got %d", k);
-    if (rows == 0) return 0;
-    topk_rows_kernel<<<rows, 1024, 0, (hipStream_t)stream>>>(logits, values, ids, vocab, k);
-    FW_LAUNCH_CHECK("topk_rows");
-    return 0;
-}
-
 // Argmax in two steps, so that a few rows of a wide vocabulary still fill the chip: grid (parts,
 // rows) finds the best key of each part of a row, then one wave per row finds the best of those.
 // Keys order by value, then by the lower id, so the result does not depend on the cut.
@@ -375,6 +342,27 @@ __global__ void fill_zero_kernel(uint32_t* __restrict__ ptr, long long words) {
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < words;
          i += (long long)gridDim.x * blockDim.x)
         ptr[i] = 0u;
+}
+
+__global__ void fill_zero_pieces_kernel(uint32_t* __restrict__ ptr, long long words_per_piece, long long stride_words) {
+    uint32_t* piece = ptr + (size_t)blockIdx.y * stride_words;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < words_per_piece; i += (long long)gridDim.x * blockDim.x)
+        piece[i] = 0u;
+}
+
+// `pieces` runs of `bytes` each, `stride_bytes` apart (a request's slot in the state of several layers
+// that lie in one allocation), cleared in one launch.
+extern "C" int fw_fill_zero_pieces(void* ptr, int pieces, long long bytes, long long stride_bytes, void* stream) {
+    FW_REQUIRE(bytes >= 0 && bytes % 4 == 0 && stride_bytes % 4 == 0 && stride_bytes >= bytes,
+               "fill_zero_pieces: %lld bytes every %lld bytes: both must be multiples of 4, the pieces apart", bytes, stride_bytes);
+    FW_REQUIRE(pieces >= 0 && pieces <= 65535, "fill_zero_pieces: %d pieces (at most 65535)", pieces);
+    if (bytes == 0 || pieces == 0) return 0;
+    const long long words = bytes / 4;
+    int blocks = fw_ceil_div(words, 256);
+    if (blocks > 256) blocks = 256;
+    fill_zero_pieces_kernel<<<dim3(blocks, pieces), 256, 0, (hipStream_t)stream>>>((uint32_t*)ptr, words, stride_bytes / 4);
+    FW_LAUNCH_CHECK("fill_zero_pieces");
+    return 0;
 }
 
 extern "C" int fw_fill_zero(void* ptr, long long bytes, void* stream) {

@@ -69,16 +69,13 @@ int fw_gemm_mfma_split(const void* a, const void* w, const float* bias, void* ou
 // the kernel leaves them zero. Calls that overlap on one device need their own of both.
 // The accumulating product can leave what the norm after it needs, as fw_gemm_decode does
 // (next_activations [M][N] bfloat16, next_squares [squares_rows][16 for M <= 16, else 64]), and
-// any mode takes such prepared activations as a, with squares / squares_rows / eps. Mode 3 is the
-// gated short convolution for single-token rows (w = [B; C; x rows], taps [N][kernel_size], state
-// [slots][N][kernel_size - 1] read and shifted, seg_slot [M]), as fw_gemm_decode's epilogue 3.
+// any mode takes such prepared activations as a, with squares / squares_rows / eps.
 int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* workspace_bytes, int* counters, int* squares_rows);
 int fw_gemm_medium(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                    int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
                    int counters_len, const float* next_norm_weight, int next_one_centered,
                    void* next_activations, float* next_squares, const float* squares, int squares_rows,
-                   float eps, const float* taps, const float* conv_bias, float* state, const int32_t* seg_slot,
-                   int kernel_size, void* stream);
+                   float eps, void* stream);
 
 // Fused product for decode steps of up to 16 rows. prologue 0: a is bfloat16 [M][K]; 1: a is
 // float32 rows, RMS-normed with norm_weight/eps (rows gathered through row_index if given) inside
@@ -186,10 +183,6 @@ int fw_argmax_rows_static(const float* logits, int32_t* ids, int32_t* also, int3
                           void* stream);
 int fw_argmax_rows_static_max_rows(void);
 
-// the k largest logits of every row, sorted by (value descending, id ascending)
-int fw_topk_rows(const float* logits, float* values, int32_t* ids, int rows, int vocab, int k,
-                 void* stream);
-
 // The next token of every row, drawn on the device: settings float32 [rows][4] = temperature (0:
 // greedy, the best candidate, ties to the lowest id), top_k (0: all candidates), top_p, min_p;
 // states [rows]: the rows' xorshift64* generators, moved on by the rows that draw. also / advance
@@ -199,6 +192,8 @@ int fw_sample_rows(const float* logits, const float* settings, unsigned long lon
                    int32_t* advance, int rows, int vocab, void* stream);
 
 int fw_fill_zero(void* ptr, long long bytes, void* stream);
+// `pieces` runs of `bytes` each, `stride_bytes` apart, cleared in one launch
+int fw_fill_zero_pieces(void* ptr, int pieces, long long bytes, long long stride_bytes, void* stream);
 
 #ifdef __cplusplus
 }

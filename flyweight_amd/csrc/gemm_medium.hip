@@ -32,8 +32,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 #define GM_DEPTH 4      // chunks in flight
 #define GM_PAD 8        // bfloat16 elements between LDS rows: spreads the rows over the banks
 
-enum { GM_STORE = 0, GM_ACCUMULATE = 1, GM_SWIGLU = 2, GM_CONV = 3 };
-#define GM_MAX_TAPS 16
+enum { GM_STORE = 0, GM_ACCUMULATE = 1, GM_SWIGLU = 2 };
 
 struct MediumArgs {
     const uint16_t* a;
@@ -56,13 +55,6 @@ struct MediumArgs {
     int squares_rows;
     float eps;
     int rotate;                     // workgroups start their walk over K at different chunks
-    // gated short convolution for single-token segments (mode 3): w = [B rows; C rows; x rows] of N
-    // channels each; every row of a is a request's one new token
-    const float* taps;              // [N][kernel_size], oldest first
-    const float* conv_bias;         // [N] or null
-    float* state;                   // [slots][N][kernel_size - 1], read and shifted
-    const int32_t* seg_slot;        // [M]
-    int kernel_size;
 };
 
 // rows of the sums of squares are 16 wide for up to 16 rows of a (the fused decode product's
@@ -81,7 +73,7 @@ template <int MT, int FW, int MODE, typename TO, bool ROTATE>
 __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArgs p) {
     constexpr int KP = 4 / FW;                  // parts of K inside the workgroup
     constexpr int CHUNK = 64 * KP;              // k per iteration of the workgroup
-    constexpr int KINDS = MODE == GM_SWIGLU ? 2 : (MODE == GM_CONV ? 3 : 1);
+    constexpr int KINDS = MODE == GM_SWIGLU ? 2 : 1;
     constexpr int SEG = CHUNK / 8;              // 16-byte pieces per row of a chunk of a
     constexpr int PIECES = MT * 16 * SEG;       // pieces per chunk of a
     constexpr int AP = (PIECES + GM_THREADS - 1) / GM_THREADS;
@@ -330,28 +322,7 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
         for (int r = 0; r < 4; ++r) {
             const int n = n_first + r;
             if (MODE == GM_SWIGLU) v[r] = gm_silu(acc[0][mt][r] * inv) * (acc[1][mt][r] * inv);
-            else if (MODE == GM_CONV) {
-                // the row is a segment of one token: B * x joins the request's last L - 1 of them, the
-                // taps are applied oldest first, the state moves on by one (shortconv.hip, the same
-                // sum in the same order); C gates the result
-                v[r] = 0.0f;
-                if (mine && n < N) {
-                    float part[3];
-#pragma unroll
-                    for (int kind = 0; kind < 3; ++kind) part[kind] = acc[kind][mt][r] * inv + (p.bias ? p.bias[n + kind * N] : 0.0f);
-                    const int history = p.kernel_size - 1;
-                    float* channel_state = p.state + ((size_t)p.seg_slot[m] * N + n) * history;
-                    const float* channel_taps = p.taps + (size_t)n * p.kernel_size;
-                    float window[GM_MAX_TAPS];
-                    for (int k = 0; k < history; ++k) window[k] = channel_state[k];
-                    window[history] = part[0] * part[2];
-                    float y = 0.0f;
-                    for (int j = 0; j < p.kernel_size; ++j) y = fmaf(channel_taps[j], window[j], y);
-                    if (p.conv_bias) y += p.conv_bias[n];
-                    for (int k = 0; k < history; ++k) channel_state[k] = window[k + 1];
-                    v[r] = part[1] * y;
-                }
-            } else v[r] = acc[0][mt][r] * inv + ((p.bias && n < N) ? p.bias[n] : 0.0f);
+            else v[r] = acc[0][mt][r] * inv + ((p.bias && n < N) ? p.bias[n] : 0.0f);
         }
         if (mine) {
             if constexpr (sizeof(TO) == 4) {
@@ -427,7 +398,7 @@ struct MediumPlan {
 static MediumPlan medium_plan(int M, int N, int K, int mode) {
     MediumPlan plan;
     plan.mt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-    const int kinds = mode == GM_SWIGLU ? 2 : (mode == GM_CONV ? 3 : 1);
+    const int kinds = mode == GM_SWIGLU ? 2 : 1;
     if (fw_ceil_div(N, 64) >= 384) {            // enough tiles of 64 features for every compute unit
         plan.fw = 4;
         plan.tiles = fw_ceil_div(N, 64);
@@ -470,8 +441,6 @@ extern "C" int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* worksp
 template <int MT, int FW, bool ROTATE>
 static void medium_launch_as(const MediumArgs& args, int out_dtype, int mode, dim3 grid, hipStream_t stream) {
     if (mode == GM_SWIGLU) gemm_medium_kernel<MT, FW, GM_SWIGLU, bf16_t, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
-    else if (mode == GM_CONV && out_dtype == FW_F32) gemm_medium_kernel<MT, FW, GM_CONV, float, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
-    else if (mode == GM_CONV) gemm_medium_kernel<MT, FW, GM_CONV, bf16_t, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
     else if (mode == GM_ACCUMULATE) gemm_medium_kernel<MT, FW, GM_ACCUMULATE, float, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
     else if (out_dtype == FW_F32) gemm_medium_kernel<MT, FW, GM_STORE, float, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
     else gemm_medium_kernel<MT, FW, GM_STORE, bf16_t, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
@@ -484,22 +453,17 @@ static void medium_launch(const MediumArgs& args, int out_dtype, int mode, dim3 
 }
 
 // mode 0: out = a . w^T (+ bias) stored as out_dtype; 1: out (float32) += a . w^T (+ bias);
-// 2: w is [2 * N][K] (gate rows, then up rows); out [M][N] bfloat16 = silu(gate) * up;
-// 3: w is [3 * N][K] (B, C, x rows); every row of a is one request's new token: out [M][N] =
-//    C * conv(B * x) with the request's state (slot seg_slot[m]) read and shifted.
+// 2: w is [2 * N][K] (gate rows, then up rows); out [M][N] bfloat16 = silu(gate) * up.
 // workspace / counters: as fw_gemm_medium_plan says for this shape. Calls that overlap on one
 // device must not share counters or workspace.
 extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
                               int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
                               int counters_len, const float* next_norm_weight, int next_one_centered,
                               void* next_activations, float* next_squares, const float* squares, int squares_rows,
-                              float eps, const float* taps, const float* conv_bias, float* state, const int32_t* seg_slot,
-                              int kernel_size, void* stream) {
+                              float eps, void* stream) {
     FW_REQUIRE(M >= 1 && M <= 64, "gemm_medium: takes 1..64 rows, got %d", M);
-    FW_REQUIRE(mode != GM_CONV || (taps && state && seg_slot && kernel_size >= 2 && kernel_size <= GM_MAX_TAPS),
-               "gemm_medium: the convolution epilogue needs taps, state, slots and a kernel size in 2..%d", GM_MAX_TAPS);
     FW_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_medium: K (%d) must be a positive multiple of 8, N (%d) positive", K, N);
-    FW_REQUIRE(mode >= 0 && mode <= 3, "gemm_medium: unknown mode %d", mode);
+    FW_REQUIRE(mode >= 0 && mode <= 2, "gemm_medium: unknown mode %d", mode);
     FW_REQUIRE(mode != GM_ACCUMULATE || out_dtype == FW_F32, "gemm_medium: accumulation needs a float32 destination");
     FW_REQUIRE(mode != GM_SWIGLU || (out_dtype == FW_BF16 && bias == nullptr), "gemm_medium: SwiGLU stores bfloat16 and takes no bias");
     FW_REQUIRE(out_dtype == FW_F32 || out_dtype == FW_BF16, "gemm_medium: unknown out dtype %d", out_dtype);
@@ -521,8 +485,7 @@ extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, v
     args.next_norm_weight = next_norm_weight; args.next_one_centered = next_one_centered;
     args.next_activations = (uint16_t*)next_activations; args.next_squares = next_squares;
     args.squares = squares; args.squares_rows = squares_rows; args.eps = eps;
-    args.taps = taps; args.conv_bias = conv_bias; args.state = state; args.seg_slot = seg_slot; args.kernel_size = kernel_size;
-    args.rotate = plan.splits == 1 && (long long)N * K * (mode == GM_SWIGLU ? 2 : (mode == GM_CONV ? 3 : 1)) > (1ll << 24);
+    args.rotate = plan.splits == 1 && (long long)N * K * (mode == GM_SWIGLU ? 2 : 1) > (1ll << 24);
     const dim3 grid(plan.tiles, plan.splits);
     hipStream_t s = (hipStream_t)stream;
     if (plan.fw == 4) {

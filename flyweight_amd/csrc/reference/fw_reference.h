@@ -46,7 +46,6 @@ int fwr_attention(const float* q, float* out, const float* k_pages, const float*
                   int num_kv_heads, int head_dim, float scale, int window, int page_size, int num_pages);
 // elementwise.hip argmax / top-k: order by value descending, then id ascending; NaN last
 int fwr_argmax_rows(const float* logits, int32_t* ids, int rows, int vocab);
-int fwr_topk_rows(const float* logits, float* values, int32_t* ids, int rows, int vocab, int k);
 // sampling.hip: settings [rows][4] = temperature (0: greedy), top_k (0: all), top_p, min_p; states: the
 // rows' xorshift64* generators, moved on by the rows that draw
 int fwr_sample_rows(const float* logits, const float* settings, unsigned long long* states, int32_t* ids, int rows, int vocab);

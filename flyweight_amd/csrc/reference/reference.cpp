@@ -230,22 +230,6 @@ int fwr_argmax_rows(const float* logits, int32_t* ids, int rows, int vocab) {
     return 0;
 }
 
-// native/src/v2_runtime.cpp:29500-29566
-int fwr_topk_rows(const float* logits, float* values, int32_t* ids, int rows, int vocab, int k) {
-    if (k < 1 || k > vocab) return fail("topk_rows: k %d outside 1..%d", k, vocab);
-    std::vector<int> order(vocab);
-    for (int r = 0; r < rows; ++r) {
-        const float* row = logits + (size_t)r * vocab;
-        for (int i = 0; i < vocab; ++i) order[i] = i;
-        std::partial_sort(order.begin(), order.begin() + k, order.end(), [&](int a, int b) { return better(row[a], a, row[b], b); });
-        for (int i = 0; i < k; ++i) {
-            ids[(size_t)r * k + i] = order[i];
-            values[(size_t)r * k + i] = row[order[i]];
-        }
-    }
-    return 0;
-}
-
 // native/src/v2_runtime.cpp:29500-29566 (the candidates), 29686-29743 (the cuts and the draw),
 // 29307-29314 (the generator): one row after the other, the whole row sorted, every sum in order
 int fwr_sample_rows(const float* logits, const float* settings, unsigned long long* states, int32_t* ids, int rows, int vocab) {

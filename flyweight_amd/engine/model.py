@@ -119,7 +119,7 @@ class CausalLM:
         final = LazyNorm(self.final_norm, x, ctx, prepared=prepared) if every_row else LazyNorm(self.final_norm, x, ctx, row_index=ctx.want_rows)
         logits = self.head.forward(final, out_dtype=torch.float32)
         if every_row and not getattr(ctx, "wants_every_row", False):
-            logits = logits[ctx.want_rows.long()]
+            logits = ops.gather_rows(logits, ctx.want_rows)
         if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0.0:
             ops.scale_softcap_(logits, self.spec.logit_scale, self.spec.logit_softcap)
         return logits

@@ -19,7 +19,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _lib = None
 
@@ -413,19 +413,23 @@ def sample_rows(logits: torch.Tensor, settings: torch.Tensor, states: torch.Tens
     return ids
 
 
-def topk_rows(logits: torch.Tensor, k: int):
-    _dev(logits)
-    _want(logits, torch.float32, "logits")
-    rows, vocab = logits.shape
-    values = torch.empty((rows, k), dtype=torch.float32, device=logits.device)
-    ids = torch.empty((rows, k), dtype=torch.int32, device=logits.device)
-    _check(library().fw_topk_rows(_p(logits), _p(values), _p(ids), rows, vocab, k, _stream()))
-    return values, ids
-
-
 def fill_zero(t: torch.Tensor) -> None:
     _dev(t)
     _check(library().fw_fill_zero(_p(t), ctypes.c_longlong(t.numel() * t.element_size()), _stream()))
+
+
+def fill_zero_pieces(first: torch.Tensor, pieces: int, stride_bytes: int) -> None:
+    """Clears ``pieces`` runs of memory the size of ``first`` (contiguous), ``stride_bytes`` apart,
+    beginning with ``first`` itself: the caller vouches that all of them lie in one allocation."""
+    _dev(first)
+    _check(library().fw_fill_zero_pieces(_p(first), int(pieces), ctypes.c_longlong(first.numel() * first.element_size()),
+                                         ctypes.c_longlong(int(stride_bytes)), _stream()))
+
+
+def gather_rows(rows: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    """rows[index] for float32 rows and an int32 index on the device (the embedding kernel: a
+    table of rows is a table of rows)."""
+    return embed_rows(rows, index)
 
 
 def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int) -> None:
@@ -570,9 +574,7 @@ def prepare_device(device: torch.device) -> None:
 
 def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int,
                      next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False,
-                     squares: Optional[torch.Tensor] = None, eps: float = 0.0, taps: Optional[torch.Tensor] = None,
-                     conv_bias: Optional[torch.Tensor] = None, state: Optional[torch.Tensor] = None,
-                     seg_slot: Optional[torch.Tensor] = None):
+                     squares: Optional[torch.Tensor] = None, eps: float = 0.0):
     """The product for 1..64 rows with K split over workgroups (fw_gemm_medium). With
     ``squares`` ``a`` holds prepared activations (x * w of an RMS norm) and the rows' 1/rms is
     formed from those sums. With ``next_norm_weight`` (accumulating product) returns what the
@@ -596,8 +598,7 @@ def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tenso
                                     ctypes.c_size_t(need_bytes.value), _p(counters),
                                     0 if counters is None else counters.numel(), _p(next_norm_weight),
                                     int(next_one_centered), _p(next_activations), _p(next_squares), _p(squares),
-                                    0 if squares is None else squares.shape[0], ctypes.c_float(eps), _p(taps), _p(conv_bias),
-                                    _p(state), _p(seg_slot), 0 if taps is None else taps.shape[1], _stream()))
+                                    0 if squares is None else squares.shape[0], ctypes.c_float(eps), _stream()))
     if next_norm_weight is not None:
         return next_activations, next_squares
     return None
@@ -606,18 +607,16 @@ def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tenso
 def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, accumulate_into: Optional[torch.Tensor] = None,
                 squares: Optional[torch.Tensor] = None, eps: float = 0.0,
-                next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False,
-                taps: Optional[torch.Tensor] = None, conv_bias: Optional[torch.Tensor] = None,
-                state: Optional[torch.Tensor] = None, seg_slot: Optional[torch.Tensor] = None):
+                next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False):
     """The medium product with the fused decode product's conventions (EPILOGUE_STORE /
-    ACCUMULATE / SWIGLU / CONV): returns the output, or for an accumulation with
-    ``next_norm_weight`` what the norm after it needs."""
-    _dev(a, w, bias, accumulate_into, squares, next_norm_weight, taps, conv_bias, state, seg_slot)
+    ACCUMULATE / SWIGLU): returns the output, or for an accumulation with ``next_norm_weight``
+    what the norm after it needs."""
+    _dev(a, w, bias, accumulate_into, squares, next_norm_weight)
     _want(a, torch.bfloat16, "a")
     _want(w, torch.bfloat16, "w")
     M, K = a.shape
-    kinds = {EPILOGUE_SWIGLU: 2, EPILOGUE_CONV: 3}.get(epilogue, 1)
-    if not 1 <= M <= MEDIUM_MAX_ROWS or w.shape[1] != K or w.shape[0] % kinds or K % 8 or epilogue not in (0, 1, 2, 3):
+    kinds = 2 if epilogue == EPILOGUE_SWIGLU else 1
+    if not 1 <= M <= MEDIUM_MAX_ROWS or w.shape[1] != K or w.shape[0] % kinds or K % 8 or epilogue not in (0, 1, 2):
         raise KernelError(f"gemm_medium: a is {tuple(a.shape)}, w is {tuple(w.shape)}, epilogue {epilogue}")
     N = w.shape[0] // kinds
     if bias is not None and (bias.dtype != torch.float32 or bias.shape != (w.shape[0],)):
@@ -625,8 +624,6 @@ def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
     if next_norm_weight is not None and (epilogue != EPILOGUE_ACCUMULATE or next_norm_weight.dtype != torch.float32
                                          or next_norm_weight.shape != (N,)):
         raise KernelError("gemm_medium: only the accumulating product prepares the next norm, whose weight is float32 [N]")
-    if epilogue == EPILOGUE_CONV:
-        _check_conv_arguments("gemm_medium", M, N, taps, conv_bias, state, seg_slot)
     if epilogue == EPILOGUE_ACCUMULATE:
         _want(accumulate_into, torch.float32, "accumulate_into")
         if accumulate_into.shape != (M, N):
@@ -635,27 +632,8 @@ def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
         return accumulate_into if left is None else left
     out_dtype = torch.bfloat16 if epilogue == EPILOGUE_SWIGLU else (out_dtype or torch.bfloat16)
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    gemm_medium_into(a, w, bias, out, _code(out_dtype), epilogue, N, squares=squares, eps=eps, taps=taps, conv_bias=conv_bias,
-                     state=state, seg_slot=seg_slot)
+    gemm_medium_into(a, w, bias, out, _code(out_dtype), epilogue, N, squares=squares, eps=eps)
     return out
-
-
-def _check_conv_arguments(name: str, M: int, N: int, taps, conv_bias, state, seg_slot) -> None:
-    """What a convolution epilogue needs: taps float32 [N, L], state float32 [slots, N, L - 1],
-    seg_slot int32 of at least M entries, an optional bias float32 [N]."""
-    if taps is None or state is None or seg_slot is None:
-        raise KernelError(f"{name}: the convolution epilogue needs taps, state and slots")
-    _want(taps, torch.float32, "taps")
-    _want(state, torch.float32, "state")
-    _want(seg_slot, torch.int32, "seg_slot")
-    if taps.dim() != 2 or taps.shape[0] != N or not 2 <= taps.shape[1] <= 16:
-        raise KernelError(f"{name}: taps are {tuple(taps.shape)}, expected [{N}, 2..16]")
-    if state.dim() != 3 or state.shape[1:] != (N, taps.shape[1] - 1) or not state.is_contiguous() or not taps.is_contiguous():
-        raise KernelError(f"{name}: state is {tuple(state.shape)}, expected [slots, {N}, {taps.shape[1] - 1}]")
-    if seg_slot.numel() < M:
-        raise KernelError(f"{name}: {seg_slot.numel()} slots for {M} rows")
-    if conv_bias is not None and (conv_bias.dtype != torch.float32 or conv_bias.shape != (N,)):
-        raise KernelError(f"{name}: the convolution's bias must be float32 [{N}]")
 
 
 def gemm_deep(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,

@@ -146,14 +146,6 @@ def argmax_rows(logits) -> np.ndarray:
     return ids
 
 
-def topk_rows(logits, k: int) -> Tuple[np.ndarray, np.ndarray]:
-    logits = _f(logits)
-    values = np.empty((logits.shape[0], k), dtype=np.float32)
-    ids = np.empty((logits.shape[0], k), dtype=np.int32)
-    _check(library().fwr_topk_rows(_p(logits), _p(values), _p(ids), logits.shape[0], logits.shape[1], int(k)))
-    return values, ids
-
-
 def sample_rows(logits, settings, states) -> Tuple[np.ndarray, np.ndarray]:
     """The next token of every row and the generators' states afterwards (``states`` uint64 [rows]
     is not changed): settings float32 [rows, 4] = temperature, top_k, top_p, min_p."""

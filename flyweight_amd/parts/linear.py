@@ -136,10 +136,9 @@ class Linear:
                           seg_slot: torch.Tensor, out_dtype: torch.dtype) -> Optional[torch.Tensor]:
         """For single-token segments: the weight holds B, C and x rows; returns C * conv(B * x)
         with the state shifted, or None when the fused kernel does not take the shape. (Beyond 16
-        rows the split-K product has the same epilogue, ``ops.gemm_medium(..., EPILOGUE_CONV)``, but
-        a workgroup must then own B, C and x of its channels, which leaves a third as many tiles
-        and a fourfold split of K: 41 us against 15.3 + 4.8 us for the product and the convolution
-        apart at 64 rows. It is not used.)"""
+        rows the product and the convolution run apart: as an epilogue of the split-K product a
+        workgroup would have to own B, C and x of its channels, which leaves a third as many tiles
+        and a fourfold split of K: 41 us against 15.3 + 4.8 us at 64 rows.)"""
         if not self._fused(a, self.out_features // 3, ops.EPILOGUE_CONV):
             return None
         return ops.gemm_decode(self._rows_of(a), self.weight, ops.EPILOGUE_CONV, bias=self.bias, out_dtype=out_dtype,

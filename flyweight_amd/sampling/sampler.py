@@ -7,13 +7,11 @@ reaches it, ``min_p`` keeps candidates at least that fraction of the best, and t
 the sorted list until the cumulative mass reaches u * kept mass
 (native/src/v2_runtime.cpp:29500-29566, 29686-29743). Each request owns an xorshift64*
 generator (:29307-29314), so what else is in the batch cannot change its draws.
-``sample_rows`` does all of it on the device (``csrc/sampling.hip``); ``draw_from_candidates``
-and ``host_candidates`` are the same rules on the host, which the kernel is tested against.
+``sample_rows`` does all of it on the device (``csrc/sampling.hip``).
 """
 
 from __future__ import annotations
 
-import math
 import time
 from typing import List, Optional, Sequence
 
@@ -46,54 +44,6 @@ def make_rng(seed: Optional[int], request_number: int) -> XorShift64Star:
     if seed is None:
         seed = (time.time_ns() ^ ((request_number + 1) * _GOLDEN)) & _MASK
     return XorShift64Star(seed)
-
-
-def draw_from_candidates(values: Sequence[float], ids: Sequence[int], config: SamplingConfig,
-                         rng: XorShift64Star) -> int:
-    """``values`` sorted descending (ties by ascending id), ``ids`` alongside. A list of one
-    candidate is drawn like any other: the generator moves on, as the reference's does
-    (native/src/v2_runtime.cpp:29722-29733)."""
-    if config.greedy:
-        return int(ids[0])
-    scaled = np.asarray(values, dtype=np.float64) / config.temperature
-    probabilities = np.where(np.isfinite(scaled), np.exp(scaled - scaled[0]), 0.0)
-    total = float(probabilities.sum())
-    if not (total > 0.0 and math.isfinite(total)):
-        return int(ids[0])
-    keep = len(probabilities)
-    if config.top_p < 1.0:
-        cumulative = 0.0
-        for index in range(len(probabilities)):
-            cumulative += probabilities[index] / total
-            if cumulative >= config.top_p:
-                keep = index + 1
-                break
-    if config.min_p > 0.0:
-        floor = config.min_p * probabilities[0]
-        kept = 1
-        while kept < keep and probabilities[kept] >= floor:
-            kept += 1
-        keep = kept
-    kept_total = 0.0
-    for index in range(keep):
-        kept_total += probabilities[index]
-    threshold = rng.uniform() * kept_total
-    cumulative = 0.0
-    for index in range(keep):
-        cumulative += probabilities[index]
-        if threshold <= cumulative:
-            return int(ids[index])
-    return int(ids[keep - 1])
-
-
-def host_candidates(logits: np.ndarray, count: int):
-    """All (count = 0) or the best ``count`` candidates by (value descending, id ascending),
-    NaN last."""
-    keyed = np.where(np.isnan(logits), -np.inf, logits)
-    order = np.lexsort((np.arange(len(logits)), -keyed))
-    if count and count < len(order):
-        order = order[:count]
-    return logits[order], order
 
 
 def pack_settings(configs: Sequence[SamplingConfig], rngs: Sequence[Optional[XorShift64Star]], vocab: int,

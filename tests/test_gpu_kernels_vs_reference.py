@@ -67,9 +67,6 @@ def test_rows_kernels(ops, ref, dtype):
     logits[1, :] = -1.0
     ld = torch.tensor(logits, device=DEV)
     assert ops.argmax_rows(ld).cpu().tolist() == ref.argmax_rows(logits).tolist()
-    values, found = ops.topk_rows(ld, 7)
-    ref_values, ref_ids = ref.topk_rows(logits, 7)
-    assert found.cpu().tolist() == ref_ids.tolist() and np.array_equal(values.cpu().numpy(), ref_values)
 
 
 def test_sampler_draws_the_reference_samplers_tokens(ops, ref):
@@ -251,11 +248,11 @@ def test_decode_attention_with_norm_rotation_and_cache_write_in_front(ops, ref, 
     close(one, want, torch.bfloat16, 2.0)
 
 
-@pytest.mark.parametrize("M,hidden,K,kernel,bias", [(20, 136, 264, 3, False), (64, 72, 1032, 4, True), (8, 200, 520, 2, True), (33, 2048, 2048, 3, False)])
+@pytest.mark.parametrize("M,hidden,K,kernel,bias", [(16, 136, 264, 3, False), (1, 72, 1032, 4, True), (8, 200, 520, 2, True), (13, 2048, 2048, 3, False)])
 def test_products_with_the_short_convolution_behind_them(ops, ref, M, hidden, K, kernel, bias):
     """in_proj with the gated convolution and the state shift in its epilogue, for single-token
-    rows of requests in scattered slots: the split-K product (any rows up to 64) and, up to 16
-    rows, the fused decode product, against the references of the product and of the convolution."""
+    rows of requests in scattered slots (the fused decode product, up to 16 rows), against the
+    references of the product and of the convolution."""
     a, a_h = rounded(RNG.normal(size=(M, K)), torch.bfloat16)
     w, w_h = rounded(RNG.normal(size=(3 * hidden, K)) / math.sqrt(K), torch.bfloat16)
     in_bias = RNG.normal(size=3 * hidden).astype(np.float32) * 0.1 if bias else None
@@ -266,8 +263,7 @@ def test_products_with_the_short_convolution_behind_them(ops, ref, M, hidden, K,
     want_state = state.copy()
     want = ref.shortconv(ref.gemm(a_h, w_h, in_bias), taps, conv_bias, want_state, np.arange(M + 1), slots)
     dev = lambda x: None if x is None else torch.tensor(x, device=DEV)      # noqa: E731
-    kernels = [ops.gemm_medium] + ([ops.gemm_decode] if M <= 16 else [])
-    for kernel_call in kernels:
+    for kernel_call in (ops.gemm_decode,):
         state_d = dev(state)
         out = kernel_call(a, w, ops.EPILOGUE_CONV, bias=dev(in_bias), out_dtype=torch.bfloat16, taps=dev(taps), conv_bias=dev(conv_bias),
                           state=state_d, seg_slot=ints(slots))

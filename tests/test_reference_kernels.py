@@ -113,19 +113,13 @@ def test_norm_rotation_cache_write_and_paged_attention(nh, nkv, hd, window, rota
     assert np.array_equal(copy, k_pages, equal_nan=True)
 
 
-def test_argmax_and_top_k_order():
+def test_argmax_order():
     logits = RNG.normal(size=(4, 300)).astype(np.float32)
     logits[0, 17] = logits[0, 250] = 50.0
     logits[1, :] = 1.0
     logits[2, 5] = np.nan
     assert ref.argmax_rows(logits).tolist() == [17, 0, int(np.nanargmax(logits[2])), int(logits[3].argmax())]
     assert ref.argmax_rows(logits[:, :1]).tolist() == [0, 0, 0, 0]
-    values, ids = ref.topk_rows(logits, 5)
-    assert ids[0, :2].tolist() == [17, 250] and ids[1].tolist() == [0, 1, 2, 3, 4]
-    for r in (0, 3):
-        order = sorted(range(300), key=lambda i: (-float(logits[r, i]), i))[:5]
-        assert ids[r].tolist() == order and np.array_equal(values[r], logits[r, order])
-    assert 5 not in ids[2].tolist() and ref.topk_rows(logits, 300)[1][2, -1] == 5        # NaN sorts last
 
 
 def sampling_cases(count, seed=0):
@@ -155,7 +149,8 @@ def test_sampler_against_the_plain_one_and_the_host_rules():
     """The C++ sampler, the plain implementation's and the package's host rules draw the same
     tokens and leave the generators in the same states, over random rows and settings."""
     import plain_lfm2
-    from flyweight_amd.sampling import SamplingConfig, XorShift64Star, draw_from_candidates, host_candidates
+    from flyweight_amd.sampling import SamplingConfig, XorShift64Star
+    from host_sampling import draw_from_candidates, host_candidates
     drawn = 0
     for logits, settings, states in sampling_cases(40):
         ids, moved_on = ref.sample_rows(logits, settings, states)

@@ -6,8 +6,8 @@ import numpy as np
 import pytest
 
 import plain_lfm2
-from flyweight_amd.sampling import (GREEDY, SamplingConfig, XorShift64Star, defaults, draw_from_candidates,
-                                    host_candidates)
+from flyweight_amd.sampling import GREEDY, SamplingConfig, XorShift64Star, defaults
+from host_sampling import draw_from_candidates, host_candidates
 
 
 def test_defaults_and_validation():
