@@ -3,8 +3,12 @@
   python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one decode step of the whole batch. Prints ONE JSON line: decoded tokens a second
-at batch 8 (``value``), the same at batch 1 and 64 (``points``), the 2,048-token prefill
-(``prefill``) and the decode step's achieved fraction of the HBM roofline (``roofline``).
+at batch 8 over the timed steps (``value``), the same at batch 1 and 64 and over all 512 tokens
+that follow the 2,048-token prompts (``points``), the 2,048-token prefill up to its first token
+(``prefill``) and the decode step's achieved fraction of the HBM roofline (``roofline``); the
+two serving workloads (64 requests behind 32,768-token prompts on the LFM2-350M shape, 128 requests
+of mixed lengths on the LFM2-2.6B shape) run at full size and give their tokens a second in
+``points`` as well.
 Peaks are the MI355X's published ones: HBM 8 TB/s, dense bfloat16 MFMA 2.5 PFLOP/s;
 ``attainable`` gives the same two fractions against a large copy and a large library product
 measured in the same run.
@@ -56,14 +60,17 @@ DECODE_STEPS_PER_TURN = 4      # decode steps the engine runs on the device befo
 
 
 def steps_per_turn(steps: int, warmup: int) -> int:
-    """The engine's decode_steps_per_turn for a run: the timed steps and the warm-up are whole turns."""
-    return DECODE_STEPS_PER_TURN if steps % DECODE_STEPS_PER_TURN == 0 and warmup % DECODE_STEPS_PER_TURN == 0 else 1
+    """The engine's decode_steps_per_turn for a run (the last turn of the warm-up and of the timed
+    steps is cut to the steps that are left, so exactly as many steps run as were asked for)."""
+    return max(1, min(DECODE_STEPS_PER_TURN, steps))
 
 
 def decode_run(torch, model, config, batch: int, steps: int, warmup: int, seed: int = 0, prompt: int = PROMPT,
                context: int = CONTEXT, sampling: dict = None):
     """``batch`` requests with prompts of ``prompt`` tokens (``sampling``: how they draw their tokens; default:
-    the most likely one); returns (seconds for ``steps`` decode steps, mean context, bytes the step must read)."""
+    the most likely one); returns (seconds for ``steps`` decode steps, mean context, bytes the step must read).
+    With ``warmup`` 0 the timed steps begin right behind the prompts' first tokens (the graph of a batch size
+    that has not run before is recorded inside the timed region then: run the same call once before)."""
     import numpy as np
     from flyweight_amd import Runtime
     from flyweight_amd.engine import accounting
@@ -137,6 +144,58 @@ def prefill_run(torch, model, config, repeats: int = 5, behind: int = 0, context
              + accounting.attention_flops(lm, PROMPT, behind))
     runtime.close()
     return statistics.median(times), flops
+
+
+def first_token_run(torch, model, config, repeats: int = 5):
+    """The median time of ``generate(prompt, 1)`` for a 2,048-token prompt: from the call to the first token
+    in the caller's hands (the request submitted and planned, the prompt's one step, the most likely token found
+    on the device and read back), as the reference times its prompt (src/flyweight/runtime_benchmark.py:129-216)."""
+    import statistics
+    import numpy as np
+    from flyweight_amd import Runtime
+    runtime = Runtime(model, context_limit=CONTEXT, parallel_sequences=1, num_pages=PROMPT // 64 + 1,
+                      max_batch_tokens=PROMPT, prefill_rows=PROMPT).prepare()
+    rng = np.random.default_rng(2)
+    times = []
+    for i in range(repeats + 1):
+        tokens = rng.integers(0, config.vocab_size, PROMPT).tolist()
+        torch.cuda.synchronize()
+        began = time.perf_counter()
+        produced = runtime.generate(tokens, 1)
+        elapsed = time.perf_counter() - began
+        assert len(produced) == 1
+        if i > 0:
+            times.append(elapsed)
+    runtime.close()
+    return statistics.median(times)
+
+
+def generation_run(torch, model, config, batch: int, new_tokens: int = 512):
+    """``batch`` requests with 2,048-token prompts that generate ``new_tokens`` tokens each, to the end: decoded
+    tokens a second from the moment every prompt has run until the last request has finished (requests admitted
+    earlier have decoded a few tokens beside the later prompts by then; those are not counted), and the mean
+    context of that stretch. The same job with eight new tokens runs first on the same runtime, so every decode
+    step of the timed stretch is a recorded one."""
+    import numpy as np
+    from flyweight_amd import Runtime
+    pages_each = (PROMPT + new_tokens + 63) // 64
+    runtime = Runtime(model, context_limit=CONTEXT, parallel_sequences=batch, num_pages=pages_each * batch,
+                      max_batch_tokens=PROMPT + batch, prefill_rows=PROMPT, decode_steps_per_turn=DECODE_STEPS_PER_TURN).prepare()
+    rng = np.random.default_rng(3)
+    for count in (8, new_tokens):
+        for _ in range(batch):
+            runtime.task_submit(rng.integers(0, config.vocab_size, PROMPT).tolist(), count)
+        while any(r.computed < len(r.prompt) for r in runtime.scheduler.requests.values()):
+            runtime.engine_step()
+        torch.cuda.synchronize()
+        began = time.perf_counter()
+        tokens = 0
+        while runtime.scheduler.has_work():
+            tokens += sum(1 for event in runtime.engine_step() if event[2] == 0)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - began
+    runtime.close()
+    return tokens / elapsed
 
 
 def attainable_run(torch):
@@ -267,11 +326,13 @@ def further_points(torch, args, points: dict) -> None:
     points["decode_b64_ctx32k_350m_frac"] = round(step_bytes / (seconds / steps) / 1e9 / HBM_PEAK_GBS, 4)
     del model
     torch.cuda.empty_cache()
-    # the two serving workloads at a quarter of their requests: whole jobs through the scheduler, tokens (prompt
-    # and generated) a second; `--workload` runs them at full size with a line of their own
-    for workload, requests in (("long-context", 16), ("mixed", 32)):
+    # the two serving workloads at full size: whole jobs through the scheduler, tokens (prompt and generated) a
+    # second; `--workload` runs one of them alone and prints a line of its own with the run's other figures
+    for workload in ("long-context", "mixed"):
+        requests = WORKLOADS[workload]["requests"]
         record = serving_run(torch, workload, requests)
         points[f"serving_{workload.replace('-', '_')}_{requests}req"] = record["value"]
+        points[f"serving_{workload.replace('-', '_')}_{requests}req_generated_per_s"] = record["generated_per_s"]
 
 
 def main() -> int:
@@ -312,10 +373,12 @@ def main() -> int:
         log(f"{args.batch * args.steps / elapsed:.1f} tokens/s")
         return 0
     log("prefill of 2,048 tokens")
-    prefill_s, prefill_flops = prefill_run(torch, model, config)
+    step_s, prefill_flops = prefill_run(torch, model, config)
     if args.only == "prefill":
-        log(f"{PROMPT / prefill_s:.1f} tokens/s")
+        log(f"{PROMPT / step_s:.1f} tokens/s")
         return 0
+    prefill_s = first_token_run(torch, model, config)
+    log(f"the prompt's step alone {step_s * 1e3:.3f} ms, generate(prompt, 1) {prefill_s * 1e3:.3f} ms")
 
     log(f"decode at batch {args.batch}: {args.warmup} warm-up and {args.steps} timed steps")
     elapsed, mean_context, step_bytes = decode_run(torch, model, config, args.batch, args.steps, args.warmup)
@@ -329,6 +392,10 @@ def main() -> int:
             seconds, _, point_bytes = decode_run(torch, model, config, batch, steps, min(args.warmup, 8))
             points[f"decode_b{batch}"] = round(batch * steps / seconds, 1)
             points[f"decode_b{batch}_frac"] = round(point_bytes / (seconds / steps) / 1e9 / HBM_PEAK_GBS, 4)
+        # the whole stretch the headline configuration names: 512 generated tokens behind 2,048-token prompts
+        for batch in (1, 8, 64):
+            log(f"decode at batch {batch}: all 512 generated tokens")
+            points[f"decode_b{batch}_512tok"] = round(generation_run(torch, model, config, batch), 1)
 
     log("a large copy and a large library product, for what the GPU gives a plain program")
     copy_gbs, product_tflops = attainable_run(torch)
@@ -344,15 +411,17 @@ def main() -> int:
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic: seeded uniform token ids, random-init weights",
         "config": config_record(config, "LFM2-1.2B shape", global_batch=args.batch, prompt_len=PROMPT, seq_len=CONTEXT,
                                 decode_steps_per_turn=steps_per_turn(args.steps, args.warmup), parallelism="single GPU"),
+        # generate(prompt, 1): to the first token in the caller's hands; step_ms: the prompt's one step alone
         "prefill": {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
-                    "frac": round(prefill_flops / prefill_s / MFMA_BF16_PEAK, 4)},
+                    "frac": round(prefill_flops / prefill_s / MFMA_BF16_PEAK, 4), "step_ms": round(step_s * 1e3, 3),
+                    "step_frac": round(prefill_flops / step_s / MFMA_BF16_PEAK, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
         "points": points,
         # the same two fractions against what was measured on this GPU instead of the published peaks
         "attainable": {"copy_gbs": round(copy_gbs, 1), "product_tflops": round(product_tflops, 1),
                        "roofline_frac": round(achieved / copy_gbs, 4),
-                       "prefill_frac": round(prefill_flops / prefill_s / (product_tflops * 1e12), 4)},
+                       "prefill_frac": round(prefill_flops / step_s / (product_tflops * 1e12), 4)},
     }), flush=True)
     return 0
 
