@@ -39,6 +39,8 @@ def _add_runtime(parser: argparse.ArgumentParser, context_default: int) -> None:
     group.add_argument("--context", "--context-window", dest="context_window", type=int, default=context_default,
                        metavar="N", help=f"maximum prompt + output tokens (default {context_default})")
     group.add_argument("--parallel", type=int, default=1, metavar="N", help="requests that may be live at once")
+    group.add_argument("--num-pages", type=int, metavar="N",
+                       help="cache pages of 64 tokens in every page group (default: every live request at the full context)")
     group.add_argument("--prefill-rows", type=int, default=512, metavar="N", help="most tokens of one prompt portion")
     group.add_argument("--max-batch-tokens", type=int, default=2048, metavar="N", help="most tokens of one step")
     group.add_argument("--decode-steps-per-turn", type=int, default=1, metavar="N",
@@ -107,7 +109,7 @@ def _runtime(args, context: Optional[int] = None):
     from .engine import Model, Runtime
     model = Model(args.model, dtype=args.dtype)
     limit = min(context or args.context_window, model.spec.max_positions)
-    return model, Runtime(model, context_limit=limit, parallel_sequences=args.parallel,
+    return model, Runtime(model, context_limit=limit, parallel_sequences=args.parallel, num_pages=args.num_pages,
                           prefill_rows=args.prefill_rows, max_batch_tokens=args.max_batch_tokens,
                           decode_steps_per_turn=args.decode_steps_per_turn).prepare()
 
@@ -157,6 +159,9 @@ def _benchmark(args) -> int:
     measured = sum(gaps)
     ordered = sorted(gaps)
     pick = lambda q: ordered[min(len(ordered) - 1, int(q * len(ordered)))] if ordered else 0.0   # noqa: E731
+    # a short stretch can overstate the sustained rate: the first and the last window side by side show a decay
+    window = min(32, max(1, len(gaps) // 2))
+    rate = lambda part: len(part) / sum(part) if sum(part) > 0 else 0.0     # noqa: E731
     report = {
         "prepare_seconds": prepare_seconds,
         "prompt_tokens": len(args.tokens),
@@ -166,6 +171,10 @@ def _benchmark(args) -> int:
         "median_seconds": statistics.median(gaps) if gaps else 0.0,
         "p90_seconds": pick(0.90),
         "p99_seconds": pick(0.99),
+        "decode_first_window_tokens_per_second": rate(gaps[:window]),
+        "decode_last_window_tokens_per_second": rate(gaps[-window:]),
+        "request_seconds": (arrivals[-1] - began) if arrivals else 0.0,
+        "generated_tokens": len(arrivals),
     }
     if ops.kernel_profile_active():
         report["kernels"] = ops.kernel_profile_report()

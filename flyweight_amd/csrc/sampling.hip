@@ -15,8 +15,10 @@
 // it is gathered without a select: everything at or above the k-th of the threads' own best. A
 // longer list (no top_k) begins with such a batch too, everything at or above the 512th of the
 // threads' best, which stays in LDS for both walks: a peaked row ends both there (81 us at top_p
-// 0.9 against 137 us when each walk selected its own first 1,024). A draw over the whole
-// vocabulary of a flat distribution takes as many batches as it walks through.
+// 0.9 against 137 us when each walk selected its own first 1,024). A long list that this batch does
+// not end (a flat distribution over the whole vocabulary) is not walked at all: the candidate at
+// which a running sum reaches its target is searched digit by digit of its key, the row's mass
+// added up per digit (sample_crossing), a dozen passes over the row whatever its shape.
 // A row whose temperature is 0 takes the best candidate and leaves its generator alone, so
 // greedy and sampled requests share one launch; a drawing row with a single candidate (top_k 1)
 // moves its generator on like any other draw. Nothing is allocated; nothing crosses to the host.
@@ -30,9 +32,18 @@
 
 struct SampleShared {
     unsigned int histogram[SAMPLE_BINS];
-    unsigned long long keys[SAMPLE_BATCH];
-    double p[SAMPLE_BATCH];
-    double running[SAMPLE_BATCH];   // the sum of p up to and including each candidate of the batch
+    union {
+        struct {
+            unsigned long long keys[SAMPLE_BATCH];
+            double p[SAMPLE_BATCH];
+            double running[SAMPLE_BATCH];   // the sum of p up to and including each candidate of the batch
+        };
+        unsigned long long bin_mass[SAMPLE_BINS];   // the search for a crossing: each digit's mass in fixed point
+    };
+    unsigned long long bin_key[SAMPLE_BINS];        // and its greatest key
+    unsigned long long above;                       // fixed-point mass of the keys above the digits found so far
+    unsigned long long found_key;
+    int found;                                      // 0: still searching, 1: the key is found, -1: the sums never get there
     unsigned long long wave_keys[SAMPLE_THREADS / 64];
     double wave_sums[SAMPLE_THREADS / 64];
     unsigned long long prefix;      // of the key being selected, the digits found so far
@@ -251,6 +262,162 @@ __device__ double sample_total(const float* __restrict__ row, int vocab, unsigne
     return total;
 }
 
+// the greatest of the threads' keys; every thread gets it
+__device__ unsigned long long sample_block_max(unsigned long long v, SampleShared& s) {
+    v = sample_wave_max(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s.wave_keys[threadIdx.x >> 6] = v;
+    __syncthreads();
+    unsigned long long best = 0ull;
+    for (int w = 0; w < SAMPLE_THREADS / 64; ++w) best = s.wave_keys[w] > best ? s.wave_keys[w] : best;
+    return best;
+}
+
+// exp((l - best) / T) / divisor of one logit (0 where the scaled logit is not finite)
+__device__ __forceinline__ double sample_part(float value, double best_scaled, double temperature, double divisor) {
+    const double scaled = (double)value / temperature;
+    return __builtin_isfinite(scaled) ? exp(scaled - best_scaled) / divisor : 0.0;
+}
+
+// The sum of the parts of the candidates with key >= at_least and key > above, in a fixed order
+// (each thread its own in the order of their ids, the threads of a wave by halving, the waves in turn).
+__device__ double sample_mass(const float* __restrict__ row, int vocab, unsigned long long at_least, unsigned long long above,
+                              double best_scaled, double temperature, double divisor, SampleShared& s) {
+    double mine = 0.0;
+    sample_for_each(row, vocab, [&](float value, int id) {
+        const unsigned long long key = candidate_key(value, id);
+        if (key >= at_least && key > above) mine += sample_part(value, best_scaled, temperature, divisor);
+    });
+#pragma unroll
+    for (int offset = 32; offset > 0; offset >>= 1) mine += __shfl_xor(mine, offset, 64);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) s.wave_sums[threadIdx.x >> 6] = mine;
+    __syncthreads();
+    double total = 0.0;
+    for (int w = 0; w < SAMPLE_THREADS / 64; ++w) total += s.wave_sums[w];
+    return total;
+}
+
+// A long list is not walked candidate by candidate. The candidate at which the running sum of the
+// parts p / divisor, taken in the list's order (greatest key first) over the candidates with key >=
+// floor_key, first reaches `target`: its key, or 0 if the sum never gets there. Found digit by digit
+// of the key like the select above, with the mass of every digit instead of its count: each pass
+// over the row adds the parts up per digit, in 64-bit fixed point (whole numbers add up to the same
+// sum in any order, so the result does not depend on timing), and the digit in which the running
+// sum passes the target is taken. A digit that holds one candidate ends the search. What fixed
+// point rounds off (2^-47 of the greatest part per candidate) can misplace the answer by a
+// neighbour where the target falls within that of a candidate's edge; the answer is therefore held
+// against the sums in floating point, in the fixed order of sample_mass, and moved to a neighbour
+// until it fits them (which it nearly always does at once). The fixed point is set so that a whole
+// row of parts of 1 stays below 2^63 (2^46 for a vocabulary of 65,536).
+__device__ unsigned long long sample_crossing(const float* __restrict__ row, int vocab, unsigned long long floor_key, double best_scaled,
+                                              double temperature, double target, double divisor, SampleShared& s) {
+    const double SAMPLE_FIXED = ldexp(1.0, 63 - (32 - __clz(vocab)));
+    const double scaled_target = target * SAMPLE_FIXED;
+    unsigned long long target_fixed = scaled_target >= 18446744073709549568.0 ? ~0ull : (unsigned long long)scaled_target;
+    if (target_fixed == 0ull) target_fixed = 1ull;      // (the first candidate reaches any target that is not above its part)
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        s.prefix = 0ull;
+        s.above = 0ull;
+        s.found = 0;
+    }
+    int shift = 64;
+    for (int level = 0; level < 6; ++level) {
+        const int bits = shift >= SAMPLE_DIGIT_BITS ? SAMPLE_DIGIT_BITS : shift;
+        shift -= bits;
+        for (int i = threadIdx.x; i < SAMPLE_BINS; i += SAMPLE_THREADS) {
+            s.histogram[i] = 0u;
+            s.bin_mass[i] = 0ull;
+            s.bin_key[i] = 0ull;
+        }
+        __syncthreads();
+        const unsigned long long prefix = s.prefix;
+        const int over = shift + bits;
+        sample_for_each(row, vocab, [&](float value, int id) {
+            const unsigned long long key = candidate_key(value, id);
+            if (key >= floor_key && (over >= 64 || (key >> over) == prefix)) {
+                const unsigned int digit = (unsigned int)(key >> shift) & ((1u << bits) - 1u);
+                const double part = sample_part(value, best_scaled, temperature, divisor) * SAMPLE_FIXED;
+                atomicAdd(&s.histogram[digit], 1u);
+                atomicAdd(&s.bin_mass[digit], part >= 18446744073709549568.0 ? ~0ull : (unsigned long long)part);
+                atomicMax(&s.bin_key[digit], key);
+            }
+        });
+        __syncthreads();
+        if (threadIdx.x < 64) {
+            const int lane = threadIdx.x, per_lane = SAMPLE_BINS / 64;
+            const int first = SAMPLE_BINS - 1 - lane * per_lane;    // lane 0 holds the highest digits
+            unsigned long long mine = 0ull;
+            for (int b = 0; b < per_lane; ++b) mine += s.bin_mass[first - b];
+            unsigned long long before = mine;
+#pragma unroll
+            for (int offset = 1; offset < 64; offset <<= 1) {
+                const unsigned long long other = __shfl_up(before, offset, 64);
+                if (lane >= offset) before += other;
+            }
+            const unsigned long long start = s.above;
+            const unsigned long long all = __shfl(before, 63, 64);
+            if (start + all < target_fixed) {
+                if (lane == 0) s.found = -1;
+            } else {
+                const unsigned long long ahead = start + (before - mine);
+                if (ahead < target_fixed && target_fixed <= ahead + mine) {     // the digit is among this lane's
+                    unsigned long long passed = ahead;
+                    int digit = first;
+                    for (int b = 0; b < per_lane; ++b) {
+                        const unsigned long long here = s.bin_mass[first - b];
+                        if (passed + here >= target_fixed) {
+                            digit = first - b;
+                            break;
+                        }
+                        passed += here;
+                    }
+                    s.prefix = (prefix << bits) | (unsigned long long)digit;
+                    s.above = passed;
+                    if (s.histogram[digit] == 1u) {
+                        s.found_key = s.bin_key[digit];
+                        s.found = 1;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        if (s.found != 0) break;
+    }
+    if (s.found < 0) return 0ull;
+    unsigned long long key = s.found > 0 ? s.found_key : s.prefix;
+    // held against the sums in floating point
+    for (int tries = 0; tries < 8; ++tries) {
+        const double before = sample_mass(row, vocab, floor_key, key, best_scaled, temperature, divisor, s);
+        const double own = sample_part(row[candidate_id(key)], best_scaled, temperature, divisor);
+        if (before >= target) {
+            // reached before this candidate: the one before it in the list (the least key above)
+            unsigned long long next = 0ull;
+            sample_for_each(row, vocab, [&](float value, int id) {
+                const unsigned long long k = candidate_key(value, id);
+                if (k > key && ~k > next) next = ~k;
+            });
+            next = sample_block_max(next, s);
+            if (next == 0ull) break;
+            key = ~next;
+        } else if (before + own < target) {
+            // not yet reached with this candidate: the one behind it (the greatest key below, inside the list)
+            unsigned long long next = 0ull;
+            sample_for_each(row, vocab, [&](float value, int id) {
+                const unsigned long long k = candidate_key(value, id);
+                if (k < key && k >= floor_key && k > next) next = k;
+            });
+            next = sample_block_max(next, s);
+            if (next == 0ull) return 0ull;      // the list ends here: the sums never get there
+            key = next;
+        } else {
+            break;
+        }
+    }
+    return key;
+}
+
 // settings: [rows][4] = temperature, top_k (a whole number), top_p, min_p. states: the rows'
 // generators, read and moved on by the rows that draw.
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float* __restrict__ logits,
@@ -319,7 +486,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
     // Up to 1,024 candidates are one batch. Everything at or above the bound is gathered at once; that
     // is the wanted candidates and usually few more (only a row with very many equal values gives more
     // than a batch holds: then the exact key of the last wanted candidate is selected first).
-    bool first_batch_ready = false;
     int first_count = 0, first_asked = 0;       // asked: how many a batch was meant to hold (fewer came: nothing is left below)
     if (candidates <= SAMPLE_BATCH) {
         // (beyond half a batch the bound lies so low that what is above it seldom fits: 768 wanted of
@@ -332,7 +498,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
             count = sample_batch(row, vocab, floor_key, ~0ull, best_scaled, temperature, s);
         }
         first_count = count < candidates ? count : (int)candidates;
-        first_batch_ready = true;
     } else {
         // The best of a longer list, gathered at once like a short list's: both walks begin with them,
         // and a peaked row ends both there. How many they are is not known beforehand (512 at least),
@@ -343,7 +508,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
             first_count = sample_batch(row, vocab, floor_key, ~0ull, best_scaled, temperature, s);
             first_asked = SAMPLE_BATCH;
         }
-        first_batch_ready = true;
     }
     // the sum over all candidates, which the shares of top_p are taken of
     double total = 1.0;
@@ -357,9 +521,9 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
     }
 
     // First walk: where the kept prefix ends (top_p, min_p) and the sum of its p. Second walk: the
-    // draw. Both go through the candidates in order, a batch at a time (with one batch it stays in
-    // LDS); inside a batch thread i holds candidate i and the running sums up to it.
-    double share_before = 0.0, mass_before = 0.0;       // of the batches walked so far
+    // draw. Both go through the batch in LDS in order: thread i holds candidate i and the running
+    // sums up to it.
+    double mass_before = 0.0;       // the sum of the kept p, once the first walk has found where they end
     long long keep = candidates;
     double threshold = 0.0;
     unsigned long long moved_on = 0ull;
@@ -372,9 +536,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
         if (candidates < vocab) floor_key = sample_select(over_row, 0ull, ~0ull, (unsigned int)candidates, s);
         mass_before = sample_total(row, vocab, floor_key, best_scaled, temperature, s);
     }
-    for (int walk = no_cuts ? 1 : 0; walk < 2; ++walk) {
-        unsigned long long ceiling = ~0ull;
-        long long position = 0;
+    bool long_list = false;
+    for (int walk = no_cuts ? 1 : 0; walk < 2 && !long_list; ++walk) {
         const long long limit = walk == 0 ? candidates : keep;
         if (walk == 1) {
             // the draw (the generator moves on exactly once per drawn token; every thread forms the same numbers)
@@ -387,66 +550,86 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_rows_kernel(const float
             threshold = u * mass_before;        // the sum of the kept p
             mass_before = 0.0;
         }
+        // the batch in LDS: made before the walks, the list's first candidates
+        const int count = first_count;
+        const int here = limit < count ? (int)limit : count;
+        const bool mine_counts = (int)threadIdx.x < here;
+        const double p = mine_counts ? s.p[threadIdx.x] : 0.0;
+        const double mass = mass_before + sample_running_sum(p, s, false);
+        s.running[threadIdx.x] = mass;
+        int first_stop = SAMPLE_BATCH;      // the first candidate of the batch at which the walk ends
         bool stopped = false;
-        while (position < limit && !stopped) {
-            int count, asked;
-            if (position == 0 && first_batch_ready) {
-                count = first_count;        // still in LDS: made before the walks, and no later batch has taken its place
-                asked = first_asked;
+        if (walk == 0) {
+            const double share = top_p < 1.0 ? sample_running_sum(p / total, s, false) : 0.0;
+            const bool below_min = min_p > 0.0 && threadIdx.x >= 1 && p < min_p;      // p of the best is 1
+            const bool reaches_top = top_p < 1.0 && share >= top_p;
+            if (mine_counts && (below_min || reaches_top)) first_stop = threadIdx.x;
+            first_stop = sample_least(first_stop, s);
+            if (first_stop < SAMPLE_BATCH) {
+                // the candidate at which it ends tells the others what is kept: up to it, without it if
+                // its p is below min_p (that is looked at first), with it if its share reaches top_p
+                if ((int)threadIdx.x == first_stop) s.keep_here = below_min ? first_stop : first_stop + 1;
+                __syncthreads();
+                keep = s.keep_here;
+                if (s.keep_here > 0) mass_before = s.running[s.keep_here - 1];
+                stopped = true;
             } else {
-                first_batch_ready = false;
-                const long long left = limit - position;
-                const unsigned int want = left < SAMPLE_BATCH ? (unsigned int)left : SAMPLE_BATCH;
-                const unsigned long long floor_key = sample_select(over_row, position == 0 ? bound : 0ull, ceiling, want, s);
-                count = sample_batch(row, vocab, floor_key, ceiling, best_scaled, temperature, s);
-                asked = (int)want;
+                __syncthreads();
+                mass_before = s.running[here - 1];      // everything in the batch is kept
             }
-            if (count == 0) break;
-            const int here = limit - position < count ? (int)(limit - position) : count;
-            const bool mine_counts = (int)threadIdx.x < here;
-            const double p = mine_counts ? s.p[threadIdx.x] : 0.0;
-            const double mass = mass_before + sample_running_sum(p, s, false);
-            s.running[threadIdx.x] = mass;
-            int first_stop = SAMPLE_BATCH;      // the first candidate of the batch at which the walk ends
-            if (walk == 0) {
-                const double share = top_p < 1.0 ? share_before + sample_running_sum(p / total, s, false) : 0.0;
-                const bool below_min = min_p > 0.0 && position + threadIdx.x >= 1 && p < min_p;      // p of the best is 1
-                const bool reaches_top = top_p < 1.0 && share >= top_p;
-                if (mine_counts && (below_min || reaches_top)) first_stop = threadIdx.x;
-                first_stop = sample_least(first_stop, s);
-                if (first_stop < SAMPLE_BATCH) {
-                    // the candidate at which it ends tells the others what is kept: up to it, without it if
-                    // its p is below min_p (that is looked at first), with it if its share reaches top_p
-                    if ((int)threadIdx.x == first_stop) s.keep_here = below_min ? first_stop : first_stop + 1;
-                    __syncthreads();
-                    keep = position + s.keep_here;
-                    if (s.keep_here > 0) mass_before = s.running[s.keep_here - 1];
-                    stopped = true;
-                } else {
-                    if ((int)threadIdx.x == here - 1) s.kept_share = share;
-                    __syncthreads();
-                    mass_before = s.running[here - 1];
-                    share_before = s.kept_share;
-                }
-            } else {
-                if (mine_counts && threshold <= mass) first_stop = threadIdx.x;
-                first_stop = sample_least(first_stop, s);
-                if (first_stop < SAMPLE_BATCH) {
-                    token = candidate_id(s.keys[first_stop]);
-                    stopped = true;
-                } else {
-                    token = candidate_id(s.keys[here - 1]);     // the last of the kept, should the sum never get there
-                    __syncthreads();
-                    mass_before = s.running[here - 1];
-                }
-            }
-            __syncthreads();
-            ceiling = s.keys[count - 1];
-            position += count;
-            if (count < asked) break;       // fewer than were asked for: nothing is left below
-            __syncthreads();
+        } else {
+            if (mine_counts && threshold <= mass) first_stop = threadIdx.x;
+            first_stop = sample_least(first_stop, s);
+            stopped = first_stop < SAMPLE_BATCH;
+            // (the last of the kept, should the sum never get there)
+            token = candidate_id(s.keys[stopped ? first_stop : here - 1]);
         }
+        __syncthreads();
+        // The walk goes on behind the batch if the list does (a batch that was selected to hold 1,024 and
+        // holds fewer has everything). A long list is not walked batch by batch: the search below.
+        if (!stopped && here < limit && !(first_asked > 0 && count < first_asked)) long_list = true;
     }
+    if (long_list) {
+        // The kept candidates are those from some key up: the last of top_k, the candidate at which the
+        // shares reach top_p, the least whose p is not below min_p (p falls along the list), whichever
+        // is greatest. Then the draw: the candidate at which the running sum reaches u times the kept sum.
+        __syncthreads();        // every wave has left the batch's arrays, which the search's bins lie over
+        unsigned long long keep_key = 0ull;
+        if (candidates < vocab) keep_key = sample_select(over_row, 0ull, ~0ull, (unsigned int)candidates, s);
+        const unsigned long long list_floor = keep_key;
+        if (top_p < 1.0) {
+            const unsigned long long reached = sample_crossing(row, vocab, list_floor, best_scaled, temperature, top_p, total, s);
+            keep_key = reached > keep_key ? reached : keep_key;
+        }
+        if (min_p > 0.0) {
+            unsigned long long least = 0ull;        // of the complements: the least key whose p holds
+            sample_for_each(row, vocab, [&](float value, int id) {
+                const unsigned long long key = candidate_key(value, id);
+                if (key >= list_floor && sample_part(value, best_scaled, temperature, 1.0) >= min_p && ~key > least) least = ~key;
+            });
+            least = sample_block_max(least, s);
+            if (least != 0ull && ~least > keep_key) keep_key = ~least;
+        }
+        const double kept_mass = sample_mass(row, vocab, keep_key, 0ull, best_scaled, temperature, 1.0, s);
+        unsigned long long x = states[r] ? states[r] : 0x9E3779B97F4A7C15ull;
+        x ^= x >> 12;
+        x ^= x << 25;
+        x ^= x >> 27;
+        moved_on = x;
+        const double u = (double)((x * 2685821657736338717ull) >> 11) * (1.0 / 9007199254740992.0);
+        unsigned long long drawn = sample_crossing(row, vocab, keep_key, best_scaled, temperature, u * kept_mass, 1.0, s);
+        if (drawn == 0ull) {
+            // the sum never got there: the last of the kept (the least key from keep_key up)
+            unsigned long long least = 0ull;
+            sample_for_each(row, vocab, [&](float value, int id) {
+                const unsigned long long key = candidate_key(value, id);
+                if (key >= keep_key && ~key > least) least = ~key;
+            });
+            drawn = ~sample_block_max(least, s);
+        }
+        token = candidate_id(drawn);
+    }
+    __syncthreads();        // (every thread has read the generator's state before it moves on)
     if (threadIdx.x == 0) states[r] = moved_on;
     leave(token);
 }

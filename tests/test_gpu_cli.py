@@ -58,6 +58,12 @@ def test_generate_with_a_seed_reproduces_and_refuses_what_it_cannot_do(folders, 
     assert status == 1 and "stop token 100000 is outside the vocabulary" in err
     status, out, err = run(capsys, "generate", folder, "--tokens", "1,100000")
     assert status == 1 and "token id 100000 at place 1" in err
+    # a cache of two pages holds 128 tokens of one request: a request that needs a third page is refused by name
+    status, out, err = run(capsys, "generate", folder, "--tokens", "1,2", "--max-tokens", "100", "--num-pages", "2", "--temperature", "0",
+                           "--ignore-eos")
+    assert status == 0 and len(out.split()) == 100
+    status, out, err = run(capsys, "generate", folder, "--tokens", "1,2", "--max-tokens", "200", "--num-pages", "2", "--ignore-eos")
+    assert status == 1 and "cache pages" in err
     status, out, err = run(capsys, "generate", folder + "-missing", "--tokens", "1,2")
     assert status == 1 and err.startswith("flyweight-amd:")
 
@@ -68,6 +74,8 @@ def test_benchmark_and_inspect_print_json(folders, capsys):
     assert status == 0 and report["prompt_tokens"] == 3 and report["iterations"] == 9
     assert report["decode_tokens_per_second"] > 0 and 0 < report["median_seconds"] <= report["p99_seconds"]
     assert report["prompt_and_first_token_seconds"] > 0 and report["prepare_seconds"] > 0
+    assert report["decode_first_window_tokens_per_second"] > 0 and report["decode_last_window_tokens_per_second"] > 0
+    assert report["generated_tokens"] == 1 + 2 + 9 and report["request_seconds"] > report["prompt_and_first_token_seconds"]
     # the same with the per-kernel profile: GPU time per kernel entry point, and steps without graphs
     from flyweight_amd.kernels import ops
     try:
