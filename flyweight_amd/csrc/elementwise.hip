@@ -16,7 +16,7 @@ void fw_set_error(const char* format, ...) {
     va_end(args);
 }
 extern "C" const char* fw_last_error(void) { return fw_error_text; }
-extern "C" int fw_abi_version(void) { return 8; }
+extern "C" int fw_abi_version(void) { return 9; }
 
 // ---- embedding -------------------------------------------------------------------------
 // The reference gathers one row per token and widens it to float32

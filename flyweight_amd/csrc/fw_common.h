@@ -158,6 +158,19 @@ __device__ __forceinline__ float block_sum(float v, float* scratch /* >= 16 floa
 
 static inline int fw_ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
+// Eight bfloat16 of a weight matrix that a decode step reads once: with `streamed` the load says
+// so (nontemporal), which keeps a stream of weights from pushing the step's activations out of the
+// caches and, on whole 1 KB pieces per wave, reads faster (a read-only kernel over 268 MB: 39.5 against
+// 43.7 us). Weights in row-major order are loaded as they always were.
+typedef __attribute__((ext_vector_type(8))) __bf16 fw_bf16x8;
+typedef __attribute__((ext_vector_type(4))) uint32_t fw_u32x4;
+template <bool STREAMED>
+__device__ __forceinline__ fw_bf16x8 fw_load_weights(const uint16_t* from) {
+    const fw_u32x4* at = reinterpret_cast<const fw_u32x4*>(from);
+    const fw_u32x4 v = STREAMED ? __builtin_nontemporal_load(at) : *at;
+    return __builtin_bit_cast(fw_bf16x8, v);
+}
+
 // ---- candidates for the next token ----------------------------------------------------
 // A candidate is ordered by (value descending, id ascending); NaN sorts last. The key packs both
 // so that one 64-bit comparison orders two candidates (a greater key comes first) and ties go to

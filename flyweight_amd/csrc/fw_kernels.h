@@ -71,7 +71,7 @@ int fw_gemm_mfma_split(const void* a, const void* w, const float* bias, void* ou
 // (next_activations [M][N] bfloat16, next_squares [squares_rows][16 for M <= 16, else 64]), and
 // any mode takes such prepared activations as a, with squares / squares_rows / eps.
 int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* workspace_bytes, int* counters, int* squares_rows);
-int fw_gemm_medium(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
+int fw_gemm_medium(const void* a, const void* w, int w_tiled, const float* bias, void* out, int out_dtype, int mode,
                    int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
                    int counters_len, const float* next_norm_weight, int next_one_centered,
                    void* next_activations, float* next_squares, const float* squares, int squares_rows,
@@ -87,8 +87,13 @@ int fw_gemm_medium(const void* a, const void* w, const float* bias, void* out, i
 // [M][N] = x_new * w_next and next_squares [fw_gemm_decode_accumulate_tiles(N)][16], per-tile sums
 // of x_new^2 of every row. A later call takes them with prologue 2 (a = those activations,
 // squares/squares_tiles = those sums, eps) and applies the row's scale in its epilogue.
+// w_tiled (here and in fw_gemm_medium): w is not row-major [rows][K] but lies in operand tiles,
+// [rows / 16][K / 32][4][16][8]: tile (i, j) holds rows 16 i .. 16 i + 15, columns 32 j .. 32 j + 31 as
+// 1 KB in the order in which a wave loads a matrix-core operand (lane = 16 * (column / 8) + row), so
+// that a wave reads whole contiguous kilobytes (rows padded with zeros to a multiple of 16; K a
+// multiple of 32). The same sums in the same order: the results are bit for bit those of row-major w.
 int fw_gemm_decode(int prologue, const void* a, const float* norm_weight, const int32_t* row_index, float eps,
-                   int one_centered, const void* w, const float* bias, void* out, int out_dtype, int epilogue,
+                   int one_centered, const void* w, int w_tiled, const float* bias, void* out, int out_dtype, int epilogue,
                    int M, int N, int K, const float* taps, const float* conv_bias, float* state,
                    const int32_t* seg_slot, int kernel_size, const float* next_norm_weight,
                    int next_one_centered, void* next_activations, float* next_squares, const float* squares,

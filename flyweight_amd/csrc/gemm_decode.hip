@@ -44,7 +44,8 @@ struct DecodeGemmArgs {
     const int32_t* row_index;   // gather of x rows, or null
     float eps;
     int one_centered;
-    const uint16_t* w;          // [tiles * tile_stride ...][K]
+    const uint16_t* w;          // [tiles * tile_stride ...][K], or the same in operand tiles (w_tiled)
+    int w_tiled;                // W lies in tiles of 16 rows x 32 columns, each 1 KB in the order of a wave's operand load
     const float* bias;          // per W row, or null
     void* out;
     int M, N, K;                // N: features per tile kind (output width)
@@ -71,7 +72,7 @@ __device__ __forceinline__ float dg_silu(float g) {
     return g * e / (1.0f + e);
 }
 
-template <int RT, int WAVES, int ROWS, int PRO, int EPI, typename TO>
+template <int RT, int WAVES, int ROWS, int PRO, int EPI, typename TO, bool WT>
 __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGemmArgs p, const int num_tiles) {
     __shared__ float partial[WAVES][RT][64][4];
     __shared__ float squares[WAVES][16];
@@ -115,7 +116,11 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
             const int feature = tile * ROWS + (ROWS == 16 ? r16 : (r16 & 7));
             const int n = TILED ? feature + rt * p.tile_stride : feature + rt * ROWS * num_tiles;
             w_ok[rt] = TILED ? feature < N : n < N;
-            w_row[rt] = p.w + (size_t)(w_ok[rt] ? n : 0) * K;
+            const int row = w_ok[rt] ? n : 0;
+            // row-major: the row's start (the column is added at each load); in operand tiles: this lane's
+            // 16 bytes of the tile row's first tile (a tile further along K lies 512 elements on)
+            w_row[rt] = WT ? p.w + ((size_t)(row >> 4) * (size_t)(K >> 5) << 9) + (((g << 4) | (row & 15)) << 3)
+                           : p.w + (size_t)row * K;
         }
         f32x4 acc[RT];
 #pragma unroll
@@ -147,9 +152,10 @@ __global__ __launch_bounds__(WAVES * 64) void decode_gemm_kernel(const DecodeGem
                 const bool ok = k + g * 8 < K;          // K is a multiple of 8: a run of 8 is in or out as a whole
                 const int from = ok ? k + g * 8 : 0;    // columns 0..7 always exist
                 const bf16x8 none = {0, 0, 0, 0, 0, 0, 0, 0};
+                const size_t w_from = WT ? (ok ? (size_t)(k >> 5) << 9 : 0) : (size_t)from;
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
-                    const bf16x8 v = *reinterpret_cast<const bf16x8*>(w_row[rt] + from);
+                    const bf16x8 v = fw_load_weights<WT>(w_row[rt] + w_from);
                     wf[rt][j] = (ok && w_ok[rt]) ? v : none;
                 }
                 if (PRO != 1) {
@@ -335,7 +341,8 @@ static int launch(const DecodeGemmArgs& args, hipStream_t stream) {
     const int tile_features = (EPI == DG_STORE || EPI == DG_ACCUMULATE) ? ROWS * RT : ROWS;
     const int num_tiles = fw_ceil_div(args.N, tile_features);
     const int blocks = num_tiles > DG_MAX_BLOCKS ? DG_MAX_BLOCKS : num_tiles;
-    decode_gemm_kernel<RT, WAVES, ROWS, PRO, EPI, TO><<<blocks, WAVES * 64, 0, stream>>>(args, num_tiles);
+    if (args.w_tiled) decode_gemm_kernel<RT, WAVES, ROWS, PRO, EPI, TO, true><<<blocks, WAVES * 64, 0, stream>>>(args, num_tiles);
+    else decode_gemm_kernel<RT, WAVES, ROWS, PRO, EPI, TO, false><<<blocks, WAVES * 64, 0, stream>>>(args, num_tiles);
     return 0;
 }
 
@@ -343,9 +350,10 @@ static int launch(const DecodeGemmArgs& args, hipStream_t stream) {
 // optional row_index); 2: a bfloat16 [M][K] = x * w left by an accumulating call together with
 // `squares` [squares_tiles][16], the row's scale is formed from those. epilogue 0: store out_dtype [M][N]; 1: float32 out += ; 2: SwiGLU, w =
 // [gate rows; up rows], out bfloat16 [M][N]; 3: gated short convolution, w = [B rows; C rows; x
-// rows] of N channels each, out_dtype [M][N], state updated.
+// rows] of N channels each, out_dtype [M][N], state updated. w_tiled: w is given in operand tiles
+// (fw_tile_weights) instead of row-major; the results are bit for bit the same.
 extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_weight, const int32_t* row_index,
-                              float eps, int one_centered, const void* w, const float* bias, void* out,
+                              float eps, int one_centered, const void* w, int w_tiled, const float* bias, void* out,
                               int out_dtype, int epilogue, int M, int N, int K, const float* taps,
                               const float* conv_bias, float* state, const int32_t* seg_slot, int kernel_size,
                               const float* next_norm_weight, int next_one_centered, void* next_activations,
@@ -353,6 +361,7 @@ extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_wei
     FW_REQUIRE(M >= 1 && M <= 16, "gemm_decode: takes 1..16 rows, got %d", M);
     FW_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_decode: K (%d) must be a positive multiple of 8, N (%d) positive", K, N);
     FW_REQUIRE(prologue >= 0 && prologue <= 2, "gemm_decode: unknown prologue %d", prologue);
+    FW_REQUIRE(!w_tiled || K % 32 == 0, "gemm_decode: weights in operand tiles need K (%d) to be a multiple of 32", K);
     FW_REQUIRE(prologue != 2 || (squares != nullptr && squares_tiles >= 1 && eps > 0.0f), "gemm_decode: the pre-normed prologue needs the partial sums of squares and eps");
     FW_REQUIRE((next_activations == nullptr) == (next_squares == nullptr) && (next_activations == nullptr) == (next_norm_weight == nullptr),
                "gemm_decode: the next norm's weight, activations and sums of squares come together");
@@ -369,7 +378,7 @@ extern "C" int fw_gemm_decode(int prologue, const void* a, const float* norm_wei
                "gemm_decode: operands must be 16-byte aligned");
     DecodeGemmArgs args;
     args.a = a; args.norm_weight = norm_weight; args.row_index = row_index; args.eps = eps; args.one_centered = one_centered;
-    args.w = (const uint16_t*)w; args.bias = bias; args.out = out; args.M = M; args.N = N; args.K = K;
+    args.w = (const uint16_t*)w; args.w_tiled = w_tiled ? 1 : 0; args.bias = bias; args.out = out; args.M = M; args.N = N; args.K = K;
     args.tile_stride = (epilogue == DG_SWIGLU || epilogue == DG_CONV) ? N : 0;
     args.taps = taps; args.conv_bias = conv_bias; args.state = state; args.seg_slot = seg_slot; args.kernel_size = kernel_size;
     args.next_norm_weight = next_norm_weight; args.next_one_centered = next_one_centered;

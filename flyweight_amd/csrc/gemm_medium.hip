@@ -37,6 +37,7 @@ enum { GM_STORE = 0, GM_ACCUMULATE = 1, GM_SWIGLU = 2 };
 struct MediumArgs {
     const uint16_t* a;
     const uint16_t* w;
+    int w_tiled;            // W lies in tiles of 16 rows x 32 columns, each 1 KB in the order of a wave's operand load
     const float* bias;
     void* out;
     int M, N, K;            // N: output features (for SwiGLU w has 2N rows: gate, then up)
@@ -69,7 +70,7 @@ __device__ __forceinline__ float gm_silu(float g) {
 
 // MT: tiles of 16 rows of a. FW: waves side by side over features (4: 64 features, no split of
 // K inside the workgroup; 2: 32 features, the two halves of a 128-k chunk go to wave pairs).
-template <int MT, int FW, int MODE, typename TO, bool ROTATE>
+template <int MT, int FW, int MODE, typename TO, bool ROTATE, bool WT>
 __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArgs p) {
     constexpr int KP = 4 / FW;                  // parts of K inside the workgroup
     constexpr int CHUNK = 64 * KP;              // k per iteration of the workgroup
@@ -97,7 +98,11 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
     const int feature = n0 + 16 * ft + r16;
     const uint16_t* w_row[KINDS];
 #pragma unroll
-    for (int kind = 0; kind < KINDS; ++kind) w_row[kind] = p.w + (size_t)((feature < N ? feature : 0) + kind * N) * K;
+    for (int kind = 0; kind < KINDS; ++kind) {
+        const int row = (feature < N ? feature : 0) + kind * N;
+        w_row[kind] = WT ? p.w + ((size_t)(row >> 4) * (size_t)(K >> 5) << 9) + (((g << 4) | (row & 15)) << 3)
+                         : p.w + (size_t)row * K;
+    }
     const uint16_t* a_piece[AP];
     int piece_row[AP], piece_k[AP];
 #pragma unroll
@@ -136,9 +141,10 @@ __global__ __launch_bounds__(GM_THREADS) void gemm_medium_kernel(const MediumArg
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             const int k = k0 + kp * 64 + ks * 32 + g * 8;
+            // (slices and chunks begin at multiples of 32, and K is one where W lies in tiles: a tile's columns are inside or outside together)
+            const size_t from = k < k_end ? (WT ? (size_t)(k >> 5) << 9 : (size_t)k) : 0;
 #pragma unroll
-            for (int kind = 0; kind < KINDS; ++kind)
-                wf[d][kind][ks] = *reinterpret_cast<const bf16x8*>(w_row[kind] + (k < k_end ? k : 0));
+            for (int kind = 0; kind < KINDS; ++kind) wf[d][kind][ks] = fw_load_weights<WT>(w_row[kind] + from);
         }
 #pragma unroll
         for (int i = 0; i < AP; ++i) {
@@ -438,25 +444,30 @@ extern "C" int fw_gemm_medium_plan(int M, int N, int K, int mode, size_t* worksp
     return 0;
 }
 
-template <int MT, int FW, bool ROTATE>
+template <int MT, int FW, bool ROTATE, bool WT>
 static void medium_launch_as(const MediumArgs& args, int out_dtype, int mode, dim3 grid, hipStream_t stream) {
-    if (mode == GM_SWIGLU) gemm_medium_kernel<MT, FW, GM_SWIGLU, bf16_t, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
-    else if (mode == GM_ACCUMULATE) gemm_medium_kernel<MT, FW, GM_ACCUMULATE, float, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
-    else if (out_dtype == FW_F32) gemm_medium_kernel<MT, FW, GM_STORE, float, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
-    else gemm_medium_kernel<MT, FW, GM_STORE, bf16_t, ROTATE><<<grid, GM_THREADS, 0, stream>>>(args);
+    if (mode == GM_SWIGLU) gemm_medium_kernel<MT, FW, GM_SWIGLU, bf16_t, ROTATE, WT><<<grid, GM_THREADS, 0, stream>>>(args);
+    else if (mode == GM_ACCUMULATE) gemm_medium_kernel<MT, FW, GM_ACCUMULATE, float, ROTATE, WT><<<grid, GM_THREADS, 0, stream>>>(args);
+    else if (out_dtype == FW_F32) gemm_medium_kernel<MT, FW, GM_STORE, float, ROTATE, WT><<<grid, GM_THREADS, 0, stream>>>(args);
+    else gemm_medium_kernel<MT, FW, GM_STORE, bf16_t, ROTATE, WT><<<grid, GM_THREADS, 0, stream>>>(args);
 }
 
 template <int MT, int FW>
 static void medium_launch(const MediumArgs& args, int out_dtype, int mode, dim3 grid, hipStream_t stream) {
-    if (args.rotate) medium_launch_as<MT, FW, true>(args, out_dtype, mode, grid, stream);
-    else medium_launch_as<MT, FW, false>(args, out_dtype, mode, grid, stream);
+    if (args.rotate) {
+        if (args.w_tiled) medium_launch_as<MT, FW, true, true>(args, out_dtype, mode, grid, stream);
+        else medium_launch_as<MT, FW, true, false>(args, out_dtype, mode, grid, stream);
+    } else {
+        if (args.w_tiled) medium_launch_as<MT, FW, false, true>(args, out_dtype, mode, grid, stream);
+        else medium_launch_as<MT, FW, false, false>(args, out_dtype, mode, grid, stream);
+    }
 }
 
 // mode 0: out = a . w^T (+ bias) stored as out_dtype; 1: out (float32) += a . w^T (+ bias);
 // 2: w is [2 * N][K] (gate rows, then up rows); out [M][N] bfloat16 = silu(gate) * up.
 // workspace / counters: as fw_gemm_medium_plan says for this shape. Calls that overlap on one
 // device must not share counters or workspace.
-extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, void* out, int out_dtype, int mode,
+extern "C" int fw_gemm_medium(const void* a, const void* w, int w_tiled, const float* bias, void* out, int out_dtype, int mode,
                               int M, int N, int K, void* workspace, size_t workspace_bytes, int* counters,
                               int counters_len, const float* next_norm_weight, int next_one_centered,
                               void* next_activations, float* next_squares, const float* squares, int squares_rows,
@@ -464,6 +475,7 @@ extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, v
     FW_REQUIRE(M >= 1 && M <= 64, "gemm_medium: takes 1..64 rows, got %d", M);
     FW_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "gemm_medium: K (%d) must be a positive multiple of 8, N (%d) positive", K, N);
     FW_REQUIRE(mode >= 0 && mode <= 2, "gemm_medium: unknown mode %d", mode);
+    FW_REQUIRE(!w_tiled || K % 32 == 0, "gemm_medium: weights in operand tiles need K (%d) to be a multiple of 32", K);
     FW_REQUIRE(mode != GM_ACCUMULATE || out_dtype == FW_F32, "gemm_medium: accumulation needs a float32 destination");
     FW_REQUIRE(mode != GM_SWIGLU || (out_dtype == FW_BF16 && bias == nullptr), "gemm_medium: SwiGLU stores bfloat16 and takes no bias");
     FW_REQUIRE(out_dtype == FW_F32 || out_dtype == FW_BF16, "gemm_medium: unknown out dtype %d", out_dtype);
@@ -479,7 +491,7 @@ extern "C" int fw_gemm_medium(const void* a, const void* w, const float* bias, v
                "gemm_medium: this shape needs %zu bytes of workspace and %d counters", plan.workspace_bytes, plan.tiles);
     FW_REQUIRE(plan.tiles <= 65535 * 16 && plan.splits <= 65535, "gemm_medium: too many tiles");
     MediumArgs args;
-    args.a = (const uint16_t*)a; args.w = (const uint16_t*)w; args.bias = bias; args.out = out;
+    args.a = (const uint16_t*)a; args.w = (const uint16_t*)w; args.w_tiled = w_tiled ? 1 : 0; args.bias = bias; args.out = out;
     args.M = M; args.N = N; args.K = K; args.k_per_split = plan.k_per_split; args.splits = plan.splits;
     args.partials = (float*)workspace; args.counters = counters;
     args.next_norm_weight = next_norm_weight; args.next_one_centered = next_one_centered;

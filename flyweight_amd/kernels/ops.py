@@ -19,7 +19,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _lib = None
 
@@ -432,14 +432,15 @@ def gather_rows(rows: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
     return embed_rows(rows, index)
 
 
-def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int) -> None:
+def _fast_gemm(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int,
+               w_tiled: Optional[torch.Tensor] = None) -> None:
     """bfloat16 operands on the matrix cores: the skinny kernel for up to 16 rows, the medium one
     (K split over workgroups) for up to 64, the tiled ones beyond (large tiles where they fill the
     chip, K cut into slices where even the small tiles are too few)."""
     M, K = a.shape
     if SKINNY_MAX_ROWS < M <= MEDIUM_MAX_ROWS or (M <= SKINNY_MAX_ROWS and w.numel() >= MEDIUM_LARGE and K % 8 == 0):
         # also a few rows of a large W (a vocabulary's head: 65,536 x 2,048 at 8 rows 52 against 61 us)
-        gemm_medium_into(a, w, bias, target, out_code, mode, N)
+        gemm_medium_into(a, w, bias, target, out_code, mode, N, w_tiled=w_tiled)
         return
     if M <= SKINNY_MAX_ROWS:
         entry = library().fw_gemm_skinny
@@ -572,9 +573,34 @@ def prepare_device(device: torch.device) -> None:
     _medium_counters(torch.device(device), 0)
 
 
+def tile_weights(w: torch.Tensor) -> Optional[torch.Tensor]:
+    """``w`` [rows, K] bfloat16 once more in operand tiles, [ceil(rows / 16), K / 32, 4, 16, 8]: what the
+    decode products read as whole contiguous kilobytes per wave (see fw_gemm_decode). None where the
+    layout does not apply (K no multiple of 32, another dtype)."""
+    if w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] % 32 or not w.is_cuda:
+        return None
+    rows, K = w.shape
+    padded = (rows + 15) // 16 * 16
+    if padded != rows:
+        w = torch.cat([w, torch.zeros((padded - rows, K), dtype=w.dtype, device=w.device)])
+    return w.view(padded // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous()
+
+
+def _tiled_for(w: torch.Tensor, w_tiled: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    """``w_tiled`` if it is ``w`` in operand tiles (checked by its shape), else an error."""
+    if w_tiled is None:
+        return None
+    rows, K = w.shape
+    if (w_tiled.dtype != torch.bfloat16 or K % 32 or tuple(w_tiled.shape) != ((rows + 15) // 16, K // 32, 4, 16, 8)
+            or not w_tiled.is_contiguous() or w_tiled.device != w.device):
+        raise KernelError(f"weights in operand tiles for w {tuple(w.shape)} are bfloat16 [{(rows + 15) // 16}, {K // 32}, 4, 16, 8], "
+                          f"found {tuple(w_tiled.shape)}")
+    return w_tiled
+
+
 def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tensor, out_code: int, mode: int, N: int,
                      next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False,
-                     squares: Optional[torch.Tensor] = None, eps: float = 0.0):
+                     squares: Optional[torch.Tensor] = None, eps: float = 0.0, w_tiled: Optional[torch.Tensor] = None):
     """The product for 1..64 rows with K split over workgroups (fw_gemm_medium). With
     ``squares`` ``a`` holds prepared activations (x * w of an RMS norm) and the rows' 1/rms is
     formed from those sums. With ``next_norm_weight`` (accumulating product) returns what the
@@ -594,7 +620,8 @@ def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tenso
     if squares is not None and (squares.dtype != torch.float32 or squares.dim() != 2 or squares.shape[1] != stride
                                 or not squares.is_contiguous()):
         raise KernelError(f"gemm_medium: sums of squares for {M} rows are float32 [n, {stride}]")
-    _check(library().fw_gemm_medium(_p(a), _p(w), _p(bias), _p(target), out_code, mode, M, N, K, _p(workspace),
+    w_tiled = _tiled_for(w, w_tiled)
+    _check(library().fw_gemm_medium(_p(a), _p(w if w_tiled is None else w_tiled), int(w_tiled is not None), _p(bias), _p(target), out_code, mode, M, N, K, _p(workspace),
                                     ctypes.c_size_t(need_bytes.value), _p(counters),
                                     0 if counters is None else counters.numel(), _p(next_norm_weight),
                                     int(next_one_centered), _p(next_activations), _p(next_squares), _p(squares),
@@ -607,7 +634,8 @@ def gemm_medium_into(a: torch.Tensor, w: torch.Tensor, bias, target: torch.Tenso
 def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, accumulate_into: Optional[torch.Tensor] = None,
                 squares: Optional[torch.Tensor] = None, eps: float = 0.0,
-                next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False):
+                next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False,
+                w_tiled: Optional[torch.Tensor] = None):
     """The medium product with the fused decode product's conventions (EPILOGUE_STORE /
     ACCUMULATE / SWIGLU): returns the output, or for an accumulation with ``next_norm_weight``
     what the norm after it needs."""
@@ -628,11 +656,11 @@ def gemm_medium(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
         _want(accumulate_into, torch.float32, "accumulate_into")
         if accumulate_into.shape != (M, N):
             raise KernelError(f"gemm_medium: destination is {tuple(accumulate_into.shape)}, expected {(M, N)}")
-        left = gemm_medium_into(a, w, bias, accumulate_into, F32, 1, N, next_norm_weight, next_one_centered, squares, eps)
+        left = gemm_medium_into(a, w, bias, accumulate_into, F32, 1, N, next_norm_weight, next_one_centered, squares, eps, w_tiled=w_tiled)
         return accumulate_into if left is None else left
     out_dtype = torch.bfloat16 if epilogue == EPILOGUE_SWIGLU else (out_dtype or torch.bfloat16)
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    gemm_medium_into(a, w, bias, out, _code(out_dtype), epilogue, N, squares=squares, eps=eps)
+    gemm_medium_into(a, w, bias, out, _code(out_dtype), epilogue, N, squares=squares, eps=eps, w_tiled=w_tiled)
     return out
 
 
@@ -666,9 +694,11 @@ def _fast_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 # ---- dispatch: which kernel serves a call ------------------------------------------------
 def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
-         out_dtype: Optional[torch.dtype] = None, accumulate_into: Optional[torch.Tensor] = None) -> torch.Tensor:
+         out_dtype: Optional[torch.dtype] = None, accumulate_into: Optional[torch.Tensor] = None,
+         w_tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a [M, K] . w [N, K]^T (+ bias): bfloat16 operands go to the matrix-core kernels,
-    everything else (float32, mixed) to the generic float32 one."""
+    everything else (float32, mixed) to the generic float32 one. ``w_tiled``: ``w`` once more in
+    operand tiles (``tile_weights``), for the kernels of few rows that read it so."""
     if not _fast_ok(a, w):
         return gemm_generic(a, w, bias, out_dtype=out_dtype, accumulate_into=accumulate_into)
     _dev(a, w, bias, accumulate_into)
@@ -682,15 +712,15 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
         _want(accumulate_into, torch.float32, "accumulate_into")
         if accumulate_into.shape != (M, N):
             raise KernelError(f"gemm: destination is {tuple(accumulate_into.shape)}, expected {(M, N)}")
-        _fast_gemm(a, w, bias, accumulate_into, F32, 1, N)
+        _fast_gemm(a, w, bias, accumulate_into, F32, 1, N, w_tiled)
         return accumulate_into
     out_dtype = out_dtype or a.dtype
     out = torch.empty((M, N), dtype=out_dtype, device=a.device)
-    _fast_gemm(a, w, bias, out, _code(out_dtype), 0, N)
+    _fast_gemm(a, w, bias, out, _code(out_dtype), 0, N, w_tiled)
     return out
 
 
-def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor, w_tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """silu(a . gate^T) * (a . up^T) with w_gate_up = [gate rows; up rows]: [M, I] in a's dtype.
     On the bfloat16 path the activation is formed from the float32 sums inside the product's
     kernel; otherwise the [M, 2I] intermediate is float32 and a second kernel forms it."""
@@ -702,7 +732,7 @@ def gemm_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
         if a.shape[1] != K:
             raise KernelError(f"gemm_swiglu: a is {tuple(a.shape)} but w is {tuple(w_gate_up.shape)}")
         out = torch.empty((a.shape[0], rows2 // 2), dtype=torch.bfloat16, device=a.device)
-        _fast_gemm(a, w_gate_up, None, out, BF16, 2, rows2 // 2)
+        _fast_gemm(a, w_gate_up, None, out, BF16, 2, rows2 // 2, w_tiled)
         return out
     return swiglu(gemm_generic(a, w_gate_up, out_dtype=torch.float32), out_dtype=a.dtype)
 
@@ -723,7 +753,8 @@ def gemm_decode(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
                 accumulate_into: Optional[torch.Tensor] = None, taps: Optional[torch.Tensor] = None,
                 conv_bias: Optional[torch.Tensor] = None, state: Optional[torch.Tensor] = None,
                 seg_slot: Optional[torch.Tensor] = None, squares: Optional[torch.Tensor] = None,
-                next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False):
+                next_norm_weight: Optional[torch.Tensor] = None, next_one_centered: bool = False,
+                w_tiled: Optional[torch.Tensor] = None):
     """One kernel for (optional RMS norm of float32 rows) -> product with bfloat16 ``w`` -> epilogue.
     With ``norm_weight`` ``a`` holds float32 rows (gathered through ``row_index`` if given), else
     bfloat16 activations. With ``next_norm_weight`` the accumulating epilogue also leaves what
@@ -777,14 +808,16 @@ def gemm_decode(a: torch.Tensor, w: torch.Tensor, epilogue: int, *, bias: Option
         raise KernelError("gemm_decode: only the accumulating product prepares the next norm, whose weight is float32 [N]")
     if epilogue == EPILOGUE_ACCUMULATE and K >= LONG_K and N <= 4096:
         # few features and a long K: the kernel that splits K over workgroups streams W faster
-        left = gemm_medium_into(a, w, bias, target, F32, 1, N, next_norm_weight, next_one_centered)
+        left = gemm_medium_into(a, w, bias, target, F32, 1, N, next_norm_weight, next_one_centered, w_tiled=w_tiled)
         return target if left is None else left
     if next_norm_weight is not None:
         next_activations = torch.empty((rows, N), dtype=torch.bfloat16, device=a.device)
         next_squares = torch.empty((library().fw_gemm_decode_accumulate_tiles(N), 16), dtype=torch.float32, device=a.device)
     prologue = 1 if normed else (2 if squares is not None else 0)
+    w_tiled = _tiled_for(w, w_tiled)
     _check(library().fw_gemm_decode(
-        prologue, _p(a), _p(norm_weight), _p(row_index), ctypes.c_float(eps), int(one_centered), _p(w), _p(bias),
+        prologue, _p(a), _p(norm_weight), _p(row_index), ctypes.c_float(eps), int(one_centered),
+        _p(w if w_tiled is None else w_tiled), int(w_tiled is not None), _p(bias),
         _p(target), _code(out_dtype), int(epilogue), rows, N, K, _p(taps), _p(conv_bias), _p(state), _p(seg_slot),
         int(kernel_size), _p(next_norm_weight), int(next_one_centered), _p(next_activations), _p(next_squares),
         _p(squares), 0 if squares is None else squares.shape[0], _stream()))

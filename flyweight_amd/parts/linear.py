@@ -31,6 +31,10 @@ class Linear:
         self.weight = weight.contiguous()
         self.bias = bias
         self.out_features, self.in_features = weight.shape
+        # The weight once more in the order in which the kernels of few rows load it (whole contiguous
+        # kilobytes per wave: a decode step is bound by how fast the weights stream); the prompt kernels
+        # read the row-major one. None where that layout does not apply.
+        self.tiled = ops.tile_weights(self.weight)
 
     # ----- which path ---------------------------------------------------------------------
     def _fused(self, a: Input, features: int, epilogue: int) -> bool:
@@ -91,11 +95,11 @@ class Linear:
         out_dtype = out_dtype or a.dtype
         if self._medium(a):
             return ops.gemm_medium(self._rows_of(a), self.weight, ops.EPILOGUE_STORE, bias=self.bias, out_dtype=out_dtype,
-                                   **self._prepared_arguments(a))
+                                   w_tiled=self.tiled, **self._prepared_arguments(a))
         if self._fused(a, self.out_features, ops.EPILOGUE_STORE):
             return ops.gemm_decode(self._rows_of(a), self.weight, ops.EPILOGUE_STORE, bias=self.bias, out_dtype=out_dtype,
-                                   **self._norm_arguments(a))
-        return ops.gemm(self._tensor_of(a), self.weight, self.bias, out_dtype=out_dtype)
+                                   w_tiled=self.tiled, **self._norm_arguments(a))
+        return ops.gemm(self._tensor_of(a), self.weight, self.bias, out_dtype=out_dtype, w_tiled=self.tiled)
 
     def accumulate(self, a: torch.Tensor, residual: torch.Tensor, then=None) -> Optional[Prepared]:
         """residual += a . W^T. ``then`` names the norm that will read the residual next, if the
@@ -108,29 +112,29 @@ class Linear:
             if parameters is not None:
                 activations, squares = ops.gemm_medium(a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias,
                                                        accumulate_into=residual, next_norm_weight=parameters[0],
-                                                       next_one_centered=parameters[2])
+                                                       next_one_centered=parameters[2], w_tiled=self.tiled)
                 return Prepared(then, activations, squares)
-            ops.gemm_medium(a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias, accumulate_into=residual)
+            ops.gemm_medium(a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias, accumulate_into=residual, w_tiled=self.tiled)
             return None
         if self._fused(a, self.out_features, ops.EPILOGUE_ACCUMULATE):
             if parameters is not None:
                 activations, squares = ops.gemm_decode(
                     a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias, accumulate_into=residual,
-                    next_norm_weight=parameters[0], next_one_centered=parameters[2])
+                    next_norm_weight=parameters[0], next_one_centered=parameters[2], w_tiled=self.tiled)
                 return Prepared(then, activations, squares)
-            ops.gemm_decode(a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias, accumulate_into=residual)
+            ops.gemm_decode(a, self.weight, ops.EPILOGUE_ACCUMULATE, bias=self.bias, accumulate_into=residual, w_tiled=self.tiled)
             return None
-        ops.gemm(a, self.weight, self.bias, accumulate_into=residual)
+        ops.gemm(a, self.weight, self.bias, accumulate_into=residual, w_tiled=self.tiled)
         return None
 
     def swiglu(self, a: Input) -> torch.Tensor:
         """The weight holds gate rows then up rows: silu(a . gate^T) * (a . up^T)."""
         if self.bias is None and self._medium(a):
-            return ops.gemm_medium(self._rows_of(a), self.weight, ops.EPILOGUE_SWIGLU, **self._prepared_arguments(a))
+            return ops.gemm_medium(self._rows_of(a), self.weight, ops.EPILOGUE_SWIGLU, w_tiled=self.tiled, **self._prepared_arguments(a))
         if self.bias is None and self._fused(a, self.out_features // 2, ops.EPILOGUE_SWIGLU):
             return ops.gemm_decode(self._rows_of(a), self.weight, ops.EPILOGUE_SWIGLU, out_dtype=torch.bfloat16,
-                                   **self._norm_arguments(a))
-        return ops.gemm_swiglu(self._tensor_of(a), self.weight)
+                                   w_tiled=self.tiled, **self._norm_arguments(a))
+        return ops.gemm_swiglu(self._tensor_of(a), self.weight, w_tiled=self.tiled)
 
     def short_conv_decode(self, a: Input, taps: torch.Tensor, conv_bias: Optional[torch.Tensor], state: torch.Tensor,
                           seg_slot: torch.Tensor, out_dtype: torch.dtype) -> Optional[torch.Tensor]:
@@ -142,4 +146,5 @@ class Linear:
         if not self._fused(a, self.out_features // 3, ops.EPILOGUE_CONV):
             return None
         return ops.gemm_decode(self._rows_of(a), self.weight, ops.EPILOGUE_CONV, bias=self.bias, out_dtype=out_dtype,
-                               taps=taps, conv_bias=conv_bias, state=state, seg_slot=seg_slot, **self._norm_arguments(a))
+                               taps=taps, conv_bias=conv_bias, state=state, seg_slot=seg_slot, w_tiled=self.tiled,
+                               **self._norm_arguments(a))

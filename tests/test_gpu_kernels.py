@@ -968,3 +968,64 @@ def test_fused_decode_product_limits(ops):
     residual = torch.zeros(16, 136, device=DEV)
     ops.gemm_decode(a, w, ops.EPILOGUE_ACCUMULATE, accumulate_into=residual)
     close(residual, back(a) @ back(w).T, torch.float32, 2.0)
+
+
+# ----- weights in operand tiles ---------------------------------------------------------------------
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("N,K", [(72, 64), (200, 96), (1000, 544), (4096, 512), (16400, 256), (2048, 4096), (40, 8192)])
+def test_weights_in_operand_tiles_change_no_bit_of_the_products_of_few_rows(ops, M, N, K):
+    """The decode products read W either row-major or once more in tiles of 16 rows x 32 columns
+    laid out as a wave loads them (``ops.tile_weights``): the same numbers from other addresses, so
+    every epilogue gives bit for bit what it gives from the row-major matrix. Feature counts that
+    are no multiple of 16 (the tiles' rows are padded with zeros), narrow and wide outputs, a K
+    long enough for the product that cuts it over workgroups, gate|up and B|C|x operands."""
+    g = torch.Generator().manual_seed(N + K + M)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    bias = torch.randn(N, generator=g).float().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(DEV)
+    tiled = ops.tile_weights(w)
+    assert tiled.shape == ((N + 15) // 16, K // 32, 4, 16, 8)
+    # tile (i, j) holds rows 16 i .., columns 32 j .., a lane's eight columns together
+    i, j, r, c = (N - 1) // 16, K // 32 - 1, (N - 1) % 16, 19
+    assert tiled[i, j, c // 8, r, c % 8] == w[N - 1, 32 * j + c]
+    assert ops.tile_weights(torch.zeros(8, 40, dtype=torch.bfloat16, device=DEV)) is None       # K no multiple of 32
+    assert ops.tile_weights(w.float()) is None
+    product = ops.gemm_decode if M <= 16 else ops.gemm_medium
+    residual = torch.randn(M, N, generator=g).float().to(DEV)
+    for epilogue, kwargs in ((ops.EPILOGUE_STORE, dict(bias=bias, out_dtype=torch.float32)),
+                             (ops.EPILOGUE_STORE, dict(out_dtype=torch.bfloat16)),
+                             (ops.EPILOGUE_ACCUMULATE, dict(bias=bias))):
+        results = []
+        for layout in (None, tiled):
+            if epilogue == ops.EPILOGUE_ACCUMULATE:
+                kwargs["accumulate_into"] = residual.clone()
+            results.append(product(a, w, epilogue, w_tiled=layout, **kwargs))
+        assert torch.equal(results[0], results[1]), f"epilogue {epilogue} {kwargs.get('out_dtype')}"
+    # with the next norm prepared, and taken by a product on tiles again
+    norm_w = (1 + 0.1 * torch.randn(N, generator=g)).float().to(DEV)
+    prepared = [product(a, w, ops.EPILOGUE_ACCUMULATE, accumulate_into=residual.clone(), next_norm_weight=norm_w, w_tiled=layout)
+                for layout in (None, tiled)]
+    # (the sums of squares hold a column per row of a; columns behind the last row are not specified)
+    assert torch.equal(prepared[0][0], prepared[1][0]) and torch.equal(prepared[0][1][:, :M], prepared[1][1][:, :M])
+    if N % 32 == 0:
+        w_next = (torch.randn(96, N, generator=g) / math.sqrt(N)).to(torch.bfloat16).to(DEV)
+        taken = [product(prepared[0][0], w_next, ops.EPILOGUE_STORE, squares=prepared[0][1], eps=1e-5, out_dtype=torch.float32, w_tiled=layout)
+                 for layout in (None, ops.tile_weights(w_next))]
+        assert torch.equal(taken[0], taken[1])
+    # gate | up, and B | C | x with the convolution behind them (up to 16 rows)
+    if N % 2 == 0:
+        gated = [product(a, w, ops.EPILOGUE_SWIGLU, w_tiled=layout) for layout in (None, tiled)]
+        assert torch.equal(gated[0], gated[1])
+    if N % 3 == 0 and M <= 16:
+        H = N // 3
+        taps = (torch.randn(H, 3, generator=g) * 0.5).float().to(DEV)
+        state = torch.randn(M + 2, H, 2, generator=g).float().to(DEV)
+        slots = torch.randperm(M + 2, generator=g)[:M].to(torch.int32).to(DEV)
+        outs, states = [], []
+        for layout in (None, tiled):
+            mine = state.clone()
+            outs.append(ops.gemm_decode(a, w, ops.EPILOGUE_CONV, taps=taps, state=mine, seg_slot=slots, out_dtype=torch.bfloat16, w_tiled=layout))
+            states.append(mine)
+        assert torch.equal(outs[0], outs[1]) and torch.equal(states[0], states[1])
+    with pytest.raises(ops.KernelError, match="operand tiles"):
+        product(a, w, ops.EPILOGUE_STORE, w_tiled=tiled[:-1].contiguous() if tiled.shape[0] > 1 else tiled.reshape(-1))
