@@ -43,7 +43,7 @@ class Linear:
         rows = a.rows if isinstance(a, LazyNorm) else a.shape[0]
         if not 1 <= rows <= ops.DECODE_MAX_ROWS:
             return False
-        if isinstance(a, LazyNorm) and (a.rms_parameters() is None or features >= self.WIDE):
+        if isinstance(a, LazyNorm) and (a.rms_parameters() is None or (features >= self.WIDE and a.prepared is None)):
             return False        # very wide outputs (a vocabulary): norming once beats norming in every workgroup
         return ops.gemm_decode_fits(rows, features, self.in_features, epilogue)
 
@@ -67,10 +67,16 @@ class Linear:
         return a.tensor() if isinstance(a, LazyNorm) else a
 
     # From this many weights on the product that splits K over workgroups also serves a few rows: its
-    # workgroups walk K from different chunks on, and a large W then streams faster than through the
-    # fused decode product (16,384 x 2,048 with SwiGLU at 8 rows: 17.6 against 19.1 us; equal at one row).
+    # workgroups walk K from different chunks on, and a large W in row-major order then streams faster
+    # than through the fused decode product (16,384 x 2,048 with SwiGLU at 8 rows: 17.6 against 19.1 us;
+    # equal at one row). From operand tiles the fused product streams faster than either (gate|up at 8
+    # rows 12.9 against 14.9 us, a vocabulary of 65,536 45.3 against 49.5 us); only the widest outputs
+    # go to the split-K product, from nine rows on, where every workgroup's own read of all of a
+    # begins to weigh (the vocabulary at 16 rows: 50.4 against 52.2 us).
     LARGE = 1 << 25
     LARGE_MIN_ROWS = 3
+    LARGE_TILED = 1 << 26
+    LARGE_TILED_MIN_ROWS = 9
 
     def _medium(self, a: Input) -> bool:
         """17..64 rows of a bfloat16 model, and fewer rows of a large weight: the product that splits
@@ -79,7 +85,10 @@ class Linear:
         if self.weight.dtype != torch.bfloat16 or a.dtype != torch.bfloat16 or self.in_features % 8:
             return False
         rows = a.rows if isinstance(a, LazyNorm) else a.shape[0]
-        few = self.LARGE_MIN_ROWS <= rows <= ops.DECODE_MAX_ROWS and self.weight.numel() >= self.LARGE
+        if self.tiled is None:
+            few = self.LARGE_MIN_ROWS <= rows <= ops.DECODE_MAX_ROWS and self.weight.numel() >= self.LARGE
+        else:
+            few = self.LARGE_TILED_MIN_ROWS <= rows <= ops.DECODE_MAX_ROWS and self.weight.numel() >= self.LARGE_TILED
         if not (few or ops.DECODE_MAX_ROWS < rows <= ops.MEDIUM_MAX_ROWS):
             return False
         return not isinstance(a, LazyNorm) or a.prepared is not None

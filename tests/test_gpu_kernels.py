@@ -973,12 +973,15 @@ def test_fused_decode_product_limits(ops):
 # ----- weights in operand tiles ---------------------------------------------------------------------
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 40, 64])
 @pytest.mark.parametrize("N,K", [(72, 64), (200, 96), (1000, 544), (4096, 512), (16400, 256), (2048, 4096), (40, 8192)])
-def test_weights_in_operand_tiles_change_no_bit_of_the_products_of_few_rows(ops, M, N, K):
+def test_weights_in_operand_tiles_change_no_bit_of_the_products_of_few_rows(ops, monkeypatch, M, N, K):
     """The decode products read W either row-major or once more in tiles of 16 rows x 32 columns
     laid out as a wave loads them (``ops.tile_weights``): the same numbers from other addresses, so
     every epilogue gives bit for bit what it gives from the row-major matrix. Feature counts that
     are no multiple of 16 (the tiles' rows are padded with zeros), narrow and wide outputs, a K
     long enough for the product that cuts it over workgroups, gate|up and B|C|x operands."""
+    # (which kernel adds a long K into few features depends on the layout, and two kernels sum in two
+    # orders: here both layouts go to the fused product, whatever the rows)
+    monkeypatch.setattr(ops, "LONG_K", 1 << 30)
     g = torch.Generator().manual_seed(N + K + M)
     a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
     bias = torch.randn(N, generator=g).float().to(DEV)
