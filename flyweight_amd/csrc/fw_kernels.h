@@ -191,8 +191,9 @@ int fw_argmax_rows_static_max_rows(void);
 // The next token of every row, drawn on the device: settings float32 [rows][4] = temperature (0:
 // greedy, the best candidate, ties to the lowest id), top_k (0: all candidates), top_p, min_p;
 // states [rows]: the rows' xorshift64* generators, moved on by the rows that draw. also / advance
-// as in fw_argmax_rows. Candidates are taken in (value descending, id ascending) order and the
-// sums are float64, in that order.
+// as in fw_argmax_rows. Candidates are taken in (value descending, id ascending) order; the sums of
+// a list of up to 1,024 candidates are float64, in that order, those of a longer one whole numbers
+// (parts in 2^-46 fixed point at 65,536 logits).
 int fw_sample_rows(const float* logits, const float* settings, unsigned long long* states, int32_t* ids, int32_t* also,
                    int32_t* advance, int rows, int vocab, void* stream);
 

@@ -99,6 +99,22 @@ def test_sampler_draws_the_reference_samplers_tokens(ops, ref):
     got = ops.sample_rows(torch.tensor(logits, device=DEV), torch.tensor(settings, device=DEV), device_states)
     assert got.cpu().tolist() == want_ids.tolist() and got.cpu().tolist()[0] == int(logits[0].argmax())
     assert np.array_equal(device_states.cpu().numpy().view(np.uint64), want_states) and want_states[0] == states[0]
+    # flat rows over the whole vocabulary (no top_k): the list is searched, not walked
+    # (where min_p alone ends the list; a row of one value and a row of two, which no bin of the value divides)
+    flat = (RNG.normal(size=(8, 65536)) * 0.02).astype(np.float32)
+    flat[5, :] = 1.5
+    flat[6, :] = np.where(RNG.random(65536) < 0.5, 0.25, -0.25)
+    flat[7, 30000:] = -np.inf
+    flat_settings = np.array([[0.8, 0, 1, 0], [0.8, 0, 0.9, 0], [1.0, 0, 0.95, 0.05], [0.7, 5000, 0.9, 0.5], [1.0, 0, 1.0, 0.9],
+                              [0.8, 0, 0.9, 0], [1.0, 0, 0.7, 0.5], [0.9, 40000, 0.99, 0]], dtype=np.float32)
+    flat_states = np.arange(11, 19, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15)
+    for draw in range(4):
+        want_ids, want_states = ref.sample_rows(flat, flat_settings, flat_states)
+        device_states = torch.tensor(flat_states.view(np.int64), device=DEV)
+        got = ops.sample_rows(torch.tensor(flat, device=DEV), torch.tensor(flat_settings, device=DEV), device_states)
+        assert got.cpu().tolist() == want_ids.tolist()
+        assert np.array_equal(device_states.cpu().numpy().view(np.uint64), want_states)
+        flat_states = want_states
 
 
 # rows that pick every product kernel: the fused decode product (<= 16), the split-K one (17..64),
