@@ -115,6 +115,17 @@ def test_sampler_draws_the_reference_samplers_tokens(ops, ref):
         assert got.cpu().tolist() == want_ids.tolist()
         assert np.array_equal(device_states.cpu().numpy().view(np.uint64), want_states)
         flat_states = want_states
+    # a larger vocabulary that is no multiple of four (rows read element by element, a coarser fixed point)
+    wide = (RNG.normal(size=(4, 150001)) * 2).astype(np.float32)
+    wide_settings = np.array([[1.0, 0, 1, 0], [0.9, 0, 0.8, 0], [1.2, 20000, 0.95, 0.001], [0.6, 0, 0.99, 0.02]], dtype=np.float32)
+    wide_states = np.arange(21, 25, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15)
+    for draw in range(3):
+        want_ids, want_states = ref.sample_rows(wide, wide_settings, wide_states)
+        device_states = torch.tensor(wide_states.view(np.int64), device=DEV)
+        got = ops.sample_rows(torch.tensor(wide, device=DEV), torch.tensor(wide_settings, device=DEV), device_states)
+        assert got.cpu().tolist() == want_ids.tolist()
+        assert np.array_equal(device_states.cpu().numpy().view(np.uint64), want_states)
+        wide_states = want_states
 
 
 # rows that pick every product kernel: the fused decode product (<= 16), the split-K one (17..64),
