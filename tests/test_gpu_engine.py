@@ -415,6 +415,37 @@ def test_drawn_tokens_come_from_recorded_steps_and_turns_like_the_most_likely_on
             assert tokens == want
 
 
+def test_draws_over_a_whole_vocabulary_beyond_a_batch_of_candidates(tmp_path):
+    """A vocabulary of 3,001 drawn from without top_k (and with one above 1,024): the sampler's path for
+    long lists, through recorded decode steps, one step or four per turn; the plain sampler's tokens
+    given the plain model's logits, in float32."""
+    from flyweight_amd.config import config_from_dict
+    from flyweight_amd.weights import write_random_model
+    from gpu_common import Loaded
+    from helpers import TINY_A
+    folder = write_random_model(str(tmp_path / "wide"), config_from_dict(dict(TINY_A, vocab_size=3001)), 5, scale="fan_in")
+    m = Loaded(folder, "float32")
+    prompts = [random_tokens(3001, n, seed=90 + n) for n in (7, 20, 3)]
+    settings = [dict(temperature=1.0, top_k=0, top_p=1.0, min_p=0.0, seed=21), dict(temperature=0.9, top_k=0, top_p=0.8, min_p=0.0005, seed=22),
+                dict(temperature=1.4, top_k=2000, top_p=0.95, min_p=0.0, seed=23)]
+    results = []
+    for steps_per_turn in (1, 4):
+        runtime = _runtime(m, parallel_sequences=4, prefill_rows=64, max_batch_tokens=128, decode_steps_per_turn=steps_per_turn)
+        ids = [runtime.task_submit(p, 14, **kw) for p, kw in zip(prompts, settings)]
+        finished = runtime.run()
+        results.append([finished[task] for task in ids])
+        assert runtime.stepper.graph_replays > 8
+    assert results[0] == results[1]
+    for prompt, kw, tokens in zip(prompts, settings, results[0]):
+        rng = plain.XorShift64Star(kw["seed"])
+        context, want = list(prompt), []
+        for _ in range(14):
+            logits = plain.forward(m.plain_config, m.plain_weights, context)[-1]
+            want.append(plain.sample(logits.astype(np.float32), kw["temperature"], kw["top_k"], kw["top_p"], kw["min_p"], rng))
+            context.append(want[-1])
+        assert tokens == want
+
+
 def test_errors_are_reported_not_hidden(loaded):
     from flyweight_amd.engine import EngineError, StepEntry, StepError
     from flyweight_amd.cache import OutOfPages
