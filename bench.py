@@ -297,7 +297,8 @@ def further_points(torch, args, points: dict) -> None:
     from flyweight_amd.config import config_from_dict
     config = config_from_dict(dict(SHAPE, max_position_embeddings=128000))
     model = Model.random(config, seed=0, dtype="bfloat16")
-    for batch, steps in ((8, min(args.steps, 64)), (64, min(args.steps, 32)), (128, min(args.steps, 32)), (256, min(args.steps, 32))):
+    # (at least 64 and 32 steps: a run of a few turns right behind a model's creation times that as well)
+    for batch, steps in ((8, max(args.steps, 64)), (64, max(args.steps, 32)), (128, max(args.steps, 32)), (256, max(args.steps, 32))):
         name = f"decode_b{batch}" + ("_maxpos128k" if batch <= 64 else "")
         log(f"decode at batch {batch}, max_position_embeddings 128,000, context {CONTEXT}")
         seconds, _, step_bytes = decode_run(torch, model, config, batch, steps, min(args.warmup, 8))
