@@ -113,6 +113,28 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_rows_kernel(
     const float w = (weight && active) ? weight[lane] : 1.0f;
 #pragma unroll
     for (int i = 0; i < QK_ROWS; ++i) page[i] = block_table[(size_t)page[i] * table_stride + pos[i] / ATTN_PAGE];
+    if (is_value && sizeof(T) == 2) {
+        // Eight rows that follow each other in one page, the first at a slot that is a multiple of eight (a
+        // prompt portion that begins at such a position): a channel's eight values are 16 bytes side by side
+        // in the transposed page and leave as one store instead of eight of 2 bytes.
+        bool together = r0 + QK_ROWS <= rows && pos[0] % 8 == 0;
+#pragma unroll
+        for (int i = 1; i < QK_ROWS; ++i) together = together && page[i] == page[0] && pos[i] == pos[0] + i;
+        if (together) {
+            const int kvh = vec - num_heads - num_kv_heads;
+            T* dest = v_pages + ((size_t)page[0] * num_kv_heads + kvh) * head_dim * ATTN_PAGE;
+            uint32_t packed[QK_ROWS / 2];
+#pragma unroll
+            for (int i = 0; i < QK_ROWS / 2; ++i)
+                packed[i] = (uint32_t)float_to_bf16_bits(v[2 * i]) | ((uint32_t)float_to_bf16_bits(v[2 * i + 1]) << 16);
+            if (active) {
+                uint32_t* to = reinterpret_cast<uint32_t*>(dest + (size_t)lane * ATTN_PAGE + pos[0] % ATTN_PAGE);
+                typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+                *reinterpret_cast<u32x4_t*>(to) = u32x4_t{packed[0], packed[1], packed[2], packed[3]};
+            }
+            return;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < QK_ROWS; ++i) {
         if (r0 + i >= rows) break;

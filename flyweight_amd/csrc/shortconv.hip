@@ -56,7 +56,10 @@ __global__ void shortconv_rows_kernel(const T* __restrict__ bcx, TO* __restrict_
 // taps sits at place j + 4 - L; the places in front are skipped. Sums in the order of the taps, as above.
 #define CONV_TILE_ROWS 8
 #define CONV_TILE_HISTORY 3
-template <typename T, typename TO>
+// C: channels side by side per thread (2: loads and stores of twice the width, where the model's width is
+// even and the input float32: 2,048 rows of 2,048 channels 19.4 -> 16.2 us; with 4, 19.2 us; a channel's
+// arithmetic is the same either way).
+template <typename T, typename TO, int C>
 __global__ __launch_bounds__(256) void shortconv_rows8_kernel(const T* __restrict__ bcx, TO* __restrict__ out,
                                                               const float* __restrict__ taps, const float* __restrict__ conv_bias,
                                                               const float* __restrict__ state, const int32_t* __restrict__ row_seg,
@@ -64,7 +67,7 @@ __global__ __launch_bounds__(256) void shortconv_rows8_kernel(const T* __restric
                                                               int rows, int hidden, int kernel_size) {
     constexpr int R = CONV_TILE_ROWS, H = CONV_TILE_HISTORY;
     const int r0 = blockIdx.y * R;
-    const int channel = blockIdx.x * blockDim.x + threadIdx.x;
+    const int channel = (blockIdx.x * blockDim.x + threadIdx.x) * C;
     if (channel >= hidden) return;
     const int history = kernel_size - 1, unused = H - history;      // places of the window in front of tap 0
     // every row's segment and place in it, asked for together and first (two dependent loads each)
@@ -73,39 +76,68 @@ __global__ __launch_bounds__(256) void shortconv_rows8_kernel(const T* __restric
     for (int i = 0; i < R; ++i) seg_of[i] = row_seg[r0 + i < rows ? r0 + i : rows - 1];
 #pragma unroll
     for (int i = 0; i < R; ++i) offset_of[i] = r0 + i - seg_row0[seg_of[i]];
+    // C values that lie side by side, as one load
+    const auto load_run = [&](const T* from, float (&values)[C]) {
+        if (C == 2 && sizeof(T) == 4) {
+            const float2 pair = *reinterpret_cast<const float2*>(from);
+            values[0] = pair.x;
+            values[C - 1] = pair.y;
+        } else {
+#pragma unroll
+            for (int c = 0; c < C; ++c) values[c] = load_as_float(from, c);
+        }
+    };
     // the products of rows r0 - 3 .. r0 + 7 (0 where that is no row of this step)
-    float product[R + H];
+    float product[R + H][C], gate[R][C];
 #pragma unroll
     for (int p = 0; p < R + H; ++p) {
         const int row = r0 - H + p;
         const bool valid = row >= 0 && row < rows;
         const T* source = bcx + (size_t)(valid ? row : 0) * 3 * hidden;
-        const float value = load_as_float(source, channel) * load_as_float(source, 2 * (size_t)hidden + channel);
-        product[p] = valid ? value : 0.0f;
-    }
-    float tap[H + 1];
+        float b[C], x[C];
+        load_run(source + channel, b);
+        load_run(source + 2 * (size_t)hidden + channel, x);
 #pragma unroll
-    for (int place = 0; place <= H; ++place)
-        tap[place] = place >= unused ? taps[(size_t)channel * kernel_size + (place - unused)] : 0.0f;
-    const float bias = conv_bias ? conv_bias[channel] : 0.0f;
+        for (int c = 0; c < C; ++c) product[p][c] = valid ? b[c] * x[c] : 0.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < R; ++i) load_run(bcx + (size_t)(r0 + i < rows ? r0 + i : rows - 1) * 3 * hidden + hidden + channel, gate[i]);
+    float tap[H + 1][C], bias[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+#pragma unroll
+        for (int place = 0; place <= H; ++place)
+            tap[place][c] = place >= unused ? taps[(size_t)(channel + c) * kernel_size + (place - unused)] : 0.0f;
+        bias[c] = conv_bias ? conv_bias[channel + c] : 0.0f;
+    }
 #pragma unroll
     for (int i = 0; i < R; ++i) {
         const int row = r0 + i;
         if (row >= rows) break;
         const int seg = seg_of[i], offset_in_segment = offset_of[i];
-        float y = 0.0f;
+        float result[C];
 #pragma unroll
-        for (int place = 0; place <= H; ++place) {
-            if (place < unused) continue;       // in front of tap 0: not this kernel's (and never multiplied, not even by 0)
-            float value = product[i + place];
-            const int offset = offset_in_segment - H + place;       // where in the segment this place lies
-            if (offset < 0)                                         // in front of the segment: the request's state
-                value = state[((size_t)seg_slot[seg] * hidden + channel) * history + history + offset];
-            y = fmaf(tap[place], value, y);
+        for (int c = 0; c < C; ++c) {
+            float y = 0.0f;
+#pragma unroll
+            for (int place = 0; place <= H; ++place) {
+                if (place < unused) continue;       // in front of tap 0: not this kernel's (and never multiplied, not even by 0)
+                float value = product[i + place][c];
+                const int offset = offset_in_segment - H + place;       // where in the segment this place lies
+                if (offset < 0)                                         // in front of the segment: the request's state
+                    value = state[((size_t)seg_slot[seg] * hidden + channel + c) * history + history + offset];
+                y = fmaf(tap[place][c], value, y);
+            }
+            y += bias[c];
+            result[c] = gate[i][c] * y;
         }
-        y += bias;
-        const float gate = load_as_float(bcx, (size_t)row * 3 * hidden + hidden + channel);
-        store_from_float(out, (size_t)row * hidden + channel, gate * y);
+        if (C == 2 && sizeof(TO) == 2) {
+            const uint32_t packed = (uint32_t)float_to_bf16_bits(result[0]) | ((uint32_t)float_to_bf16_bits(result[C - 1]) << 16);
+            *reinterpret_cast<uint32_t*>(out + (size_t)row * hidden + channel) = packed;
+        } else {
+#pragma unroll
+            for (int c = 0; c < C; ++c) store_from_float(out, (size_t)row * hidden + channel + c, result[c]);
+        }
     }
 }
 
@@ -161,10 +193,14 @@ static void launch(const void* bcx, void* out, const float* taps, const float* c
             (const T*)bcx, (TO*)out, taps, conv_bias, state, seg_slot, hidden, kernel_size);
         return;
     }
-    if (kernel_size <= CONV_TILE_HISTORY + 1 && rows >= 4 * CONV_TILE_ROWS)
-        shortconv_rows8_kernel<T, TO><<<dim3(bx, fw_ceil_div(rows, CONV_TILE_ROWS)), 256, 0, stream>>>(
-            (const T*)bcx, (TO*)out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, rows, hidden, kernel_size);
-    else
+    if (kernel_size <= CONV_TILE_HISTORY + 1 && rows >= 4 * CONV_TILE_ROWS) {
+        if (hidden % 2 == 0 && sizeof(T) == 4)
+            shortconv_rows8_kernel<T, TO, 2><<<dim3(fw_ceil_div(hidden / 2, 256), fw_ceil_div(rows, CONV_TILE_ROWS)), 256, 0, stream>>>(
+                (const T*)bcx, (TO*)out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, rows, hidden, kernel_size);
+        else
+            shortconv_rows8_kernel<T, TO, 1><<<dim3(bx, fw_ceil_div(rows, CONV_TILE_ROWS)), 256, 0, stream>>>(
+                (const T*)bcx, (TO*)out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, rows, hidden, kernel_size);
+    } else
         shortconv_rows_kernel<T, TO><<<dim3(bx, rows), 256, 0, stream>>>(
             (const T*)bcx, (TO*)out, taps, conv_bias, state, row_seg, seg_row0, seg_slot, hidden, kernel_size);
     shortconv_state_kernel<T><<<dim3(bx, segments), 256, 0, stream>>>(
