@@ -84,14 +84,19 @@ __global__ __launch_bounds__(256) void rmsnorm_rows4_kernel(const float* __restr
     const int row = blockIdx.x;
     const f32x4* source = reinterpret_cast<const f32x4*>(x + (size_t)(row_index ? row_index[row] : row) * hidden);
     const int pieces = hidden / 4;
-    f32x4 held[4];
+    f32x4 held[4], scale[4];
     float sum = 0.0f;
+    // (the weight is asked for with the row, not behind the sum over the block. A wave per row, whose sum needs
+    // neither LDS nor a barrier, was slower: 6.8 against 6.4 us for 2,048 rows of 2,048.)
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const int piece = threadIdx.x + u * 256;
         held[u] = piece < pieces ? source[piece] : f32x4{0.f, 0.f, 0.f, 0.f};
-        sum += (held[u][0] * held[u][0] + held[u][1] * held[u][1]) + (held[u][2] * held[u][2] + held[u][3] * held[u][3]);
+        scale[u] = reinterpret_cast<const f32x4*>(weight)[piece < pieces ? piece : 0];
     }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        sum += (held[u][0] * held[u][0] + held[u][1] * held[u][1]) + (held[u][2] * held[u][2] + held[u][3] * held[u][3]);
     sum = block_sum(sum, scratch);
     const float inv = rsqrtf(sum / (float)hidden + eps);
     const float one = one_centered ? 1.0f : 0.0f;
@@ -99,7 +104,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rows4_kernel(const float* __restr
     for (int u = 0; u < 4; ++u) {
         const int piece = threadIdx.x + u * 256;
         if (piece >= pieces) break;
-        const f32x4 w = reinterpret_cast<const f32x4*>(weight)[piece];
+        const f32x4 w = scale[u];
         f32x4 y;
 #pragma unroll
         for (int e = 0; e < 4; ++e) y[e] = held[u][e] * inv * (w[e] + one);
